@@ -1,0 +1,268 @@
+// C-ABI entry points of the matrix-multiplication engine (declared in
+// include/dragon_hip_gemm.h).  Each one validates its arguments, translates the
+// reference's (N, M, K, ...) argument list into the operand bounds of the one
+// guarded kernel, and launches on streams[0].
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <mutex>
+#include "gemm_mfma.h"
+#include "../../include/dragon_hip_gemm.h"
+
+using namespace dragon;
+
+namespace {
+
+constexpr int MAX_STREAMS = 10;  // the reference copies the handles into jlong streams[10]
+
+inline bool aligned16(int64_t a) { return (a & 15) == 0; }
+inline bool x4(int v) { return (v & 3) == 0; }
+
+int num_compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            n <= 0)
+            n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+int check_common(const int64_t* streams, int length, int64_t dA, int64_t dB, int64_t dC) {
+    if (streams == nullptr || length < 1 || length > MAX_STREAMS) return hipErrorInvalidValue;
+    if (dA == 0 || dB == 0 || dC == 0) return hipErrorInvalidValue;
+    if (!aligned16(dA) || !aligned16(dB) || !aligned16(dC)) return hipErrorInvalidValue;
+    return hipSuccess;
+}
+
+// 2-D products, optionally cut into gz K slices.
+int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t dA, int64_t dB,
+              int64_t dC, int64_t dCbuf, int N, int M, int K) {
+    int e = check_common(streams, length, dA, dB, dC);
+    if (e) return e;
+    if (N <= 0 || M <= 0 || K <= 0 || gz < 1) return hipErrorInvalidValue;
+    if (!x4(N) || !x4(M) || !x4(K)) return hipErrorInvalidValue;
+    if (gz > 1 && (dCbuf == 0 || !aligned16(dCbuf))) return hipErrorInvalidValue;
+    if ((long long)N * M > 0x7fffffffLL) return hipErrorInvalidValue;
+
+    GemmParams p = {};
+    p.A = (const float*)(intptr_t)dA;
+    p.B = (const float*)(intptr_t)dB;
+    p.C = (float*)(intptr_t)dC;
+    p.Cbuf = (float*)(intptr_t)dCbuf;
+    p.rows = N;
+    p.cols = M;
+    p.k_total = K;
+    p.ldc = M;
+    switch (variant) {
+        case GEMM_NN:  // A[N,K], B[K,M]
+            p.lda = K; p.a_outer = N; p.a_inner = K;
+            p.ldb = M; p.b_outer = K; p.b_inner = M;
+            break;
+        case GEMM_T1:  // A[K,N], B[K,M]
+            p.lda = N; p.a_outer = K; p.a_inner = N;
+            p.ldb = M; p.b_outer = K; p.b_inner = M;
+            break;
+        default:       // GEMM_T2: A[N,K], B[M,K]
+            p.lda = K; p.a_outer = N; p.a_inner = K;
+            p.ldb = K; p.b_outer = M; p.b_inner = K;
+            break;
+    }
+    p.nz = gz;
+    if (gz > 1) {
+        // K_slice = (K / GZ) >> 3 << 3   (reference: MM/micro.cuh:92)
+        p.k_slice = ((K / gz) >> 3) << 3;
+        p.sizeC = (long long)N * M;
+        p.split = 1;  // a zero K_slice leaves every slice but the last empty: they write zeros
+    }
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, num_compute_units());
+    return gemm_launch(variant, p, tile, (hipStream_t)(intptr_t)streams[0]);
+}
+
+}  // namespace
+
+extern "C" {
+
+int dragon_Cuda_matMul_matMul(const int64_t* streams, int32_t length, int64_t dA, int64_t dB,
+                              int64_t dC, int32_t N, int32_t M, int32_t K) {
+    return matmul_2d(GEMM_NN, streams, length, 1, dA, dB, dC, 0, N, M, K);
+}
+int dragon_Cuda_matMul_matMulT1(const int64_t* streams, int32_t length, int64_t dA, int64_t dB,
+                                int64_t dC, int32_t N, int32_t M, int32_t K) {
+    return matmul_2d(GEMM_T1, streams, length, 1, dA, dB, dC, 0, N, M, K);
+}
+int dragon_Cuda_matMul_matMulT2(const int64_t* streams, int32_t length, int64_t dA, int64_t dB,
+                                int64_t dC, int32_t N, int32_t M, int32_t K) {
+    return matmul_2d(GEMM_T2, streams, length, 1, dA, dB, dC, 0, N, M, K);
+}
+
+int dragon_Cuda_matMul_matMulSK(const int64_t* streams, int32_t length, int32_t GridZ, int64_t dA,
+                                int64_t dB, int64_t dC, int64_t dCbuf, int32_t N, int32_t M,
+                                int32_t K) {
+    return matmul_2d(GEMM_NN, streams, length, GridZ, dA, dB, dC, dCbuf, N, M, K);
+}
+int dragon_Cuda_matMul_matMulT1SK(const int64_t* streams, int32_t length, int32_t GridZ,
+                                  int64_t dA, int64_t dB, int64_t dC, int64_t dCbuf, int32_t N,
+                                  int32_t M, int32_t K) {
+    return matmul_2d(GEMM_T1, streams, length, GridZ, dA, dB, dC, dCbuf, N, M, K);
+}
+int dragon_Cuda_matMul_matMulT2SK(const int64_t* streams, int32_t length, int32_t GridZ,
+                                  int64_t dA, int64_t dB, int64_t dC, int64_t dCbuf, int32_t N,
+                                  int32_t M, int32_t K) {
+    return matmul_2d(GEMM_T2, streams, length, GridZ, dA, dB, dC, dCbuf, N, M, K);
+}
+
+int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC, int32_t part,
+                                     int32_t sizeC) {
+    if (dC == 0 || sizeC <= 0 || part < 0 || !x4(sizeC) || !aligned16(dC))
+        return hipErrorInvalidValue;
+    if (part > 0 && (dCbuf == 0 || !aligned16(dCbuf))) return hipErrorInvalidValue;
+    if (part == 0) return hipSuccess;
+    return skbuf_summary_launch((hipStream_t)(intptr_t)stream, (const float*)(intptr_t)dCbuf,
+                                (float*)(intptr_t)dC, part, sizeC);
+}
+
+// ---- batched ---------------------------------------------------------------------
+
+int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length, int64_t dA,
+                                        int64_t dB, int64_t dC, int32_t Batch, int32_t N,
+                                        int32_t M, int32_t BK, int32_t AK) {
+    int e = check_common(streams, length, dA, dB, dC);
+    if (e) return e;
+    if (Batch <= 0 || N <= 0 || M <= 0 || BK <= 0 || AK < BK) return hipErrorInvalidValue;
+    if (!x4(M) || !x4(AK)) return hipErrorInvalidValue;
+    GemmParams p = {};
+    p.A = (const float*)(intptr_t)dA;   // A[Batch, N, AK]
+    p.B = (const float*)(intptr_t)dB;   // B[Batch, BK, M]
+    p.C = (float*)(intptr_t)dC;         // C[Batch, N, M]
+    p.rows = N; p.cols = M; p.k_total = AK;
+    p.lda = AK; p.a_outer = N;  p.a_inner = AK;
+    p.ldb = M;  p.b_outer = BK; p.b_inner = M;
+    p.ldc = M;
+    p.sA = (long long)N * AK; p.sB = (long long)BK * M; p.sC = (long long)N * M;
+    p.nz = Batch;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, num_compute_units());
+    return gemm_launch(GEMM_NN, p, tile, (hipStream_t)(intptr_t)streams[0]);
+}
+
+int dragon_Cuda_batchMatMul_batchMatMul_texture(const int64_t* streams, int32_t length,
+                                                int64_t dA, int64_t dB, int64_t dC, int32_t Batch,
+                                                int32_t N, int32_t M, int32_t BK, int32_t AK) {
+    return dragon_Cuda_batchMatMul_batchMatMul(streams, length, dA, dB, dC, Batch, N, M, BK, AK);
+}
+
+int dragon_Cuda_batchMatMul_batchMatMulT1(const int64_t* streams, int32_t length, int64_t dA,
+                                          int64_t dB, int64_t dC, int32_t Batch, int32_t CN,
+                                          int32_t AN, int32_t M, int32_t K) {
+    int e = check_common(streams, length, dA, dB, dC);
+    if (e) return e;
+    if (Batch <= 0 || CN <= 0 || AN < CN || M <= 0 || K <= 0) return hipErrorInvalidValue;
+    if (!x4(AN) || !x4(M)) return hipErrorInvalidValue;
+    GemmParams p = {};
+    p.A = (const float*)(intptr_t)dA;   // A[Batch, K, AN]
+    p.B = (const float*)(intptr_t)dB;   // B[Batch, K, M]
+    p.C = (float*)(intptr_t)dC;         // C[Batch, CN, M]
+    p.rows = CN; p.cols = M; p.k_total = K;
+    p.lda = AN; p.a_outer = K; p.a_inner = AN;
+    p.ldb = M;  p.b_outer = K; p.b_inner = M;
+    p.ldc = M;
+    p.sA = (long long)K * AN; p.sB = (long long)K * M; p.sC = (long long)CN * M;
+    p.nz = Batch;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, num_compute_units());
+    return gemm_launch(GEMM_T1, p, tile, (hipStream_t)(intptr_t)streams[0]);
+}
+
+int dragon_Cuda_batchMatMul_batchMatMulT2(const int64_t* streams, int32_t length, int64_t dA,
+                                          int64_t dB, int64_t dC, int32_t Batch, int32_t N,
+                                          int32_t CM, int32_t BM, int32_t K) {
+    int e = check_common(streams, length, dA, dB, dC);
+    if (e) return e;
+    if (Batch <= 0 || N <= 0 || CM <= 0 || BM <= 0 || BM > CM || K <= 0) return hipErrorInvalidValue;
+    if (!x4(CM) || !x4(K)) return hipErrorInvalidValue;
+    GemmParams p = {};
+    p.A = (const float*)(intptr_t)dA;   // A[Batch, N, K]
+    p.B = (const float*)(intptr_t)dB;   // B[Batch, BM, K]
+    p.C = (float*)(intptr_t)dC;         // C[Batch, N, CM]
+    p.rows = N; p.cols = CM; p.k_total = K;
+    p.lda = K; p.a_outer = N;  p.a_inner = K;
+    p.ldb = K; p.b_outer = BM; p.b_inner = K;
+    p.ldc = CM;
+    p.sA = (long long)N * K; p.sB = (long long)BM * K; p.sC = (long long)N * CM;
+    p.nz = Batch;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, num_compute_units());
+    return gemm_launch(GEMM_T2, p, tile, (hipStream_t)(intptr_t)streams[0]);
+}
+
+int dragon_Cuda_batchMatMul_batchMatMulT2_texture(const int64_t* streams, int32_t length,
+                                                  int64_t dA, int64_t dB, int64_t dC,
+                                                  int32_t Batch, int32_t N, int32_t CM,
+                                                  int32_t BM, int32_t K) {
+    return dragon_Cuda_batchMatMul_batchMatMulT2(streams, length, dA, dB, dC, Batch, N, CM, BM, K);
+}
+
+// ---- *_mma: forward to the FP32 path ---------------------------------------------
+
+int dragon_Cuda_matMul_matMul_mma(const int64_t* streams, int32_t length, int64_t dA, int64_t dB,
+                                  int64_t dC, int32_t N, int32_t M, int32_t K) {
+    return dragon_Cuda_matMul_matMul(streams, length, dA, dB, dC, N, M, K);
+}
+int dragon_Cuda_matMul_matMulT1_mma(const int64_t* streams, int32_t length, int64_t dA,
+                                    int64_t dB, int64_t dC, int32_t N, int32_t M, int32_t K) {
+    return dragon_Cuda_matMul_matMulT1(streams, length, dA, dB, dC, N, M, K);
+}
+int dragon_Cuda_matMul_matMulT2_mma(const int64_t* streams, int32_t length, int64_t dA,
+                                    int64_t dB, int64_t dC, int32_t N, int32_t M, int32_t K) {
+    return dragon_Cuda_matMul_matMulT2(streams, length, dA, dB, dC, N, M, K);
+}
+int dragon_Cuda_batchMatMul_batchMatMul_mma(int32_t, const int64_t* streams, int32_t length,
+                                            int64_t dA, int64_t dB, int64_t dC, int32_t Batch,
+                                            int32_t N, int32_t M, int32_t BK, int32_t AK) {
+    return dragon_Cuda_batchMatMul_batchMatMul(streams, length, dA, dB, dC, Batch, N, M, BK, AK);
+}
+int dragon_Cuda_batchMatMul_batchMatMulT1_mma(const int64_t* streams, int32_t length, int64_t dA,
+                                              int64_t dB, int64_t dC, int32_t Batch, int32_t CN,
+                                              int32_t AN, int32_t M, int32_t K) {
+    return dragon_Cuda_batchMatMul_batchMatMulT1(streams, length, dA, dB, dC, Batch, CN, AN, M, K);
+}
+int dragon_Cuda_batchMatMul_batchMatMulT2_mma(int32_t, const int64_t* streams, int32_t length,
+                                              int64_t dA, int64_t dB, int64_t dC, int32_t Batch,
+                                              int32_t N, int32_t CM, int32_t BM, int32_t K) {
+    return dragon_Cuda_batchMatMul_batchMatMulT2(streams, length, dA, dB, dC, Batch, N, CM, BM, K);
+}
+
+// ---- host heuristics ---------------------------------------------------------------
+
+static int tile_classes(int n, bool count_full) {
+    // Number of tile classes (128, 64, 32, 16, 8, 4) a dimension decomposes into; the
+    // 128 class counts once per full tile when count_full is set.
+    int c = 0;
+    if (n > 127) c += count_full ? (n >> 7) : 1;
+    n &= 127;
+    for (int bit = 64; bit >= 4; bit >>= 1)
+        if (n & bit) c++;
+    return c;
+}
+
+int32_t dragon_Cuda_matMul_blockNum(int32_t N, int32_t M) {
+    return tile_classes(N, true) * tile_classes(M, true);
+}
+
+static int stream_classes(int n) { return ((n & (n - 1)) == 0) ? 1 : tile_classes(n, false); }
+
+int32_t dragon_Cuda_matMul_nstream(int32_t N, int32_t M) {
+    const int size = stream_classes(N) * stream_classes(M);
+    return size < MAX_STREAMS ? size : MAX_STREAMS;
+}
+
+int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M) {
+    int size = stream_classes(N) * stream_classes(M);
+    if (size < 1) size = 1;
+    return size < MAX_STREAMS ? size : MAX_STREAMS;
+}
+
+void dragon_gemm_force_tile(int32_t tile) { gemm_force_tile(tile); }
+
+}  // extern "C"

@@ -1,0 +1,50 @@
+// Internal interface between the C-ABI entry points and the gfx950 GEMM kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace dragon {
+
+enum GemmVariant { GEMM_NN = 0, GEMM_T1 = 1, GEMM_T2 = 2 };
+
+enum GemmTile {
+    TILE_AUTO = -1,
+    TILE_128x128 = 0,
+    TILE_64x64 = 1,
+    TILE_256x64 = 2,
+    TILE_64x256 = 3,
+    TILE_128x64 = 4,
+    TILE_64x128 = 5,
+    TILE_COUNT = 6
+};
+
+// One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
+//   K-inner operand (k contiguous): outer bound = number of rows that exist (exact),
+//                                   inner bound = k extent (multiple of 4).
+//   K-outer operand (k is the row): outer bound = number of k rows that exist (exact),
+//                                   inner bound = row length (multiple of 4).
+struct GemmParams {
+    const float* A;
+    const float* B;
+    float* C;
+    float* Cbuf;            // split-K partials: slice z >= 1 goes to Cbuf + (z-1)*sizeC
+    int rows, cols;         // stored extent of C: rows exact, cols a multiple of 4
+    int k_total;            // contraction length
+    int lda, ldb, ldc;      // leading strides in floats (multiples of 4)
+    int a_outer, a_inner;
+    int b_outer, b_inner;
+    long long sA, sB, sC;   // batch strides in floats
+    int nz;                 // grid depth: batches, or K slices when split is set
+    int split;              // non-zero selects split-K
+    int k_slice;            // slice z covers [z*k_slice, (z+1)*k_slice), the last runs to k_total
+    long long sizeC;        // floats per split-K partial
+    int tiles_m, tiles_n;   // filled by the launcher
+};
+
+int gemm_choose_tile(int rows, int cols, int nz, int num_cu);
+void gemm_force_tile(int tile);
+hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
+
+// C[i] += sum_p Cbuf[p*sizeC + i], Kahan-compensated, p ascending.
+hipError_t skbuf_summary_launch(hipStream_t stream, const float* Cbuf, float* C, int part, int sizeC);
+
+}  // namespace dragon

@@ -1,0 +1,325 @@
+"""Python access to the gfx950 FP32 matrix-multiplication engine.
+
+Thin, one-to-one wrappers over the C ABI (no compute happens in Python):
+
+  Cuda             -- runtime natives of the reference's z.dragon.engine.cuda.impl.Cuda
+  Cuda_matMul      -- natives + heuristics of ...impl.math.Cuda_matMul
+  Cuda_batchMatMul -- natives + heuristics of ...impl.math.Cuda_batchMatMul
+  CudaException    -- the error type the reference's natives throw
+
+Method names and argument order follow the Java declarations
+(source/alpha-Dragon-v1.2/src/z/dragon/engine/cuda/impl/Cuda.java,
+ .../impl/math/Cuda_matMul.java, .../impl/math/Cuda_batchMatMul.java).
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+
+lib = _lib.load()
+
+
+class CudaException(RuntimeError):
+    """Mirror of z.dragon.engine.cuda.impl.CudaException: carries the runtime error code."""
+
+    def __init__(self, code):
+        self.code = int(code)
+        name = lib.dragon_Cuda_getExceptionName(self.code)
+        info = lib.dragon_Cuda_getExceptionInfo(self.code)
+        super().__init__("%s (%d): %s" % ((name or b"?").decode(), self.code,
+                                           (info or b"").decode()))
+
+
+def _check(code):
+    if code != 0:
+        raise CudaException(code)
+
+
+def _stream_array(streams):
+    arr = (ctypes.c_int64 * len(streams))(*[int(s) for s in streams])
+    return arr, len(streams)
+
+
+def _host_ptr(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+class Cuda:
+    """Runtime natives (Cuda.java:66-194)."""
+
+    @staticmethod
+    def malloc(size):
+        addr = lib.dragon_Cuda_malloc(int(size))
+        if addr == 0:
+            raise CudaException(lib.dragon_Cuda_getLastExceptionType() or 2)
+        return addr
+
+    @staticmethod
+    def free(address):
+        _check(lib.dragon_Cuda_free(address))
+
+    @staticmethod
+    def mallocHost(size):
+        addr = lib.dragon_Cuda_mallocHost(int(size))
+        if addr == 0:
+            raise CudaException(lib.dragon_Cuda_getLastExceptionType() or 2)
+        return addr
+
+    @staticmethod
+    def freeHost(address):
+        _check(lib.dragon_Cuda_freeHost(address))
+
+    @staticmethod
+    def memsetAsync(stream, address, value, size):
+        _check(lib.dragon_Cuda_memsetAsync(stream, address, value, size))
+
+    @staticmethod
+    def memcpyAsyncDeviceToDevice(stream, dst, src, size):
+        _check(lib.dragon_Cuda_memcpyAsyncDeviceToDevice(stream, dst, src, size))
+
+    @staticmethod
+    def getDeviceId():
+        return lib.dragon_Cuda_getDeviceId()
+
+    @staticmethod
+    def getDeviceCount():
+        return lib.dragon_Cuda_getDeviceCount()
+
+    @staticmethod
+    def setDevice(dev_id):
+        _check(lib.dragon_Cuda_setDevice(dev_id))
+
+    @staticmethod
+    def deviceSynchronize():
+        _check(lib.dragon_Cuda_deviceSynchronize())
+
+    @staticmethod
+    def multiProcessorCount(dev_id=0):
+        return lib.dragon_CudaDevice_multiProcessorCount(dev_id)
+
+    @staticmethod
+    def newStream_Blocking():
+        s = lib.dragon_Cuda_newStream_Blocking()
+        if s == 0:
+            raise CudaException(lib.dragon_Cuda_getLastExceptionType() or 1)
+        return s
+
+    @staticmethod
+    def newStream_NonBlocking():
+        s = lib.dragon_Cuda_newStream_NonBlocking()
+        if s == 0:
+            raise CudaException(lib.dragon_Cuda_getLastExceptionType() or 1)
+        return s
+
+    @staticmethod
+    def deleteStream(stream):
+        _check(lib.dragon_Cuda_deleteStream(stream))
+
+    @staticmethod
+    def streamQuery(stream):
+        r = lib.dragon_Cuda_streamQuery(stream)
+        if r < 0:
+            raise CudaException(lib.dragon_Cuda_getLastExceptionType() or 1)
+        return bool(r)
+
+    @staticmethod
+    def streamSynchronize(stream):
+        _check(lib.dragon_Cuda_streamSynchronize(stream))
+
+    @staticmethod
+    def newEvent_Default():
+        return lib.dragon_Cuda_newEvent_Default()
+
+    @staticmethod
+    def newEvent_DisableTiming():
+        return lib.dragon_Cuda_newEvent_DisableTiming()
+
+    @staticmethod
+    def deleteEvent(event):
+        _check(lib.dragon_Cuda_deleteEvent(event))
+
+    @staticmethod
+    def eventRecord(event, stream_or_streams, length=None):
+        if isinstance(stream_or_streams, (list, tuple)):
+            arr, n = _stream_array(stream_or_streams)
+            _check(lib.dragon_Cuda_eventRecord_streams(event, arr, n if length is None else length))
+        else:
+            _check(lib.dragon_Cuda_eventRecord(event, stream_or_streams))
+
+    @staticmethod
+    def eventSynchronize(event):
+        _check(lib.dragon_Cuda_eventSynchronize(event))
+
+    @staticmethod
+    def eventSync_Del(event):
+        _check(lib.dragon_Cuda_eventSync_Del(event))
+
+    @staticmethod
+    def eventElapsedTime(start_event, stop_event):
+        ms = lib.dragon_Cuda_eventElapsedTime(start_event, stop_event)
+        if ms < 0:
+            raise CudaException(lib.dragon_Cuda_getLastExceptionType() or 1)
+        return ms
+
+    @staticmethod
+    def streamWaitEvent_default(stream, event):
+        _check(lib.dragon_Cuda_streamWaitEvent_default(stream, event))
+
+    @staticmethod
+    def getLastExceptionType():
+        return lib.dragon_Cuda_getLastExceptionType()
+
+    @staticmethod
+    def set1D(stream, address, value, length):
+        if isinstance(value, (int, float)):
+            _check(lib.dragon_Cuda_set1D_value(stream, address, float(value), length))
+        else:
+            _check(lib.dragon_Cuda_set1D(stream, address, _host_ptr(value), length))
+
+    @staticmethod
+    def set2D(stream, address, value, height, width, stride):
+        if isinstance(value, (int, float)):
+            _check(lib.dragon_Cuda_set2D_value(stream, address, float(value), height, width, stride))
+        else:
+            _check(lib.dragon_Cuda_set2D(stream, address, _host_ptr(value), height, width, stride))
+
+    @staticmethod
+    def get1D(stream, address, value, length):
+        _check(lib.dragon_Cuda_get1D(stream, address, _host_ptr(value), length))
+
+    @staticmethod
+    def get2D(stream, address, value, height, width, stride):
+        _check(lib.dragon_Cuda_get2D(stream, address, _host_ptr(value), height, width, stride))
+
+
+class Cuda_matMul:
+    """Natives and helpers of Cuda_matMul.java."""
+
+    blockNum = staticmethod(lambda N, M: lib.dragon_Cuda_matMul_blockNum(N, M))
+    nstream = staticmethod(lambda N, M: lib.dragon_Cuda_matMul_nstream(N, M))
+
+    @staticmethod
+    def SKbuf_summary(stream, dCbuf, dC, part, sizeC):
+        _check(lib.dragon_Cuda_matMul_SKbuf_summary(stream, dCbuf, dC, part, sizeC))
+
+    @staticmethod
+    def matMul(streams, length, dA, dB, dC, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMul(arr, length, dA, dB, dC, N, M, K))
+
+    @staticmethod
+    def matMulT1(streams, length, dA, dB, dC, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulT1(arr, length, dA, dB, dC, N, M, K))
+
+    @staticmethod
+    def matMulT2(streams, length, dA, dB, dC, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulT2(arr, length, dA, dB, dC, N, M, K))
+
+    @staticmethod
+    def matMulSK(streams, length, GZ, dA, dB, dC, dCbuf, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulSK(arr, length, GZ, dA, dB, dC, dCbuf, N, M, K))
+
+    @staticmethod
+    def matMulT1SK(streams, length, GZ, dA, dB, dC, dCbuf, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulT1SK(arr, length, GZ, dA, dB, dC, dCbuf, N, M, K))
+
+    @staticmethod
+    def matMulT2SK(streams, length, GZ, dA, dB, dC, dCbuf, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulT2SK(arr, length, GZ, dA, dB, dC, dCbuf, N, M, K))
+
+    @staticmethod
+    def matMul_mma(streams, length, dA, dB, dC, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMul_mma(arr, length, dA, dB, dC, N, M, K))
+
+    @staticmethod
+    def matMulT1_mma(streams, length, dA, dB, dC, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulT1_mma(arr, length, dA, dB, dC, N, M, K))
+
+    @staticmethod
+    def matMulT2_mma(streams, length, dA, dB, dC, N, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulT2_mma(arr, length, dA, dB, dC, N, M, K))
+
+
+class Cuda_batchMatMul:
+    """Natives and helpers of Cuda_batchMatMul.java."""
+
+    streamSize = staticmethod(lambda N, M: lib.dragon_Cuda_batchMatMul_streamSize(N, M))
+
+    @staticmethod
+    def batchMatMul(streams, length, dA, dB, dC, Batch, N, M, BK, AK):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_batchMatMul_batchMatMul(arr, length, dA, dB, dC, Batch, N, M, BK, AK))
+
+    @staticmethod
+    def batchMatMul_texture(streams, length, dA, dB, dC, Batch, N, M, BK, AK):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_batchMatMul_batchMatMul_texture(arr, length, dA, dB, dC, Batch, N, M,
+                                                               BK, AK))
+
+    @staticmethod
+    def batchMatMulT1(streams, length, dA, dB, dC, Batch, CN, AN, M, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_batchMatMul_batchMatMulT1(arr, length, dA, dB, dC, Batch, CN, AN, M, K))
+
+    @staticmethod
+    def batchMatMulT2(streams, length, dA, dB, dC, Batch, N, CM, BM, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_batchMatMul_batchMatMulT2(arr, length, dA, dB, dC, Batch, N, CM, BM, K))
+
+    @staticmethod
+    def batchMatMulT2_texture(streams, length, dA, dB, dC, Batch, N, CM, BM, K):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_batchMatMul_batchMatMulT2_texture(arr, length, dA, dB, dC, Batch, N,
+                                                                 CM, BM, K))
+
+
+def force_tile(tile):
+    """Force one kernel tile shape (-1 = automatic).  Benchmark / test hook."""
+    lib.dragon_gemm_force_tile(int(tile))
+
+
+class DeviceArray:
+    """A float32 device allocation filled from / read back into a numpy array.
+
+    Test and benchmark plumbing: owns one Cuda.malloc block of `a.size` floats."""
+
+    def __init__(self, host=None, size=None, zero=True):
+        n = int(host.size if host is not None else size)
+        self.size = n
+        self.address = Cuda.malloc(max(n, 4) * 4)
+        if host is not None:
+            h = np.ascontiguousarray(host, dtype=np.float32).reshape(-1)
+            Cuda.set1D(0, self.address, h, n)
+        elif zero:
+            Cuda.memsetAsync(0, self.address, 0, n * 4)
+            Cuda.streamSynchronize(0)
+
+    def get(self, shape=None):
+        out = np.empty(self.size, dtype=np.float32)
+        Cuda.get1D(0, self.address, out, self.size)
+        return out.reshape(shape) if shape is not None else out
+
+    def fill(self, value):
+        Cuda.set1D(0, self.address, float(value), self.size)
+        Cuda.streamSynchronize(0)
+
+    def free(self):
+        if self.address:
+            Cuda.free(self.address)
+            self.address = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass

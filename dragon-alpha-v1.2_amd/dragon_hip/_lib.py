@@ -1,0 +1,106 @@
+"""ctypes binding of libdragon_hip.so: the C ABI declared in include/dragon_hip_gemm.h
+and include/dragon_hip_runtime.h.
+
+The library is loaded from the package directory.  There is no fallback: if the shared
+object is missing or a symbol cannot be resolved the import fails, and every compute
+entry point needs a GPU.
+"""
+import ctypes
+import os
+from ctypes import c_int32, c_int64, c_float, c_void_p, c_char_p, POINTER
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libdragon_hip.so")
+
+i32, i64, f32 = c_int32, c_int64, c_float
+p_i64 = POINTER(c_int64)
+p_f32 = POINTER(c_float)
+
+# name -> (restype, argtypes); mirrors the two public headers one to one
+_MM2D = [p_i64, i32, i64, i64, i64, i32, i32, i32]
+_MMSK = [p_i64, i32, i32, i64, i64, i64, i64, i32, i32, i32]
+_BMM = [p_i64, i32, i64, i64, i64, i32, i32, i32, i32, i32]
+SIGNATURES = {
+    # include/dragon_hip_gemm.h
+    "dragon_Cuda_matMul_matMul": (i32, _MM2D),
+    "dragon_Cuda_matMul_matMulT1": (i32, _MM2D),
+    "dragon_Cuda_matMul_matMulT2": (i32, _MM2D),
+    "dragon_Cuda_matMul_matMulSK": (i32, _MMSK),
+    "dragon_Cuda_matMul_matMulT1SK": (i32, _MMSK),
+    "dragon_Cuda_matMul_matMulT2SK": (i32, _MMSK),
+    "dragon_Cuda_matMul_SKbuf_summary": (i32, [i64, i64, i64, i32, i32]),
+    "dragon_Cuda_batchMatMul_batchMatMul": (i32, _BMM),
+    "dragon_Cuda_batchMatMul_batchMatMul_texture": (i32, _BMM),
+    "dragon_Cuda_batchMatMul_batchMatMulT1": (i32, _BMM),
+    "dragon_Cuda_batchMatMul_batchMatMulT2": (i32, _BMM),
+    "dragon_Cuda_batchMatMul_batchMatMulT2_texture": (i32, _BMM),
+    "dragon_Cuda_matMul_matMul_mma": (i32, _MM2D),
+    "dragon_Cuda_matMul_matMulT1_mma": (i32, _MM2D),
+    "dragon_Cuda_matMul_matMulT2_mma": (i32, _MM2D),
+    "dragon_Cuda_batchMatMul_batchMatMul_mma": (i32, [i32] + _BMM),
+    "dragon_Cuda_batchMatMul_batchMatMulT1_mma": (i32, _BMM),
+    "dragon_Cuda_batchMatMul_batchMatMulT2_mma": (i32, [i32] + _BMM),
+    "dragon_Cuda_matMul_blockNum": (i32, [i32, i32]),
+    "dragon_Cuda_matMul_nstream": (i32, [i32, i32]),
+    "dragon_Cuda_batchMatMul_streamSize": (i32, [i32, i32]),
+    "dragon_gemm_force_tile": (None, [i32]),
+    # include/dragon_hip_runtime.h
+    "dragon_Cuda_malloc": (i64, [i64]),
+    "dragon_Cuda_free": (i32, [i64]),
+    "dragon_Cuda_mallocHost": (i64, [i64]),
+    "dragon_Cuda_freeHost": (i32, [i64]),
+    "dragon_Cuda_memsetAsync": (i32, [i64, i64, i32, i64]),
+    "dragon_Cuda_memcpyAsyncHostToDevice": (i32, [i64, i64, i64, i64]),
+    "dragon_Cuda_memcpyAsyncHostToHost": (i32, [i64, i64, i64, i64]),
+    "dragon_Cuda_memcpyAsyncDeviceToHost": (i32, [i64, i64, i64, i64]),
+    "dragon_Cuda_memcpyAsyncDeviceToDevice": (i32, [i64, i64, i64, i64]),
+    "dragon_Cuda_memcpyAsyncDefault": (i32, [i64, i64, i64, i64]),
+    "dragon_Cuda_getDeviceId": (i32, []),
+    "dragon_Cuda_getDeviceCount": (i32, []),
+    "dragon_Cuda_setDevice": (i32, [i32]),
+    "dragon_Cuda_deviceSynchronize": (i32, []),
+    "dragon_CudaDevice_multiProcessorCount": (i32, [i32]),
+    "dragon_Cuda_newStream_Blocking": (i64, []),
+    "dragon_Cuda_newStream_NonBlocking": (i64, []),
+    "dragon_Cuda_deleteStream": (i32, [i64]),
+    "dragon_Cuda_deleteStreams": (i32, [p_i64, i32]),
+    "dragon_Cuda_streamQuery": (i32, [i64]),
+    "dragon_Cuda_streamSynchronize": (i32, [i64]),
+    "dragon_Cuda_streamsSynchronize": (i32, [p_i64, i32]),
+    "dragon_Cuda_newEvent_Default": (i64, []),
+    "dragon_Cuda_newEvent_BlockingSync": (i64, []),
+    "dragon_Cuda_newEvent_DisableTiming": (i64, []),
+    "dragon_Cuda_deleteEvent": (i32, [i64]),
+    "dragon_Cuda_eventRecord": (i32, [i64, i64]),
+    "dragon_Cuda_eventRecord_streams": (i32, [i64, p_i64, i32]),
+    "dragon_Cuda_eventSynchronize": (i32, [i64]),
+    "dragon_Cuda_eventSync_Del": (i32, [i64]),
+    "dragon_Cuda_eventElapsedTime": (f32, [i64, i64]),
+    "dragon_Cuda_streamWaitEvent_default": (i32, [i64, i64]),
+    "dragon_Cuda_streamsWaitEvent_default": (i32, [p_i64, i32, i64]),
+    "dragon_Cuda_getExceptionName": (c_char_p, [i32]),
+    "dragon_Cuda_getExceptionInfo": (c_char_p, [i32]),
+    "dragon_Cuda_getLastExceptionType": (i32, []),
+    "dragon_Cuda_set1D_value": (i32, [i64, i64, f32, i32]),
+    "dragon_Cuda_set2D_value": (i32, [i64, i64, f32, i32, i32, i32]),
+    "dragon_Cuda_get1D": (i32, [i64, i64, c_void_p, i32]),
+    "dragon_Cuda_get2D": (i32, [i64, i64, c_void_p, i32, i32, i32]),
+    "dragon_Cuda_set1D": (i32, [i64, i64, c_void_p, i32]),
+    "dragon_Cuda_set2D": (i32, [i64, i64, c_void_p, i32, i32, i32]),
+    "dragon_Cuda_get1D_v2": (i32, [i64, i64, c_void_p, i64, i32]),
+    "dragon_Cuda_get2D_v2": (i32, [i64, i64, c_void_p, i64, i32, i32, i32]),
+    "dragon_Cuda_set1D_v2": (i32, [i64, i64, c_void_p, i64, i32]),
+    "dragon_Cuda_set2D_v2": (i32, [i64, i64, c_void_p, i64, i32, i32, i32]),
+}
+
+
+def load(path=LIB_PATH):
+    if not os.path.exists(path):
+        raise ImportError(
+            "libdragon_hip.so is not built (%s); run dragon-alpha-v1.2_amd/csrc/build.sh" % path)
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing: fail loudly
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib

@@ -1,0 +1,173 @@
+/*
+ * dragon_hip_gemm.h -- C ABI of the gfx950 FP32 matrix-multiplication engine.
+ *
+ * Each entry point takes exactly the argument list of one `static native` method of
+ * the reference's z.dragon.engine.cuda.impl.math.Cuda_matMul / Cuda_batchMatMul
+ * classes, i.e. of one JNI function of Cuda_matMul.dll / Cuda_batchMatMul.dll, minus
+ * the (JNIEnv*, jclass) pair:  jlong -> int64_t (a raw device address or a stream
+ * handle), jint -> int32_t, jlongArray -> const int64_t*.  Where the JNI functions
+ * return void and throw z.dragon.engine.cuda.impl.CudaException(int), these return
+ * the hipError_t value as int (0 = success); a JNI shim turns a non-zero value into
+ * the exception.
+ *
+ * Reference paths below are relative to source/ of the reference tree:
+ *   MM  = engine-cuda-base/Cuda_matMul/Cuda_matMul
+ *   BMM = engine-cuda-base/Cuda_batchMatMul/Cuda_batchMatMul
+ *   JM  = alpha-Dragon-v1.2/src/z/dragon/engine/cuda/impl/math
+ *
+ * Conventions shared by all entry points (same as the reference):
+ *   - Letters follow the reference: N = rows of C, M = columns of C, K = contraction.
+ *   - Row-major FP32.  Addresses are device pointers owned by the caller, 16-byte
+ *     aligned; nothing is allocated, freed or retained here.
+ *   - C is overwritten (no alpha/beta).  Padded rows/columns of C receive exact zeros.
+ *   - streams[0..length) are valid stream handles, 1 <= length <= 10.  Work is issued
+ *     asynchronously on streams[0]; the other handles are left idle (the caller joins
+ *     all of them into streams[0] anyway).  The call returns without waiting.
+ *   - Callable from any host thread; no host-side global state is modified.
+ *   - Errors: hipErrorInvalidValue (1) for a null address, a non-positive dimension, a
+ *     stream count outside 1..10, a dimension that violates the x4 padding contract, or
+ *     a misaligned address; otherwise the launch status.
+ */
+#ifndef DRAGON_HIP_GEMM_H
+#define DRAGON_HIP_GEMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- 2-D products: N, M, K are multiples of 4 (caller-padded with zeros) -------- */
+
+/* C[N,M] = A[N,K] * B[K,M].
+ * Replaces Java_z_dragon_engine_cuda_impl_math_Cuda_1matMul_matMul (MM/A.cu:41-56,
+ * declared JM/Cuda_matMul.java:109) and its dispatcher matMul4x (MM/matMul.cuh:47-119). */
+int dragon_Cuda_matMul_matMul(const int64_t* streams, int32_t length,
+                              int64_t dA, int64_t dB, int64_t dC,
+                              int32_t N, int32_t M, int32_t K);
+
+/* C[N,M] = A[K,N]^T * B[K,M].
+ * Replaces ..._Cuda_1matMul_matMulT1 (MM/A.cu:90-105, JM/Cuda_matMul.java:206,
+ * dispatcher MM/matMulT1.cuh:42-89). */
+int dragon_Cuda_matMul_matMulT1(const int64_t* streams, int32_t length,
+                                int64_t dA, int64_t dB, int64_t dC,
+                                int32_t N, int32_t M, int32_t K);
+
+/* C[N,M] = A[N,K] * B[M,K]^T.
+ * Replaces ..._Cuda_1matMul_matMulT2 (MM/A.cu:139-154, JM/Cuda_matMul.java:315,
+ * dispatcher MM/matMulT2.cuh:44-107). */
+int dragon_Cuda_matMul_matMulT2(const int64_t* streams, int32_t length,
+                                int64_t dA, int64_t dB, int64_t dC,
+                                int32_t N, int32_t M, int32_t K);
+
+/* ---- split-K stage 1: K is cut into GridZ slices of K_slice = (K/GridZ)>>3<<3, the
+ * last slice takes the remainder; slice 0 is written to C, slice z >= 1 to
+ * Cbuf + (z-1)*N*M.  Cbuf holds (GridZ-1)*N*M floats.  GridZ >= 1.
+ * Replace ..._Cuda_1matMul_matMulSK / matMulT1SK / matMulT2SK (MM/A.cu:59-79, 108-128,
+ * 157-178; JM/Cuda_matMul.java:137, 251, 343; slice rule MM/micro.cuh:92 and
+ * MM/matMulSK_kernel.cuh:124-131). */
+int dragon_Cuda_matMul_matMulSK(const int64_t* streams, int32_t length, int32_t GridZ,
+                                int64_t dA, int64_t dB, int64_t dC, int64_t dCbuf,
+                                int32_t N, int32_t M, int32_t K);
+int dragon_Cuda_matMul_matMulT1SK(const int64_t* streams, int32_t length, int32_t GridZ,
+                                  int64_t dA, int64_t dB, int64_t dC, int64_t dCbuf,
+                                  int32_t N, int32_t M, int32_t K);
+int dragon_Cuda_matMul_matMulT2SK(const int64_t* streams, int32_t length, int32_t GridZ,
+                                  int64_t dA, int64_t dB, int64_t dC, int64_t dCbuf,
+                                  int32_t N, int32_t M, int32_t K);
+
+/* ---- split-K stage 2: C[i] += sum_{p < part} Cbuf[p*sizeC + i], Kahan-compensated,
+ * p ascending, starting from the value already in C.  sizeC is a multiple of 4.
+ * Bit-identical to the reference's operation order.
+ * Replaces ..._Cuda_1matMul_SKbuf_1summary (MM/A.cu:20-30, JM/Cuda_matMul.java:69,
+ * kernel MM/SKbufsum.cuh:29-81). */
+int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC,
+                                     int32_t part, int32_t sizeC);
+
+/* ---- batched products (grid depth = Batch) --------------------------------------- */
+
+/* C[b][N,M] = A[b][N,AK] * B[b][BK,M], k < BK.  M and AK are multiples of 4, N and BK
+ * are arbitrary; batch strides N*AK, BK*M, N*M.
+ * Replaces ..._Cuda_1batchMatMul_batchMatMul and batchMatMul_texture (BMM/A.cu:20-62,
+ * JM/Cuda_batchMatMul.java:90,137, dispatcher BMM/batchMatMul.cuh:48-254).  The texture
+ * entry is the same computation (textures only served the reference's edge tiles). */
+int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length,
+                                        int64_t dA, int64_t dB, int64_t dC,
+                                        int32_t Batch, int32_t N, int32_t M,
+                                        int32_t BK, int32_t AK);
+int dragon_Cuda_batchMatMul_batchMatMul_texture(const int64_t* streams, int32_t length,
+                                                int64_t dA, int64_t dB, int64_t dC,
+                                                int32_t Batch, int32_t N, int32_t M,
+                                                int32_t BK, int32_t AK);
+
+/* C[b][CN,M] = A[b][K,AN]^T * B[b][K,M].  AN and M are multiples of 4, CN <= AN and K
+ * are arbitrary; batch strides K*AN, K*M, CN*M.
+ * Replaces ..._Cuda_1batchMatMul_batchMatMulT1 (BMM/A.cu:71-89,
+ * JM/Cuda_batchMatMul.java:209, dispatcher BMM/batchMatMulT1.cuh:45-155). */
+int dragon_Cuda_batchMatMul_batchMatMulT1(const int64_t* streams, int32_t length,
+                                          int64_t dA, int64_t dB, int64_t dC,
+                                          int32_t Batch, int32_t CN, int32_t AN,
+                                          int32_t M, int32_t K);
+
+/* C[b][N,CM] = A[b][N,K] * B[b][BM,K]^T.  CM and K are multiples of 4, N and BM <= CM
+ * are arbitrary; columns BM..CM-1 of C are written as zeros; batch strides N*K, BM*K,
+ * N*CM.
+ * Replaces ..._Cuda_1batchMatMul_batchMatMulT2 and batchMatMulT2_texture
+ * (BMM/A.cu:98-143, JM/Cuda_batchMatMul.java:283,327, dispatcher
+ * BMM/batchMatMulT2.cuh:48-248). */
+int dragon_Cuda_batchMatMul_batchMatMulT2(const int64_t* streams, int32_t length,
+                                          int64_t dA, int64_t dB, int64_t dC,
+                                          int32_t Batch, int32_t N, int32_t CM,
+                                          int32_t BM, int32_t K);
+int dragon_Cuda_batchMatMul_batchMatMulT2_texture(const int64_t* streams, int32_t length,
+                                                  int64_t dA, int64_t dB, int64_t dC,
+                                                  int32_t Batch, int32_t N, int32_t CM,
+                                                  int32_t BM, int32_t K);
+
+/* ---- *_mma entries: the reference declares TF32 tensor-core variants
+ * (JM/Cuda_matMul.java:163,278,369; JM/Cuda_batchMatMul.java:166,236,355) whose native
+ * source is not published and which are off by default.  gfx950 has no reduced-precision
+ * FP32 matrix instruction, so these forward to the FP32 path above (results are at least
+ * as accurate as TF32). */
+int dragon_Cuda_matMul_matMul_mma(const int64_t* streams, int32_t length,
+                                  int64_t dA, int64_t dB, int64_t dC,
+                                  int32_t N, int32_t M, int32_t K);
+int dragon_Cuda_matMul_matMulT1_mma(const int64_t* streams, int32_t length,
+                                    int64_t dA, int64_t dB, int64_t dC,
+                                    int32_t N, int32_t M, int32_t K);
+int dragon_Cuda_matMul_matMulT2_mma(const int64_t* streams, int32_t length,
+                                    int64_t dA, int64_t dB, int64_t dC,
+                                    int32_t N, int32_t M, int32_t K);
+int dragon_Cuda_batchMatMul_batchMatMul_mma(int32_t useTexture,
+                                            const int64_t* streams, int32_t length,
+                                            int64_t dA, int64_t dB, int64_t dC,
+                                            int32_t Batch, int32_t N, int32_t M,
+                                            int32_t BK, int32_t AK);
+int dragon_Cuda_batchMatMul_batchMatMulT1_mma(const int64_t* streams, int32_t length,
+                                              int64_t dA, int64_t dB, int64_t dC,
+                                              int32_t Batch, int32_t CN, int32_t AN,
+                                              int32_t M, int32_t K);
+int dragon_Cuda_batchMatMul_batchMatMulT2_mma(int32_t useTexture,
+                                              const int64_t* streams, int32_t length,
+                                              int64_t dA, int64_t dB, int64_t dC,
+                                              int32_t Batch, int32_t N, int32_t CM,
+                                              int32_t BM, int32_t K);
+
+/* ---- host heuristics the Java side keeps as static methods; exported so a non-Java
+ * host can reproduce its decisions.
+ * blockNum: JM/Cuda_matMul.java:18-38; nstream: JM/Cuda_matMul.java:41-65;
+ * streamSize: JM/Cuda_batchMatMul.java:18-42. */
+int32_t dragon_Cuda_matMul_blockNum(int32_t N, int32_t M);
+int32_t dragon_Cuda_matMul_nstream(int32_t N, int32_t M);
+int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M);
+
+/* ---- tuning hook (no counterpart in the reference): force one tile shape for every
+ * following launch of this process, -1 restores the automatic choice.  For benchmarks
+ * and tests that sweep the kernel variants; not thread-safe against concurrent calls.
+ * Shapes: 0 = 128x128, 1 = 64x64, 2 = 256x64, 3 = 64x256, 4 = 128x64, 5 = 64x128. */
+void dragon_gemm_force_tile(int32_t tile);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRAGON_HIP_GEMM_H */
