@@ -1,0 +1,119 @@
+"""The drop-in boundary without a GPU: the shared library loads, exports every symbol
+the public headers declare, and its host-side helpers and argument validation behave.
+No compute entry point is executed here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("dragon_hip_gemm.h", "dragon_hip_runtime.h")]
+INVALID_VALUE = 1   # hipErrorInvalidValue
+
+
+def declared_symbols():
+    names = []
+    for h in HEADERS:
+        text = open(h).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)   # drop comments
+        names += re.findall(r"\b(dragon_\w+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_headers_declare_something():
+    names = declared_symbols()
+    assert len(names) >= 60
+    for must in ("dragon_Cuda_matMul_matMul", "dragon_Cuda_matMul_matMulT1SK",
+                 "dragon_Cuda_matMul_SKbuf_summary", "dragon_Cuda_batchMatMul_batchMatMulT2_texture",
+                 "dragon_Cuda_malloc", "dragon_Cuda_eventRecord_streams"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(dh):
+    lib = ctypes.CDLL(dh._lib.LIB_PATH)
+    missing = [n for n in declared_symbols() if not hasattr(lib, n)]
+    assert not missing, "declared in include/*.h but not exported: %s" % missing
+
+
+def test_binding_covers_every_declared_symbol(dh):
+    assert sorted(dh._lib.SIGNATURES) == declared_symbols()
+
+
+def test_heuristics_match_the_oracle(dh):
+    MM, BMM = dh.Cuda_matMul, dh.Cuda_batchMatMul
+    for N in list(range(1, 300)) + [512, 1000, 1024, 4096, 4100]:
+        for M in (1, 3, 4, 7, 64, 96, 100, 128, 255, 256, 388, 780, 4096):
+            if N % 4 == 0 and M % 4 == 0:
+                assert MM.blockNum(N, M) == oracle.blockNum(N, M)
+                assert MM.nstream(N, M) == oracle.nstream(N, M)
+            assert BMM.streamSize(N, M) == oracle.streamSize(N, M)   # N may be unpadded here
+    assert MM.blockNum(4096, 4096) == 1024 and MM.nstream(1000, 780) == 10
+
+
+def _streams(n):
+    return (ctypes.c_int64 * max(n, 1))(*([0] * max(n, 1)))
+
+
+def test_argument_validation_rejects_before_touching_the_device(dh):
+    lib = dh.lib
+    s = _streams(1)
+    ok_ptr = 0x1000   # aligned, never dereferenced: every call below must fail validation
+    f = lib.dragon_Cuda_matMul_matMul
+    assert f(s, 1, 0, ok_ptr, ok_ptr, 4, 4, 4) == INVALID_VALUE          # null A
+    assert f(s, 1, ok_ptr, 0, ok_ptr, 4, 4, 4) == INVALID_VALUE          # null B
+    assert f(s, 1, ok_ptr, ok_ptr, 0, 4, 4, 4) == INVALID_VALUE          # null C
+    assert f(s, 1, ok_ptr, ok_ptr, ok_ptr, 0, 4, 4) == INVALID_VALUE     # N <= 0
+    assert f(s, 1, ok_ptr, ok_ptr, ok_ptr, 4, -4, 4) == INVALID_VALUE    # M <= 0
+    assert f(s, 1, ok_ptr, ok_ptr, ok_ptr, 4, 4, 0) == INVALID_VALUE     # K <= 0
+    assert f(s, 1, ok_ptr, ok_ptr, ok_ptr, 5, 4, 4) == INVALID_VALUE     # N not padded to x4
+    assert f(s, 1, ok_ptr + 4, ok_ptr, ok_ptr, 4, 4, 4) == INVALID_VALUE  # misaligned
+    assert f(s, 0, ok_ptr, ok_ptr, ok_ptr, 4, 4, 4) == INVALID_VALUE     # no stream
+    assert f(_streams(11), 11, ok_ptr, ok_ptr, ok_ptr, 4, 4, 4) == INVALID_VALUE  # > 10 streams
+    assert f(None, 1, ok_ptr, ok_ptr, ok_ptr, 4, 4, 4) == INVALID_VALUE  # null stream array
+    for name in ("dragon_Cuda_matMul_matMulT1", "dragon_Cuda_matMul_matMulT2",
+                 "dragon_Cuda_matMul_matMul_mma"):
+        assert getattr(lib, name)(s, 1, 0, ok_ptr, ok_ptr, 4, 4, 4) == INVALID_VALUE
+    sk = lib.dragon_Cuda_matMul_matMulT1SK
+    assert sk(s, 1, 4, ok_ptr, ok_ptr, ok_ptr, 0, 4, 4, 64) == INVALID_VALUE   # split without Cbuf
+    assert sk(s, 1, 0, ok_ptr, ok_ptr, ok_ptr, ok_ptr, 4, 4, 64) == INVALID_VALUE  # GridZ < 1
+    sm = lib.dragon_Cuda_matMul_SKbuf_summary
+    assert sm(0, ok_ptr, 0, 3, 64) == INVALID_VALUE
+    assert sm(0, 0, ok_ptr, 3, 64) == INVALID_VALUE
+    assert sm(0, ok_ptr, ok_ptr, 3, 62) == INVALID_VALUE    # sizeC not x4
+    assert sm(0, ok_ptr, ok_ptr, -1, 64) == INVALID_VALUE
+    b = lib.dragon_Cuda_batchMatMul_batchMatMul
+    assert b(s, 1, ok_ptr, ok_ptr, ok_ptr, 0, 4, 4, 4, 4) == INVALID_VALUE      # Batch <= 0
+    assert b(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 5, 6, 4, 4) == INVALID_VALUE      # M not x4
+    assert b(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 5, 8, 5, 4) == INVALID_VALUE      # AK < BK
+    t1 = lib.dragon_Cuda_batchMatMul_batchMatMulT1
+    assert t1(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 9, 8, 4, 3) == INVALID_VALUE     # AN < CN
+    t2 = lib.dragon_Cuda_batchMatMul_batchMatMulT2
+    assert t2(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 5, 8, 9, 4) == INVALID_VALUE     # BM > CM
+    assert t2(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 5, 8, 7, 6) == INVALID_VALUE     # K not x4
+
+
+def test_python_wrapper_raises_the_exception_type(dh):
+    with pytest.raises(dh.CudaException) as e:
+        dh.Cuda_matMul.matMul([0], 1, 0, 0, 0, 4, 4, 4)
+    assert e.value.code == INVALID_VALUE
+
+
+def test_synthetic_generator_is_the_documented_stream(dh):
+    from dragon_hip import synthetic
+    g = synthetic.SplitMix64(1234567)   # published splitmix64 test vector
+    assert [int(v) for v in g.next(3)] == [6457827717110365317, 3203168211198807973,
+                                            9817491932198370423]
+    a = synthetic.stream_for(5).uniform((4, 7), -1, 1)
+    b = synthetic.stream_for(5).uniform((4, 7), -1, 1)
+    assert np.array_equal(a, b) and a.dtype == np.float32
+    assert (a >= -1).all() and (a < 1).all()
+    n = synthetic.stream_for(2).normal((200000,), 0, 1)
+    assert abs(float(n.mean())) < 0.01 and abs(float(n.std()) - 1) < 0.01
+    x = np.arange(15, dtype=np.float32).reshape(3, 5)
+    p = synthetic.to_device_layout(x, pad_first=True)
+    assert p.shape == (4, 8) and np.array_equal(p[:3, :5], x) and p[3].sum() == 0 and p[:, 5:].sum() == 0
+    assert np.array_equal(synthetic.from_device_layout(p.reshape(-1), (3, 5)), x)

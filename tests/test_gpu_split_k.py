@@ -1,0 +1,100 @@
+"""GPU parity of the two-stage split-K path (matMul*SK + SKbuf_summary)."""
+import numpy as np
+import pytest
+
+from oracle import oracle
+from helpers import NN, T1, T2, VARIANT_NAMES, assert_within_tolerance, logical_operands, pad2, rel_fro
+
+pytestmark = pytest.mark.gpu
+
+
+def run_sk(gpu, variant, A, B, GZ, summary=True, fill=9.0):
+    """A, B already padded to x4.  Returns (C, Cbuf) as written by stage 1 (and stage 2)."""
+    MM, Cuda = gpu.Cuda_matMul, gpu.Cuda
+    if variant == NN:
+        (N, K), M = A.shape, B.shape[1]
+    elif variant == T1:
+        (K, N), M = A.shape, B.shape[1]
+    else:
+        (N, K), M = A.shape, B.shape[0]
+    dA, dB = gpu.DeviceArray(A), gpu.DeviceArray(B)
+    dC, dCbuf = gpu.DeviceArray(size=N * M), gpu.DeviceArray(size=N * M * max(GZ - 1, 1))
+    dC.fill(fill)
+    dCbuf.fill(fill)
+    [MM.matMulSK, MM.matMulT1SK, MM.matMulT2SK][variant]([0], 1, GZ, dA.address, dB.address,
+                                                           dC.address, dCbuf.address, N, M, K)
+    if summary:
+        MM.SKbuf_summary(0, dCbuf.address, dC.address, GZ - 1, N * M)
+    Cuda.streamSynchronize(0)
+    C, Cbuf = dC.get((N, M)), dCbuf.get((max(GZ - 1, 1), N, M))[:GZ - 1]
+    for x in (dA, dB, dC, dCbuf):
+        x.free()
+    return C, Cbuf
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("shape_gz", [((64, 64, 256), 2), ((128, 132, 1000), 6), ((36, 260, 1532), 2),
+                                      ((256, 256, 4096), 16), ((100, 52, 904), 7), ((8, 8, 40), 4)])
+def test_stage1_partials_follow_the_slice_rule_bitwise(gpu, variant, shape_gz):
+    # integer inputs: each slice's partial product is exact, so slice bounds that are off
+    # by a single k show up as a bit mismatch against the oracle's partials
+    (N, M, K), GZ = shape_gz
+    rng = np.random.default_rng(K + GZ)
+    A, B = logical_operands(variant, rng, N, M, K, dist="int")
+    C, Cbuf = run_sk(gpu, variant, A, B, GZ, summary=False)
+    C0, Cb0 = oracle.matMulSK(variant, GZ, A, B)
+    assert np.array_equal(C, C0)
+    assert np.array_equal(Cbuf, Cb0)
+    # after stage 2 the product is complete
+    C, _ = run_sk(gpu, variant, A, B, GZ, summary=True)
+    assert np.array_equal(C, oracle.matmul(variant, A, B))
+
+
+def test_stage2_summary_is_bit_identical_to_the_reference_order(gpu):
+    rng = np.random.default_rng(77)
+    MM, Cuda = gpu.Cuda_matMul, gpu.Cuda
+    for part, sizeC in [(1, 4), (3, 64), (7, 252), (15, 256), (127, 65536), (33, 100004), (9, 1 << 20)]:
+        C = (rng.standard_normal(sizeC) * 100).astype(np.float32)
+        Cbuf = rng.standard_normal((part, sizeC)).astype(np.float32)
+        Cbuf[::2] *= 1e-4                       # mixed magnitudes exercise the compensation
+        dC, dCbuf = gpu.DeviceArray(C), gpu.DeviceArray(Cbuf)
+        MM.SKbuf_summary(0, dCbuf.address, dC.address, part, sizeC)
+        Cuda.streamSynchronize(0)
+        got = dC.get()
+        assert np.array_equal(got, oracle.SKbuf_summary(Cbuf, C, part)), (part, sizeC)
+        exact = C.astype(np.float64) + Cbuf.astype(np.float64).sum(axis=0)
+        assert np.abs(got - exact).max() <= 2 * np.spacing(np.abs(exact).max().astype(np.float32))
+        dC.free(); dCbuf.free()
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_split_k_equals_unsplit_within_tolerance(gpu, variant):
+    rng = np.random.default_rng(3 + variant)
+    N, M, K = 256, 128, 8192
+    A, B = logical_operands(variant, rng, N, M, K, dist="normal")
+    R32 = oracle.matmul(variant, A, B)
+    R64 = oracle.matmul_f64(variant, A, B)
+    for GZ in (2, 8, 32):
+        C, _ = run_sk(gpu, variant, A, B, GZ)
+        assert_within_tolerance(C, R32, K, A, B, "%s GZ=%d vs FP32 oracle" % (VARIANT_NAMES[variant], GZ))
+        assert_within_tolerance(C, R64, K, A, B, "%s GZ=%d vs FP64 oracle" % (VARIANT_NAMES[variant], GZ))
+        # and against the oracle's own two-stage computation
+        C0, Cb0 = oracle.matMulSK(variant, GZ, A, B)
+        assert rel_fro(C, oracle.SKbuf_summary(Cb0, C0, GZ - 1)) < 2e-6
+
+
+def test_degenerate_slices(gpu):
+    # K smaller than 8*GridZ: K_slice = 0, every slice but the last is empty and must be
+    # written as zeros; the last carries the whole product
+    rng = np.random.default_rng(11)
+    A, B = logical_operands(T1, rng, 32, 36, 24, dist="int")
+    C, Cbuf = run_sk(gpu, T1, A, B, 4, summary=False)
+    assert oracle.SK_K_slice(24, 4) == 0
+    assert np.count_nonzero(C) == 0 and np.count_nonzero(Cbuf[:2]) == 0
+    assert np.array_equal(Cbuf[2], oracle.matmul(T1, A, B))
+    # GridZ = 1 through the split-K entry is the plain product (Cbuf unused)
+    MM = gpu.Cuda_matMul
+    dA, dB, dC = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(size=32 * 36)
+    MM.matMulT1SK([0], 1, 1, dA.address, dB.address, dC.address, 0, 32, 36, 24)
+    gpu.Cuda.streamSynchronize(0)
+    assert np.array_equal(dC.get((32, 36)), oracle.matmul(T1, A, B))

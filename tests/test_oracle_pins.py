@@ -1,0 +1,309 @@
+"""Pins the CPU oracle independently of its own formulas (CPU only).
+
+The reference holds no golden vectors for this path (its tests draw unseeded random
+inputs and check a tolerance), so the oracle is pinned by what the mathematics fixes:
+exact integer products, data-movement cases, transpose identities, FP64 products within
+the forward error bound, enumeration of the split-K slice rule, and the hand-derived
+heuristics table.  Where oracle/_ref is built, the reference's own micro.cuh helpers
+are compared as well.
+"""
+import numpy as np
+import pytest
+
+from oracle import oracle
+from helpers import NN, T1, T2
+
+RNG = np.random.default_rng(20240521)
+
+
+def _ops(variant, N, M, K, ints=False):
+    shA = (K, N) if variant == T1 else (N, K)
+    shB = (M, K) if variant == T2 else (K, M)
+    if ints:
+        return (RNG.integers(-4, 5, shA).astype(np.float32),
+                RNG.integers(-4, 5, shB).astype(np.float32))
+    return (RNG.uniform(-1, 1, shA).astype(np.float32),
+            RNG.uniform(-1, 1, shB).astype(np.float32))
+
+
+def _logical(variant, A, B):
+    return (A.T if variant == T1 else A), (B.T if variant == T2 else B)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (17, 33, 129), (64, 48, 300)])
+def test_integer_inputs_are_exact(variant, shape):
+    # |a|,|b| <= 4, K <= 300: every partial sum is an integer below 2^24, so any
+    # correct summation order gives exactly the int64 product.  A dropped term, a
+    # wrong index or a transposed operand changes the integer result.
+    N, M, K = shape
+    A, B = _ops(variant, N, M, K, ints=True)
+    La, Lb = _logical(variant, A, B)
+    exact = La.astype(np.int64) @ Lb.astype(np.int64)
+    for fn in (oracle.multiply_literal, oracle.matmul):
+        C = fn(variant, A, B)
+        assert np.array_equal(C.astype(np.int64), exact)
+        assert np.array_equal(C, exact.astype(np.float32))
+    assert np.array_equal(oracle.matmul_f64(variant, A, B), exact.astype(np.float64))
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_identity_and_one_hot_move_data_only(variant):
+    n = 37
+    X = RNG.uniform(-1, 1, (n, n)).astype(np.float32)
+    I = np.eye(n, dtype=np.float32)
+    # op(A) = X, op(B) = I  ->  C = X exactly
+    A = X.T.copy() if variant == T1 else X
+    assert np.array_equal(oracle.matmul(variant, A, I), X)
+    # op(A) = I, op(B) = X  ->  C = X exactly
+    B = X.T.copy() if variant == T2 else X
+    assert np.array_equal(oracle.matmul(variant, I, B), X)
+    # one-hot row selector picks row 5 of op(B)
+    sel = np.zeros((1, n), np.float32)
+    sel[0, 5] = 1
+    A1 = sel.T.copy() if variant == T1 else sel
+    assert np.array_equal(oracle.matmul(variant, A1, B)[0], X[5])
+
+
+def test_all_ones_gives_K():
+    for K in (1, 4, 1000, 4099):
+        C = oracle.matmul(NN, np.ones((3, K), np.float32), np.ones((K, 5), np.float32))
+        assert np.all(C == K)
+
+
+@pytest.mark.parametrize("shape", [(5, 7, 11), (33, 20, 257), (130, 70, 64)])
+def test_transposed_variants_equal_plain_product_bitwise(shape):
+    # matMulT1(A,B) == matMul(A^T,B) and matMulT2(A,B) == matMul(A,B^T), element by
+    # element with the same k order, hence bit-identical.
+    N, M, K = shape
+    A, B = _ops(NN, N, M, K)
+    C = oracle.matmul(NN, A, B)
+    assert np.array_equal(oracle.matmul(T1, A.T.copy(), B), C)
+    assert np.array_equal(oracle.matmul(T2, A, B.T.copy()), C)
+    assert np.array_equal(oracle.multiply_literal(T1, A.T.copy(), B), C)
+    assert np.array_equal(oracle.multiply_literal(T2, A, B.T.copy()), C)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("shape", [(1, 1, 5), (50, 49, 131), (257, 300, 515), (96, 520, 260)])
+def test_fast_is_bitwise_the_literal_loop(variant, shape):
+    A, B = _ops(variant, *shape)
+    assert np.array_equal(oracle.matmul(variant, A, B), oracle.multiply_literal(variant, A, B))
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_fp32_oracle_within_forward_error_bound_of_fp64(variant):
+    # |fl(sum) - sum| <= gamma_K * sum |a_k b_k| for recursive summation, gamma_K ~ K*u.
+    N, M, K = 40, 52, 1000
+    A, B = _ops(variant, N, M, K)
+    La, Lb = _logical(variant, A, B)
+    exact = La.astype(np.float64) @ Lb.astype(np.float64)
+    absprod = np.abs(La).astype(np.float64) @ np.abs(Lb).astype(np.float64)
+    u = 2.0 ** -24
+    gamma = (K + 1) * u / (1 - (K + 1) * u)
+    C = oracle.matmul(variant, A, B)
+    assert np.all(np.abs(C - exact) <= gamma * absprod)
+    C64 = oracle.matmul_f64(variant, A, B)
+    assert np.allclose(C64, exact, rtol=1e-13, atol=1e-13)
+    # and not trivially equal: FP32 accumulation does round
+    assert np.abs(C - exact).max() > 0
+
+
+def test_fp32_oracle_is_sequential_k_ascending():
+    # 2^24 + 1 + 1 ... in FP32: adding 1.0 to 2^24 one at a time never moves it,
+    # while any pairwise/blocked order would.  Pins "k ascending, one add at a time".
+    K = 64
+    a = np.ones((1, K), np.float32)
+    b = np.ones((K, 1), np.float32)
+    a[0, 0] = 2.0 ** 24
+    for fn in (oracle.multiply_literal, oracle.matmul):
+        assert fn(NN, a, b)[0, 0] == np.float32(2.0 ** 24)
+    # descending order would give 2^24 + 63 -> rounds to 2^24 + 64
+    a2 = a[:, ::-1].copy()
+    assert oracle.matmul(NN, a2, b)[0, 0] == np.float32(2.0 ** 24 + 64)
+
+
+def test_no_fma_contraction():
+    # a*b + c with a single rounding differs from round(round(a*b) + c) here.
+    a = np.float32(1 + 2.0 ** -12)
+    prod_rounded = np.float32(a * a)                 # 1 + 2^-11 (the 2^-24 term is lost)
+    c = np.float32(-prod_rounded)
+    A = np.array([[1.0, a]], np.float32)             # k=0 contributes c, k=1 contributes a*a
+    B = np.array([[c], [a]], np.float32)
+    got = oracle.matmul(NN, A, B)[0, 0]
+    assert got == np.float32(0.0)                    # separate rounding: exactly cancels
+    assert np.float64(a) * np.float64(a) + np.float64(c) != 0.0   # a fused multiply-add would not
+
+
+# ---- batched ---------------------------------------------------------------------------
+def _bmm_case(variant, Batch, N, M, K):
+    """Logical batched operands laid out in the reference's padded memory layout."""
+    p4 = lambda v: (v + 3) // 4 * 4
+    if variant == NN:      # A[B,N,AK], B[B,BK,CM]
+        AK, CM = p4(K), p4(M)
+        A = np.zeros((Batch, N, AK), np.float32); A[:, :, :K] = RNG.uniform(-1, 1, (Batch, N, K))
+        B = np.zeros((Batch, K, CM), np.float32); B[:, :, :M] = RNG.uniform(-1, 1, (Batch, K, M))
+        dims = (N, CM, K, AK)
+        ref = A[:, :, :K].astype(np.float64) @ B.astype(np.float64)
+    elif variant == T1:    # A[B,K,AN], B[B,K,CM] -> C[B,CN,CM]
+        AN, CM = p4(N), p4(M)
+        A = np.zeros((Batch, K, AN), np.float32); A[:, :, :N] = RNG.uniform(-1, 1, (Batch, K, N))
+        B = np.zeros((Batch, K, CM), np.float32); B[:, :, :M] = RNG.uniform(-1, 1, (Batch, K, M))
+        dims = (N, AN, CM, K)
+        ref = np.transpose(A[:, :, :N], (0, 2, 1)).astype(np.float64) @ B.astype(np.float64)
+    else:                  # A[B,N,K4], B[B,BM,K4] -> C[B,N,CM]
+        K4, CM = p4(K), p4(M)
+        A = np.zeros((Batch, N, K4), np.float32); A[:, :, :K] = RNG.uniform(-1, 1, (Batch, N, K))
+        B = np.zeros((Batch, M, K4), np.float32); B[:, :, :K] = RNG.uniform(-1, 1, (Batch, M, K))
+        dims = (N, CM, M, K4)
+        ref = np.zeros((Batch, N, CM))
+        ref[:, :, :M] = A.astype(np.float64) @ np.transpose(B, (0, 2, 1)).astype(np.float64)
+    return A, B, dims, ref
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("shape", [(3, 5, 6, 7), (4, 33, 21, 9), (2, 70, 130, 50)])
+def test_batched_oracle(variant, shape):
+    Batch, N, M, K = shape
+    A, B, dims, ref = _bmm_case(variant, Batch, N, M, K)
+    C1 = oracle.bmm_literal(variant, A, B, Batch, *dims)
+    C2 = oracle.bmm(variant, A, B, Batch, *dims)
+    assert np.array_equal(C1, C2)
+    assert np.allclose(C1, ref, rtol=0, atol=2e-5 * np.sqrt(K))
+    # batched == loop of 2-D products on the logical slices, bit for bit
+    for b in range(Batch):
+        if variant == NN:
+            c = oracle.matmul(NN, A[b][:, :K], B[b])
+        elif variant == T1:
+            c = oracle.matmul(T1, A[b][:, :N], B[b])
+        else:
+            c = np.zeros_like(C1[b])
+            c[:, :M] = oracle.matmul(T2, A[b], B[b])
+        assert np.array_equal(C1[b], c)
+
+
+# ---- split-K -----------------------------------------------------------------------------
+def test_split_k_slice_rule_enumerated():
+    for K in list(range(8, 300, 4)) + [1532, 4096, 131072]:
+        for GZ in (1, 2, 3, 4, 7, 16, 36, 128):
+            ks = oracle.SK_K_slice(K, GZ)
+            assert ks % 8 == 0 and ks == (K // GZ) // 8 * 8
+            total, prev_end = 0, 0
+            for z in range(GZ):
+                a, b = oracle.SK_bounds(K, GZ, z)
+                assert a == prev_end and b >= a
+                if z < GZ - 1:
+                    assert b - a == ks
+                else:
+                    assert b == K            # the last slice takes the remainder
+                total += b - a
+                prev_end = b
+            assert total == K
+    assert oracle.SK_K_slice(131072, 128) == 1024
+    assert oracle.SK_K_slice(131072, 36) == 3640
+    assert oracle.SK_K_slice(1532, 2) == 760
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_split_k_partials_sum_to_product(variant):
+    N, M, K, GZ = 24, 36, 1000, 6
+    A, B = _ops(variant, N, M, K, ints=True)
+    La, Lb = _logical(variant, A, B)
+    exact = (La.astype(np.int64) @ Lb.astype(np.int64)).astype(np.float32)
+    C0, Cbuf = oracle.matMulSK(variant, GZ, A, B)
+    assert Cbuf.shape == (GZ - 1, N, M)
+    # each partial is the exact product over its own k range
+    for z in range(GZ):
+        a, b = oracle.SK_bounds(K, GZ, z)
+        part = (La[:, a:b].astype(np.int64) @ Lb[a:b].astype(np.int64)).astype(np.float32)
+        assert np.array_equal(C0 if z == 0 else Cbuf[z - 1], part)
+    assert np.array_equal(oracle.SKbuf_summary(Cbuf, C0, GZ - 1), exact)
+
+
+def test_kahan_summary_beats_plain_sum_and_matches_fp64():
+    # one large value followed by many small ones: plain FP32 accumulation loses them,
+    # the compensated sum keeps them.
+    part, sizeC = 127, 64
+    C = np.full(sizeC, 1.0e4, np.float32)
+    Cbuf = RNG.uniform(1e-4, 2e-4, (part, sizeC)).astype(np.float32)
+    exact = C.astype(np.float64) + Cbuf.astype(np.float64).sum(axis=0)
+    got = oracle.SKbuf_summary(Cbuf, C, part)
+    plain = C.copy()
+    for p in range(part):
+        plain = plain + Cbuf[p]
+    assert np.abs(got - exact).max() <= np.spacing(np.float32(1.0e4))   # within 1 ulp
+    assert np.abs(plain - exact).max() > 5 * np.abs(got - exact).max()
+    # part = 0 leaves C untouched
+    assert np.array_equal(oracle.SKbuf_summary(Cbuf, C, 0), C)
+
+
+# ---- heuristics ------------------------------------------------------------------------------
+def _tile_count_bruteforce(n):
+    """Greedy carve of n (multiple of 4) into 128,64,32,16,8,4 tiles: number of tiles."""
+    cnt = 0
+    for t in (128, 64, 32, 16, 8, 4):
+        cnt += n // t
+        n %= t
+    return cnt
+
+
+def _class_count_bruteforce(n):
+    if n & (n - 1) == 0:
+        return 1
+    cnt = 0
+    for t in (128, 64, 32, 16, 8, 4):
+        if n >= t:
+            cnt += 1
+        n %= t
+    return cnt
+
+
+def test_blockNum_and_nstream_against_bruteforce():
+    for N in range(4, 1300, 4):
+        for M in (4, 8, 12, 64, 100, 128, 252, 256, 780, 1000, 1028):
+            assert oracle.blockNum(N, M) == _tile_count_bruteforce(N) * _tile_count_bruteforce(M)
+            ns = min(10, _class_count_bruteforce(N) * _class_count_bruteforce(M))
+            assert oracle.nstream(N, M) == ns
+            assert oracle.streamSize(N, M) == max(1, ns)
+
+
+def test_heuristics_known_answers():
+    # hand-derived from the Java sources
+    assert oracle.blockNum(4096, 4096) == 1024
+    assert oracle.blockNum(256, 256) == 4
+    assert oracle.blockNum(1000, 780) == 80
+    assert oracle.blockNum(512, 512) == 16
+    assert oracle.nstream(4096, 4096) == 1
+    assert oracle.nstream(1000, 780) == 10
+    assert oracle.smooth_maxPart(256) == 128
+    assert oracle.smooth_maxPart(38) == 40
+    assert oracle.smooth_maxPart(10) == 16
+    assert oracle.smooth_maxPart(30) == 32
+    # BASELINE shapes with 256 compute units
+    for kind in (oracle.MATMUL, oracle.MATMUL_T1, oracle.MATMUL_T2):
+        assert oracle.gridZ(kind, 4096, 4096, 4096, 256) == 1
+        assert oracle.gridZ(kind, 1000, 780, 1532, 256) == 2
+    assert oracle.gridZ(oracle.MATMUL_T1, 256, 256, 131072, 256) == 128
+    # the same weight-gradient shape on a 38-SM device
+    assert oracle.gridZ(oracle.MATMUL_T1, 256, 256, 131072, 38) == 36
+    # below the threshold nothing splits
+    assert oracle.gridZ(oracle.MATMUL, 128, 128, 508, 256) == 1
+
+
+def test_reference_micro_helpers_when_built():
+    ref = oracle.load_ref()
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (reference tree absent at build time)")
+    for N in range(4, 1100, 4):
+        for M in (4, 60, 128, 388, 780, 1024):
+            assert ref.ref_blockNum(N, M) == oracle.blockNum(N, M)
+    for K in (8, 100, 1532, 4096, 131072):
+        for GZ in (1, 2, 5, 36, 128):
+            assert ref.ref_SK_K_slice(K, GZ) == oracle.SK_K_slice(K, GZ)
+
+
+def test_samePercent_relative_rule():
+    a = np.array([1.0, 2.0, 0.0, 5.0, np.nan], np.float32)
+    b = np.array([1.0005, 2.1, 0.0, 5.0, np.nan], np.float32)
+    # 1.0 vs 1.0005: 2.5e-4 < 1e-3 same; 2.0 vs 2.1: 2.4e-2 different; equal; equal; NaN pair same
+    assert oracle.samePercent_relative(a, b) == pytest.approx(4 / 5)
