@@ -1,18 +1,29 @@
 #!/bin/bash
-# Builds libdragon_hip.so (kernels + C ABI + runtime bridge) for gfx950, in-tree.
-set -euo pipefail
+# Builds libdragon_hip.so for gfx950, in-tree: HIP kernels + C ABI + runtime bridge
+# (hipcc) and the host-side engine mirror (g++, plain C++ above the C ABI).
+set -uo pipefail
 cd "$(dirname "$0")"
 HIPCC=${HIPCC:-/opt/rocm/bin/hipcc}
-FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Wall -Wno-unused-function \
+HIPFLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Wall -Wno-unused-function \
   -Xclang -target-feature -Xclang -packed-fp32-ops"
-SRCS="gemm_mfma.hip skbuf_summary.hip c_abi_gemm.hip runtime.hip"
-OBJS=""
 mkdir -p build
-for s in $SRCS; do
+OBJS=""
+PIDS=""
+for s in gemm_mfma.hip skbuf_summary.hip c_abi_gemm.hip runtime.hip; do
   o=build/${s%.hip}.o
-  $HIPCC $FLAGS -c "$s" -o "$o" 2> >(grep -v "packed-fp32-ops" >&2) &
+  # the host pass does not know the packed-fp32 target feature and says so: harmless
+  ( $HIPCC $HIPFLAGS -c "$s" -o "$o" 2>&1 | grep -v "packed-fp32-ops" >&2; exit ${PIPESTATUS[0]} ) &
+  PIDS="$PIDS $!"
   OBJS="$OBJS $o"
 done
-wait
-$HIPCC --offload-arch=gfx950 -shared -fPIC -o ../libdragon_hip.so $OBJS
+for s in ../engine/dragon_engine.cpp ../engine/engine_c_api.cpp; do
+  o=build/$(basename "${s%.cpp}").o
+  g++ -O2 -std=c++17 -fPIC -Wall -c "$s" -o "$o" &
+  PIDS="$PIDS $!"
+  OBJS="$OBJS $o"
+done
+for p in $PIDS; do
+  wait "$p" || { echo "build.sh: a compile step failed" >&2; exit 1; }
+done
+$HIPCC --offload-arch=gfx950 -shared -fPIC -o ../libdragon_hip.so $OBJS || exit 1
 echo "built $(cd .. && pwd)/libdragon_hip.so"

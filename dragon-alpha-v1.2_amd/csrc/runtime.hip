@@ -42,6 +42,13 @@ __global__ void fill2d_kernel(float* __restrict__ X, float value, int height, in
     }
 }
 
+// dst[i] = src[i] as float4: the plain copy that HBM byte counters are calibrated against
+__global__ void copy4_kernel(v4f* __restrict__ dst, const v4f* __restrict__ src, long long n4) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride)
+        dst[i] = src[i];
+}
+
 int launch_blocks(long long n, int threads) {
     long long b = (n + threads - 1) / threads;
     if (b < 1) b = 1;
@@ -242,6 +249,15 @@ int dragon_Cuda_set2D_value(int64_t stream, int64_t address, float value, int32_
     hipLaunchKernelGGL(fill2d_kernel, dim3(launch_blocks((long long)height * stride, 256)),
                        dim3(256), 0, as_stream(stream), (float*)as_ptr(address), value, height,
                        width, stride);
+    return note(hipGetLastError());
+}
+
+int dragon_Cuda_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t length) {
+    if (dst == 0 || src == 0 || length <= 0 || (length & 3) || ((dst | src) & 15))
+        return note(hipErrorInvalidValue);
+    const long long n4 = length >> 2;
+    hipLaunchKernelGGL(copy4_kernel, dim3(launch_blocks(n4, 256)), dim3(256), 0, as_stream(stream),
+                       (v4f*)as_ptr(dst), (const v4f*)as_ptr(src), n4);
     return note(hipGetLastError());
 }
 

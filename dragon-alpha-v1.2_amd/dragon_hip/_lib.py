@@ -1,5 +1,5 @@
 """ctypes binding of libdragon_hip.so: the C ABI declared in include/dragon_hip_gemm.h
-and include/dragon_hip_runtime.h.
+and include/dragon_hip_runtime.h, and the host-side engine of include/dragon_hip_engine.h.
 
 The library is loaded from the package directory.  There is no fallback: if the shared
 object is missing or a symbol cannot be resolved the import fails, and every compute
@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "libdragon_hip.so")
 i32, i64, f32 = c_int32, c_int64, c_float
 p_i64 = POINTER(c_int64)
 p_f32 = POINTER(c_float)
+p_i32 = POINTER(c_int32)
 
 # name -> (restype, argtypes); mirrors the two public headers one to one
 _MM2D = [p_i64, i32, i64, i64, i64, i32, i32, i32]
@@ -91,6 +92,34 @@ SIGNATURES = {
     "dragon_Cuda_get2D_v2": (i32, [i64, i64, c_void_p, i64, i32, i32, i32]),
     "dragon_Cuda_set1D_v2": (i32, [i64, i64, c_void_p, i64, i32]),
     "dragon_Cuda_set2D_v2": (i32, [i64, i64, c_void_p, i64, i32, i32, i32]),
+    "dragon_Cuda_copy1D_kernel": (i32, [i64, i64, i64, i64]),
+    # include/dragon_hip_engine.h
+    "dragon_engine_last_error": (c_char_p, []),
+    "dragon_engine_last_cuda_code": (i32, []),
+    "dragon_engine_cuda_float32": (c_void_p, [i32, i32]),
+    "dragon_engine_delete": (None, [c_void_p]),
+    "dragon_engine_check": (i32, [c_void_p, i32]),
+    "dragon_engine_sync": (i32, [c_void_p, i32]),
+    "dragon_engine_set_param": (i32, [c_void_p, c_char_p, i32]),
+    "dragon_engine_get_param": (i32, [c_void_p, c_char_p]),
+    "dragon_engine_gridZ": (i32, [c_void_p, i32, i32, i32, i32]),
+    "dragon_policy_gridZ": (i32, [i32, i32, i32, i32, i32]),
+    "dragon_policy_smooth_maxPart": (i32, [i32]),
+    "dragon_engine_empty": (c_void_p, [c_void_p, p_i32, i32]),
+    "dragon_engine_zeros": (c_void_p, [c_void_p, p_i32, i32]),
+    "dragon_engine_tensor": (c_void_p, [c_void_p, c_void_p, i32, p_i32, i32]),
+    "dragon_engine_set": (i32, [c_void_p, c_void_p, c_void_p, i32]),
+    "dragon_engine_valueOf": (i32, [c_void_p, c_void_p, c_void_p, i32]),
+    "dragon_engine_delete_tensor": (i32, [c_void_p, c_void_p]),
+    "dragon_tensor_c": (i32, [c_void_p]),
+    "dragon_tensor_ndim": (i32, [c_void_p]),
+    "dragon_tensor_dim": (i32, [c_void_p, i32]),
+    "dragon_tensor_length": (i32, [c_void_p]),
+    "dragon_tensor_lengthv": (i32, [c_void_p]),
+    "dragon_tensor_length_4x": (i32, [c_void_p]),
+    "dragon_tensor_address": (i64, [c_void_p]),
+    "dragon_engine_product": (c_void_p, [c_void_p, i32, i32, c_void_p, c_void_p]),
+    "dragon_engine_product_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
 }
 
 

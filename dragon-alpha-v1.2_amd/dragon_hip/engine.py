@@ -1,0 +1,173 @@
+"""Python face of the host-side engine mirror: Engine / Tensor with the reference's method
+names (alpha.engine.cuda_float32, eg.tensor, eg.matMul, eg.batchMatMulT2, eg.valueOf ...).
+All logic lives in the C++ classes behind include/dragon_hip_engine.h."""
+import ctypes
+
+import numpy as np
+
+from . import lib, CudaException
+
+
+class NullPointerException(RuntimeError):
+    pass
+
+
+class IllegalArgumentException(ValueError):
+    pass
+
+
+def _raise(code):
+    msg = (lib.dragon_engine_last_error() or b"").decode()
+    if code == 1:
+        raise NullPointerException(msg)
+    if code == 2:
+        raise IllegalArgumentException(msg)
+    if code == 3:
+        raise CudaException(lib.dragon_engine_last_cuda_code())
+    raise RuntimeError(msg)
+
+
+def _last_code():
+    # pointer-returning entry points report through the thread's last error only
+    msg = (lib.dragon_engine_last_error() or b"").decode()
+    return msg
+
+
+def _dims(dim):
+    arr = (ctypes.c_int32 * len(dim))(*[int(d) for d in dim])
+    return arr, len(dim)
+
+
+class Tensor:
+    def __init__(self, eg, handle):
+        self._eg, self._h = eg, handle
+
+    def c(self):
+        rc = lib.dragon_tensor_c(self._h)
+        if rc:
+            _raise(rc)
+        return self
+
+    @property
+    def dim(self):
+        return [lib.dragon_tensor_dim(self._h, i) for i in range(lib.dragon_tensor_ndim(self._h))]
+
+    def ndim(self):
+        return lib.dragon_tensor_ndim(self._h)
+
+    length = property(lambda self: lib.dragon_tensor_length(self._h))
+    lengthv = property(lambda self: lib.dragon_tensor_lengthv(self._h))
+    length_4x = property(lambda self: lib.dragon_tensor_length_4x(self._h))
+    address = property(lambda self: lib.dragon_tensor_address(self._h))
+
+    def value(self):
+        return self._eg.valueOf(self)
+
+
+MATMUL, MATMUL_T1, MATMUL_T2, BMM, BMM_T1, BMM_T2 = range(6)
+
+
+class Engine:
+    """alpha.engine.cuda_float32(deviceId, ...)"""
+
+    def __init__(self, device_id=0, stream_pool_size=32):
+        self._h = lib.dragon_engine_cuda_float32(device_id, stream_pool_size)
+        if not self._h:
+            msg = _last_code()
+            code = lib.dragon_engine_last_cuda_code()
+            raise CudaException(code) if code else RuntimeError(msg)
+
+    def close(self):
+        if self._h:
+            lib.dragon_engine_delete(self._h)
+            self._h = None
+
+    def check(self, flag):
+        lib.dragon_engine_check(self._h, int(flag))
+        return self
+
+    def sync(self, flag):
+        lib.dragon_engine_sync(self._h, int(flag))
+        return self
+
+    def set_param(self, name, value):
+        rc = lib.dragon_engine_set_param(self._h, name.encode(), int(value))
+        if rc:
+            _raise(rc)
+        return self
+
+    def get_param(self, name):
+        return lib.dragon_engine_get_param(self._h, name.encode())
+
+    def gridZ(self, kind, N, M, K):
+        return lib.dragon_engine_gridZ(self._h, kind, N, M, K)
+
+    # ---- tensors ----
+    def _wrap(self, h):
+        if not h:
+            msg = _last_code()
+            if "null" in msg.lower():
+                raise NullPointerException(msg)
+            code = lib.dragon_engine_last_cuda_code()
+            if msg.startswith("hip") and code:
+                raise CudaException(code)
+            raise IllegalArgumentException(msg)
+        return Tensor(self, h)
+
+    def empty(self, *dim):
+        arr, n = _dims(dim)
+        return self._wrap(lib.dragon_engine_empty(self._h, arr, n))
+
+    def zeros(self, *dim):
+        arr, n = _dims(dim)
+        return self._wrap(lib.dragon_engine_zeros(self._h, arr, n))
+
+    def tensor(self, value, *dim):
+        v = np.ascontiguousarray(value, dtype=np.float32).reshape(-1)
+        arr, n = _dims(dim)
+        return self._wrap(lib.dragon_engine_tensor(self._h, v.ctypes.data, v.size, arr, n))
+
+    def valueOf(self, ts):
+        out = np.empty(ts.length, dtype=np.float32)
+        rc = lib.dragon_engine_valueOf(self._h, ts._h, out.ctypes.data, out.size)
+        if rc:
+            _raise(rc)
+        return out
+
+    def delete(self, *tensors):
+        for t in tensors:
+            if t is not None and t._h:
+                lib.dragon_engine_delete_tensor(self._h, t._h)
+                t._h = None
+
+    # ---- products ----
+    def _product(self, op, args, likeA=True):
+        hs = [a._h if a is not None else None for a in args]
+        if len(args) == 2:
+            return self._wrap(lib.dragon_engine_product(self._h, op, int(likeA), hs[0], hs[1]))
+        rc = lib.dragon_engine_product_into(self._h, op, hs[0], hs[1], hs[2])
+        if rc:
+            _raise(rc)
+        return args[0]
+
+    def matMul(self, *t):
+        return self._product(MATMUL, t)
+
+    def matMulT1(self, *t):
+        return self._product(MATMUL_T1, t)
+
+    def matMulT2(self, *t):
+        return self._product(MATMUL_T2, t)
+
+    def batchMatMul(self, *t, likeA=True):
+        return self._product(BMM, t, likeA)
+
+    def batchMatMulT1(self, *t, likeA=True):
+        return self._product(BMM_T1, t, likeA)
+
+    def batchMatMulT2(self, *t, likeA=True):
+        return self._product(BMM_T2, t, likeA)
+
+
+def cuda_float32(device_id=0, stream_pool_size=32):
+    return Engine(device_id, stream_pool_size)

@@ -1,0 +1,835 @@
+// Implementation of the host-side mirror declared in dragon_engine.hpp.  Every device
+// action goes through the C ABI (dragon_Cuda_* entry points); no HIP call is made here.
+#include "dragon_engine.hpp"
+
+#include <string.h>
+
+#include "../../include/dragon_hip_gemm.h"
+#include "../../include/dragon_hip_runtime.h"
+
+namespace dragon {
+
+namespace {
+
+inline int pad4(int x) { return ((x + 3) >> 2) << 2; }
+
+inline void cu(int code) {
+    if (code != 0) throw CudaException(code);
+}
+inline int64_t cu_handle(int64_t h) {
+    if (h == 0) {
+        int code = dragon_Cuda_getLastExceptionType();
+        throw CudaException(code ? code : 2);
+    }
+    return h;
+}
+
+std::string fmt(const char* f, long long a = 0, long long b = 0) {
+    char buf[256];
+    snprintf(buf, sizeof(buf), f, a, b);
+    return buf;
+}
+
+// streams -> streams[0]  (CudaFloat32EngineBase.java:649-654)
+void sync_streamArray_2_stream0(const std::vector<int64_t>& streams) {
+    int64_t event1 = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+    cu(dragon_Cuda_eventRecord_streams(event1, streams.data(), (int)streams.size()));
+    cu(dragon_Cuda_streamWaitEvent_default(streams[0], event1));
+    cu(dragon_Cuda_deleteEvent(event1));
+}
+
+// CudaFloat32EngineBase.java:657-694
+class StreamArraySyncer : public Syncer {
+public:
+    StreamArraySyncer(CudaStreamPool* pool, std::vector<int64_t> streams)
+        : pool_(pool), streams_(std::move(streams)) {
+        sync_streamArray_2_stream0(streams_);
+        event_ = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        cu(dragon_Cuda_eventRecord(event_, streams_[0]));
+    }
+    // The reference's finalizer drops the event without waiting; waiting is the safe
+    // reading of the same protocol, and a completed syncer makes this a no-op.
+    ~StreamArraySyncer() override {
+        try { sync(); } catch (...) {}
+    }
+    void sync() override {
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            if (called_) return;
+            cu(dragon_Cuda_eventSync_Del(event_));
+            called_ = true;
+        }
+        pool_->returnStreamArray(streams_);
+    }
+private:
+    CudaStreamPool* pool_;
+    std::vector<int64_t> streams_;
+    int64_t event_ = 0;
+    bool called_ = false;
+    std::mutex mu_;
+};
+
+// CudaFloat32EngineBase.java:1008-1054: completion of the reduction on streams[0], then the
+// partial-product buffer goes back to the core
+class SplitKSyncer : public Syncer {
+public:
+    SplitKSyncer(EngineCore* core, EngineCore::Block block, CudaStreamPool* pool,
+                 std::vector<int64_t> streams)
+        : core_(core), block_(block), pool_(pool), streams_(std::move(streams)) {
+        event_ = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        cu(dragon_Cuda_eventRecord(event_, streams_[0]));
+    }
+    ~SplitKSyncer() override {
+        try { sync(); } catch (...) {}
+    }
+    void sync() override {
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            if (called_) return;
+            cu(dragon_Cuda_eventSync_Del(event_));
+            called_ = true;
+        }
+        core_->free(block_.size, block_.address);
+        pool_->returnStreamArray(streams_);
+    }
+private:
+    EngineCore* core_;
+    EngineCore::Block block_;
+    CudaStreamPool* pool_;
+    std::vector<int64_t> streams_;
+    int64_t event_ = 0;
+    bool called_ = false;
+    std::mutex mu_;
+};
+
+// one stream, one event (StreamSyncer of the reference, used by memset)
+class StreamSyncer : public Syncer {
+public:
+    StreamSyncer(CudaStreamPool* pool, int64_t stream) : pool_(pool), stream_(stream) {
+        event_ = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        cu(dragon_Cuda_eventRecord(event_, stream_));
+    }
+    ~StreamSyncer() override {
+        try { sync(); } catch (...) {}
+    }
+    void sync() override {
+        if (called_) return;
+        cu(dragon_Cuda_eventSync_Del(event_));
+        called_ = true;
+        pool_->returnStream(stream_);
+    }
+private:
+    CudaStreamPool* pool_;
+    int64_t stream_, event_ = 0;
+    bool called_ = false;
+};
+
+std::mutex g_cuda_class_lock;  // the reference serialises setDevice+malloc/free on Cuda.class
+
+}  // namespace
+
+CudaException::CudaException(int c)
+    : std::runtime_error(std::string(dragon_Cuda_getExceptionName(c) ? dragon_Cuda_getExceptionName(c)
+                                                                      : "hipError") +
+                         " (" + std::to_string(c) + ")"),
+      code(c) {}
+
+// ---- CudaDevice ----------------------------------------------------------------------------
+CudaDevice::CudaDevice(int id) : id_(id), sm_count_(0) {
+    sm_count_ = dragon_CudaDevice_multiProcessorCount(id);
+    if (sm_count_ <= 0) throw CudaException(dragon_Cuda_getLastExceptionType());
+}
+
+// ---- CudaStreamPool ---------------------------------------------------------------------------
+CudaStreamPool::CudaStreamPool(const CudaDevice& dev, int max_streamsize, int max_getsize_oneturn)
+    : dev_id_(dev.getId()), max_streamsize_(max_streamsize),
+      max_getsize_oneturn_(max_getsize_oneturn) {
+    if (max_streamsize <= 0) throw IllegalArgumentException("max_streamsize must be positive");
+    if (max_getsize_oneturn_ > max_streamsize_) max_getsize_oneturn_ = max_streamsize_;
+}
+CudaStreamPool::~CudaStreamPool() {
+    if (!gc_.empty()) dragon_Cuda_deleteStreams(gc_.data(), (int)gc_.size());
+}
+void CudaStreamPool::init() {
+    std::lock_guard<std::mutex> g(g_cuda_class_lock);
+    cu(dragon_Cuda_setDevice(dev_id_));
+    for (int i = 0; i < max_streamsize_; i++) gc_.push_back(cu_handle(dragon_Cuda_newStream_Blocking()));
+}
+int64_t CudaStreamPool::getStream() {
+    std::lock_guard<std::mutex> g(mu_);
+    if (!inited_) { init(); inited_ = true; }
+    int64_t s = gc_[gc_index_];
+    gc_index_ = (gc_index_ + 1) % max_streamsize_;
+    return s;
+}
+std::vector<int64_t> CudaStreamPool::getStreamArray(int length) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (!inited_) { init(); inited_ = true; }
+    if (length > max_getsize_oneturn_) length = max_getsize_oneturn_;
+    std::vector<int64_t> streams((size_t)length);
+    for (int i = 0; i < length; i++) {
+        streams[i] = gc_[gc_index_];
+        gc_index_ = (gc_index_ + 1) % max_streamsize_;
+    }
+    return streams;
+}
+int CudaStreamPool::total_stream_size() {
+    std::lock_guard<std::mutex> g(mu_);
+    return (int)gc_.size();
+}
+
+// ---- CudaFloat32EngineBase ------------------------------------------------------------------------
+CudaFloat32EngineBase::CudaFloat32EngineBase(int deviceId, int streamPool_maxsize)
+    : dev_(deviceId) {
+    streamPool_.reset(new CudaStreamPool(dev_, streamPool_maxsize, 16));
+    recomputeMaxParts();
+}
+
+void CudaFloat32EngineBase::recomputeMaxParts() {     // CudaFloat32EngineBase.java:86-92
+    const int SM_count = dev_.multiProcessorCount();
+    matMul_sk_maxPart = policy_smooth_maxPart(SM_count);
+    matMulT1_sk_maxPart = policy_smooth_maxPart(SM_count);
+    matMulT2_sk_maxPart = policy_smooth_maxPart(SM_count);
+}
+
+static void check_threshold(int threshold) {
+    if (threshold <= 0 || (threshold & (threshold - 1)) != 0)
+        throw IllegalArgumentException(fmt("threshold { got %lld } must be a power of 2", threshold));
+}
+static void check_maxPart(int maxPart) {
+    if (maxPart < 4) throw IllegalArgumentException(fmt("maxPartNum { got %lld } must >= 4", maxPart));
+}
+void CudaFloat32EngineBase::matMul_splitK_threshold(int t) { check_threshold(t); matMul_sk_threshold = t; }
+void CudaFloat32EngineBase::matMul_splitK_maxPart(int p) { check_maxPart(p); matMul_sk_maxPart = p; }
+void CudaFloat32EngineBase::matMulT1_splitK_threshold(int t) { check_threshold(t); matMulT1_sk_threshold = t; }
+void CudaFloat32EngineBase::matMulT1_maxPart(int p) { check_maxPart(p); matMulT1_sk_maxPart = p; }
+void CudaFloat32EngineBase::matMulT2_splitK_threshold(int t) { check_threshold(t); matMulT2_sk_threshold = t; }
+void CudaFloat32EngineBase::matMulT2_splitK_maxPart(int p) { check_maxPart(p); matMulT2_sk_maxPart = p; }
+void CudaFloat32EngineBase::tf32(bool flag) {
+    matMul_tf32 = matMulT1_tf32 = matMulT2_tf32 = flag;
+    batchMatMul_tf32 = batchMatMulT1_tf32 = batchMatMulT2_tf32 = flag;
+}
+
+// ---- split-K policy as pure functions of (shape, unit count, knobs) ---------------------------
+// The restriction block shared by the three products (e.g. CudaFloat32EngineBase.java:1551-1562).
+// All arithmetic in float, truncation where Java casts to int.
+static int policy_clamp(float fGridZ, int K, int b, int SM, float maxBlock, int maxPart) {
+    if (fGridZ < 1.8f) return 1;
+    int GridZ = (int)fGridZ;
+    int GridZ2 = K >> 8;
+    if (GridZ > GridZ2) GridZ = GridZ2;
+    float coef = (float)K / ((float)K + 4096.0f);
+    int GridZ3 = (int)((float)SM * maxBlock * coef / (float)b);
+    if (GridZ > GridZ3) GridZ = GridZ3;
+    if (GridZ < 2) GridZ = 2; else GridZ = (GridZ + 3) >> 2 << 2;
+    if (GridZ > maxPart) GridZ = maxPart;
+    return GridZ;
+}
+
+int policy_smooth_maxPart(int x) {   // CudaFloat32EngineBase.java:70-74
+    if (x <= 32) x = (x + 3) >> 2 << 2; else x = (x + 7) >> 3 << 3;
+    return x < 16 ? 16 : (x > 128 ? 128 : x);
+}
+
+int policy_matMul_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k) {   // :1523-1532
+    float fGridZ = 1; int b0 = 1;
+    if (K >= k.threshold) {
+        b0 = dragon_Cuda_matMul_blockNum(N, M);
+        float expect_block_perSM = k.minBlock_perSM + 0.4f * (float)K / ((float)K + 1024.0f);
+        if ((float)b0 < (float)SM * expect_block_perSM) {
+            int b1 = dragon_Cuda_matMul_blockNum(K, M);
+            int b2 = dragon_Cuda_matMul_blockNum(N, K);
+            fGridZ = (float)(b1 + b2) / ((float)b0 * 2.0f);
+        }
+    }
+    return policy_clamp(fGridZ, K, b0, SM, k.maxBlock_perSM, k.maxPart);
+}
+
+int policy_matMulT1_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k) {  // :1740-1749
+    float fGridZ = 1; int b1 = 1;
+    if (K >= k.threshold) {
+        b1 = dragon_Cuda_matMul_blockNum(N, M);
+        float expect_block_perSM = k.minBlock_perSM + (float)K / ((float)K + 1024.0f);
+        if ((float)b1 < (float)SM * expect_block_perSM) {
+            int b0 = dragon_Cuda_matMul_blockNum(K, N);
+            int b2 = dragon_Cuda_matMul_blockNum(K, M);
+            fGridZ = (float)(b0 + b2) / ((float)b1 * 2.0f);
+        }
+    }
+    return policy_clamp(fGridZ, K, b1, SM, k.maxBlock_perSM, k.maxPart);
+}
+
+// :1859-1867 and :1894 -- the reference tests blockNum(N,K) against the matMul (not matMulT2)
+// block constants here and clamps with them; threshold and maxPart are the T2 fields.
+int policy_matMulT2_gridZ(int N, int M, int K, int SM, const SplitKKnobs& t2, const SplitKKnobs& mm) {
+    float fGridZ = 1; int b2 = 1;
+    if (K >= t2.threshold) {
+        b2 = dragon_Cuda_matMul_blockNum(N, K);
+        float expect_block_perSM = mm.minBlock_perSM + (float)K / ((float)K + 1024.0f);
+        if ((float)b2 < (float)SM * expect_block_perSM) {
+            int b0 = dragon_Cuda_matMul_blockNum(N, M);
+            int b1 = dragon_Cuda_matMul_blockNum(K, M);
+            fGridZ = (float)(b1 + b2) / ((float)b0 * 2.0f);
+        }
+    }
+    return policy_clamp(fGridZ, K, b2, SM, mm.maxBlock_perSM, t2.maxPart);
+}
+
+int CudaFloat32EngineBase::matMul_gridZ(int N, int M, int K) const {
+    SplitKKnobs k = {matMul_sk_threshold, matMul_sk_maxPart, matMul_sk_minBlock_perSM, matMul_sk_maxBlock_perSM};
+    return policy_matMul_gridZ(N, M, K, dev_.multiProcessorCount(), k);
+}
+int CudaFloat32EngineBase::matMulT1_gridZ(int N, int M, int K) const {
+    SplitKKnobs k = {matMulT1_sk_threshold, matMulT1_sk_maxPart, matMulT1_sk_minBlock_perSM, matMulT1_sk_maxBlock_perSM};
+    return policy_matMulT1_gridZ(N, M, K, dev_.multiProcessorCount(), k);
+}
+int CudaFloat32EngineBase::matMulT2_gridZ(int N, int M, int K) const {
+    SplitKKnobs t2 = {matMulT2_sk_threshold, matMulT2_sk_maxPart, matMulT2_sk_minBlock_perSM, matMulT2_sk_maxBlock_perSM};
+    SplitKKnobs mm = {matMul_sk_threshold, matMul_sk_maxPart, matMul_sk_minBlock_perSM, matMul_sk_maxBlock_perSM};
+    return policy_matMulT2_gridZ(N, M, K, dev_.multiProcessorCount(), t2, mm);
+}
+
+int64_t CudaFloat32EngineBase::malloc(int64_t memsize) {   // :1148-1156
+    std::lock_guard<std::mutex> g(g_cuda_class_lock);
+    cu(dragon_Cuda_setDevice(dev_.getId()));
+    return cu_handle(dragon_Cuda_malloc(memsize));
+}
+void CudaFloat32EngineBase::free(int64_t address) {        // :1158-1164
+    std::lock_guard<std::mutex> g(g_cuda_class_lock);
+    cu(dragon_Cuda_setDevice(dev_.getId()));
+    cu(dragon_Cuda_free(address));
+}
+SyncerPtr CudaFloat32EngineBase::memset(int64_t address, int value, int64_t memsize) {  // :1166-1171
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_memsetAsync(stream, address, value, memsize));
+    return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
+}
+void CudaFloat32EngineBase::get1D(int64_t address, float* value, int length) {
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_get1D(stream, address, value, length));
+    streamPool_->returnStream(stream);
+}
+void CudaFloat32EngineBase::get2D(int64_t address, float* value, int height, int width, int stride) {
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_get2D(stream, address, value, height, width, stride));
+    streamPool_->returnStream(stream);
+}
+void CudaFloat32EngineBase::set1D(int64_t address, const float* value, int length) {
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_set1D(stream, address, value, length));
+    streamPool_->returnStream(stream);
+}
+void CudaFloat32EngineBase::set2D(int64_t address, const float* value, int height, int width, int stride) {
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_set2D(stream, address, value, height, width, stride));
+    streamPool_->returnStream(stream);
+}
+
+// Shared body of matMul / matMulT1 / matMulT2 (:1534-1589, :1751-1806, :1870-1925)
+SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64_t A, int64_t B,
+                                        int N, int M, int K) {
+    const int length = dragon_Cuda_matMul_nstream(N, M);
+    std::vector<int64_t> streamArray = streamPool_->getStreamArray(length);
+    const int n = (int)streamArray.size();
+    last_gridZ = GridZ;
+    last_stream_count = n;
+    const bool big = (N > 127) && (M > 127) && (K % 8 == 0);
+    if (GridZ < 2) {   // no need to split
+        int rc;
+        if (variant == 0)
+            rc = (matMul_tf32 && big)
+                     ? dragon_Cuda_matMul_matMul_mma(streamArray.data(), n, A, B, C, N, M, K)
+                     : dragon_Cuda_matMul_matMul(streamArray.data(), n, A, B, C, N, M, K);
+        else if (variant == 1)
+            rc = (matMulT1_tf32 && big)
+                     ? dragon_Cuda_matMul_matMulT1_mma(streamArray.data(), n, A, B, C, N, M, K)
+                     : dragon_Cuda_matMul_matMulT1(streamArray.data(), n, A, B, C, N, M, K);
+        else
+            rc = (matMulT2_tf32 && big)
+                     ? dragon_Cuda_matMul_matMulT2_mma(streamArray.data(), n, A, B, C, N, M, K)
+                     : dragon_Cuda_matMul_matMulT2(streamArray.data(), n, A, B, C, N, M, K);
+        cu(rc);
+        return SyncerPtr(new StreamArraySyncer(streamPool_.get(), streamArray));
+    }
+    // split K to improve parallelism
+    const int part = GridZ - 1;
+    const int sizeC = N * M;
+    if (core_ == nullptr) throw NullPointerException("engine core is not bound");
+    EngineCore::Block block = core_->malloc(sizeC * part);
+    const int64_t Cbuf = block.address;
+    try {
+        // stage 1: local products
+        int rc;
+        if (variant == 0)
+            rc = dragon_Cuda_matMul_matMulSK(streamArray.data(), n, GridZ, A, B, C, Cbuf, N, M, K);
+        else if (variant == 1)
+            rc = dragon_Cuda_matMul_matMulT1SK(streamArray.data(), n, GridZ, A, B, C, Cbuf, N, M, K);
+        else
+            rc = dragon_Cuda_matMul_matMulT2SK(streamArray.data(), n, GridZ, A, B, C, Cbuf, N, M, K);
+        cu(rc);
+        // stage 2: global reduction on streams[0] once every stream has finished stage 1
+        int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        cu(dragon_Cuda_eventRecord_streams(event, streamArray.data(), n));
+        const int64_t stream = streamArray[0];
+        cu(dragon_Cuda_streamWaitEvent_default(stream, event));
+        cu(dragon_Cuda_matMul_SKbuf_summary(stream, Cbuf, C, part, sizeC));
+        cu(dragon_Cuda_deleteEvent(event));
+    } catch (...) {
+        core_->free(block.size, block.address);
+        throw;
+    }
+    return SyncerPtr(new SplitKSyncer(core_, block, streamPool_.get(), streamArray));
+}
+
+SyncerPtr CudaFloat32EngineBase::matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K) {
+    return run_2d(0, matMul_gridZ(N, M, K), C, A, B, N, M, K);
+}
+SyncerPtr CudaFloat32EngineBase::matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K) {
+    return run_2d(1, matMulT1_gridZ(N, M, K), C, A, B, N, M, K);
+}
+SyncerPtr CudaFloat32EngineBase::matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K) {
+    return run_2d(2, matMulT2_gridZ(N, M, K), C, A, B, N, M, K);
+}
+
+SyncerPtr CudaFloat32EngineBase::batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N,
+                                             int M, int BK, int AK) {   // :1939-1959
+    const int length = dragon_Cuda_batchMatMul_streamSize(N, M);
+    std::vector<int64_t> s = streamPool_->getStreamArray(length);
+    const int n = (int)s.size();
+    last_gridZ = 1; last_stream_count = n;
+    int rc;
+    if (batchMatMul_tf32 && (N > 127) && (M > 127) && (BK % 2 == 0) && (BK > 7))
+        rc = dragon_Cuda_batchMatMul_batchMatMul_mma(batchMatMul_useTexture, s.data(), n, A, B, C,
+                                                     Batch, N, M, BK, AK);
+    else if (batchMatMul_useTexture)
+        rc = dragon_Cuda_batchMatMul_batchMatMul_texture(s.data(), n, A, B, C, Batch, N, M, BK, AK);
+    else
+        rc = dragon_Cuda_batchMatMul_batchMatMul(s.data(), n, A, B, C, Batch, N, M, BK, AK);
+    cu(rc);
+    return SyncerPtr(new StreamArraySyncer(streamPool_.get(), s));
+}
+
+SyncerPtr CudaFloat32EngineBase::batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN,
+                                               int AN, int M, int K) {  // :1966-1981
+    const int length = dragon_Cuda_batchMatMul_streamSize(CN, M);
+    std::vector<int64_t> s = streamPool_->getStreamArray(length);
+    const int n = (int)s.size();
+    last_gridZ = 1; last_stream_count = n;
+    int rc;
+    if (batchMatMulT1_tf32 && (CN > 127) && (M > 127) && (K > 7))
+        rc = dragon_Cuda_batchMatMul_batchMatMulT1_mma(s.data(), n, A, B, C, Batch, CN, AN, M, K);
+    else
+        rc = dragon_Cuda_batchMatMul_batchMatMulT1(s.data(), n, A, B, C, Batch, CN, AN, M, K);
+    cu(rc);
+    return SyncerPtr(new StreamArraySyncer(streamPool_.get(), s));
+}
+
+SyncerPtr CudaFloat32EngineBase::batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N,
+                                               int CM, int BM, int K) { // :1995-2017
+    const int length = dragon_Cuda_batchMatMul_streamSize(N, CM);
+    std::vector<int64_t> s = streamPool_->getStreamArray(length);
+    const int n = (int)s.size();
+    last_gridZ = 1; last_stream_count = n;
+    const bool useTexture = batchMatMulT2_useTexture && (N > 47) && (CM > 47);
+    int rc;
+    if (batchMatMulT2_tf32 && (N > 127) && (CM > 127) && (K > 7))
+        rc = dragon_Cuda_batchMatMul_batchMatMulT2_mma(batchMatMulT2_useTexture, s.data(), n, A, B, C,
+                                                       Batch, N, CM, BM, K);
+    else if (useTexture)
+        rc = dragon_Cuda_batchMatMul_batchMatMulT2_texture(s.data(), n, A, B, C, Batch, N, CM, BM, K);
+    else
+        rc = dragon_Cuda_batchMatMul_batchMatMulT2(s.data(), n, A, B, C, Batch, N, CM, BM, K);
+    cu(rc);
+    return SyncerPtr(new StreamArraySyncer(streamPool_.get(), s));
+}
+
+// ---- EngineCore ---------------------------------------------------------------------------------------
+EngineCore::EngineCore(CudaFloat32EngineBase* base, bool chk) : check(chk), base_(base) {
+    base_->engineCore(this);
+}
+
+EngineCore::Block EngineCore::malloc(int mem_length) {
+    if (check && mem_length <= 0)
+        throw IllegalArgumentException(fmt("mem_length { got %lld } must be positive", mem_length));
+    Block b;
+    b.size = (int64_t)mem_length * 4;
+    b.address = base_->malloc(b.size);
+    std::lock_guard<std::mutex> g(mu_);
+    live_blocks_++;
+    return b;
+}
+void EngineCore::free(int64_t, int64_t address) {
+    if (address == 0) return;
+    base_->free(address);
+    std::lock_guard<std::mutex> g(mu_);
+    live_blocks_--;
+}
+SyncerPtr EngineCore::memset(int64_t address, int value, int length) {
+    if (check) {
+        if (address == 0) throw NullPointerException("Tensor is null");
+        if (length <= 0) throw IllegalArgumentException(fmt("length { got %lld } must > 0", length));
+    }
+    return base_->memset(address, value, (int64_t)length * 4);
+}
+void EngineCore::get1D(int64_t address, float* value, int length) {
+    if (check && address == 0) throw NullPointerException("Tensor is null");
+    base_->get1D(address, value, length);
+}
+void EngineCore::get2D(int64_t address, float* value, int height, int width) {
+    if (check && address == 0) throw NullPointerException("Tensor is null");
+    base_->get2D(address, value, height, width, pad4(width));
+}
+void EngineCore::set1D(int64_t address, const float* value, int length) {
+    if (check && address == 0) throw NullPointerException("Tensor is null");
+    base_->set1D(address, value, length);
+}
+void EngineCore::set2D(int64_t address, const float* value, int length, int width) {
+    if (check) {
+        if (address == 0) throw NullPointerException("Tensor is null");
+        if (width <= 0 || length % width != 0)
+            throw IllegalArgumentException(fmt("value.length { got %lld } %% width { got %lld } != 0", length, width));
+    }
+    base_->set2D(address, value, length / width, width, pad4(width));
+}
+
+void EngineCore::matMul_check(int64_t C, int64_t A, int64_t B, int N, int M, int K) const {  // :695-705
+    if (C == 0) throw NullPointerException("Tensor C is null");
+    if (B == 0) throw NullPointerException("Tensor B is null");
+    if (A == 0) throw NullPointerException("Tensor A is null");
+    if (N <= 0) throw IllegalArgumentException(fmt("N { got %lld } must > 0", N));
+    if (M <= 0) throw IllegalArgumentException(fmt("M { got %lld } must > 0", M));
+    if (K <= 0) throw IllegalArgumentException(fmt("K { got %lld } must > 0", K));
+}
+
+SyncerPtr EngineCore::matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K) {    // :708-717
+    if (check) matMul_check(C, A, B, N, M, K);
+    return base_->matMul(C, A, B, pad4(N), pad4(M), pad4(K));
+}
+SyncerPtr EngineCore::matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K) {  // :743-752
+    if (check) matMul_check(C, A, B, N, M, K);
+    return base_->matMulT1(C, A, B, pad4(N), pad4(M), pad4(K));
+}
+SyncerPtr EngineCore::matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K) {  // :755-764
+    if (check) matMul_check(C, A, B, N, M, K);
+    return base_->matMulT2(C, A, B, pad4(N), pad4(M), pad4(K));
+}
+SyncerPtr EngineCore::batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K) {  // :767-780
+    if (check) {
+        if (Batch <= 0) throw IllegalArgumentException("Batch MatMul: Batch must be positive");
+        matMul_check(C, A, B, N, M, K);
+    }
+    // A[Batch, N, AK] * B[Batch, BK, M] = C[Batch, N, M]
+    return base_->batchMatMul(C, A, B, pad4(Batch), N, pad4(M), K, pad4(K));
+}
+SyncerPtr EngineCore::batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K) {  // :782-795
+    if (check) {
+        if (Batch <= 0) throw IllegalArgumentException("Batch MatMul: Batch must be positive");
+        matMul_check(C, A, B, N, M, K);
+    }
+    // (A[Batch, K, AN])^T * B[Batch, K, M] = C[Batch, CN, M]
+    return base_->batchMatMulT1(C, A, B, pad4(Batch), N, pad4(N), pad4(M), K);
+}
+SyncerPtr EngineCore::batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K) {  // :797-810
+    if (check) {
+        if (Batch <= 0) throw IllegalArgumentException("Batch MatMul: Batch must be positive");
+        matMul_check(C, A, B, N, M, K);
+    }
+    // A[Batch, N, K] * (B[Batch, BM, K])^T = C[Batch, N, CM]
+    return base_->batchMatMulT2(C, A, B, pad4(Batch), N, pad4(M), M, pad4(K));
+}
+
+// ---- Tensor --------------------------------------------------------------------------------------------
+Tensor::Tensor(bool check, const std::vector<int>& d) {   // Tensor.java:206-239
+    if (check) {
+        if (d.empty()) throw IllegalArgumentException("Tensor.ndim == 0");
+        for (size_t i = 0; i < d.size(); i++)
+            if (d[i] <= 0)
+                throw IllegalArgumentException(fmt("dim[%lld] { got %lld } must be positive", (long long)i, d[i]));
+    }
+    const int firstDim = d[0], firstDim_4x = pad4(firstDim);
+    long long L4, Lv, L;
+    if (d.size() == 1) {
+        L4 = firstDim_4x; Lv = firstDim_4x; L = firstDim;
+    } else {
+        const int lastDim = d.back(), lastDim_4x = pad4(lastDim);
+        long long midlen = 1;
+        for (size_t i = 1; i + 1 < d.size(); i++) midlen *= d[i];
+        L4 = (long long)firstDim_4x * midlen * lastDim_4x;
+        Lv = (long long)firstDim * midlen * lastDim_4x;
+        L = (long long)firstDim * midlen * lastDim;
+    }
+    if (L4 <= 0 || L4 > 0x7fffffffLL)
+        throw IllegalArgumentException("the length of Tensor is exceed the upper limit");
+    length_4x = (int)L4; lengthv = (int)Lv; length = (int)L;
+    dim = d;
+}
+Tensor& Tensor::c() {
+    if (syncer_) { syncer_->sync(); syncer_.reset(); }
+    return *this;
+}
+
+// ---- Engine ------------------------------------------------------------------------------------------------
+Engine::Engine(int deviceId, int streamPool_maxsize) {
+    base_.reset(new CudaFloat32EngineBase(deviceId, streamPool_maxsize));
+    core_.reset(new EngineCore(base_.get(), true));
+}
+Engine::~Engine() {}
+
+static void equals(int a, const char* an, int b, const char* bn) {
+    if (a != b)
+        throw IllegalArgumentException(std::string(an) + " { got " + std::to_string(a) + " } != " + bn +
+                                       " { got " + std::to_string(b) + " }");
+}
+static void must_greater_equal(int a, const char* an, int b) {
+    if (a < b)
+        throw IllegalArgumentException(std::string(an) + " { got " + std::to_string(a) + " } must >= " +
+                                       std::to_string(b));
+}
+static void require(Tensor* t, const char* name) {
+    if (t == nullptr) throw NullPointerException(std::string("Tensor ") + name + " is null");
+}
+
+void Engine::finish(Tensor* C, SyncerPtr sc) {
+    if (sync_) sc->sync(); else C->setSyncer(std::move(sc));
+}
+
+Tensor* Engine::empty(const std::vector<int>& dim) {   // Engine.java:522-532
+    std::unique_ptr<Tensor> ts(new Tensor(check_, dim));
+    EngineCore::Block b = core_->malloc(ts->length_4x);
+    ts->mem_size = b.size; ts->address = b.address;
+    if (ts->length_4x > ts->length) {   // padded: the pad must read as zero
+        SyncerPtr sc = core_->memset(ts->address, 0, ts->length_4x);
+        if (sync_) sc->sync(); else ts->setSyncer(std::move(sc));
+    }
+    return ts.release();
+}
+Tensor* Engine::zeros(const std::vector<int>& dim) {   // Engine.java:545-551
+    std::unique_ptr<Tensor> ts(new Tensor(check_, dim));
+    EngineCore::Block b = core_->malloc(ts->length_4x);
+    ts->mem_size = b.size; ts->address = b.address;
+    SyncerPtr sc = core_->memset(ts->address, 0, ts->length_4x);
+    if (sync_) sc->sync(); else ts->setSyncer(std::move(sc));
+    return ts.release();
+}
+Tensor* Engine::tensor(const float* value, int value_length, const std::vector<int>& dim_in) {  // :671-676
+    if (value == nullptr) throw NullPointerException("value is null");
+    std::vector<int> dim = dim_in;
+    int neg = -1; long long known = 1;
+    for (size_t i = 0; i < dim.size(); i++) {
+        if (dim[i] == -1 && neg < 0) neg = (int)i; else known *= dim[i];
+    }
+    if (neg >= 0) {
+        if (known <= 0 || value_length % known != 0)
+            throw IllegalArgumentException("value.length is not a multiple of the known dimensions");
+        dim[neg] = (int)(value_length / known);
+    }
+    Tensor* ts = empty(dim);
+    try {
+        ts->c();
+        set(ts, value, value_length);
+    } catch (...) { deleteTensor(ts); throw; }
+    return ts;
+}
+Tensor* Engine::set(Tensor* X, const float* value, int value_length) {   // Engine.java:824-837
+    if (check_) {
+        require(X, "X");
+        equals(value_length, "value<float>.length", X->length, "X.length");
+    }
+    if (X->ndim() == 1) core_->set1D(X->address, value, value_length);
+    else {
+        const int width = X->lastDim();
+        if ((width & 3) == 0) core_->set1D(X->address, value, value_length);
+        else core_->set2D(X->address, value, value_length, width);
+    }
+    return X;
+}
+std::vector<float> Engine::valueOf(Tensor* ts) {   // Engine.java:908-914
+    require(ts, "ts");
+    std::vector<float> out((size_t)ts->length);
+    ts->c();
+    if (ts->ndim() == 1) { core_->get1D(ts->address, out.data(), ts->length); return out; }
+    const int width = ts->lastDim();
+    if ((width & 3) == 0) core_->get1D(ts->address, out.data(), ts->length);
+    else core_->get2D(ts->address, out.data(), ts->length / width, width);
+    return out;
+}
+void Engine::deleteTensor(Tensor* ts) {
+    if (ts == nullptr) return;
+    ts->c();
+    core_->free(ts->mem_size, ts->address);
+    delete ts;
+}
+
+// 2-D products (Engine.java:958-995, 1042-1077, 1080-1118)
+Tensor* Engine::matMul(Tensor* A, Tensor* B) {
+    require(A, "A"); require(B, "B");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2");
+        equals(A->dimAt(1), "A.width", B->dimAt(0), "B.height");
+    }
+    const int AH = A->dim[0], AW = A->dimAt(1), BW = B->dim[1];
+    Tensor* C = &empty({AH, BW})->c();
+    try { finish(C, core_->matMul(C->address, A->address, B->address, AH, BW, AW)); }
+    catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::matMul(Tensor* C, Tensor* A, Tensor* B) {
+    require(C, "C"); require(A, "A"); require(B, "B");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2"); equals(C->ndim(), "C.ndim", 2, "2");
+        equals(C->dimAt(0), "C.height", A->dimAt(0), "A.height");
+        equals(C->dimAt(1), "C.width", B->dimAt(1), "B.width");
+        equals(A->dimAt(1), "A.width", B->dimAt(0), "B.height");
+    }
+    finish(C, core_->matMul(C->address, A->address, B->address, A->dim[0], B->dim[1], A->dimAt(1)));
+    return C;
+}
+Tensor* Engine::matMulT1(Tensor* A, Tensor* B) {
+    require(A, "A"); require(B, "B");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2");
+        equals(A->dimAt(0), "A.height", B->dimAt(0), "B.height");
+    }
+    const int AH = A->dim[0], AW = A->dim[1], BW = B->dim[1];   // A[K, N], B[K, M]
+    Tensor* C = &empty({AW, BW})->c();
+    try { finish(C, core_->matMulT1(C->address, A->address, B->address, AW, BW, AH)); }
+    catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::matMulT1(Tensor* C, Tensor* A, Tensor* B) {
+    require(C, "C"); require(A, "A"); require(B, "B");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2"); equals(C->ndim(), "C.ndim", 2, "2");
+        equals(C->dimAt(0), "C.height", A->dimAt(1), "A.width");
+        equals(C->dimAt(1), "C.width", B->dimAt(1), "B.width");
+        equals(A->dimAt(0), "A.height", B->dimAt(0), "B.height");
+    }
+    finish(C, core_->matMulT1(C->address, A->address, B->address, A->dim[1], B->dim[1], A->dim[0]));
+    return C;
+}
+Tensor* Engine::matMulT2(Tensor* A, Tensor* B) {
+    require(A, "A"); require(B, "B");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2");
+        equals(A->dimAt(1), "A.width", B->dimAt(1), "B.width");
+    }
+    const int AH = A->dim[0], AW = A->dim[1], BH = B->dim[0];   // A[N, K], B[M, K]
+    Tensor* C = &empty({AH, BH})->c();
+    try { finish(C, core_->matMulT2(C->address, A->address, B->address, AH, BH, AW)); }
+    catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::matMulT2(Tensor* C, Tensor* A, Tensor* B) {
+    require(C, "C"); require(A, "A"); require(B, "B");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2"); equals(C->ndim(), "C.ndim", 2, "2");
+        equals(C->dimAt(0), "C.height", A->dimAt(0), "A.height");
+        equals(C->dimAt(1), "C.width", B->dimAt(0), "B.height");
+        equals(A->dimAt(1), "A.width", B->dimAt(1), "B.width");
+    }
+    finish(C, core_->matMulT2(C->address, A->address, B->address, A->dim[0], B->dim[0], A->dim[1]));
+    return C;
+}
+
+// batched products (Engine.java:1121-1312): batch = product of the leading dimensions
+static std::vector<int> batched_dimC(bool likeA, Tensor* A, Tensor* B, int rows, int cols) {
+    Tensor* L = likeA ? A : B;
+    std::vector<int> dimC(L->dim.begin(), L->dim.end());
+    dimC[dimC.size() - 2] = rows;
+    dimC[dimC.size() - 1] = cols;
+    return dimC;
+}
+static int batch_of(Tensor* T) { return T->length / (T->dimAt(-2) * T->dimAt(-1)); }
+
+Tensor* Engine::batchMatMul(bool likeA, Tensor* A, Tensor* B) {
+    require(A, "A"); require(B, "B");
+    if (A->ndim() == 2 && B->ndim() == 2) return matMul(A, B);
+    if (check_) {
+        must_greater_equal(A->ndim(), "A.ndim", 3); must_greater_equal(B->ndim(), "B.ndim", 3);
+        equals(A->dimAt(-1), "A.width", B->dimAt(-2), "B.height");
+        equals(batch_of(A), "A.batch", batch_of(B), "B.batch");
+    }
+    const int AH = A->dimAt(-2), AW = A->dimAt(-1), BW = B->dimAt(-1);
+    Tensor* C = &empty(batched_dimC(likeA, A, B, AH, BW))->c();
+    try { finish(C, core_->batchMatMul(C->address, A->address, B->address, batch_of(A), AH, BW, AW)); }
+    catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::batchMatMul(Tensor* C, Tensor* A, Tensor* B) {
+    require(C, "C"); require(A, "A"); require(B, "B");
+    if (A->ndim() == 2 && B->ndim() == 2 && C->ndim() == 2) return matMul(C, A, B);
+    if (check_) {
+        must_greater_equal(A->ndim(), "A.ndim", 3); must_greater_equal(B->ndim(), "B.ndim", 3);
+        must_greater_equal(C->ndim(), "C.ndim", 3);
+        equals(C->dimAt(-2), "C.height", A->dimAt(-2), "A.height");
+        equals(C->dimAt(-1), "C.width", B->dimAt(-1), "B.width");
+        equals(A->dimAt(-1), "A.width", B->dimAt(-2), "B.height");
+        equals(batch_of(A), "A.batch", batch_of(B), "B.batch");
+        equals(batch_of(A), "A.batch", batch_of(C), "C.batch");
+    }
+    finish(C, core_->batchMatMul(C->address, A->address, B->address, batch_of(A), A->dimAt(-2),
+                                 B->dimAt(-1), A->dimAt(-1)));
+    return C;
+}
+Tensor* Engine::batchMatMulT1(bool likeA, Tensor* A, Tensor* B) {
+    require(A, "A"); require(B, "B");
+    if (A->ndim() == 2 && B->ndim() == 2) return matMulT1(A, B);
+    if (check_) {
+        must_greater_equal(A->ndim(), "A.ndim", 3); must_greater_equal(B->ndim(), "B.ndim", 3);
+        equals(A->dimAt(-2), "A.height", B->dimAt(-2), "B.height");
+        equals(batch_of(A), "A.batch", batch_of(B), "B.batch");
+    }
+    const int AH = A->dimAt(-2), AW = A->dimAt(-1), BW = B->dimAt(-1);   // A^T[N: AW, K: AH]
+    Tensor* C = &empty(batched_dimC(likeA, A, B, AW, BW))->c();
+    try { finish(C, core_->batchMatMulT1(C->address, A->address, B->address, batch_of(A), AW, BW, AH)); }
+    catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::batchMatMulT1(Tensor* C, Tensor* A, Tensor* B) {
+    require(C, "C"); require(A, "A"); require(B, "B");
+    if (A->ndim() == 2 && B->ndim() == 2 && C->ndim() == 2) return matMulT1(C, A, B);
+    if (check_) {
+        must_greater_equal(A->ndim(), "A.ndim", 3); must_greater_equal(B->ndim(), "B.ndim", 3);
+        must_greater_equal(C->ndim(), "C.ndim", 3);
+        equals(C->dimAt(-2), "C.height", A->dimAt(-1), "A.width");
+        equals(C->dimAt(-1), "C.width", B->dimAt(-1), "B.width");
+        equals(A->dimAt(-2), "A.height", B->dimAt(-2), "B.height");
+        equals(batch_of(A), "A.batch", batch_of(B), "B.batch");
+        equals(batch_of(A), "A.batch", batch_of(C), "C.batch");
+    }
+    finish(C, core_->batchMatMulT1(C->address, A->address, B->address, batch_of(A), A->dimAt(-1),
+                                   B->dimAt(-1), A->dimAt(-2)));
+    return C;
+}
+Tensor* Engine::batchMatMulT2(bool likeA, Tensor* A, Tensor* B) {
+    require(A, "A"); require(B, "B");
+    if (A->ndim() == 2 && B->ndim() == 2) return matMulT2(A, B);
+    if (check_) {
+        must_greater_equal(A->ndim(), "A.ndim", 3); must_greater_equal(B->ndim(), "B.ndim", 3);
+        equals(A->dimAt(-1), "A.width", B->dimAt(-1), "B.width");
+        equals(batch_of(A), "A.batch", batch_of(B), "B.batch");
+    }
+    const int AH = A->dimAt(-2), AW = A->dimAt(-1), BH = B->dimAt(-2);   // B^T[K: BW, M: BH]
+    Tensor* C = &empty(batched_dimC(likeA, A, B, AH, BH))->c();
+    try { finish(C, core_->batchMatMulT2(C->address, A->address, B->address, batch_of(A), AH, BH, AW)); }
+    catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::batchMatMulT2(Tensor* C, Tensor* A, Tensor* B) {
+    require(C, "C"); require(A, "A"); require(B, "B");
+    if (A->ndim() == 2 && B->ndim() == 2 && C->ndim() == 2) return matMulT2(C, A, B);
+    if (check_) {
+        must_greater_equal(A->ndim(), "A.ndim", 3); must_greater_equal(B->ndim(), "B.ndim", 3);
+        must_greater_equal(C->ndim(), "C.ndim", 3);
+        equals(C->dimAt(-2), "C.height", A->dimAt(-2), "A.height");
+        equals(C->dimAt(-1), "C.width", B->dimAt(-2), "B.height");
+        equals(A->dimAt(-1), "A.width", B->dimAt(-1), "B.width");
+        equals(batch_of(A), "A.batch", batch_of(B), "B.batch");
+        equals(batch_of(A), "A.batch", batch_of(C), "C.batch");
+    }
+    finish(C, core_->batchMatMulT2(C->address, A->address, B->address, batch_of(A), A->dimAt(-2),
+                                   B->dimAt(-2), A->dimAt(-1)));
+    return C;
+}
+
+}  // namespace dragon

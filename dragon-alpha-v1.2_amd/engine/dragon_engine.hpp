@@ -1,0 +1,234 @@
+// Host side of the matrix-multiplication path, above the C ABI: a C++ mirror of the
+// Java classes that drive the reference's native libraries, with the same names,
+// argument meaning and error behaviour.  It calls nothing but the C ABI of
+// include/dragon_hip_gemm.h and include/dragon_hip_runtime.h -- exactly what the
+// reference's Java code would call through JNI.
+//
+//   CudaDevice             z/dragon/engine/cuda/impl/CudaDevice.java (multiProcessorCount only)
+//   CudaStreamPool         z/dragon/engine/cuda/impl/CudaStreamp1.java:34-63 (round-robin, never blocks)
+//   Syncer and its kinds   z/dragon/engine/cuda/CudaFloat32EngineBase.java:649-694, 1008-1054
+//   CudaFloat32EngineBase  z/dragon/engine/cuda/CudaFloat32EngineBase.java:70-92, 1148-1260, 1471-2020
+//   EngineCore             z/dragon/engine/EngineCore.java:693-811 (checks and x4 padding)
+//   Tensor                 z/dragon/engine/Tensor.java:206-239 (length / lengthv / length_4x)
+//   Engine                 z/dragon/engine/Engine.java:522-551, 671-676, 824-837, 908-914, 955-1312
+// (paths relative to source/alpha-Dragon-v1.2/src of the reference tree)
+#pragma once
+#include <stdint.h>
+#include <memory>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace dragon {
+
+// ---- exceptions: the Java types the reference throws ---------------------------------
+struct NullPointerException : std::runtime_error { using std::runtime_error::runtime_error; };
+struct IllegalArgumentException : std::runtime_error { using std::runtime_error::runtime_error; };
+struct CudaException : std::runtime_error {
+    int code;
+    explicit CudaException(int c);
+};
+
+// ---- device ----------------------------------------------------------------------------
+class CudaDevice {
+public:
+    explicit CudaDevice(int id = 0);
+    int getId() const { return id_; }
+    int multiProcessorCount() const { return sm_count_; }
+    // lets a test drive the split-K policy as a device with another unit count would
+    void overrideMultiProcessorCount(int n) { sm_count_ = n; }
+private:
+    int id_, sm_count_;
+};
+
+// ---- stream pool: hands out streams round-robin, returning them is a no-op ----------------
+class CudaStreamPool {
+public:
+    CudaStreamPool(const CudaDevice& dev, int max_streamsize, int max_getsize_oneturn);
+    ~CudaStreamPool();
+    int64_t getStream();
+    std::vector<int64_t> getStreamArray(int length);
+    void returnStream(int64_t) {}
+    void returnStreamArray(const std::vector<int64_t>&) {}
+    int total_stream_size();
+private:
+    void init();
+    int dev_id_, max_streamsize_, max_getsize_oneturn_;
+    std::vector<int64_t> gc_;
+    int gc_index_ = 0;
+    bool inited_ = false;
+    std::mutex mu_;
+};
+
+// ---- completion handles ----------------------------------------------------------------------
+class Syncer {
+public:
+    virtual ~Syncer() {}
+    virtual void sync() = 0;
+};
+typedef std::unique_ptr<Syncer> SyncerPtr;
+
+class EngineCore;
+
+// ---- split-K policy, usable without a device ---------------------------------------------------
+struct SplitKKnobs {
+    int threshold;          // K below this never splits (default 512)
+    int maxPart;            // upper bound of GridZ (default smooth(SM count))
+    float minBlock_perSM;   // 1.2f for matMul, 1.14f for matMulT1 / matMulT2
+    float maxBlock_perSM;   // 4.0f
+};
+int policy_smooth_maxPart(int x);
+int policy_matMul_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
+int policy_matMulT1_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
+int policy_matMulT2_gridZ(int N, int M, int K, int SM, const SplitKKnobs& t2, const SplitKKnobs& mm);
+
+// ---- the engine "plugin": split-K policy, stream checkout, event protocol -----------------------
+class CudaFloat32EngineBase {
+public:
+    CudaFloat32EngineBase(int deviceId, int streamPool_maxsize);
+    CudaDevice& device() { return dev_; }
+    CudaStreamPool& streamPool() { return *streamPool_; }
+    void engineCore(EngineCore* core) { core_ = core; }
+
+    // knobs (same names and defaults as the Java fields)
+    int matMul_sk_threshold = 512, matMul_sk_maxPart = 16;
+    float matMul_sk_minBlock_perSM = 1.2f, matMul_sk_maxBlock_perSM = 4.0f;
+    int matMulT1_sk_threshold = 512, matMulT1_sk_maxPart = 16;
+    float matMulT1_sk_minBlock_perSM = 1.14f, matMulT1_sk_maxBlock_perSM = 4.0f;
+    int matMulT2_sk_threshold = 512, matMulT2_sk_maxPart = 16;
+    float matMulT2_sk_minBlock_perSM = 1.14f, matMulT2_sk_maxBlock_perSM = 4.0f;
+    bool matMul_tf32 = false, matMulT1_tf32 = false, matMulT2_tf32 = false;
+    bool batchMatMul_tf32 = false, batchMatMulT1_tf32 = false, batchMatMulT2_tf32 = false;
+    bool batchMatMul_useTexture = true, batchMatMulT2_useTexture = true;
+
+    void matMul_splitK_threshold(int threshold);     // must be a positive power of two
+    void matMul_splitK_maxPart(int maxPart);         // must be >= 4
+    void matMulT1_splitK_threshold(int threshold);
+    void matMulT1_maxPart(int maxPart);
+    void matMulT2_splitK_threshold(int threshold);
+    void matMulT2_splitK_maxPart(int maxPart);
+    void tf32(bool flag);
+    void recomputeMaxParts();                        // maxPart = smooth(SM count), as the constructor does
+
+    // the split-K decisions on their own (1 = no split), for inspection
+    int matMul_gridZ(int N, int M, int K) const;
+    int matMulT1_gridZ(int N, int M, int K) const;
+    int matMulT2_gridZ(int N, int M, int K) const;
+
+    // memory operations
+    int64_t malloc(int64_t memsize);
+    void free(int64_t address);
+    SyncerPtr memset(int64_t address, int value, int64_t memsize);
+    void get1D(int64_t address, float* value, int length);
+    void get2D(int64_t address, float* value, int height, int width, int stride);
+    void set1D(int64_t address, const float* value, int length);
+    void set2D(int64_t address, const float* value, int height, int width, int stride);
+
+    // products; dims arrive already padded by EngineCore
+    SyncerPtr matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int BK, int AK);
+    SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN, int AN, int M, int K);
+    SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int CM, int BM, int K);
+
+    // what the last product call decided (test introspection)
+    int last_gridZ = 1, last_stream_count = 0;
+
+private:
+    SyncerPtr run_2d(int variant, int gridZ, int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    CudaDevice dev_;
+    std::unique_ptr<CudaStreamPool> streamPool_;
+    EngineCore* core_ = nullptr;
+};
+
+// ---- EngineCore: argument checks, x4 padding, memory blocks ----------------------------------------
+class EngineCore {
+public:
+    explicit EngineCore(CudaFloat32EngineBase* base, bool check = true);
+    CudaFloat32EngineBase* engineBase() { return base_; }
+    bool check;
+
+    // a block is {size in bytes, address}; the pool behind it is the caller's business in
+    // the reference, here every block is its own device allocation
+    struct Block { int64_t size, address; };
+    Block malloc(int mem_length);
+    void free(int64_t size, int64_t address);
+    int64_t live_blocks() const { return live_blocks_; }
+    SyncerPtr memset(int64_t address, int value, int length);
+    void get1D(int64_t address, float* value, int length);
+    void get2D(int64_t address, float* value, int height, int width);
+    void set1D(int64_t address, const float* value, int length);
+    void set2D(int64_t address, const float* value, int length, int width);
+
+    SyncerPtr matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
+    SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
+    SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
+
+private:
+    void matMul_check(int64_t C, int64_t A, int64_t B, int N, int M, int K) const;
+    CudaFloat32EngineBase* base_;
+    int64_t live_blocks_ = 0;
+    std::mutex mu_;
+};
+
+// ---- Tensor: row-major, last dimension stored with a stride rounded up to 4 ---------------------------
+class Tensor {
+public:
+    Tensor(bool check, const std::vector<int>& dim);
+    std::vector<int> dim;
+    int length = 0;      // logical element count
+    int lengthv = 0;     // firstDim * mid * lastDim_4x
+    int length_4x = 0;   // firstDim_4x * mid * lastDim_4x: what is allocated
+    int64_t mem_size = 0, address = 0;
+    int ndim() const { return (int)dim.size(); }
+    int dimAt(int i) const { return i < 0 ? dim[dim.size() + i] : dim[i]; }
+    int lastDim() const { return dim.back(); }
+    void setSyncer(SyncerPtr sc) { syncer_ = std::move(sc); }
+    Tensor& c();         // wait for the pending operation that produces this tensor
+private:
+    SyncerPtr syncer_;
+};
+
+// ---- Engine: the tensor-level API ------------------------------------------------------------------------
+class Engine {
+public:
+    Engine(int deviceId, int streamPool_maxsize);
+    ~Engine();
+    EngineCore& engineCore() { return *core_; }
+    CudaFloat32EngineBase& engineBase() { return *base_; }
+    Engine& check(bool flag) { check_ = flag; core_->check = flag; return *this; }
+    Engine& sync(bool flag) { sync_ = flag; return *this; }
+
+    Tensor* empty(const std::vector<int>& dim);
+    Tensor* zeros(const std::vector<int>& dim);
+    Tensor* tensor(const float* value, int value_length, const std::vector<int>& dim);
+    Tensor* set(Tensor* X, const float* value, int value_length);
+    std::vector<float> valueOf(Tensor* ts);
+    void deleteTensor(Tensor* ts);
+
+    Tensor* matMul(Tensor* A, Tensor* B);
+    Tensor* matMul(Tensor* C, Tensor* A, Tensor* B);
+    Tensor* matMulT1(Tensor* A, Tensor* B);
+    Tensor* matMulT1(Tensor* C, Tensor* A, Tensor* B);
+    Tensor* matMulT2(Tensor* A, Tensor* B);
+    Tensor* matMulT2(Tensor* C, Tensor* A, Tensor* B);
+    Tensor* batchMatMul(bool likeA, Tensor* A, Tensor* B);
+    Tensor* batchMatMul(Tensor* C, Tensor* A, Tensor* B);
+    Tensor* batchMatMulT1(bool likeA, Tensor* A, Tensor* B);
+    Tensor* batchMatMulT1(Tensor* C, Tensor* A, Tensor* B);
+    Tensor* batchMatMulT2(bool likeA, Tensor* A, Tensor* B);
+    Tensor* batchMatMulT2(Tensor* C, Tensor* A, Tensor* B);
+
+private:
+    void finish(Tensor* C, SyncerPtr sc);
+    std::unique_ptr<CudaFloat32EngineBase> base_;
+    std::unique_ptr<EngineCore> core_;
+    bool check_ = true, sync_ = true;
+};
+
+}  // namespace dragon

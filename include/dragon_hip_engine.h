@@ -1,0 +1,88 @@
+/*
+ * dragon_hip_engine.h -- C access to the host-side engine mirror (C++ classes named after
+ * the reference's Java classes: Engine, EngineCore, CudaFloat32EngineBase, Tensor, Syncer).
+ *
+ * This is NOT the drop-in boundary (that is dragon_hip_gemm.h / dragon_hip_runtime.h, the
+ * level of the reference's JNI functions).  It exposes the layer above it -- the logic the
+ * reference keeps in Java -- to hosts without a JVM: tests, benchmarks, C programs.
+ * Reference: source/alpha-Dragon-v1.2/src/z/dragon/engine/Engine.java:522-551, 671-676,
+ * 824-837, 908-914, 955-1312; EngineCore.java:693-811; cuda/CudaFloat32EngineBase.java:70-92,
+ * 649-694, 1008-1054, 1471-2020; Tensor.java:206-239.
+ *
+ * Errors: functions returning int give 0 on success, else DRAGON_E_*; functions returning a
+ * pointer give NULL on failure.  dragon_engine_last_error() describes the last failure of
+ * the calling thread; for DRAGON_E_CUDA dragon_engine_last_cuda_code() holds the runtime code.
+ */
+#ifndef DRAGON_HIP_ENGINE_H
+#define DRAGON_HIP_ENGINE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dragon_engine dragon_engine;   /* z.dragon.engine.Engine over CudaFloat32EngineBase */
+typedef struct dragon_tensor dragon_tensor;   /* z.dragon.engine.Tensor */
+
+enum {
+    DRAGON_OK = 0,
+    DRAGON_E_NULL_POINTER = 1,       /* java.lang.NullPointerException */
+    DRAGON_E_ILLEGAL_ARGUMENT = 2,   /* java.lang.IllegalArgumentException */
+    DRAGON_E_CUDA = 3,               /* z.dragon.engine.cuda.impl.CudaException */
+    DRAGON_E_OTHER = 4
+};
+const char* dragon_engine_last_error(void);
+int32_t dragon_engine_last_cuda_code(void);
+
+/* alpha.engine.cuda_float32(deviceId, ...) with a stream pool of the given size (32 in the
+ * reference's default constructor). */
+dragon_engine* dragon_engine_cuda_float32(int32_t device_id, int32_t stream_pool_size);
+void dragon_engine_delete(dragon_engine* eg);
+int dragon_engine_check(dragon_engine* eg, int32_t flag);   /* Engine.check(boolean) */
+int dragon_engine_sync(dragon_engine* eg, int32_t flag);    /* Engine.sync(boolean)  */
+
+/* knobs of CudaFloat32EngineBase; names as in Java: "matMul_splitK_threshold",
+ * "matMul_splitK_maxPart", "matMulT1_splitK_threshold", "matMulT1_maxPart",
+ * "matMulT2_splitK_threshold", "matMulT2_splitK_maxPart", "tf32", "batchMatMul_useTexture",
+ * "batchMatMulT2_useTexture", and "multiProcessorCount" (test hook: pretend another unit
+ * count and recompute maxPart from it). */
+int dragon_engine_set_param(dragon_engine* eg, const char* name, int32_t value);
+int32_t dragon_engine_get_param(dragon_engine* eg, const char* name);   /* also "last_gridZ",
+    "last_stream_count", "live_blocks", "stream_pool_size" */
+
+/* split-K decision for padded dims; kind 0 matMul, 1 matMulT1, 2 matMulT2; 1 = no split */
+int32_t dragon_engine_gridZ(dragon_engine* eg, int32_t kind, int32_t N, int32_t M, int32_t K);
+/* the same decision as a pure function of the unit count, with the default knobs
+ * (threshold 512, maxPart smooth(SM), minBlock 1.2 / 1.14, maxBlock 4.0); needs no device */
+int32_t dragon_policy_gridZ(int32_t kind, int32_t N, int32_t M, int32_t K, int32_t SM);
+int32_t dragon_policy_smooth_maxPart(int32_t x);
+
+/* tensors */
+dragon_tensor* dragon_engine_empty(dragon_engine* eg, const int32_t* dim, int32_t ndim);
+dragon_tensor* dragon_engine_zeros(dragon_engine* eg, const int32_t* dim, int32_t ndim);
+dragon_tensor* dragon_engine_tensor(dragon_engine* eg, const float* value, int32_t value_length,
+                                    const int32_t* dim, int32_t ndim);
+int dragon_engine_set(dragon_engine* eg, dragon_tensor* X, const float* value, int32_t value_length);
+int dragon_engine_valueOf(dragon_engine* eg, dragon_tensor* ts, float* out, int32_t out_length);
+int dragon_engine_delete_tensor(dragon_engine* eg, dragon_tensor* ts);
+int dragon_tensor_c(dragon_tensor* ts);                      /* Tensor.c(): wait for its producer */
+int32_t dragon_tensor_ndim(const dragon_tensor* ts);
+int32_t dragon_tensor_dim(const dragon_tensor* ts, int32_t i);
+int32_t dragon_tensor_length(const dragon_tensor* ts);
+int32_t dragon_tensor_lengthv(const dragon_tensor* ts);
+int32_t dragon_tensor_length_4x(const dragon_tensor* ts);
+int64_t dragon_tensor_address(const dragon_tensor* ts);
+
+/* products: op 0 matMul, 1 matMulT1, 2 matMulT2, 3 batchMatMul, 4 batchMatMulT1,
+ * 5 batchMatMulT2.  The first form allocates C (likeA picks whose leading dims C copies in
+ * the batched forms), the second writes into an existing C. */
+dragon_tensor* dragon_engine_product(dragon_engine* eg, int32_t op, int32_t likeA,
+                                     dragon_tensor* A, dragon_tensor* B);
+int dragon_engine_product_into(dragon_engine* eg, int32_t op, dragon_tensor* C,
+                               dragon_tensor* A, dragon_tensor* B);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRAGON_HIP_ENGINE_H */
