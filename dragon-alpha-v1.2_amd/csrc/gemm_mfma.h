@@ -14,7 +14,11 @@ enum GemmTile {
     TILE_64x256 = 3,
     TILE_128x64 = 4,
     TILE_64x128 = 5,
-    TILE_COUNT = 6
+    TILE_128x128_K32 = 6,   // the same shapes with 32 k per LDS stage
+    TILE_64x64_K32 = 7,
+    TILE_128x64_K32 = 8,
+    TILE_64x128_K32 = 9,
+    TILE_COUNT = 10
 };
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
@@ -40,7 +44,7 @@ struct GemmParams {
     int tiles_m, tiles_n;   // filled by the launcher
 };
 
-int gemm_choose_tile(int rows, int cols, int nz, int num_cu);
+int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu);
 void gemm_force_tile(int tile);
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
 

@@ -20,8 +20,11 @@
 // Operand layouts.  An operand is either "K-inner" (k is the contiguous index:
 // A of NN/T2, B of T2) or "K-outer" (k is the row index: B of NN/T1, A of T1).
 // Neither is transposed on its way through LDS:
-//   K-inner tile  -> LDS [row][k] (+4 floats of row padding); a lane reads 4
-//                    consecutive k with one ds_read_b128 and feeds 4 MFMA steps.
+//   K-inner tile  -> LDS [row][k] in 16-byte chunks, chunk c of row r stored at chunk
+//                    position c ^ swizzle(r) so that both the staging stores (lanes
+//                    walk along a row) and the fragment reads (lanes walk down the
+//                    rows) touch every bank once; a lane reads 4 consecutive k with
+//                    one ds_read_b128 and feeds 4 MFMA steps.
 //   K-outer tile  -> LDS [k][row]; a lane reads T consecutive rows with one
 //                    ds_read, and those T values belong to T different MFMA
 //                    blocks (block b of a wave holds rows {T*p + b}).  The
@@ -64,15 +67,25 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
 // Tile staging: global -> registers -> LDS
 // ---------------------------------------------------------------------------
 
-// K-inner operand: R rows of KT consecutive k.  LDS row stride KT+4 floats.
+// Chunk swizzle of a K-inner tile.  Rows hold CPR = KT/4 chunks of 16 bytes with no
+// padding.  With 4 chunks per row two rows share the 32 banks, so the row pair index
+// (r>>1)&3 permutes the chunks; with 8 chunks per row the row index r&7 does.
+template <int KT>
+__device__ __forceinline__ int kin_swizzle(int row) {
+    static_assert(KT == 16 || KT == 32, "k per stage: 16 or 32");
+    return (KT == 16) ? ((row >> 1) & 3) : (row & 7);
+}
+
+// K-inner operand: R rows of KT consecutive k.  LDS row stride KT floats, chunks swizzled.
 template <int R, int KT>
 struct KInner {
     static constexpr int CPR = KT / 4;            // float4 chunks per row
     static constexpr int RPP = NTHREADS / CPR;    // rows per pass
     static constexpr int PASSES = R / RPP;
-    static constexpr int LDS_STRIDE = KT + 4;
+    static constexpr int LDS_STRIDE = KT;
     static constexpr int LDS_FLOATS = R * LDS_STRIDE;
     static_assert(R % RPP == 0 && PASSES >= 1, "tile does not divide over the workgroup");
+    static_assert(RPP % 8 == 0, "the swizzle must repeat from pass to pass");
 
     int off[PASSES];   // byte offset of this thread's chunk, or OOB_OFFSET if its row is outside
     int kcol;          // k offset of this thread's chunk inside the tile
@@ -81,7 +94,7 @@ struct KInner {
     __device__ __forceinline__ void init(int t, int row0, int outer_bound, int ld) {
         const int c = t % CPR, r0 = t / CPR;
         kcol = c * 4;
-        lds_at = r0 * LDS_STRIDE + c * 4;
+        lds_at = r0 * LDS_STRIDE + 4 * (c ^ kin_swizzle<KT>(r0));
 #pragma unroll
         for (int s = 0; s < PASSES; s++) {
             const int r = r0 + s * RPP;
@@ -151,10 +164,11 @@ struct KOuter {
 template <int T, int KT>
 __device__ __forceinline__ void read_frag_kinner(float (&frag)[T][4], const float* lds,
                                                  int wave_row0, int g, int r, int h) {
-    constexpr int S = KT + 4;
+    // wave_row0 and b*32 are multiples of 32, so the swizzle depends on r alone
+    const int chunk = (g * 2 + h) ^ kin_swizzle<KT>(r);
 #pragma unroll
     for (int b = 0; b < T; b++) {
-        const v4f v = *(const v4f*)(lds + (wave_row0 + b * 32 + r) * S + g * 8 + h * 4);
+        const v4f v = *(const v4f*)(lds + (wave_row0 + b * 32 + r) * KT + chunk * 4);
         frag[b][0] = v.x; frag[b][1] = v.y; frag[b][2] = v.z; frag[b][3] = v.w;
     }
 }
@@ -184,20 +198,27 @@ __device__ __forceinline__ void read_frag_kouter(float (&frag)[T][4], const floa
 //   WM x WN       : wavefront grid in the workgroup (WM*WN == 4)
 //   TM x TN       : 32x32 MFMA blocks per wavefront
 //   KT            : k per LDS stage
+//
+// Workgroups are persistent: workgroup w works on the logical tiles w, w+G, w+2G, ...
+// (G = grid size, chosen by the launcher as what the device keeps resident).  The
+// first LDS stage of the next tile is fetched during the last k-step of the current
+// one, and the stores of a finished tile drain while the next tile computes, so a
+// stream of short tiles (small K, large C) keeps the matrix cores busy.
 // ---------------------------------------------------------------------------
-template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT>
-__global__ __launch_bounds__(NTHREADS) void gemm_f32_mfma(const GemmParams p) {
-    static_assert(WM * WN == 4, "four wavefronts per workgroup");
-    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
-    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT>, KOuter<BN, KT>>::type;
+struct TileCtx {
+    const float* a_ptr;   // A at (row0, k0) of this tile's batch / slice
+    const float* b_ptr;
+    float* c_ptr;         // C (or split-K partial) of this tile's batch / slice
+    int row0, col0;
+    int k0;               // first k of the slice
+    int ka_lim, kb_lim;   // first k each operand may no longer touch
+    int nstage;           // LDS stages to run (>= 1; an empty slice runs one all-zero stage)
+};
 
-    __shared__ __attribute__((aligned(16))) float As[2][LoadA::LDS_FLOATS];
-    __shared__ __attribute__((aligned(16))) float Bs[2][LoadB::LDS_FLOATS];
-
-    // ---- which tile, which batch / K slice -------------------------------------
+template <bool A_KIN, bool B_KIN, int BM, int BN, int KT, typename LoadA, typename LoadB>
+__device__ __forceinline__ TileCtx decode_tile(const GemmParams& p, int lid) {
+    TileCtx c;
     const int tiles = p.tiles_m * p.tiles_n;
-    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int z = lid / tiles;
     int tt = lid - z * tiles;
     // bands of 8 tile rows, walked row-fastest, keep one XCD's concurrent tiles compact
@@ -207,10 +228,10 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_mfma(const GemmParams p) {
     const int first_m = band * BAND;
     const int band_rows = (p.tiles_m - first_m < BAND) ? (p.tiles_m - first_m) : BAND;
     tt -= band * band_sz;
-    const int tile_m = first_m + tt % band_rows;
     const int tile_n = tt / band_rows;
-    const int row0 = tile_m * BM, col0 = tile_n * BN;
-
+    const int tile_m = first_m + (tt - tile_n * band_rows);
+    c.row0 = tile_m * BM;
+    c.col0 = tile_n * BN;
     const float* A = p.A;
     const float* B = p.B;
     float* C = p.C;
@@ -224,122 +245,203 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_mfma(const GemmParams p) {
         B += (size_t)z * p.sB;
         C += (size_t)z * p.sC;
     }
-    // k range each operand may touch
-    const int ka_lim = min(k1, A_KIN ? p.a_inner : p.a_outer);
-    const int kb_lim = min(k1, B_KIN ? p.b_inner : p.b_outer);
+    c.k0 = k0;
+    c.ka_lim = min(k1, A_KIN ? p.a_inner : p.a_outer);
+    c.kb_lim = min(k1, B_KIN ? p.b_inner : p.b_outer);
+    const int n = (k1 - k0 + KT - 1) / KT;
+    c.nstage = n > 0 ? n : 1;
+    c.a_ptr = LoadA::tile_base(A, c.row0, k0, p.lda);
+    c.b_ptr = LoadB::tile_base(B, c.col0, k0, p.ldb);
+    c.c_ptr = C;
+    return c;
+}
+
+// Wavefronts per SIMD the register allocator should leave room for: as many workgroups
+// as the LDS footprint lets a compute unit hold (160 KiB), at most 4.
+template <bool A_KIN, bool B_KIN, int BM, int BN, int KT>
+constexpr int target_occupancy() {
+    const int lds = 2 * 4 * (BM * KT + BN * KT);
+    const int fit = (160 * 1024) / lds;
+    return fit > 4 ? 4 : (fit < 1 ? 1 : fit);
+}
+
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT>
+__global__ __launch_bounds__(NTHREADS, (target_occupancy<A_KIN, B_KIN, WM * TM * 32, WN * TN * 32, KT>()))
+void gemm_f32_mfma(const GemmParams p) {
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
+    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT>, KOuter<BN, KT>>::type;
+
+    __shared__ __attribute__((aligned(16))) float As[2][LoadA::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float Bs[2][LoadB::LDS_FLOATS];
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
+    const size_t a_step = LoadA::k_advance(p.lda), b_step = LoadB::k_advance(p.ldb);
 
+    const int total = p.tiles_m * p.tiles_n * p.nz;
+    const int G = gridDim.x;
+    int lid = xcd_contiguous_id(blockIdx.x, G);   // G <= total, so lid is a valid tile
+
+    TileCtx cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid);
     LoadA la;
     LoadB lb;
-    la.init(t, row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
-    lb.init(t, col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
-    const float* a_ptr = LoadA::tile_base(A, row0, k0, p.lda);
-    const float* b_ptr = LoadB::tile_base(B, col0, k0, p.ldb);
-    const size_t a_step = LoadA::k_advance(p.lda), b_step = LoadB::k_advance(p.ldb);
+    la.init(t, cur.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+    lb.init(t, cur.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
 
     v16f acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+        for (int j = 0; j < TN; j++) acc[i][j] = (v16f)(0.0f);
 
     v4f ra[LoadA::PASSES], rb[LoadB::PASSES];
-    const int ntile = (k1 - k0 + KT - 1) / KT;
 
-    // prologue: stage 0
-    la.load(ra, a_ptr, ka_lim - k0);
-    lb.load(rb, b_ptr, kb_lim - k0);
+    // stage 0 of the first tile
+    la.load(ra, cur.a_ptr, cur.ka_lim - cur.k0);
+    lb.load(rb, cur.b_ptr, cur.kb_lim - cur.k0);
     la.store(ra, As[0]);
     lb.store(rb, Bs[0]);
     __syncthreads();
+    int buf = 0;
 
-    for (int it = 0; it < ntile; it++) {
-        const int cur = it & 1;
-        const int knext = k0 + (it + 1) * KT;
-        if (it + 1 < ntile) {        // prefetch the next stage into registers
-            a_ptr += a_step;
-            b_ptr += b_step;
-            la.load(ra, a_ptr, ka_lim - knext);
-            lb.load(rb, b_ptr, kb_lim - knext);
+    for (;;) {
+        const bool has_next = lid + G < total;
+        TileCtx nxt = cur;
+        const float* a_ptr = cur.a_ptr;
+        const float* b_ptr = cur.b_ptr;
+        for (int it = 0; it < cur.nstage; it++) {
+            const bool last = (it + 1 == cur.nstage);
+            bool fetched = false;
+            if (!last) {                 // next stage of this tile -> registers
+                a_ptr += a_step;
+                b_ptr += b_step;
+                const int knext = cur.k0 + (it + 1) * KT;
+                la.load(ra, a_ptr, cur.ka_lim - knext);
+                lb.load(rb, b_ptr, cur.kb_lim - knext);
+                fetched = true;
+            } else if (has_next) {       // first stage of the next tile -> registers
+                nxt = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid + G);
+                la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+                lb.init(t, nxt.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+                la.load(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0);
+                lb.load(rb, nxt.b_ptr, nxt.kb_lim - nxt.k0);
+                fetched = true;
+            }
+            const float* as = As[buf];
+            const float* bs = Bs[buf];
+#pragma unroll
+            for (int g = 0; g < KT / 8; g++) {
+                float fa[TM][4], fb[TN][4];
+                if constexpr (A_KIN) read_frag_kinner<TM, KT>(fa, as, wm * TM * 32, g, r, h);
+                else                 read_frag_kouter<TM, BM>(fa, as, wm * TM * 32, g, r, h);
+                if constexpr (B_KIN) read_frag_kinner<TN, KT>(fb, bs, wn * TN * 32, g, r, h);
+                else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q],
+                                                                             acc[i][j], 0, 0, 0);
+            }
+            if (fetched) {
+                la.store(ra, As[buf ^ 1]);
+                lb.store(rb, Bs[buf ^ 1]);
+            }
+            __syncthreads();
+            buf ^= 1;
         }
-        const float* as = As[cur];
-        const float* bs = Bs[cur];
-#pragma unroll
-        for (int g = 0; g < KT / 8; g++) {
-            float fa[TM][4], fb[TN][4];
-            if constexpr (A_KIN) read_frag_kinner<TM, KT>(fa, as, wm * TM * 32, g, r, h);
-            else                 read_frag_kouter<TM, BM>(fa, as, wm * TM * 32, g, r, h);
-            if constexpr (B_KIN) read_frag_kinner<TN, KT>(fb, bs, wn * TN * 32, g, r, h);
-            else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
-#pragma unroll
-            for (int q = 0; q < 4; q++)
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q],
-                                                                         acc[i][j], 0, 0, 0);
-        }
-        if (it + 1 < ntile) {
-            la.store(ra, As[cur ^ 1]);
-            lb.store(rb, Bs[cur ^ 1]);
-        }
-        __syncthreads();
-    }
 
-    // ---- epilogue: predicated stores ------------------------------------------
-    // MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
-    // K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
+        // ---- epilogue: predicated stores (they drain while the next tile computes) ----
+        // MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
+        // K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+        for (int i = 0; i < TM; i++) {
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-            const int mrow = 8 * (e / 4) + 4 * h + (e % 4);
-            const int row = row0 + wm * TM * 32 + (A_KIN ? (i * 32 + mrow) : (TM * mrow + i));
-            if (row >= p.rows) continue;
-            float* crow = C + (size_t)row * p.ldc;
-            if constexpr (B_KIN) {
+            for (int e = 0; e < 16; e++) {
+                const int mrow = 8 * (e / 4) + 4 * h + (e % 4);
+                const int row = cur.row0 + wm * TM * 32 + (A_KIN ? (i * 32 + mrow) : (TM * mrow + i));
+                if (row < p.rows) {
+                    float* crow = cur.c_ptr + (size_t)row * p.ldc;
+                    if constexpr (B_KIN) {
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int col = col0 + wn * TN * 32 + j * 32 + r;
-                    if (col < p.cols) crow[col] = acc[i][j][e];
-                }
-            } else {
-                const int col = col0 + wn * TN * 32 + TN * r;
-                if (col < p.cols) {
-                    if constexpr (TN == 1) {
-                        crow[col] = acc[i][0][e];
-                    } else if constexpr (TN == 2) {
-                        v2f v = {acc[i][0][e], acc[i][1][e]};
-                        *(v2f*)(crow + col) = v;
+                        for (int j = 0; j < TN; j++) {
+                            const int col = cur.col0 + wn * TN * 32 + j * 32 + r;
+                            if (col < p.cols) crow[col] = acc[i][j][e];
+                        }
                     } else {
-                        v4f v = {acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
-                        *(v4f*)(crow + col) = v;
+                        const int col = cur.col0 + wn * TN * 32 + TN * r;
+                        if (col < p.cols) {
+                            if constexpr (TN == 1) {
+                                crow[col] = acc[i][0][e];
+                            } else if constexpr (TN == 2) {
+                                v2f v = {acc[i][0][e], acc[i][1][e]};
+                                *(v2f*)(crow + col) = v;
+                            } else {
+                                v4f v = {acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
+                                *(v4f*)(crow + col) = v;
+                            }
+                        }
                     }
                 }
             }
         }
+        if (!has_next) break;
+        for (int i = 0; i < TM; i++)
+            for (int j = 0; j < TN; j++) acc[i][j] = (v16f)(0.0f);
+        cur = nxt;
+        lid += G;
     }
 }
 
 // ---------------------------------------------------------------------------
 // Host side: tile choice and launch
 // ---------------------------------------------------------------------------
+struct DeviceInfo { int num_cu; };
+
+static int device_num_cu() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT>
 static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    auto kernel = gemm_f32_mfma<A_KIN, B_KIN, WM, WN, TM, TN, KT>;
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
-    const long long nwg = (long long)p.tiles_m * p.tiles_n * p.nz;
-    if (nwg <= 0 || nwg > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((gemm_f32_mfma<A_KIN, B_KIN, WM, WN, TM, TN, KT>), dim3((unsigned)nwg),
-                       dim3(NTHREADS), 0, stream, p);
+    const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
+    if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidValue;
+    // workgroups the device keeps resident: one persistent workgroup per slot
+    static int resident_per_cu = 0;   // per instantiation; a benign race fills it with the same value
+    if (resident_per_cu == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NTHREADS, 0) != hipSuccess || n < 1)
+            n = 1;
+        resident_per_cu = n;
+    }
+    // One persistent workgroup per resident slot, trimmed so that every workgroup gets the
+    // same number of tiles (+-1): a static schedule has no tail to balance a ragged last round.
+    const long long slots = (long long)device_num_cu() * resident_per_cu;
+    long long grid = total;
+    if (total > slots) {
+        const long long rounds = (total + slots - 1) / slots;
+        grid = (total + rounds - 1) / rounds;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -352,6 +454,10 @@ static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stre
         case TILE_64x256:  return launch_cfg<A_KIN, B_KIN, 1, 4, 2, 2, 16>(p, stream);
         case TILE_128x64:  return launch_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 16>(p, stream);
         case TILE_64x128:  return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 2, 16>(p, stream);
+        case TILE_128x128_K32: return launch_cfg<A_KIN, B_KIN, 2, 2, 2, 2, 32>(p, stream);
+        case TILE_64x64_K32:   return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 32>(p, stream);
+        case TILE_128x64_K32:  return launch_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 32>(p, stream);
+        case TILE_64x128_K32:  return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 2, 32>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -359,28 +465,44 @@ static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stre
 static int g_forced_tile = TILE_AUTO;
 void gemm_force_tile(int tile) { g_forced_tile = tile; }
 
-static const int kTileM[TILE_COUNT] = {128, 64, 256, 64, 128, 64};
-static const int kTileN[TILE_COUNT] = {128, 64, 64, 256, 64, 128};
+// What the tile shapes are worth, measured on MI355X (fractions of a compute unit's
+// FP32 matrix peak): `alone` is what one resident workgroup sustains by itself (its
+// global-load latency is exposed), `cap` what a full compute unit reaches with
+// `resident` workgroups sharing it.
+struct TileTraits { int bm, bn, kt, resident; float alone, cap; };
+static const TileTraits kTiles[TILE_COUNT] = {
+    /* TILE_128x128     */ {128, 128, 16, 4, 0.62f, 0.92f},
+    /* TILE_64x64       */ { 64,  64, 16, 8, 0.35f, 0.82f},
+    /* TILE_256x64      */ {256,  64, 16, 4, 0.62f, 0.88f},
+    /* TILE_64x256      */ { 64, 256, 16, 4, 0.62f, 0.88f},
+    /* TILE_128x64      */ {128,  64, 16, 6, 0.48f, 0.85f},
+    /* TILE_64x128      */ { 64, 128, 16, 6, 0.48f, 0.85f},
+    /* TILE_128x128_K32 */ {128, 128, 32, 2, 0.65f, 0.88f},
+    /* TILE_64x64_K32   */ { 64,  64, 32, 5, 0.42f, 0.82f},
+    /* TILE_128x64_K32  */ {128,  64, 32, 3, 0.52f, 0.84f},
+    /* TILE_64x128_K32  */ { 64, 128, 32, 3, 0.52f, 0.84f},
+};
 
-// Pick the tile shape with the lowest estimated cost: work actually issued to the
-// matrix cores (padded tiles), stretched by how unevenly the workgroups fill the
-// compute units.
-int gemm_choose_tile(int rows, int cols, int nz, int num_cu) {
+// Pick the tile shape with the lowest estimated time: the matrix work of the busiest
+// compute unit (padded tiles, k rounded up to the stage), divided by what that unit
+// sustains with the workgroups it gets.
+int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu) {
     if (g_forced_tile != TILE_AUTO) return g_forced_tile;
     int best = TILE_128x128;
     double best_cost = 1e300;
     for (int tile = 0; tile < TILE_COUNT; tile++) {
-        const int bm = kTileM[tile], bn = kTileN[tile];
-        const long long tm = (rows + bm - 1) / bm, tn = (cols + bn - 1) / bn;
-        const long long nwg = tm * tn * nz;
-        // workgroups resident per CU: the small tiles leave room for more
-        const int resident = (bm * bn >= 128 * 128) ? 2 : 4;
-        const long long slots = (long long)num_cu * resident;
-        const long long rounds = (nwg + slots - 1) / slots;
-        // time ~ rounds * (tile work / resident sharing) ; small tiles pay a fixed overhead
-        const double per_tile = (double)bm * bn * (1.0 + 1024.0 / (bm * bn) * 4.0);
-        const double cost = (double)rounds * per_tile * resident;
-        if (cost < best_cost * 0.999) { best_cost = cost; best = tile; }
+        const TileTraits& tt = kTiles[tile];
+        const long long tm = (rows + tt.bm - 1) / tt.bm, tn = (cols + tt.bn - 1) / tt.bn;
+        const long long total = tm * tn * nz;
+        const long long per_cu = (total + num_cu - 1) / num_cu;       // tiles on the busiest unit
+        const long long together = per_cu < tt.resident ? per_cu : tt.resident;
+        double eff = together * (double)tt.alone;
+        if (eff > tt.cap) eff = tt.cap;
+        const long long kp = ((long long)k + tt.kt - 1) / tt.kt * tt.kt;
+        // a short tile pays for filling and draining its pipeline: about two stages' worth
+        const double work = (double)per_cu * tt.bm * tt.bn * (double)(kp + 2 * tt.kt);
+        const double cost = work / eff;
+        if (cost < best_cost * 0.98) { best_cost = cost; best = tile; }
     }
     return best;
 }

@@ -123,7 +123,10 @@ SIGNATURES = {
 }
 
 
-def load(path=LIB_PATH):
+def load(path=None):
+    """Loads the library from the package directory, or from $DRAGON_HIP_LIBRARY when set
+    (for trying out another build of the same ABI)."""
+    path = path or os.environ.get("DRAGON_HIP_LIBRARY") or LIB_PATH
     if not os.path.exists(path):
         raise ImportError(
             "libdragon_hip.so is not built (%s); run dragon-alpha-v1.2_amd/csrc/build.sh" % path)

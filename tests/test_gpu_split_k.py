@@ -83,6 +83,21 @@ def test_split_k_equals_unsplit_within_tolerance(gpu, variant):
         assert rel_fro(C, oracle.SKbuf_summary(Cb0, C0, GZ - 1)) < 2e-6
 
 
+@pytest.mark.parametrize("tile", [1, 6, 7, 9])
+def test_split_k_with_every_stage_depth(gpu, tile):
+    # K slices that are not multiples of the k stage (16 or 32), on forced tile shapes
+    rng = np.random.default_rng(50 + tile)
+    gpu.force_tile(tile)
+    try:
+        for variant in (NN, T1, T2):
+            A, B = logical_operands(variant, rng, 132, 68, 1000, dist="int")
+            C, Cbuf = run_sk(gpu, variant, A, B, 6, summary=False)
+            C0, Cb0 = oracle.matMulSK(variant, 6, A, B)
+            assert np.array_equal(C, C0) and np.array_equal(Cbuf, Cb0)
+    finally:
+        gpu.force_tile(-1)
+
+
 def test_degenerate_slices(gpu):
     # K smaller than 8*GridZ: K_slice = 0, every slice but the last is empty and must be
     # written as zeros; the last carries the whole product
