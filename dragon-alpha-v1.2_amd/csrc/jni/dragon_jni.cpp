@@ -1,0 +1,312 @@
+// JNI shim: the exact symbols the reference's Java classes bind
+//   z.dragon.engine.cuda.impl.math.Cuda_matMul        (reference: Cuda_matMul/Cuda_matMul/A.cu:20-178)
+//   z.dragon.engine.cuda.impl.math.Cuda_batchMatMul   (reference: Cuda_batchMatMul/Cuda_batchMatMul/A.cu:20-143)
+//   z.dragon.engine.cuda.impl.Cuda (the subset this path uses; reference: Cuda/Cuda/Cuda_memory.cuh,
+//   Cuda_Stream.cuh, Cuda_Event.cuh, Cuda_Device.cuh, Cuda_float.cuh)
+// each forwarding to the C ABI of include/dragon_hip_gemm.h / dragon_hip_runtime.h and turning a
+// non-zero status into z.dragon.engine.cuda.impl.CudaException(int), as the reference's
+// handleError / throwCudaException do (Cuda_matMul/Cuda_matMul/JNITool.cuh:9-25).
+//
+// Built only where a JDK provides <jni.h> (build_jni.sh next to this file); the rest of the
+// library does not depend on it.
+#if __has_include(<jni.h>)
+#include <jni.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <vector>
+
+#include "../../../include/dragon_hip_gemm.h"
+#include "../../../include/dragon_hip_runtime.h"
+
+namespace {
+
+JavaVM* g_jvm = nullptr;
+
+void throwCudaException(JNIEnv* env, int code) {
+    jclass cls = env->FindClass("z/dragon/engine/cuda/impl/CudaException");
+    if (cls == nullptr) return;                       // NoClassDefFoundError is already pending
+    jmethodID ctor = env->GetMethodID(cls, "<init>", "(I)V");
+    if (ctor == nullptr) return;
+    jobject ex = env->NewObject(cls, ctor, (jint)code);
+    if (ex != nullptr) env->Throw((jthrowable)ex);
+}
+inline void handle(JNIEnv* env, int code) {
+    if (code != 0) throwCudaException(env, code);
+}
+inline jlong handle_addr(JNIEnv* env, int64_t v) {
+    if (v == 0) {
+        int code = dragon_Cuda_getLastExceptionType();
+        throwCudaException(env, code ? code : 2);
+    }
+    return (jlong)v;
+}
+
+// The reference copies the handles into a fixed jlong streams[10]; a longer array is an
+// error here instead of a buffer overrun.
+struct Streams {
+    int64_t s[10];
+    int n;
+    bool ok;
+    Streams(JNIEnv* env, jlongArray arr, jint length) : n(length), ok(false) {
+        if (arr == nullptr || length < 1 || length > 10 || env->GetArrayLength(arr) < length) {
+            throwCudaException(env, 1);
+            return;
+        }
+        jlong tmp[10];
+        env->GetLongArrayRegion(arr, 0, length, tmp);
+        for (int i = 0; i < length; i++) s[i] = (int64_t)tmp[i];
+        ok = true;
+    }
+};
+
+std::vector<int64_t> long_array(JNIEnv* env, jlongArray arr, jint length) {
+    std::vector<int64_t> v;
+    if (arr == nullptr || length <= 0) return v;
+    std::vector<jlong> tmp((size_t)length);
+    env->GetLongArrayRegion(arr, 0, length, tmp.data());
+    v.assign(tmp.begin(), tmp.end());
+    return v;
+}
+
+}  // namespace
+
+#define MM(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1matMul_##name
+#define BMM(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1batchMatMul_##name
+#define RT(name) Java_z_dragon_engine_cuda_impl_Cuda_##name
+
+extern "C" {
+
+JNIEXPORT jint JNICALL JNI_OnLoad(JavaVM* vm, void*) {   // reference: Cuda/Cuda/JNIConfig.cuh:12-20
+    g_jvm = vm;
+    return JNI_VERSION_1_8;
+}
+
+// ---- Cuda_matMul -------------------------------------------------------------------------
+JNIEXPORT void JNICALL MM(SKbuf_1summary)(JNIEnv* env, jclass, jlong stream, jlong dCbuf, jlong dC,
+                                          jint part, jint sizeC) {
+    handle(env, dragon_Cuda_matMul_SKbuf_summary(stream, dCbuf, dC, part, sizeC));
+}
+
+#define DEF_MM2D(jname, cname)                                                                   \
+    JNIEXPORT void JNICALL MM(jname)(JNIEnv* env, jclass, jlongArray streamArray, jint length,   \
+                                     jlong dA, jlong dB, jlong dC, jint N, jint M, jint K) {     \
+        Streams st(env, streamArray, length);                                                    \
+        if (!st.ok) return;                                                                      \
+        handle(env, cname(st.s, st.n, dA, dB, dC, N, M, K));                                     \
+    }
+DEF_MM2D(matMul, dragon_Cuda_matMul_matMul)
+DEF_MM2D(matMulT1, dragon_Cuda_matMul_matMulT1)
+DEF_MM2D(matMulT2, dragon_Cuda_matMul_matMulT2)
+DEF_MM2D(matMul_1mma, dragon_Cuda_matMul_matMul_mma)
+DEF_MM2D(matMulT1_1mma, dragon_Cuda_matMul_matMulT1_mma)
+DEF_MM2D(matMulT2_1mma, dragon_Cuda_matMul_matMulT2_mma)
+
+#define DEF_MMSK(jname, cname)                                                                   \
+    JNIEXPORT void JNICALL MM(jname)(JNIEnv* env, jclass, jlongArray streamArray, jint length,   \
+                                     jint GridZ, jlong dA, jlong dB, jlong dC, jlong dCbuf,      \
+                                     jint N, jint M, jint K) {                                   \
+        Streams st(env, streamArray, length);                                                    \
+        if (!st.ok) return;                                                                      \
+        handle(env, cname(st.s, st.n, GridZ, dA, dB, dC, dCbuf, N, M, K));                       \
+    }
+DEF_MMSK(matMulSK, dragon_Cuda_matMul_matMulSK)
+DEF_MMSK(matMulT1SK, dragon_Cuda_matMul_matMulT1SK)
+DEF_MMSK(matMulT2SK, dragon_Cuda_matMul_matMulT2SK)
+
+// ---- Cuda_batchMatMul -------------------------------------------------------------------------
+#define DEF_BMM(jname, cname)                                                                    \
+    JNIEXPORT void JNICALL BMM(jname)(JNIEnv* env, jclass, jlongArray streamArray, jint length,  \
+                                      jlong dA, jlong dB, jlong dC, jint Batch, jint d0,         \
+                                      jint d1, jint d2, jint d3) {                               \
+        Streams st(env, streamArray, length);                                                    \
+        if (!st.ok) return;                                                                      \
+        handle(env, cname(st.s, st.n, dA, dB, dC, Batch, d0, d1, d2, d3));                       \
+    }
+DEF_BMM(batchMatMul, dragon_Cuda_batchMatMul_batchMatMul)
+DEF_BMM(batchMatMul_1texture, dragon_Cuda_batchMatMul_batchMatMul_texture)
+DEF_BMM(batchMatMulT1, dragon_Cuda_batchMatMul_batchMatMulT1)
+DEF_BMM(batchMatMulT1_1mma, dragon_Cuda_batchMatMul_batchMatMulT1_mma)
+DEF_BMM(batchMatMulT2, dragon_Cuda_batchMatMul_batchMatMulT2)
+DEF_BMM(batchMatMulT2_1texture, dragon_Cuda_batchMatMul_batchMatMulT2_texture)
+
+#define DEF_BMM_MMA(jname, cname)                                                                \
+    JNIEXPORT void JNICALL BMM(jname)(JNIEnv* env, jclass, jboolean useTexture,                  \
+                                      jlongArray streamArray, jint length, jlong dA, jlong dB,   \
+                                      jlong dC, jint Batch, jint d0, jint d1, jint d2, jint d3) {\
+        Streams st(env, streamArray, length);                                                    \
+        if (!st.ok) return;                                                                      \
+        handle(env, cname(useTexture ? 1 : 0, st.s, st.n, dA, dB, dC, Batch, d0, d1, d2, d3));   \
+    }
+DEF_BMM_MMA(batchMatMul_1mma, dragon_Cuda_batchMatMul_batchMatMul_mma)
+DEF_BMM_MMA(batchMatMulT2_1mma, dragon_Cuda_batchMatMul_batchMatMulT2_mma)
+
+// ---- Cuda: memory ---------------------------------------------------------------------------------
+JNIEXPORT jlong JNICALL RT(malloc)(JNIEnv* env, jclass, jlong size) {
+    return handle_addr(env, dragon_Cuda_malloc(size));
+}
+JNIEXPORT void JNICALL RT(free)(JNIEnv* env, jclass, jlong address) { handle(env, dragon_Cuda_free(address)); }
+JNIEXPORT jlong JNICALL RT(mallocHost)(JNIEnv* env, jclass, jlong size) {
+    return handle_addr(env, dragon_Cuda_mallocHost(size));
+}
+JNIEXPORT void JNICALL RT(freeHost)(JNIEnv* env, jclass, jlong address) { handle(env, dragon_Cuda_freeHost(address)); }
+JNIEXPORT void JNICALL RT(memsetAsync)(JNIEnv* env, jclass, jlong stream, jlong address, jint value, jlong size) {
+    handle(env, dragon_Cuda_memsetAsync(stream, address, value, size));
+}
+JNIEXPORT void JNICALL RT(memcpyAsyncHostToDevice)(JNIEnv* env, jclass, jlong s, jlong dst, jlong src, jlong n) {
+    handle(env, dragon_Cuda_memcpyAsyncHostToDevice(s, dst, src, n));
+}
+JNIEXPORT void JNICALL RT(memcpyAsyncDeviceToHost)(JNIEnv* env, jclass, jlong s, jlong dst, jlong src, jlong n) {
+    handle(env, dragon_Cuda_memcpyAsyncDeviceToHost(s, dst, src, n));
+}
+JNIEXPORT void JNICALL RT(memcpyAsyncDeviceToDevice)(JNIEnv* env, jclass, jlong s, jlong dst, jlong src, jlong n) {
+    handle(env, dragon_Cuda_memcpyAsyncDeviceToDevice(s, dst, src, n));
+}
+JNIEXPORT void JNICALL RT(memcpyAsyncHostToHost)(JNIEnv* env, jclass, jlong s, jlong dst, jlong src, jlong n) {
+    handle(env, dragon_Cuda_memcpyAsyncHostToHost(s, dst, src, n));
+}
+JNIEXPORT void JNICALL RT(memcpyAsyncDefault)(JNIEnv* env, jclass, jlong s, jlong dst, jlong src, jlong n) {
+    handle(env, dragon_Cuda_memcpyAsyncDefault(s, dst, src, n));
+}
+
+// ---- Cuda: device ----------------------------------------------------------------------------------
+JNIEXPORT jint JNICALL RT(getDeviceId)(JNIEnv*, jclass) { return dragon_Cuda_getDeviceId(); }
+JNIEXPORT jint JNICALL RT(getDeviceCount)(JNIEnv*, jclass) { return dragon_Cuda_getDeviceCount(); }
+JNIEXPORT void JNICALL RT(setDevice)(JNIEnv* env, jclass, jint id) { handle(env, dragon_Cuda_setDevice(id)); }
+JNIEXPORT void JNICALL RT(deviceSynchronize)(JNIEnv* env, jclass) { handle(env, dragon_Cuda_deviceSynchronize()); }
+
+// ---- Cuda: streams (overloads carry the JNI signature suffix) -------------------------------------------
+JNIEXPORT jlong JNICALL RT(newStream_1Blocking__)(JNIEnv* env, jclass) {
+    return handle_addr(env, dragon_Cuda_newStream_Blocking());
+}
+JNIEXPORT jlong JNICALL RT(newStream_1Blocking__I)(JNIEnv* env, jclass, jint) {   // priority ignored
+    return handle_addr(env, dragon_Cuda_newStream_Blocking());
+}
+JNIEXPORT jlong JNICALL RT(newStream_1NonBlocking__)(JNIEnv* env, jclass) {
+    return handle_addr(env, dragon_Cuda_newStream_NonBlocking());
+}
+JNIEXPORT jlong JNICALL RT(newStream_1NonBlocking__I)(JNIEnv* env, jclass, jint) {
+    return handle_addr(env, dragon_Cuda_newStream_NonBlocking());
+}
+JNIEXPORT void JNICALL RT(deleteStream__J)(JNIEnv* env, jclass, jlong stream) {
+    handle(env, dragon_Cuda_deleteStream(stream));
+}
+JNIEXPORT void JNICALL RT(deleteStream___3JI)(JNIEnv* env, jclass, jlongArray arr, jint length) {
+    std::vector<int64_t> v = long_array(env, arr, length);
+    handle(env, dragon_Cuda_deleteStreams(v.data(), (int)v.size()));
+}
+JNIEXPORT jboolean JNICALL RT(streamQuery)(JNIEnv* env, jclass, jlong stream) {
+    int r = dragon_Cuda_streamQuery(stream);
+    if (r < 0) { throwCudaException(env, dragon_Cuda_getLastExceptionType()); return JNI_FALSE; }
+    return r ? JNI_TRUE : JNI_FALSE;
+}
+JNIEXPORT void JNICALL RT(streamSynchronize__J)(JNIEnv* env, jclass, jlong stream) {
+    handle(env, dragon_Cuda_streamSynchronize(stream));
+}
+JNIEXPORT void JNICALL RT(streamSynchronize___3JI)(JNIEnv* env, jclass, jlongArray arr, jint length) {
+    std::vector<int64_t> v = long_array(env, arr, length);
+    handle(env, dragon_Cuda_streamsSynchronize(v.data(), (int)v.size()));
+}
+
+// ---- Cuda: events -------------------------------------------------------------------------------------------
+JNIEXPORT jlong JNICALL RT(newEvent_1Default)(JNIEnv* env, jclass) { return handle_addr(env, dragon_Cuda_newEvent_Default()); }
+JNIEXPORT jlong JNICALL RT(newEvent_1BlockingSync)(JNIEnv* env, jclass) { return handle_addr(env, dragon_Cuda_newEvent_BlockingSync()); }
+JNIEXPORT jlong JNICALL RT(newEvent_1DisableTiming)(JNIEnv* env, jclass) { return handle_addr(env, dragon_Cuda_newEvent_DisableTiming()); }
+JNIEXPORT void JNICALL RT(deleteEvent)(JNIEnv* env, jclass, jlong event) { handle(env, dragon_Cuda_deleteEvent(event)); }
+JNIEXPORT void JNICALL RT(eventRecord__JJ)(JNIEnv* env, jclass, jlong event, jlong stream) {
+    handle(env, dragon_Cuda_eventRecord(event, stream));
+}
+JNIEXPORT void JNICALL RT(eventRecord__J_3JI)(JNIEnv* env, jclass, jlong event, jlongArray arr, jint length) {
+    std::vector<int64_t> v = long_array(env, arr, length);
+    handle(env, dragon_Cuda_eventRecord_streams(event, v.data(), (int)v.size()));
+}
+JNIEXPORT void JNICALL RT(eventSynchronize)(JNIEnv* env, jclass, jlong event) { handle(env, dragon_Cuda_eventSynchronize(event)); }
+JNIEXPORT void JNICALL RT(eventSync_1Del)(JNIEnv* env, jclass, jlong event) { handle(env, dragon_Cuda_eventSync_Del(event)); }
+JNIEXPORT void JNICALL RT(eventSynchronize_1delete)(JNIEnv* env, jclass, jlong event) { handle(env, dragon_Cuda_eventSync_Del(event)); }
+JNIEXPORT jfloat JNICALL RT(eventElapsedTime)(JNIEnv* env, jclass, jlong e0, jlong e1) {
+    float ms = dragon_Cuda_eventElapsedTime(e0, e1);
+    if (ms < 0) throwCudaException(env, dragon_Cuda_getLastExceptionType());
+    return ms;
+}
+JNIEXPORT void JNICALL RT(streamWaitEvent_1default)(JNIEnv* env, jclass, jlong stream, jlong event) {
+    handle(env, dragon_Cuda_streamWaitEvent_default(stream, event));
+}
+JNIEXPORT void JNICALL RT(streamsWaitEvent_1default)(JNIEnv* env, jclass, jlongArray arr, jint length, jlong event) {
+    std::vector<int64_t> v = long_array(env, arr, length);
+    handle(env, dragon_Cuda_streamsWaitEvent_default(v.data(), (int)v.size(), event));
+}
+
+// ---- Cuda: errors -----------------------------------------------------------------------------------------------
+JNIEXPORT jstring JNICALL RT(getExceptionName)(JNIEnv* env, jclass, jint type) {
+    return env->NewStringUTF(dragon_Cuda_getExceptionName(type));
+}
+JNIEXPORT jstring JNICALL RT(getExceptionInfo)(JNIEnv* env, jclass, jint type) {
+    return env->NewStringUTF(dragon_Cuda_getExceptionInfo(type));
+}
+JNIEXPORT jint JNICALL RT(getLastExceptionType)(JNIEnv*, jclass) { return dragon_Cuda_getLastExceptionType(); }
+
+// ---- Cuda: float fill / transfer -------------------------------------------------------------------------------------
+JNIEXPORT void JNICALL RT(set1D__JJFI)(JNIEnv* env, jclass, jlong stream, jlong address, jfloat value, jint length) {
+    handle(env, dragon_Cuda_set1D_value(stream, address, value, length));
+}
+JNIEXPORT void JNICALL RT(set2D__JJFIII)(JNIEnv* env, jclass, jlong stream, jlong address, jfloat value,
+                                         jint height, jint width, jint stride) {
+    handle(env, dragon_Cuda_set2D_value(stream, address, value, height, width, stride));
+}
+JNIEXPORT void JNICALL RT(get1D)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value, jint length) {
+    std::vector<float> x((size_t)(length > 0 ? length : 0));
+    int rc = dragon_Cuda_get1D(stream, address, x.data(), length);
+    if (rc) { throwCudaException(env, rc); return; }
+    env->SetFloatArrayRegion(value, 0, length, x.data());
+}
+JNIEXPORT void JNICALL RT(get2D)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value,
+                                 jint height, jint width, jint stride) {
+    std::vector<float> x((size_t)height * (size_t)width);
+    int rc = dragon_Cuda_get2D(stream, address, x.data(), height, width, stride);
+    if (rc) { throwCudaException(env, rc); return; }
+    env->SetFloatArrayRegion(value, 0, height * width, x.data());
+}
+JNIEXPORT void JNICALL RT(get1D_1v2)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value,
+                                     jlong buf, jint length) {
+    std::vector<float> x((size_t)(length > 0 ? length : 0));
+    int rc = dragon_Cuda_get1D_v2(stream, address, x.data(), buf, length);
+    if (rc) { throwCudaException(env, rc); return; }
+    env->SetFloatArrayRegion(value, 0, length, x.data());
+}
+JNIEXPORT void JNICALL RT(get2D_1v2)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value,
+                                     jlong buf, jint height, jint width, jint stride) {
+    std::vector<float> x((size_t)height * (size_t)width);
+    int rc = dragon_Cuda_get2D_v2(stream, address, x.data(), buf, height, width, stride);
+    if (rc) { throwCudaException(env, rc); return; }
+    env->SetFloatArrayRegion(value, 0, height * width, x.data());
+}
+JNIEXPORT void JNICALL RT(set1D__JJ_3FI)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value, jint length) {
+    jfloat* x = env->GetFloatArrayElements(value, nullptr);
+    int rc = dragon_Cuda_set1D(stream, address, x, length);
+    env->ReleaseFloatArrayElements(value, x, JNI_ABORT);
+    handle(env, rc);
+}
+JNIEXPORT void JNICALL RT(set2D__JJ_3FIII)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value,
+                                           jint height, jint width, jint stride) {
+    jfloat* x = env->GetFloatArrayElements(value, nullptr);
+    int rc = dragon_Cuda_set2D(stream, address, x, height, width, stride);
+    env->ReleaseFloatArrayElements(value, x, JNI_ABORT);
+    handle(env, rc);
+}
+JNIEXPORT void JNICALL RT(set1D_1v2__JJ_3FJI)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value,
+                                              jlong buf, jint length) {
+    jfloat* x = env->GetFloatArrayElements(value, nullptr);
+    int rc = dragon_Cuda_set1D_v2(stream, address, x, buf, length);
+    env->ReleaseFloatArrayElements(value, x, JNI_ABORT);
+    handle(env, rc);
+}
+JNIEXPORT void JNICALL RT(set2D_1v2__JJ_3FJIII)(JNIEnv* env, jclass, jlong stream, jlong address, jfloatArray value,
+                                                jlong buf, jint height, jint width, jint stride) {
+    jfloat* x = env->GetFloatArrayElements(value, nullptr);
+    int rc = dragon_Cuda_set2D_v2(stream, address, x, buf, height, width, stride);
+    env->ReleaseFloatArrayElements(value, x, JNI_ABORT);
+    handle(env, rc);
+}
+
+}  // extern "C"
+#endif  // __has_include(<jni.h>)

@@ -1,0 +1,31 @@
+"""Writes tests/golden/jni_symbols.txt: the JNI export names the reference's native
+libraries define for the matrix-multiplication path and the runtime subset it uses,
+read as text from the reference's source files (nothing is imported or run).
+
+usage: python tests/golden/make_jni_symbols.py [/root/reference]
+"""
+import os
+import re
+import sys
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+CU = os.path.join(REF, "source", "engine-cuda-base")
+FILES = [
+    "Cuda_matMul/Cuda_matMul/A.cu",
+    "Cuda_batchMatMul/Cuda_batchMatMul/A.cu",
+    "Cuda/Cuda/Cuda_memory.cuh",
+    "Cuda/Cuda/Cuda_Stream.cuh",
+    "Cuda/Cuda/Cuda_Event.cuh",
+    "Cuda/Cuda/Cuda_Device.cuh",
+    "Cuda/Cuda/Cuda_Exception.cuh",
+    "Cuda/Cuda/Cuda_float.cuh",
+]
+out = []
+for f in FILES:
+    text = open(os.path.join(CU, f), encoding="utf-8", errors="replace").read()
+    for name in re.findall(r"\b(Java_z_dragon_engine_cuda_impl_\w+)\s*\(", text):
+        out.append("%s %s" % (f, name))
+dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "jni_symbols.txt")
+with open(dst, "w") as fh:
+    fh.write("\n".join(out) + "\n")
+print("wrote %d names to %s" % (len(out), dst))
