@@ -18,7 +18,12 @@ enum GemmTile {
     TILE_64x64_K32 = 7,
     TILE_128x64_K32 = 8,
     TILE_64x128_K32 = 9,
-    TILE_COUNT = 10
+    TILE_64x64_K64 = 10,    // long stages: one workgroup per compute unit still covers its load latency
+    TILE_64x64_K128 = 11,
+    TILE_128x128_K64 = 12,
+    TILE_128x64_K64 = 13,
+    TILE_64x128_K64 = 14,
+    TILE_COUNT = 15
 };
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.

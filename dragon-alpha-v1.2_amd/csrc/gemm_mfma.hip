@@ -69,10 +69,11 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
 
 // Chunk swizzle of a K-inner tile.  Rows hold CPR = KT/4 chunks of 16 bytes with no
 // padding.  With 4 chunks per row two rows share the 32 banks, so the row pair index
-// (r>>1)&3 permutes the chunks; with 8 chunks per row the row index r&7 does.
+// (r>>1)&3 permutes the chunks; with 8 or more chunks per row every row starts at bank 0
+// and the row index r&7 permutes the low three bits of the chunk index.
 template <int KT>
 __device__ __forceinline__ int kin_swizzle(int row) {
-    static_assert(KT == 16 || KT == 32, "k per stage: 16 or 32");
+    static_assert(KT == 16 || KT == 32 || KT == 64 || KT == 128, "k per stage: 16, 32, 64 or 128");
     return (KT == 16) ? ((row >> 1) & 3) : (row & 7);
 }
 
@@ -357,7 +358,8 @@ void gemm_f32_mfma(const GemmParams p) {
             buf ^= 1;
         }
 
-        // ---- epilogue: predicated stores (they drain while the next tile computes) ----
+        // ---- epilogue: predicated streaming stores (C is written once and never read back
+        // here; they drain while the next tile computes) ----
         // MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
         // K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
 #pragma unroll
@@ -372,19 +374,19 @@ void gemm_f32_mfma(const GemmParams p) {
 #pragma unroll
                         for (int j = 0; j < TN; j++) {
                             const int col = cur.col0 + wn * TN * 32 + j * 32 + r;
-                            if (col < p.cols) crow[col] = acc[i][j][e];
+                            if (col < p.cols) __builtin_nontemporal_store(acc[i][j][e], crow + col);
                         }
                     } else {
                         const int col = cur.col0 + wn * TN * 32 + TN * r;
                         if (col < p.cols) {
                             if constexpr (TN == 1) {
-                                crow[col] = acc[i][0][e];
+                                __builtin_nontemporal_store(acc[i][0][e], crow + col);
                             } else if constexpr (TN == 2) {
                                 v2f v = {acc[i][0][e], acc[i][1][e]};
-                                *(v2f*)(crow + col) = v;
+                                __builtin_nontemporal_store(v, (v2f*)(crow + col));
                             } else {
                                 v4f v = {acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
-                                *(v4f*)(crow + col) = v;
+                                __builtin_nontemporal_store(v, (v4f*)(crow + col));
                             }
                         }
                     }
@@ -458,6 +460,11 @@ static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stre
         case TILE_64x64_K32:   return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 32>(p, stream);
         case TILE_128x64_K32:  return launch_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 32>(p, stream);
         case TILE_64x128_K32:  return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 2, 32>(p, stream);
+        case TILE_64x64_K64:   return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 64>(p, stream);
+        case TILE_64x64_K128:  return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 128>(p, stream);
+        case TILE_128x128_K64: return launch_cfg<A_KIN, B_KIN, 2, 2, 2, 2, 64>(p, stream);
+        case TILE_128x64_K64:  return launch_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 64>(p, stream);
+        case TILE_64x128_K64:  return launch_cfg<A_KIN, B_KIN, 2, 2, 1, 2, 64>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -481,6 +488,11 @@ static const TileTraits kTiles[TILE_COUNT] = {
     /* TILE_64x64_K32   */ { 64,  64, 32, 5, 0.42f, 0.82f},
     /* TILE_128x64_K32  */ {128,  64, 32, 3, 0.52f, 0.84f},
     /* TILE_64x128_K32  */ { 64, 128, 32, 3, 0.52f, 0.84f},
+    /* TILE_64x64_K64   */ { 64,  64, 64, 2, 0.55f, 0.80f},
+    /* TILE_64x64_K128  */ { 64,  64, 128, 1, 0.65f, 0.65f},
+    /* TILE_128x128_K64 */ {128, 128, 64, 1, 0.80f, 0.80f},
+    /* TILE_128x64_K64  */ {128,  64, 64, 1, 0.70f, 0.70f},
+    /* TILE_64x128_K64  */ { 64, 128, 64, 1, 0.70f, 0.70f},
 };
 
 // Pick the tile shape with the lowest estimated time: the matrix work of the busiest

@@ -6,9 +6,10 @@
 // result is bit-identical to it.  The additions carry no multiply, so there is
 // nothing for the compiler to contract; reassociation is off by default.
 //
-// HBM-bound: reads part*sizeC floats once.  One float4 per thread per partial;
-// the loads of 8 partials are issued before the dependent Kahan chain consumes
-// them so that enough bytes are in flight.
+// HBM-bound: reads part*sizeC floats once.  The sum over the partials is a serial
+// chain per element, so the bytes in flight come from the elements: a C of at least
+// 1M floats uses one float4 per thread, a smaller one a single float per thread (four
+// times the threads), and the loads of 16 partials are issued ahead of the chain.
 #include <hip/hip_runtime.h>
 #include "gemm_mfma.h"
 
@@ -16,47 +17,56 @@ namespace dragon {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void kahan_step(v4f& v, v4f& c, v4f vbuf) {
+template <typename V>
+__device__ __forceinline__ void kahan_step(V& v, V& c, V vbuf) {
     vbuf = vbuf - c;          // subtract the error of the previous addition
-    const v4f t = v + vbuf;
+    const V t = v + vbuf;
     c = (t - v) - vbuf;       // recover what the addition lost
     v = t;
 }
 
+template <typename V>
 __global__ __launch_bounds__(256) void skbuf_summary_kernel(const float* __restrict__ Cbuf,
                                                             float* __restrict__ C,
-                                                            int part, int size4, size_t sizeC) {
+                                                            int part, int nvec, size_t sizeC) {
+    constexpr int W = sizeof(V) / sizeof(float);
+    constexpr int AHEAD = 16;
     const int stride = gridDim.x * blockDim.x;
-    for (int i4 = blockIdx.x * blockDim.x + threadIdx.x; i4 < size4; i4 += stride) {
-        const size_t at = (size_t)i4 * 4;
-        v4f v = *(const v4f*)(C + at);
-        v4f c = {0.f, 0.f, 0.f, 0.f};
+    for (int iv = blockIdx.x * blockDim.x + threadIdx.x; iv < nvec; iv += stride) {
+        const size_t at = (size_t)iv * W;
+        V v = *(const V*)(C + at);
+        V c = (V)(0.0f);
         const float* src = Cbuf + at;
         int p = 0;
-        for (; p + 8 <= part; p += 8) {
-            v4f b[8];
+        for (; p + AHEAD <= part; p += AHEAD) {
+            V b[AHEAD];
 #pragma unroll
-            for (int u = 0; u < 8; u++)
-                b[u] = __builtin_nontemporal_load((const v4f*)(src + (size_t)(p + u) * sizeC));
+            for (int u = 0; u < AHEAD; u++)
+                b[u] = __builtin_nontemporal_load((const V*)(src + (size_t)(p + u) * sizeC));
 #pragma unroll
-            for (int u = 0; u < 8; u++) kahan_step(v, c, b[u]);
+            for (int u = 0; u < AHEAD; u++) kahan_step(v, c, b[u]);
         }
         for (; p < part; p++)
-            kahan_step(v, c, __builtin_nontemporal_load((const v4f*)(src + (size_t)p * sizeC)));
-        *(v4f*)(C + at) = v;
+            kahan_step(v, c, __builtin_nontemporal_load((const V*)(src + (size_t)p * sizeC)));
+        *(V*)(C + at) = v;
     }
 }
 
 hipError_t skbuf_summary_launch(hipStream_t stream, const float* Cbuf, float* C, int part,
                                 int sizeC) {
-    const int size4 = sizeC >> 2;
-    if (size4 <= 0) return hipSuccess;
-    // 64 threads per workgroup spreads a small C over many compute units.
-    const int threads = 64;
-    int blocks = (size4 + threads - 1) / threads;
-    if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(skbuf_summary_kernel, dim3(blocks), dim3(threads), 0, stream, Cbuf, C, part,
-                       size4, (size_t)sizeC);
+    if (sizeC <= 0) return hipSuccess;
+    const int threads = 64;   // small workgroups spread a small C over many compute units
+    if (sizeC >= (1 << 20)) {
+        const int nvec = sizeC >> 2;
+        int blocks = (nvec + threads - 1) / threads;
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(skbuf_summary_kernel<v4f>, dim3(blocks), dim3(threads), 0, stream, Cbuf,
+                           C, part, nvec, (size_t)sizeC);
+    } else {
+        const int blocks = (sizeC + threads - 1) / threads;
+        hipLaunchKernelGGL(skbuf_summary_kernel<float>, dim3(blocks), dim3(threads), 0, stream, Cbuf,
+                           C, part, sizeC, (size_t)sizeC);
+    }
     return hipGetLastError();
 }
 
