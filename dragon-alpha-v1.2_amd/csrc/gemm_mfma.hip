@@ -67,14 +67,17 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
 // Tile staging: global -> registers -> LDS
 // ---------------------------------------------------------------------------
 
-// Chunk swizzle of a K-inner tile.  Rows hold CPR = KT/4 chunks of 16 bytes with no
-// padding.  With 4 chunks per row two rows share the 32 banks, so the row pair index
-// (r>>1)&3 permutes the chunks; with 8 or more chunks per row every row starts at bank 0
-// and the row index r&7 permutes the low three bits of the chunk index.
+// Chunk swizzle of a K-inner tile.  Rows hold CPR = KT/4 chunks of 16 bytes, no padding.
+// Measured on gfx950: a ds_read_b128 serves 16 lanes per cycle from 16 chunk slots (256
+// bytes wide), a ds_write_b128 8 lanes per cycle from 8 slots.  The fragment reads walk
+// DOWN the rows (16 consecutive rows, same logical chunk), the staging stores walk ALONG
+// a row; XOR-ing the chunk index with the index of the row's 256-byte group puts the 16
+// rows of a read on 16 different slots and leaves the stores a permutation of a
+// contiguous run.
 template <int KT>
 __device__ __forceinline__ int kin_swizzle(int row) {
     static_assert(KT == 16 || KT == 32 || KT == 64 || KT == 128, "k per stage: 16, 32, 64 or 128");
-    return (KT == 16) ? ((row >> 1) & 3) : (row & 7);
+    return (KT == 16) ? ((row >> 2) & 3) : (KT == 32) ? ((row >> 1) & 7) : (row & 15);
 }
 
 // K-inner operand: R rows of KT consecutive k.  LDS row stride KT floats, chunks swizzled.
@@ -86,16 +89,17 @@ struct KInner {
     static constexpr int LDS_STRIDE = KT;
     static constexpr int LDS_FLOATS = R * LDS_STRIDE;
     static_assert(R % RPP == 0 && PASSES >= 1, "tile does not divide over the workgroup");
-    static_assert(RPP % 8 == 0, "the swizzle must repeat from pass to pass");
 
     int off[PASSES];   // byte offset of this thread's chunk, or OOB_OFFSET if its row is outside
     int kcol;          // k offset of this thread's chunk inside the tile
-    int lds_at;        // float index of the first chunk in the LDS tile
+    int row_first;     // tile row of the first pass
+    int chunk;         // logical chunk index in the row
 
     __device__ __forceinline__ void init(int t, int row0, int outer_bound, int ld) {
         const int c = t % CPR, r0 = t / CPR;
         kcol = c * 4;
-        lds_at = r0 * LDS_STRIDE + 4 * (c ^ kin_swizzle<KT>(r0));
+        row_first = r0;
+        chunk = c;
 #pragma unroll
         for (int s = 0; s < PASSES; s++) {
             const int r = r0 + s * RPP;
@@ -110,7 +114,10 @@ struct KInner {
     }
     __device__ __forceinline__ void store(const v4f (&reg)[PASSES], float* lds) const {
 #pragma unroll
-        for (int s = 0; s < PASSES; s++) *(v4f*)(lds + lds_at + s * RPP * LDS_STRIDE) = reg[s];
+        for (int s = 0; s < PASSES; s++) {
+            const int r = row_first + s * RPP;
+            *(v4f*)(lds + r * LDS_STRIDE + 4 * (chunk ^ kin_swizzle<KT>(r))) = reg[s];
+        }
     }
     __device__ __forceinline__ static const float* tile_base(const float* X, int row0, int k, int ld) {
         return X + (size_t)row0 * ld + k;
