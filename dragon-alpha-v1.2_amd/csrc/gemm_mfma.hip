@@ -339,6 +339,9 @@ void gemm_f32_mfma(const GemmParams p) {
                 lb.load(rb, nxt.b_ptr, nxt.kb_lim - nxt.k0);
                 fetched = true;
             }
+            // the prefetch must be in flight before the matrix work starts: keep the scheduler
+            // from sinking the loads down to their first use
+            __builtin_amdgcn_sched_barrier(0);
             const float* as = As[buf];
             const float* bs = Bs[buf];
 #pragma unroll
