@@ -30,6 +30,9 @@ for _p in (ROOT, os.path.join(ROOT, "dragon-alpha-v1.2_amd")):
 
 PEAK_TFLOPS = 157.3      # FP32 MFMA, dense
 HBM_PEAK_GBS = 8000.0
+# HBM-side bytes per 4096^3 launch read off the hardware counters (FETCH_SIZE scaled x2.000 by a
+# known copy, plus WRITE_SIZE); source: profiles/gemm_f32_mfma_4096cubed.md
+MEASURED_TRAFFIC_BYTES = {"A*B": 785.9 * 2 ** 20, "A*B^T": 811.3 * 2 ** 20, "A^T*B": 775.6 * 2 ** 20}
 
 
 def log(*a):
@@ -150,7 +153,10 @@ def main():
     achieved = flop / (kernel_ms[slowest] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "gemm_f32_mfma %s 4096^3" % slowest,
                 "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None}
+                "frac": round(achieved / PEAK_TFLOPS, 4),
+                "traffic": round(MEASURED_TRAFFIC_BYTES[slowest]),
+                "traffic_note": "bytes per launch at the L2-fabric boundary from rocprofv3 counters "
+                                "(includes Infinity-Cache hits); algorithmic = 201326592"}
 
     # ---------------- CPU baseline: the oracle on the same three products ---------------------
     cpu_baseline = None
