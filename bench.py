@@ -12,7 +12,8 @@ HBM before the timed region.  Prints ONE JSON line:
                HIP events on the launch stream
   cpu_baseline the CPU oracle (a port of the reference's CPU matmul loops) timed on this
                host's cores on the same three products
-  per_config   every BASELINE workload (split-K, batched, ragged) in TFLOP/s and % of peak
+  per_config   every BASELINE workload (split-K, batched, ragged) and the biased fully-connected
+               layer in TFLOP/s and % of peak
 
 usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--headline-only]
        python bench.py --calibrate-copy     (profiling aid, see --help)
@@ -82,8 +83,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5",
-                    help="which of the other BASELINE workloads to time (default 3,4,5)")
+    ap.add_argument("--configs", default="3,4,5,bias",
+                    help="which of the other workloads to time (default 3,4,5,bias): BASELINE configs "
+                         "3, 4, 5 and the biased fully-connected layer")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
                          "(the known-size copy that FETCH_SIZE / WRITE_SIZE are scaled by)")
@@ -298,6 +300,36 @@ def main():
             S, 1, da.address, db.address, dc.address, p4(Bt5), n5, p4(m5), k5, p4(k5)), iters=100)
         record("cfg5 batchMatMul batch33 257x129 by 129x385", 2.0 * Bt5 * n5 * m5 * k5, ms)
         for x in (da, db, dc):
+            x.free()
+
+    if "bias" in extra:
+        # fully-connected layer with bias, Y[8192,4096] = X[8192,4096] * W[4096,4096] + b: the bias row
+        # inside the product's launch against the reference's two launches, and the row kernel alone
+        log("biased fully-connected layer ...")
+        Nb, Mb, Kb = 8192, 4096, 4096
+        g = synthetic.stream_for(6)
+        dX = dh.DeviceArray(g.normal((Nb, Kb), 0.0, 1.0))
+        dW = dh.DeviceArray(g.normal((Kb, Mb), 0.0, 0.02))
+        db = dh.DeviceArray(g.normal((Mb,), 0.0, 1.0))
+        dY = dh.DeviceArray(size=Nb * Mb)
+        FN = dh.Cuda_function
+        flb = 2.0 * Nb * Mb * Kb
+
+        def two_launches():
+            MM.matMul(S, 1, dX.address, dW.address, dY.address, Nb, Mb, Kb)
+            FN.linear_dual2D_row(stream, dY.address, db.address, Mb, 1.0, 1.0, 0.0, dY.address, Nb * Mb,
+                                 Mb, Mb)
+        ms = timer.per_launch_ms(lambda: MM.matMul_biased(
+            S, 1, dX.address, dW.address, dY.address, db.address, Nb, Mb, Kb, Nb * Mb, Mb), iters=20)
+        record("fullconnect_biased 8192x4096x4096 bias in the product's launch", flb, ms)
+        ms = timer.per_launch_ms(two_launches, iters=20)
+        record("fullconnect_biased 8192x4096x4096 product + linear_dual2D_row", flb, ms)
+        ms = timer.per_launch_ms(lambda: FN.linear_dual2D_row(
+            stream, dY.address, db.address, Mb, 1.0, 1.0, 0.0, dY.address, Nb * Mb, Mb, Mb), iters=50)
+        per_config["linear_dual2D_row 8192x4096 (HBM-bound)"] = {
+            "ms": round(ms, 4), "alg_GBps": round(8.0 * Nb * Mb / (ms * 1e-3) / 1e9, 1),
+            "pct_hbm_peak": round(100 * 8.0 * Nb * Mb / (ms * 1e-3) / 8e12, 1)}
+        for x in (dX, dW, db, dY):
             x.free()
 
     Cuda.deleteStream(stream)

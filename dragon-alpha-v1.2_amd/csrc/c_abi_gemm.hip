@@ -39,7 +39,8 @@ int check_common(const int64_t* streams, int length, int64_t dA, int64_t dB, int
 
 // 2-D products, optionally cut into gz K slices.
 int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t dA, int64_t dB,
-              int64_t dC, int64_t dCbuf, int N, int M, int K) {
+              int64_t dC, int64_t dCbuf, int N, int M, int K, int64_t dBias = 0, int bias_rows = 0,
+              int bias_width = 0) {
     int e = check_common(streams, length, dA, dB, dC);
     if (e) return e;
     if (N <= 0 || M <= 0 || K <= 0 || gz < 1) return hipErrorInvalidValue;
@@ -70,6 +71,9 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
             p.ldb = K; p.b_outer = M; p.b_inner = K;
             break;
     }
+    p.bias = (const float*)(intptr_t)dBias;
+    p.bias_rows = dBias ? bias_rows : 0;
+    p.bias_width = dBias ? bias_width : 0;
     p.nz = gz;
     if (gz > 1) {
         // K_slice = (K / GZ) >> 3 << 3   (reference: MM/micro.cuh:92)
@@ -122,6 +126,29 @@ int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC, 
     if (part == 0) return hipSuccess;
     return skbuf_summary_launch((hipStream_t)(intptr_t)stream, (const float*)(intptr_t)dCbuf,
                                 (float*)(intptr_t)dC, part, sizeC);
+}
+
+int dragon_Cuda_matMul_matMul_biased(const int64_t* streams, int32_t length, int64_t dA, int64_t dB,
+                                     int64_t dC, int64_t dBias, int32_t N, int32_t M, int32_t K,
+                                     int32_t lengthv, int32_t width) {
+    if (dBias == 0 || !aligned16(dBias) || width <= 0 || width > M || lengthv <= 0 || M <= 0 ||
+        lengthv % M != 0 || lengthv / M > N)
+        return hipErrorInvalidValue;
+    return matmul_2d(GEMM_NN, streams, length, 1, dA, dB, dC, 0, N, M, K, dBias, lengthv / M, width);
+}
+
+int dragon_Cuda_function_linear_dual2D_row(int64_t stream, int64_t dX1, int64_t dX2,
+                                           int32_t row_lengthv, float alpha, float beta, float gamma,
+                                           int64_t dY, int32_t lengthv, int32_t width, int32_t stride) {
+    if (dX1 == 0 || dX2 == 0 || dY == 0 || !aligned16(dX1) || !aligned16(dX2) || !aligned16(dY))
+        return hipErrorInvalidValue;
+    if (lengthv <= 0 || row_lengthv <= 0 || stride <= 0 || width <= 0 || width > stride ||
+        !x4(lengthv) || !x4(row_lengthv) || !x4(stride) || lengthv % stride != 0 ||
+        lengthv % row_lengthv != 0 || row_lengthv % stride != 0)
+        return hipErrorInvalidValue;
+    return linear_dual2D_row_launch((hipStream_t)(intptr_t)stream, (const float*)(intptr_t)dX1,
+                                    (const float*)(intptr_t)dX2, row_lengthv, alpha, beta, gamma,
+                                    (float*)(intptr_t)dY, lengthv, width, stride);
 }
 
 // ---- batched ---------------------------------------------------------------------

@@ -46,12 +46,22 @@ struct GemmParams {
     int split;              // non-zero selects split-K
     int k_slice;            // slice z covers [z*k_slice, (z+1)*k_slice), the last runs to k_total
     long long sizeC;        // floats per split-K partial
+    const float* bias;      // optional row vector added to C[i][j] for i < bias_rows, j < bias_width
+    int bias_rows, bias_width;
     int tiles_m, tiles_n;   // filled by the launcher
 };
 
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu);
 void gemm_force_tile(int tile);
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
+// the GEMM_NN product with p.bias added in the epilogue (what gemm_launch forwards to when p.bias is set)
+hipError_t gemm_launch_nn_biased(const GemmParams& p, int tile, hipStream_t stream);
+
+// Y[i] = alpha*X1[i] + beta*X2[i % row_lengthv] + gamma over lengthv floats laid out in rows of
+// `stride`, elements at or beyond `width` in a row written as zero.
+hipError_t linear_dual2D_row_launch(hipStream_t stream, const float* X1, const float* X2, int row_lengthv,
+                                    float alpha, float beta, float gamma, float* Y, int lengthv,
+                                    int width, int stride);
 
 // C[i] += sum_p Cbuf[p*sizeC + i], Kahan-compensated, p ascending.
 hipError_t skbuf_summary_launch(hipStream_t stream, const float* Cbuf, float* C, int part, int sizeC);

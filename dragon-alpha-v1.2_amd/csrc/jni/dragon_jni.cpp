@@ -74,6 +74,7 @@ std::vector<int64_t> long_array(JNIEnv* env, jlongArray arr, jint length) {
 #define MM(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1matMul_##name
 #define BMM(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1batchMatMul_##name
 #define RT(name) Java_z_dragon_engine_cuda_impl_Cuda_##name
+#define FN(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1function_##name
 
 extern "C" {
 
@@ -113,6 +114,27 @@ DEF_MM2D(matMulT2_1mma, dragon_Cuda_matMul_matMulT2_mma)
 DEF_MMSK(matMulSK, dragon_Cuda_matMul_matMulSK)
 DEF_MMSK(matMulT1SK, dragon_Cuda_matMul_matMulT1SK)
 DEF_MMSK(matMulT2SK, dragon_Cuda_matMul_matMulT2SK)
+
+// One launch for matMul + bias row.  The reference has no such native: a maintainer who wants it
+// declares `public static native void matMul_biased(long[] streamArray, int length, long dA_address,
+// long dB_address, long dC_address, long dBias_address, int N, int M, int K, int lengthv, int width)`
+// in Cuda_matMul.java and calls it from the unsplit branch of CudaFloat32EngineBase.matMul_biased.
+JNIEXPORT void JNICALL MM(matMul_1biased)(JNIEnv* env, jclass, jlongArray streamArray, jint length,
+                                          jlong dA, jlong dB, jlong dC, jlong dBias, jint N, jint M,
+                                          jint K, jint lengthv, jint width) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_matMul_matMul_biased(st.s, st.n, dA, dB, dC, dBias, N, M, K, lengthv, width));
+}
+
+// ---- Cuda_function: the bias row (reference: Cuda_function/Cuda_function/A.cu:287-303) ---------
+JNIEXPORT void JNICALL FN(linear_1dual2D_1row)(JNIEnv* env, jclass, jlong stream, jlong dX1, jlong dX2,
+                                               jint row_lengthv, jfloat alpha, jfloat beta,
+                                               jfloat gamma, jlong dY, jint lengthv, jint width,
+                                               jint stride) {
+    handle(env, dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta, gamma,
+                                                       dY, lengthv, width, stride));
+}
 
 // ---- Cuda_batchMatMul -------------------------------------------------------------------------
 #define DEF_BMM(jname, cname)                                                                    \

@@ -5,6 +5,7 @@ Thin, one-to-one wrappers over the C ABI (no compute happens in Python):
   Cuda             -- runtime natives of the reference's z.dragon.engine.cuda.impl.Cuda
   Cuda_matMul      -- natives + heuristics of ...impl.math.Cuda_matMul
   Cuda_batchMatMul -- natives + heuristics of ...impl.math.Cuda_batchMatMul
+  Cuda_function    -- linear_dual2D_row of ...impl.math.Cuda_function (the bias row)
   CudaException    -- the error type the reference's natives throw
 
 Method names and argument order follow the Java declarations
@@ -235,6 +236,13 @@ class Cuda_matMul:
         _check(lib.dragon_Cuda_matMul_matMulT2SK(arr, length, GZ, dA, dB, dC, dCbuf, N, M, K))
 
     @staticmethod
+    def matMul_biased(streams, length, dA, dB, dC, dBias, N, M, K, lengthv, width):
+        """One launch for matMul followed by the bias row; no native of this name in the reference."""
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMul_biased(arr, length, dA, dB, dC, dBias, N, M, K,
+                                                    lengthv, width))
+
+    @staticmethod
     def matMul_mma(streams, length, dA, dB, dC, N, M, K):
         arr, _ = _stream_array(streams)
         _check(lib.dragon_Cuda_matMul_matMul_mma(arr, length, dA, dB, dC, N, M, K))
@@ -248,6 +256,16 @@ class Cuda_matMul:
     def matMulT2_mma(streams, length, dA, dB, dC, N, M, K):
         arr, _ = _stream_array(streams)
         _check(lib.dragon_Cuda_matMul_matMulT2_mma(arr, length, dA, dB, dC, N, M, K))
+
+
+class Cuda_function:
+    """The one native of Cuda_function.java the biased products use."""
+
+    @staticmethod
+    def linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta, gamma, dY, lengthv, width,
+                          stride):
+        _check(lib.dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta,
+                                                          gamma, dY, lengthv, width, stride))
 
 
 class Cuda_batchMatMul:

@@ -30,6 +30,8 @@ SIGNATURES = {
     "dragon_Cuda_matMul_matMulT1SK": (i32, _MMSK),
     "dragon_Cuda_matMul_matMulT2SK": (i32, _MMSK),
     "dragon_Cuda_matMul_SKbuf_summary": (i32, [i64, i64, i64, i32, i32]),
+    "dragon_Cuda_function_linear_dual2D_row": (i32, [i64, i64, i64, i32, f32, f32, f32, i64, i32, i32, i32]),
+    "dragon_Cuda_matMul_matMul_biased": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_batchMatMul_batchMatMul": (i32, _BMM),
     "dragon_Cuda_batchMatMul_batchMatMul_texture": (i32, _BMM),
     "dragon_Cuda_batchMatMul_batchMatMulT1": (i32, _BMM),
@@ -120,6 +122,9 @@ SIGNATURES = {
     "dragon_tensor_address": (i64, [c_void_p]),
     "dragon_engine_product": (c_void_p, [c_void_p, i32, i32, c_void_p, c_void_p]),
     "dragon_engine_product_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
+    "dragon_engine_fullconnect": (c_void_p, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
+    "dragon_engine_fullconnect_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "dragon_engine_linear2_row": (c_void_p, [c_void_p, i32, c_void_p, c_void_p, f32, f32, f32]),
 }
 
 

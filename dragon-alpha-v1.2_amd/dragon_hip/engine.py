@@ -168,6 +168,44 @@ class Engine:
     def batchMatMulT2(self, *t, likeA=True):
         return self._product(BMM_T2, t, likeA)
 
+    # ---- fully connected layer and bias row ----
+    def _fullconnect(self, op, t, n_in):
+        """t = inputs, or (output, inputs...) when one more tensor than n_in is given."""
+        hs = [a._h if a is not None else None for a in t]
+        if len(t) == n_in:
+            hs += [None] * (3 - n_in)
+            return self._wrap(lib.dragon_engine_fullconnect(self._h, op, hs[0], hs[1], hs[2]))
+        hs += [None] * (4 - len(hs))
+        rc = lib.dragon_engine_fullconnect_into(self._h, op, hs[0], hs[1], hs[2], hs[3])
+        if rc:
+            _raise(rc)
+        return t[0]
+
+    def fullconnect(self, *t):
+        return self._fullconnect(0, t, 2)
+
+    def fullconnect_biased(self, *t):
+        return self._fullconnect(1, t, 3)
+
+    def fullconnect_deltaX(self, deltaY, W):
+        return self._fullconnect(2, (deltaY, W), 2)
+
+    def fullconnect_deltaW(self, X, deltaY):
+        return self._fullconnect(3, (X, deltaY), 2)
+
+    def matMul_biased(self, *t):
+        return self._fullconnect(4, t, 3)
+
+    def linear2_row(self, inplace, X1, X2, alpha, beta, gamma):
+        h = lib.dragon_engine_linear2_row(self._h, int(inplace), X1._h if X1 else None,
+                                          X2._h if X2 else None, alpha, beta, gamma)
+        if inplace and h:
+            return X1
+        return self._wrap(h)
+
+    def add_row(self, inplace, X1, X2):
+        return self.linear2_row(inplace, X1, X2, 1.0, 1.0, 0.0)
+
 
 def cuda_float32(device_id=0, stream_pool_size=32):
     return Engine(device_id, stream_pool_size)

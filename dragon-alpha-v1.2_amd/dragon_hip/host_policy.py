@@ -1,9 +1,9 @@
 """The split-K decision of the host engine as a pure function of the compute-unit count
-(reference: CudaFloat32EngineBase.java:1519-1562, 1736-1779, 1855-1896), computed by the
+(reference: CudaFloat32EngineBase.java:1519-1562, 1604-1613, 1736-1779, 1855-1896), computed by the
 library's C++ engine mirror.  Needs no device."""
 from . import lib
 
-MATMUL, MATMUL_T1, MATMUL_T2 = 0, 1, 2
+MATMUL, MATMUL_T1, MATMUL_T2, MATMUL_BIASED = 0, 1, 2, 3
 
 
 def gridZ(kind, N, M, K, SM):

@@ -245,6 +245,21 @@ int policy_matMul_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k) {   /
     return policy_clamp(fGridZ, K, b0, SM, k.maxBlock_perSM, k.maxPart);
 }
 
+// :1604-1613 -- the same test as matMul without the 0.4 factor on K/(K+1024)
+int policy_matMul_biased_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k) {
+    float fGridZ = 1; int b0 = 1;
+    if (K >= k.threshold) {
+        b0 = dragon_Cuda_matMul_blockNum(N, M);
+        float expect_block_perSM = k.minBlock_perSM + (float)K / ((float)K + 1024.0f);
+        if ((float)b0 < (float)SM * expect_block_perSM) {
+            int b1 = dragon_Cuda_matMul_blockNum(K, M);
+            int b2 = dragon_Cuda_matMul_blockNum(N, K);
+            fGridZ = (float)(b1 + b2) / ((float)b0 * 2.0f);
+        }
+    }
+    return policy_clamp(fGridZ, K, b0, SM, k.maxBlock_perSM, k.maxPart);
+}
+
 int policy_matMulT1_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k) {  // :1740-1749
     float fGridZ = 1; int b1 = 1;
     if (K >= k.threshold) {
@@ -278,6 +293,10 @@ int policy_matMulT2_gridZ(int N, int M, int K, int SM, const SplitKKnobs& t2, co
 int CudaFloat32EngineBase::matMul_gridZ(int N, int M, int K) const {
     SplitKKnobs k = {matMul_sk_threshold, matMul_sk_maxPart, matMul_sk_minBlock_perSM, matMul_sk_maxBlock_perSM};
     return policy_matMul_gridZ(N, M, K, dev_.multiProcessorCount(), k);
+}
+int CudaFloat32EngineBase::matMul_biased_gridZ(int N, int M, int K) const {
+    SplitKKnobs k = {matMul_sk_threshold, matMul_sk_maxPart, matMul_sk_minBlock_perSM, matMul_sk_maxBlock_perSM};
+    return policy_matMul_biased_gridZ(N, M, K, dev_.multiProcessorCount(), k);
 }
 int CudaFloat32EngineBase::matMulT1_gridZ(int N, int M, int K) const {
     SplitKKnobs k = {matMulT1_sk_threshold, matMulT1_sk_maxPart, matMulT1_sk_minBlock_perSM, matMulT1_sk_maxBlock_perSM};
@@ -325,9 +344,10 @@ void CudaFloat32EngineBase::set2D(int64_t address, const float* value, int heigh
     streamPool_->returnStream(stream);
 }
 
-// Shared body of matMul / matMulT1 / matMulT2 (:1534-1589, :1751-1806, :1870-1925)
+// Shared body of matMul / matMulT1 / matMulT2 (:1534-1589, :1751-1806, :1870-1925) and, with a
+// Bias address, of matMul_biased (:1615-1686): the bias row is the last thing issued on streams[0].
 SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64_t A, int64_t B,
-                                        int N, int M, int K) {
+                                        int N, int M, int K, int64_t Bias, int lengthv, int width) {
     const int length = dragon_Cuda_matMul_nstream(N, M);
     std::vector<int64_t> streamArray = streamPool_->getStreamArray(length);
     const int n = (int)streamArray.size();
@@ -336,6 +356,25 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
     const bool big = (N > 127) && (M > 127) && (K % 8 == 0);
     if (GridZ < 2) {   // no need to split
         int rc;
+        if (Bias != 0) {
+            const bool mma = matMul_tf32 && big;
+            if (matMul_biased_fused && !mma) {
+                cu(dragon_Cuda_matMul_matMul_biased(streamArray.data(), n, A, B, C, Bias, N, M, K,
+                                                    lengthv, width));
+            } else {
+                cu(mma ? dragon_Cuda_matMul_matMul_mma(streamArray.data(), n, A, B, C, N, M, K)
+                       : dragon_Cuda_matMul_matMul(streamArray.data(), n, A, B, C, N, M, K));
+                int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+                cu(dragon_Cuda_eventRecord_streams(event, streamArray.data(), n));
+                cu(dragon_Cuda_streamWaitEvent_default(streamArray[0], event));
+                cu(dragon_Cuda_function_linear_dual2D_row(streamArray[0], C, Bias, M, 1.0f, 1.0f, 0.0f,
+                                                          C, lengthv, width, M));
+                cu(dragon_Cuda_deleteEvent(event));
+            }
+            // the reference's BiasedForwardSyncer (:924-956) waits on streams[0] alone, where the
+            // bias row ran; the stream-array syncer joins the idle streams first, same result
+            return SyncerPtr(new StreamArraySyncer(streamPool_.get(), streamArray));
+        }
         if (variant == 0)
             rc = (matMul_tf32 && big)
                      ? dragon_Cuda_matMul_matMul_mma(streamArray.data(), n, A, B, C, N, M, K)
@@ -374,6 +413,10 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
         cu(dragon_Cuda_streamWaitEvent_default(stream, event));
         cu(dragon_Cuda_matMul_SKbuf_summary(stream, Cbuf, C, part, sizeC));
         cu(dragon_Cuda_deleteEvent(event));
+        // stage 3 of matMul_biased: the bias row, after the reduction
+        if (Bias != 0)
+            cu(dragon_Cuda_function_linear_dual2D_row(stream, C, Bias, M, 1.0f, 1.0f, 0.0f, C, lengthv,
+                                                      width, M));
     } catch (...) {
         core_->free(block.size, block.address);
         throw;
@@ -383,6 +426,19 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
 
 SyncerPtr CudaFloat32EngineBase::matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K) {
     return run_2d(0, matMul_gridZ(N, M, K), C, A, B, N, M, K);
+}
+SyncerPtr CudaFloat32EngineBase::matMul_biased(int64_t C, int64_t A, int64_t B, int N, int M, int K,
+                                               int64_t Bias, int lengthv, int width) {   // :1594-1688
+    if (Bias == 0) throw NullPointerException("Tensor Bias is null");
+    return run_2d(0, matMul_biased_gridZ(N, M, K), C, A, B, N, M, K, Bias, lengthv, width);
+}
+SyncerPtr CudaFloat32EngineBase::linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv,
+                                                float alpha, float beta, float gamma, int lengthv,
+                                                int width, int stride) {   // :4517-4530
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_function_linear_dual2D_row(stream, X1, X2, row_lengthv, alpha, beta, gamma, Y,
+                                              lengthv, width, stride));
+    return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
 }
 SyncerPtr CudaFloat32EngineBase::matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K) {
     return run_2d(1, matMulT1_gridZ(N, M, K), C, A, B, N, M, K);
@@ -501,6 +557,37 @@ void EngineCore::matMul_check(int64_t C, int64_t A, int64_t B, int N, int M, int
     if (K <= 0) throw IllegalArgumentException(fmt("K { got %lld } must > 0", K));
 }
 
+void EngineCore::func_param_check_row(int lengthv, int row_lengthv, int width, int stride) const {  // :1613-1622
+    auto s = [](int v) { return std::to_string(v); };
+    if (lengthv < row_lengthv)
+        throw IllegalArgumentException("lengthv { got " + s(lengthv) + " } < row_lengthv { " + s(row_lengthv) + " }");
+    if (width <= 0) throw IllegalArgumentException("width { got " + s(width) + " } <= 0");
+    if (lengthv % row_lengthv != 0)
+        throw IllegalArgumentException("lengthv { got " + s(lengthv) + " } % row_lengthv { " + s(row_lengthv) + " } != 0");
+    if (row_lengthv % stride != 0)
+        throw IllegalArgumentException("row_lengthv { " + s(row_lengthv) + " } % stride { " + s(stride) + " } != 0");
+}
+SyncerPtr EngineCore::matMul_biased(int64_t C, int64_t A, int64_t B, int N, int M, int K, int64_t Bias,
+                                    int lengthv) {   // :719-740
+    const int M_4x = pad4(M);
+    if (check) {
+        matMul_check(C, A, B, N, M, K);
+        if (Bias == 0) throw NullPointerException("Tensor Bias is null");
+        func_param_check_row(lengthv, M_4x, M, M_4x);
+    }
+    return base_->matMul_biased(C, A, B, pad4(N), M_4x, pad4(K), Bias, lengthv, M);
+}
+SyncerPtr EngineCore::linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
+                                     float beta, float gamma, int lengthv, int width) {   // :1965-1983
+    const int stride = pad4(width);
+    if (check) {
+        if (Y == 0) throw NullPointerException("Tensor Y is null");
+        if (X1 == 0) throw NullPointerException("Tensor X1 is null");
+        if (X2 == 0) throw NullPointerException("Tensor X2 is null");
+        func_param_check_row(lengthv, row_lengthv, width, stride);
+    }
+    return base_->linear2_2D_row(Y, X1, X2, row_lengthv, alpha, beta, gamma, lengthv, width, stride);
+}
 SyncerPtr EngineCore::matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K) {    // :708-717
     if (check) matMul_check(C, A, B, N, M, K);
     return base_->matMul(C, A, B, pad4(N), pad4(M), pad4(K));
@@ -684,6 +771,35 @@ Tensor* Engine::matMul(Tensor* C, Tensor* A, Tensor* B) {
     finish(C, core_->matMul(C->address, A->address, B->address, A->dim[0], B->dim[1], A->dimAt(1)));
     return C;
 }
+// C = A * B + Bias (Engine.java:998-1039)
+Tensor* Engine::matMul_biased(Tensor* A, Tensor* B, Tensor* Bias) {
+    require(A, "A"); require(B, "B"); require(Bias, "Bias");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2");
+        equals(A->dimAt(1), "A.width", B->dimAt(0), "B.height");
+        equals(Bias->lastDim(), "Bias.lastDim", B->dimAt(1), "B.width");
+    }
+    const int AH = A->dim[0], AW = A->dimAt(1), BW = B->dim[1];
+    Tensor* C = &empty({AH, BW})->c();
+    try {
+        finish(C, core_->matMul_biased(C->address, A->address, B->address, AH, BW, AW, Bias->address,
+                                       C->lengthv));
+    } catch (...) { deleteTensor(C); throw; }
+    return C;
+}
+Tensor* Engine::matMul_biased(Tensor* C, Tensor* A, Tensor* B, Tensor* Bias) {
+    require(C, "C"); require(A, "A"); require(B, "B"); require(Bias, "Bias");
+    if (check_) {
+        equals(A->ndim(), "A.ndim", 2, "2"); equals(B->ndim(), "B.ndim", 2, "2"); equals(C->ndim(), "C.ndim", 2, "2");
+        equals(C->dimAt(0), "C.height", A->dimAt(0), "A.height");
+        equals(C->dimAt(1), "C.width", B->dimAt(1), "B.width");
+        equals(A->dimAt(1), "A.width", B->dimAt(0), "B.height");
+        equals(Bias->lastDim(), "Bias.lastDim", B->dimAt(1), "B.width");
+    }
+    finish(C, core_->matMul_biased(C->address, A->address, B->address, A->dim[0], B->dim[1], A->dimAt(1),
+                                   Bias->address, C->lengthv));
+    return C;
+}
 Tensor* Engine::matMulT1(Tensor* A, Tensor* B) {
     require(A, "A"); require(B, "B");
     if (check_) {
@@ -830,6 +946,119 @@ Tensor* Engine::batchMatMulT2(Tensor* C, Tensor* A, Tensor* B) {
     finish(C, core_->batchMatMulT2(C->address, A->address, B->address, batch_of(A), A->dimAt(-2),
                                    B->dimAt(-2), A->dimAt(-1)));
     return C;
+}
+
+// ---- fully connected layer: the 2-D products over a tensor of any rank, rows = length / lastDim
+// (Engine.java:1315-1470).  Only the last dimension carries a padded stride, so the leading
+// dimensions fold into one row count without moving data.
+static std::vector<int> with_last(const Tensor* X, int last) {
+    std::vector<int> d = X->dim;
+    d.back() = last;
+    return d;
+}
+Tensor* Engine::fullconnect(Tensor* X, Tensor* W) {
+    require(X, "X"); require(W, "W");
+    if (X->ndim() == 2) return matMul(X, W);
+    if (check_) {
+        must_greater_equal(X->ndim(), "X.ndim", 3);
+        equals(W->ndim(), "W.ndim", 2, "2");
+        equals(X->dimAt(-1), "X.features", W->dimAt(0), "W.in_features");
+    }
+    const int WOW = W->dim[1], XIW = X->dimAt(-1), GN = X->length / XIW;
+    Tensor* Y = &empty(with_last(X, WOW))->c();
+    try { finish(Y, core_->matMul(Y->address, X->address, W->address, GN, WOW, XIW)); }
+    catch (...) { deleteTensor(Y); throw; }
+    return Y;
+}
+Tensor* Engine::fullconnect(Tensor* Y, Tensor* X, Tensor* W) {
+    require(Y, "Y"); require(X, "X"); require(W, "W");
+    if (X->ndim() == 2 && Y->ndim() == 2) return matMul(Y, X, W);
+    if (check_) {
+        must_greater_equal(Y->ndim(), "Y.ndim", 2); must_greater_equal(X->ndim(), "X.ndim", 2);
+        equals(W->ndim(), "W.ndim", 2, "2");
+        equals(X->dimAt(-1), "X.features", W->dimAt(0), "W.in_features");
+        equals(Y->dimAt(-1), "Y.features", W->dimAt(1), "W.out_features");
+        equals(X->length / X->dimAt(-1), "(X.batch * X.height)", Y->length / Y->dimAt(-1), "(Y.batch * Y.height)");
+    }
+    const int WOW = W->dim[1], XIW = X->dimAt(-1), GN = X->length / XIW;
+    finish(Y, core_->matMul(Y->address, X->address, W->address, GN, WOW, XIW));
+    return Y;
+}
+Tensor* Engine::fullconnect_biased(Tensor* X, Tensor* W, Tensor* Bias) {
+    require(X, "X"); require(W, "W"); require(Bias, "Bias");
+    if (X->ndim() == 2) return matMul_biased(X, W, Bias);
+    if (check_) {
+        must_greater_equal(X->ndim(), "X.ndim", 3);
+        equals(W->ndim(), "W.ndim", 2, "2");
+        equals(X->dimAt(-1), "X.features", W->dimAt(0), "W.in_features");
+        equals(Bias->length, "Bias.length", W->dimAt(1), "W.out_features");
+    }
+    const int WOW = W->dim[1], XIW = X->dimAt(-1), GN = X->length / XIW;
+    Tensor* Y = &empty(with_last(X, WOW))->c();
+    try {
+        finish(Y, core_->matMul_biased(Y->address, X->address, W->address, GN, WOW, XIW, Bias->address,
+                                       Y->lengthv));
+    } catch (...) { deleteTensor(Y); throw; }
+    return Y;
+}
+Tensor* Engine::fullconnect_biased(Tensor* Y, Tensor* X, Tensor* W, Tensor* Bias) {
+    require(Y, "Y"); require(X, "X"); require(W, "W"); require(Bias, "Bias");
+    if (X->ndim() == 2 && Y->ndim() == 2) return matMul_biased(Y, X, W, Bias);
+    if (check_) {
+        must_greater_equal(Y->ndim(), "Y.ndim", 2); must_greater_equal(X->ndim(), "X.ndim", 2);
+        equals(W->ndim(), "W.ndim", 2, "2");
+        equals(X->dimAt(-1), "X.features", W->dimAt(0), "W.in_features");
+        equals(Y->dimAt(-1), "Y.features", W->dimAt(1), "W.out_features");
+        equals(X->length / X->dimAt(-1), "(X.batch * X.height)", Y->length / Y->dimAt(-1), "(Y.batch * Y.height)");
+        equals(Bias->length, "Bias.length", W->dimAt(1), "W.out_features");
+    }
+    const int WOW = W->dim[1], XIW = X->dimAt(-1), GN = X->length / XIW;
+    finish(Y, core_->matMul_biased(Y->address, X->address, W->address, GN, WOW, XIW, Bias->address,
+                                   Y->lengthv));
+    return Y;
+}
+Tensor* Engine::fullconnect_deltaX(Tensor* deltaY, Tensor* W) {   // deltaX = deltaY * W^T
+    require(deltaY, "deltaY"); require(W, "W");
+    if (deltaY->ndim() == 2) return matMulT2(deltaY, W);
+    if (check_) {
+        must_greater_equal(deltaY->ndim(), "deltaY.ndim", 3);
+        equals(W->ndim(), "W.ndim", 2, "2");
+        equals(deltaY->dimAt(-1), "deltaY.features", W->dimAt(1), "W.out_features");
+    }
+    const int WIW = W->dim[0], YOW = deltaY->dimAt(-1), GN = deltaY->length / YOW;
+    Tensor* deltaX = &empty(with_last(deltaY, WIW))->c();
+    try { finish(deltaX, core_->matMulT2(deltaX->address, deltaY->address, W->address, GN, WIW, YOW)); }
+    catch (...) { deleteTensor(deltaX); throw; }
+    return deltaX;
+}
+Tensor* Engine::fullconnect_deltaW(Tensor* X, Tensor* deltaY) {   // deltaW = X^T * deltaY
+    require(X, "X"); require(deltaY, "deltaY");
+    if (deltaY->ndim() == 2 && X->ndim() == 2) return matMulT1(X, deltaY);
+    if (check_) {
+        must_greater_equal(X->ndim(), "X.ndim", 3); must_greater_equal(deltaY->ndim(), "deltaY.ndim", 3);
+        equals(X->length / X->dimAt(-1), "(X.batch * X.height)", deltaY->length / deltaY->dimAt(-1),
+               "(deltaY.batch * Y.height)");
+    }
+    const int XIW = X->dimAt(-1), YOW = deltaY->dimAt(-1), GK = deltaY->length / YOW;
+    Tensor* deltaW = &empty({XIW, YOW})->c();
+    try { finish(deltaW, core_->matMulT1(deltaW->address, X->address, deltaY->address, XIW, YOW, GK)); }
+    catch (...) { deleteTensor(deltaW); throw; }
+    return deltaW;
+}
+
+// Engine.java:4185-4207, check_row :3781-3788
+Tensor* Engine::linear2_row(bool inplace, Tensor* X1, Tensor* X2, float alpha, float beta, float gamma) {
+    require(X1, "X1"); require(X2, "X2");
+    if (check_) {
+        must_greater_equal(X1->ndim(), "X1.ndim", 2);
+        equals(X1->lastDim(), "X1.lastDim", X2->lastDim(), "X2.lastDim");
+    }
+    Tensor* Y = inplace ? X1 : &empty(X1->dim)->c();
+    try {
+        finish(Y, core_->linear2_2D_row(Y->address, X1->address, X2->address, X2->lengthv, alpha, beta,
+                                        gamma, X1->lengthv, X1->lastDim()));
+    } catch (...) { if (!inplace) deleteTensor(Y); throw; }
+    return Y;
 }
 
 }  // namespace dragon

@@ -7,10 +7,12 @@
 //   CudaDevice             z/dragon/engine/cuda/impl/CudaDevice.java (multiProcessorCount only)
 //   CudaStreamPool         z/dragon/engine/cuda/impl/CudaStreamp1.java:34-63 (round-robin, never blocks)
 //   Syncer and its kinds   z/dragon/engine/cuda/CudaFloat32EngineBase.java:649-694, 1008-1054
-//   CudaFloat32EngineBase  z/dragon/engine/cuda/CudaFloat32EngineBase.java:70-92, 1148-1260, 1471-2020
+//   CudaFloat32EngineBase  z/dragon/engine/cuda/CudaFloat32EngineBase.java:70-92, 1148-1260, 1471-2020,
+//                          4517-4530 (linear2_2D_row)
 //   EngineCore             z/dragon/engine/EngineCore.java:693-811 (checks and x4 padding)
 //   Tensor                 z/dragon/engine/Tensor.java:206-239 (length / lengthv / length_4x)
-//   Engine                 z/dragon/engine/Engine.java:522-551, 671-676, 824-837, 908-914, 955-1312
+//   Engine                 z/dragon/engine/Engine.java:522-551, 671-676, 824-837, 908-914, 955-1470,
+//                          4185-4207 (add_row / linear2_row)
 // (paths relative to source/alpha-Dragon-v1.2/src of the reference tree)
 #pragma once
 #include <stdint.h>
@@ -80,6 +82,7 @@ struct SplitKKnobs {
 };
 int policy_smooth_maxPart(int x);
 int policy_matMul_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
+int policy_matMul_biased_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
 int policy_matMulT1_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
 int policy_matMulT2_gridZ(int N, int M, int K, int SM, const SplitKKnobs& t2, const SplitKKnobs& mm);
 
@@ -101,6 +104,9 @@ public:
     bool matMul_tf32 = false, matMulT1_tf32 = false, matMulT2_tf32 = false;
     bool batchMatMul_tf32 = false, batchMatMulT1_tf32 = false, batchMatMulT2_tf32 = false;
     bool batchMatMul_useTexture = true, batchMatMulT2_useTexture = true;
+    // Not a field of the Java class: when set (the default) an unsplit matMul_biased adds the bias
+    // row inside the product's launch; when cleared it issues the reference's two launches.
+    bool matMul_biased_fused = true;
 
     void matMul_splitK_threshold(int threshold);     // must be a positive power of two
     void matMul_splitK_maxPart(int maxPart);         // must be >= 4
@@ -113,6 +119,7 @@ public:
 
     // the split-K decisions on their own (1 = no split), for inspection
     int matMul_gridZ(int N, int M, int K) const;
+    int matMul_biased_gridZ(int N, int M, int K) const;
     int matMulT1_gridZ(int N, int M, int K) const;
     int matMulT2_gridZ(int N, int M, int K) const;
 
@@ -127,8 +134,12 @@ public:
 
     // products; dims arrive already padded by EngineCore
     SyncerPtr matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr matMul_biased(int64_t C, int64_t A, int64_t B, int N, int M, int K, int64_t Bias,
+                            int lengthv, int width);
     SyncerPtr matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K);
     SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
+                             float beta, float gamma, int lengthv, int width, int stride);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int BK, int AK);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN, int AN, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int CM, int BM, int K);
@@ -137,7 +148,8 @@ public:
     int last_gridZ = 1, last_stream_count = 0;
 
 private:
-    SyncerPtr run_2d(int variant, int gridZ, int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr run_2d(int variant, int gridZ, int64_t C, int64_t A, int64_t B, int N, int M, int K,
+                     int64_t Bias = 0, int lengthv = 0, int width = 0);
     CudaDevice dev_;
     std::unique_ptr<CudaStreamPool> streamPool_;
     EngineCore* core_ = nullptr;
@@ -163,14 +175,19 @@ public:
     void set2D(int64_t address, const float* value, int length, int width);
 
     SyncerPtr matMul(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr matMul_biased(int64_t C, int64_t A, int64_t B, int N, int M, int K, int64_t Bias,
+                            int lengthv);
     SyncerPtr matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K);
     SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
+    SyncerPtr linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
+                             float beta, float gamma, int lengthv, int width);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
 
 private:
     void matMul_check(int64_t C, int64_t A, int64_t B, int N, int M, int K) const;
+    void func_param_check_row(int lengthv, int row_lengthv, int width, int stride) const;
     CudaFloat32EngineBase* base_;
     int64_t live_blocks_ = 0;
     std::mutex mu_;
@@ -213,6 +230,8 @@ public:
 
     Tensor* matMul(Tensor* A, Tensor* B);
     Tensor* matMul(Tensor* C, Tensor* A, Tensor* B);
+    Tensor* matMul_biased(Tensor* A, Tensor* B, Tensor* Bias);
+    Tensor* matMul_biased(Tensor* C, Tensor* A, Tensor* B, Tensor* Bias);
     Tensor* matMulT1(Tensor* A, Tensor* B);
     Tensor* matMulT1(Tensor* C, Tensor* A, Tensor* B);
     Tensor* matMulT2(Tensor* A, Tensor* B);
@@ -223,6 +242,18 @@ public:
     Tensor* batchMatMulT1(Tensor* C, Tensor* A, Tensor* B);
     Tensor* batchMatMulT2(bool likeA, Tensor* A, Tensor* B);
     Tensor* batchMatMulT2(Tensor* C, Tensor* A, Tensor* B);
+
+    // fully connected layer over the last dimension of a tensor of any rank >= 2
+    Tensor* fullconnect(Tensor* X, Tensor* W);
+    Tensor* fullconnect(Tensor* Y, Tensor* X, Tensor* W);
+    Tensor* fullconnect_biased(Tensor* X, Tensor* W, Tensor* Bias);
+    Tensor* fullconnect_biased(Tensor* Y, Tensor* X, Tensor* W, Tensor* Bias);
+    Tensor* fullconnect_deltaX(Tensor* deltaY, Tensor* W);
+    Tensor* fullconnect_deltaW(Tensor* X, Tensor* deltaY);
+
+    // Y = alpha*X1 + beta*X2 + gamma with the row vector X2 broadcast over the rows of X1
+    Tensor* add_row(bool inplace, Tensor* X1, Tensor* X2) { return linear2_row(inplace, X1, X2, 1.0f, 1.0f, 0.0f); }
+    Tensor* linear2_row(bool inplace, Tensor* X1, Tensor* X2, float alpha, float beta, float gamma);
 
 private:
     void finish(Tensor* C, SyncerPtr sc);

@@ -74,6 +74,7 @@ int dragon_engine_set_param(dragon_engine* eg, const char* name, int32_t v) {
         else if (n == "matMulT2_splitK_threshold") b.matMulT2_splitK_threshold(v);
         else if (n == "matMulT2_splitK_maxPart") b.matMulT2_splitK_maxPart(v);
         else if (n == "tf32") b.tf32(v != 0);
+        else if (n == "matMul_biased_fused") b.matMul_biased_fused = (v != 0);
         else if (n == "batchMatMul_useTexture") b.batchMatMul_useTexture = (v != 0);
         else if (n == "batchMatMulT2_useTexture") b.batchMatMulT2_useTexture = (v != 0);
         else if (n == "multiProcessorCount") {
@@ -95,6 +96,7 @@ int32_t dragon_engine_get_param(dragon_engine* eg, const char* name) {
         else if (n == "matMulT1_maxPart") out = b.matMulT1_sk_maxPart;
         else if (n == "matMulT2_splitK_threshold") out = b.matMulT2_sk_threshold;
         else if (n == "matMulT2_splitK_maxPart") out = b.matMulT2_sk_maxPart;
+        else if (n == "matMul_biased_fused") out = b.matMul_biased_fused ? 1 : 0;
         else if (n == "multiProcessorCount") out = b.device().multiProcessorCount();
         else if (n == "last_gridZ") out = b.last_gridZ;
         else if (n == "last_stream_count") out = b.last_stream_count;
@@ -111,7 +113,7 @@ int32_t dragon_engine_gridZ(dragon_engine* eg, int32_t kind, int32_t N, int32_t 
         if (!eg) throw NullPointerException("engine");
         CudaFloat32EngineBase& b = eg->eg.engineBase();
         out = kind == 0 ? b.matMul_gridZ(N, M, K) : kind == 1 ? b.matMulT1_gridZ(N, M, K)
-                                                             : b.matMulT2_gridZ(N, M, K);
+            : kind == 3 ? b.matMul_biased_gridZ(N, M, K) : b.matMulT2_gridZ(N, M, K);
     });
     return out;
 }
@@ -121,6 +123,7 @@ int32_t dragon_policy_gridZ(int32_t kind, int32_t N, int32_t M, int32_t K, int32
     mm.maxPart = t.maxPart = policy_smooth_maxPart(SM);
     if (kind == 0) return policy_matMul_gridZ(N, M, K, SM, mm);
     if (kind == 1) return policy_matMulT1_gridZ(N, M, K, SM, t);
+    if (kind == 3) return policy_matMul_biased_gridZ(N, M, K, SM, mm);
     return policy_matMulT2_gridZ(N, M, K, SM, t, mm);
 }
 
@@ -212,6 +215,47 @@ int dragon_engine_product_into(dragon_engine* eg, int32_t op, dragon_tensor* C, 
             default: throw IllegalArgumentException("unknown product");
         }
     });
+}
+
+dragon_tensor* dragon_engine_fullconnect(dragon_engine* eg, int32_t op, dragon_tensor* X,
+                                         dragon_tensor* W, dragon_tensor* Bias) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        Engine& e = eg->eg;
+        switch (op) {
+            case 0: t = e.fullconnect(T(X), T(W)); break;
+            case 1: t = e.fullconnect_biased(T(X), T(W), T(Bias)); break;
+            case 2: t = e.fullconnect_deltaX(T(X), T(W)); break;
+            case 3: t = e.fullconnect_deltaW(T(X), T(W)); break;
+            case 4: t = e.matMul_biased(T(X), T(W), T(Bias)); break;
+            default: throw IllegalArgumentException("unknown fullconnect operation");
+        }
+    });
+    return t ? wrap(t) : nullptr;
+}
+int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor* Y, dragon_tensor* X,
+                                   dragon_tensor* W, dragon_tensor* Bias) {
+    return guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        Engine& e = eg->eg;
+        switch (op) {
+            case 0: e.fullconnect(T(Y), T(X), T(W)); break;
+            case 1: e.fullconnect_biased(T(Y), T(X), T(W), T(Bias)); break;
+            case 4: e.matMul_biased(T(Y), T(X), T(W), T(Bias)); break;
+            default: throw IllegalArgumentException("unknown fullconnect operation");
+        }
+    });
+}
+dragon_tensor* dragon_engine_linear2_row(dragon_engine* eg, int32_t inplace, dragon_tensor* X1,
+                                         dragon_tensor* X2, float alpha, float beta, float gamma) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        t = eg->eg.linear2_row(inplace != 0, T(X1), T(X2), alpha, beta, gamma);
+    });
+    if (!t) return nullptr;
+    return inplace ? X1 : wrap(t);
 }
 
 }  // extern "C"

@@ -51,7 +51,8 @@ int dragon_engine_set_param(dragon_engine* eg, const char* name, int32_t value);
 int32_t dragon_engine_get_param(dragon_engine* eg, const char* name);   /* also "last_gridZ",
     "last_stream_count", "live_blocks", "stream_pool_size" */
 
-/* split-K decision for padded dims; kind 0 matMul, 1 matMulT1, 2 matMulT2; 1 = no split */
+/* split-K decision for padded dims; kind 0 matMul, 1 matMulT1, 2 matMulT2, 3 matMul_biased;
+ * 1 = no split */
 int32_t dragon_engine_gridZ(dragon_engine* eg, int32_t kind, int32_t N, int32_t M, int32_t K);
 /* the same decision as a pure function of the unit count, with the default knobs
  * (threshold 512, maxPart smooth(SM), minBlock 1.2 / 1.14, maxBlock 4.0); needs no device */
@@ -81,6 +82,24 @@ dragon_tensor* dragon_engine_product(dragon_engine* eg, int32_t op, int32_t like
                                      dragon_tensor* A, dragon_tensor* B);
 int dragon_engine_product_into(dragon_engine* eg, int32_t op, dragon_tensor* C,
                                dragon_tensor* A, dragon_tensor* B);
+
+/* fully connected layer over the last dimension (Engine.java:1315-1470) and the biased
+ * 2-D product (Engine.java:998-1039):
+ *   op 0 fullconnect(X, W)            Y = X * W                  Bias ignored
+ *   op 1 fullconnect_biased(X, W, B)  Y = X * W + B
+ *   op 2 fullconnect_deltaX(dY, W)    dX = dY * W^T              X is deltaY, Bias ignored
+ *   op 3 fullconnect_deltaW(X, dY)    dW = X^T * dY              W is deltaY, Bias ignored
+ *   op 4 matMul_biased(A, B, Bias)    C = A * B + Bias, 2-D only
+ * The into-form takes ops 0, 1 and 4. */
+dragon_tensor* dragon_engine_fullconnect(dragon_engine* eg, int32_t op, dragon_tensor* X,
+                                         dragon_tensor* W, dragon_tensor* Bias);
+int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor* Y,
+                                   dragon_tensor* X, dragon_tensor* W, dragon_tensor* Bias);
+
+/* linear2_row / add_row (Engine.java:4185-4207): Y = alpha*X1 + beta*X2 + gamma, the row vector
+ * X2 broadcast over the rows of X1.  inplace != 0 writes into X1 and returns X1 itself. */
+dragon_tensor* dragon_engine_linear2_row(dragon_engine* eg, int32_t inplace, dragon_tensor* X1,
+                                         dragon_tensor* X2, float alpha, float beta, float gamma);
 
 #ifdef __cplusplus
 }

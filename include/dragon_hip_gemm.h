@@ -84,6 +84,35 @@ int dragon_Cuda_matMul_matMulT2SK(const int64_t* streams, int32_t length, int32_
 int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC,
                                      int32_t part, int32_t sizeC);
 
+/* ---- bias row -------------------------------------------------------------------- */
+
+/* Y[i] = alpha*X1[i] + beta*X2[i % row_lengthv] + gamma for i < lengthv, then elements whose
+ * column (i % stride) is >= width are multiplied by zero.  X2 is a row vector of row_lengthv
+ * floats broadcast over the rows of X1; Y may alias X1.  lengthv, row_lengthv and stride are
+ * multiples of 4, row_lengthv a multiple of stride, lengthv a multiple of row_lengthv.
+ * Issued on `stream`.  With (alpha, beta, gamma) = (1, 1, 0) this is the bias addition of
+ * matMul_biased / fullconnect_biased
+ * (alpha-Dragon-v1.2/src/z/dragon/engine/cuda/CudaFloat32EngineBase.java:1626-1634, 1676-1680).
+ * Replaces Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear_1dual2D_1row
+ * (engine-cuda-base/Cuda_function/Cuda_function/A.cu:287-303, declared JM/Cuda_function.java:489,
+ * kernel .../type1_linear_dual2D_row.cuh:43-84). */
+int dragon_Cuda_function_linear_dual2D_row(int64_t stream, int64_t dX1, int64_t dX2,
+                                           int32_t row_lengthv, float alpha, float beta,
+                                           float gamma, int64_t dY, int32_t lengthv,
+                                           int32_t width, int32_t stride);
+
+/* C[N,M] = A[N,K] * B[K,M], then C[i][j] += Bias[j] for the first lengthv/M rows and j < width,
+ * in one launch: the bias row is added to the accumulators before they are stored.  Every bit
+ * of C equals what dragon_Cuda_matMul_matMul followed by
+ * dragon_Cuda_function_linear_dual2D_row(streams[0], C, Bias, M, 1, 1, 0, C, lengthv, width, M)
+ * leaves.  lengthv is a multiple of M with lengthv/M <= N (the unpadded row count), width <= M.
+ * No native counterpart in the reference, which issues the two launches above from Java
+ * (CudaFloat32EngineBase.java:1594-1638); a host that owns that method calls this instead. */
+int dragon_Cuda_matMul_matMul_biased(const int64_t* streams, int32_t length,
+                                     int64_t dA, int64_t dB, int64_t dC, int64_t dBias,
+                                     int32_t N, int32_t M, int32_t K,
+                                     int32_t lengthv, int32_t width);
+
 /* ---- batched products (grid depth = Batch) --------------------------------------- */
 
 /* C[b][N,M] = A[b][N,AK] * B[b][BK,M], k < BK.  M and AK are multiples of 4, N and BK

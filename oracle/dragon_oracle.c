@@ -396,6 +396,29 @@ int oracle_gridZ(int kind, int N, int M, int K, int SM,
 }
 
 /* ------------------------------------------------------------------------ */
+/* Bias row                                                                  */
+/* ------------------------------------------------------------------------ */
+
+/* Y[i] = alpha*X1[i] + beta*X2[i % row_lengthv] + gamma, then the element is multiplied by
+ * the 0/1 flag "column (i % stride) < width"
+ * (engine-cuda-base/Cuda_function/Cuda_function/type1_linear_dual2D_row.cuh:43-66,
+ * within_width: Cuda_function/micro.cuh:61-65).  Each product and sum is rounded to float
+ * on its own (this file is built with contraction off); the reference's compiler may fuse a
+ * product into a sum, which changes nothing for (alpha, beta, gamma) = (1, 1, 0), the bias
+ * addition of matMul_biased (CudaFloat32EngineBase.java:1626-1634).  Y may alias X1. */
+void oracle_linear_dual2D_row(const float* X1, const float* X2, int row_lengthv, float alpha,
+                              float beta, float gamma, float* Y, int lengthv, int width,
+                              int stride) {
+    for (int i = 0; i < lengthv; i++) {
+        float p1 = alpha * X1[i];
+        float p2 = beta * X2[i % row_lengthv];
+        float y = (p1 + p2) + gamma;
+        y *= ((i % stride) < width) ? 1.0f : 0.0f;
+        Y[i] = y;
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* Error metrics used by the parity tests                                    */
 /* ------------------------------------------------------------------------ */
 

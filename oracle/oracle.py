@@ -47,6 +47,7 @@ for _name, _res, _args in [
     ("oracle_streamSize", c_int, [c_int, c_int]),
     ("oracle_smooth_maxPart", c_int, [c_int]),
     ("oracle_gridZ", c_int, [c_int] * 6 + [c_float, c_float, c_int]),
+    ("oracle_linear_dual2D_row", None, [_P, _P, c_int, c_float, c_float, c_float, _P, c_int, c_int, c_int]),
     ("oracle_samePercent_relative", c_float, [_P, _P, c_int, c_float]),
     ("oracle_num_threads", c_int, []),
 ]:
@@ -180,6 +181,19 @@ def gridZ(kind, N, M, K, SM, threshold=512, minBlock=None, maxBlock=4.0, maxPart
     if maxPart is None:
         maxPart = smooth_maxPart(SM)
     return _o.oracle_gridZ(kind, N, M, K, SM, threshold, minBlock, maxBlock, maxPart)
+
+
+def linear_dual2D_row(X1, X2, alpha, beta, gamma, width):
+    """X1: device-layout matrix [rows, stride] (stride a multiple of 4), X2: row vector of
+    `stride` floats.  Returns alpha*X1 + beta*X2 + gamma with columns >= width times zero."""
+    X1, p1 = _f32(X1)
+    X2, p2 = _f32(np.ravel(X2))
+    rows, stride = X1.shape
+    assert stride % 4 == 0 and X2.size == stride and 0 < width <= stride
+    Y = np.empty_like(X1)
+    _o.oracle_linear_dual2D_row(p1, p2, stride, alpha, beta, gamma, Y.ctypes.data_as(_P),
+                                rows * stride, width, stride)
+    return Y
 
 
 def samePercent_relative(a, b, threshold=1e-3):

@@ -19,11 +19,16 @@ FILES = [
     "Cuda/Cuda/Cuda_Device.cuh",
     "Cuda/Cuda/Cuda_Exception.cuh",
     "Cuda/Cuda/Cuda_float.cuh",
+    "Cuda_function/Cuda_function/A.cu",
 ]
+# of the element-wise library only the bias row belongs to the path
+ONLY = {"Cuda_function/Cuda_function/A.cu": {"Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear_1dual2D_1row"}}
 out = []
 for f in FILES:
     text = open(os.path.join(CU, f), encoding="utf-8", errors="replace").read()
     for name in re.findall(r"\b(Java_z_dragon_engine_cuda_impl_\w+)\s*\(", text):
+        if f in ONLY and name not in ONLY[f]:
+            continue
         out.append("%s %s" % (f, name))
 dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "jni_symbols.txt")
 with open(dst, "w") as fh:

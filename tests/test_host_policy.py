@@ -14,6 +14,11 @@ def test_known_answers(dh):
     assert hp.gridZ(hp.MATMUL_T1, 256, 256, 131072, 256) == 128    # config 3 on 256 units
     assert hp.gridZ(hp.MATMUL_T1, 256, 256, 131072, 38) == 36      # the same on 38 units
     assert hp.gridZ(hp.MATMUL, 64, 64, 508, 256) == 1              # K below the threshold
+    # matMul_biased tests blockNum against 1.2 + K/(K+1024) units where matMul uses 1.2 + 0.4*K/(K+1024):
+    # 512 blocks of 2048x4096 at K = 16384 lie between 256*1.58 = 404 and 256*2.14 = 548, so only the
+    # biased product splits; fGridZ = (4096 + 2048)/(2*512) = 6, capped by 256*4*0.8/512 = 1 -> raised to 2
+    assert hp.gridZ(hp.MATMUL, 2048, 4096, 16384, 256) == 1
+    assert hp.gridZ(hp.MATMUL_BIASED, 2048, 4096, 16384, 256) == 2
 
 
 def test_policy_matches_oracle_over_a_grid(dh):
@@ -25,8 +30,8 @@ def test_policy_matches_oracle_over_a_grid(dh):
         for N in dims:
             for M in dims:
                 for K in ks:
-                    for kind in (0, 1, 2):
+                    for kind in (0, 1, 2, 3):
                         assert hp.gridZ(kind, N, M, K, SM) == oracle.gridZ(kind, N, M, K, SM), \
                             (kind, N, M, K, SM)
                         n += 1
-    assert n > 30000
+    assert n > 40000

@@ -11,13 +11,14 @@ GOLDEN = os.path.join(ROOT, "tests", "golden", "jni_symbols.txt")
 
 PREFIX = {"MM": "Java_z_dragon_engine_cuda_impl_math_Cuda_1matMul_",
           "BMM": "Java_z_dragon_engine_cuda_impl_math_Cuda_1batchMatMul_",
-          "RT": "Java_z_dragon_engine_cuda_impl_Cuda_"}
+          "RT": "Java_z_dragon_engine_cuda_impl_Cuda_",
+          "FN": "Java_z_dragon_engine_cuda_impl_math_Cuda_1function_"}
 
 
 def shim_names():
     text = open(SHIM).read()
     names = set()
-    for macro, arg in re.findall(r"JNICALL\s+(MM|BMM|RT)\((\w+)\)\s*\(", text):
+    for macro, arg in re.findall(r"JNICALL\s+(MM|BMM|RT|FN)\((\w+)\)\s*\(", text):
         names.add(PREFIX[macro] + arg)
     for kind, arg in re.findall(r"^DEF_(MM2D|MMSK|BMM|BMM_MMA)\((\w+),", text, flags=re.M):
         names.add(PREFIX["MM" if kind.startswith("MM") else "BMM"] + arg)
@@ -34,6 +35,13 @@ def test_every_matmul_native_of_the_reference_is_in_the_shim():
     gemm = {n for n, f in g.items() if "Cuda_matMul" in f or "Cuda_batchMatMul" in f}
     assert len(gemm) == 12           # 7 in Cuda_matMul/A.cu, 5 in Cuda_batchMatMul/A.cu
     assert gemm <= s, sorted(gemm - s)
+
+
+def test_bias_row_native_is_in_the_shim():
+    g, s = golden(), shim_names()
+    rows = {n for n, f in g.items() if "Cuda_function" in f}
+    assert rows == {PREFIX["FN"] + "linear_1dual2D_1row"}
+    assert rows <= s
 
 
 def test_runtime_subset_names_exist_in_the_reference():

@@ -290,6 +290,48 @@ def test_heuristics_known_answers():
     assert oracle.gridZ(oracle.MATMUL, 128, 128, 508, 256) == 1
 
 
+def test_biased_policy_known_answer():
+    # hand-derived (see the arithmetic in test_host_policy.test_known_answers)
+    assert oracle.blockNum(2048, 4096) == 512
+    assert oracle.gridZ(oracle.MATMUL, 2048, 4096, 16384, 256) == 1
+    assert oracle.gridZ(oracle.MATMUL_BIASED, 2048, 4096, 16384, 256) == 2
+    # where both split they agree: the clamp is shared
+    assert oracle.gridZ(oracle.MATMUL_BIASED, 1000, 780, 1532, 256) == 2
+
+
+def test_bias_row_is_an_exact_add_and_zeroes_the_pad():
+    rows, width = 37, 50
+    stride = 52
+    X1 = np.zeros((rows, stride), np.float32)
+    X1[:, :width] = RNG.uniform(-3, 3, (rows, width)).astype(np.float32)
+    X1[:, width:] = 7.0            # garbage in the pad must come out as zero
+    X2 = np.zeros(stride, np.float32)
+    X2[:width] = RNG.uniform(-1, 1, width).astype(np.float32)
+    Y = oracle.linear_dual2D_row(X1, X2, 1.0, 1.0, 0.0, width)
+    assert np.array_equal(Y[:, :width], X1[:, :width] + X2[None, :width])   # numpy adds in float32
+    assert np.all(Y[:, width:] == 0)
+    # integers: exact whatever the rounding order
+    Xi = RNG.integers(-100, 100, (8, 8)).astype(np.float32)
+    bi = RNG.integers(-100, 100, 8).astype(np.float32)
+    Yi = oracle.linear_dual2D_row(Xi, bi, 3.0, -2.0, 5.0, 8)
+    assert np.array_equal(Yi, 3 * Xi - 2 * bi[None, :] + 5)
+
+
+def test_bias_row_general_coefficients_within_rounding_of_fp64():
+    rows, width, stride = 64, 33, 36
+    X1 = np.zeros((rows, stride), np.float32)
+    X1[:, :width] = RNG.normal(size=(rows, width)).astype(np.float32)
+    X2 = np.zeros(stride, np.float32)
+    X2[:width] = RNG.normal(size=width).astype(np.float32)
+    a, b, g = np.float32(0.37), np.float32(-1.91), np.float32(0.123)
+    Y = oracle.linear_dual2D_row(X1, X2, a, b, g, width)
+    ref = np.float64(a) * X1.astype(np.float64) + np.float64(b) * X2.astype(np.float64)[None, :] + np.float64(g)
+    mag = np.abs(np.float64(a) * X1) + np.abs(np.float64(b) * X2)[None, :] + abs(np.float64(g))
+    # four roundings, each at most half an ulp of a partial result no larger than mag
+    assert np.all(np.abs(Y[:, :width] - ref[:, :width]) <= 4 * 2.0 ** -24 * mag[:, :width])
+    assert np.all(Y[:, width:] == 0)
+
+
 def test_reference_micro_helpers_when_built():
     ref = oracle.load_ref()
     if ref is None:
