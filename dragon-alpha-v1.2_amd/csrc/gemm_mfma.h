@@ -23,7 +23,12 @@ enum GemmTile {
     TILE_128x128_K64 = 12,
     TILE_128x64_K64 = 13,
     TILE_64x128_K64 = 14,
-    TILE_COUNT = 15
+    TILE_COUNT = 15,        // the shapes above use register-staged double buffering
+    // direct global->LDS staging through 4 stage buffers
+    TILE_DMA_128x128_S4 = 15,
+    TILE_DMA_64x64_S4 = 16,
+    TILE_DMA_64x64_K32_S4 = 17,
+    TILE_ALL_COUNT = 18
 };
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
@@ -54,6 +59,8 @@ struct GemmParams {
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu);
 void gemm_force_tile(int tile);
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
+// the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
+hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // the GEMM_NN product with p.bias added in the epilogue (what gemm_launch forwards to when p.bias is set)
 hipError_t gemm_launch_nn_biased(const GemmParams& p, int tile, hipStream_t stream);
 

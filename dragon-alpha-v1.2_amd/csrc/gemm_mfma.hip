@@ -12,7 +12,7 @@ void gemm_force_tile(int tile) { g_forced_tile = tile; }
 // global-load latency is exposed), `cap` what a full compute unit reaches with
 // `resident` workgroups sharing it.
 struct TileTraits { int bm, bn, kt, resident; float alone, cap; };
-static const TileTraits kTiles[TILE_COUNT] = {
+static const TileTraits kTiles[TILE_ALL_COUNT] = {
     /* TILE_128x128     */ {128, 128, 16, 4, 0.62f, 0.92f},
     /* TILE_64x64       */ { 64,  64, 16, 8, 0.35f, 0.82f},
     /* TILE_256x64      */ {256,  64, 16, 4, 0.62f, 0.88f},
@@ -28,6 +28,11 @@ static const TileTraits kTiles[TILE_COUNT] = {
     /* TILE_128x128_K64 */ {128, 128, 64, 1, 0.80f, 0.80f},
     /* TILE_128x64_K64  */ {128,  64, 64, 1, 0.70f, 0.70f},
     /* TILE_64x128_K64  */ { 64, 128, 64, 1, 0.70f, 0.70f},
+    // direct-to-LDS staging, three stages in flight: the best a lone workgroup does; with company
+    // its larger LDS footprint (fewer resident workgroups) loses to the register-staged shapes
+    /* TILE_DMA_128x128_S4   */ {128, 128, 16, 2, 0.60f, 0.86f},
+    /* TILE_DMA_64x64_S4     */ { 64,  64, 16, 5, 0.40f, 0.78f},
+    /* TILE_DMA_64x64_K32_S4 */ { 64,  64, 32, 2, 0.69f, 0.78f},
 };
 
 // Pick the tile shape with the lowest estimated time: the matrix work of the busiest
@@ -37,7 +42,7 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu) {
     if (g_forced_tile != TILE_AUTO) return g_forced_tile;
     int best = TILE_128x128;
     double best_cost = 1e300;
-    for (int tile = 0; tile < TILE_COUNT; tile++) {
+    for (int tile = 0; tile < TILE_ALL_COUNT; tile++) {
         const TileTraits& tt = kTiles[tile];
         const long long tm = (rows + tt.bm - 1) / tt.bm, tn = (cols + tt.bn - 1) / tt.bn;
         const long long total = tm * tn * nz;
@@ -57,6 +62,7 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu) {
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream) {
     if (p.bias != nullptr)   // the bias row exists for the forward product only
         return variant == GEMM_NN ? gemm_launch_nn_biased(p, tile, stream) : hipErrorInvalidValue;
+    if (tile >= TILE_COUNT) return gemm_launch_dma(variant, p, tile, stream);
     switch (variant) {
         case GEMM_NN: return launch_variant<true, false, false>(p, tile, stream);
         case GEMM_T1: return launch_variant<false, false, false>(p, tile, stream);

@@ -62,6 +62,34 @@ __device__ __forceinline__ v4f buffer_load_f4(const float* base, int byte_offset
     return __builtin_bit_cast(v4f, x);
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave writes
+// lds_wave_base + 16*l (the base must be the same for the whole wave; it travels in M0).  A lane
+// whose offset is out of range writes zeros.  Completion is counted by vmcnt like any other
+// vector-memory load.
+// Written as inline assembly on purpose: the compiler then knows nothing of a transfer in flight
+// and inserts no waits of its own before LDS reads (its alias analysis gives up on merged
+// ds_read2 instructions and would wait for EVERY transfer, serialising the pipeline); the kernel
+// waits explicitly.  Transfers the compiler does not know of can only make the waits it inserts
+// for its own loads and stores longer, never too short, because vmcnt retires in issue order.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // M0 is "reserved": it is exactly what this changes
+__device__ __forceinline__ void dma_f4(const float* base, float* lds_wave_base, int byte_offset) {
+    const unsigned long long b = (unsigned long long)base;
+    const v4u rsrc = {(unsigned)b, (unsigned)(b >> 32) & 0xffffu, (unsigned)RSRC_RECORDS, (unsigned)RSRC_FLAGS};
+    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(unsigned long long)(__attribute__((address_space(3))) void*)lds_wave_base);
+    // one wait state is required between writing M0 and the transfer that reads it
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(byte_offset), "s"(rsrc)
+                 : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+// s_waitcnt for the vector-memory counter alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
+// expcnt 6:4 and lgkmcnt 11:8 left at "no wait")
+constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with a private L2.
 // Re-number them so that one XCD owns a contiguous range of logical ids.
 __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
@@ -126,6 +154,25 @@ struct KInner {
             *(v4f*)(lds + r * LDS_STRIDE + 4 * (chunk ^ kin_swizzle<KT>(r))) = reg[s];
         }
     }
+    // ---- direct global -> LDS staging (no registers).  The hardware places lane l's 16 bytes at
+    // (wave's LDS base) + 16*l, so thread t fills LDS chunk position s*NTHREADS + t and the swizzle
+    // moves to the global side: the thread at slot c of row r fetches logical chunk c ^ swizzle(r).
+    int dma_kcol[PASSES];
+    __device__ __forceinline__ void init_dma(int t, int row0, int outer_bound, int ld) {
+        const int slot = t % CPR, r0 = t / CPR;
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const int r = r0 + s * RPP;
+            const int c = slot ^ kin_swizzle<KT>(r);
+            dma_kcol[s] = c * 4;
+            off[s] = (row0 + r < outer_bound) ? (r * ld + c * 4) * 4 : OOB_OFFSET;
+        }
+    }
+    __device__ __forceinline__ void issue(float* lds, const float* base, int k_left, int wave) const {
+#pragma unroll
+        for (int s = 0; s < PASSES; s++)
+            dma_f4(base, lds + (s * NTHREADS + wave * 64) * 4, dma_kcol[s] < k_left ? off[s] : OOB_OFFSET);
+    }
     __device__ __forceinline__ static const float* tile_base(const float* X, int row0, int k, int ld) {
         return X + (size_t)row0 * ld + k;
     }
@@ -166,6 +213,13 @@ struct KOuter {
 #pragma unroll
         for (int s = 0; s < PASSES; s++) *(v4f*)(lds + lds_at + s * RPP * LDS_STRIDE) = reg[s];
     }
+    // direct global -> LDS staging: thread t's chunk of pass s already sits at LDS chunk s*NTHREADS + t
+    __device__ __forceinline__ void init_dma(int t, int col0, int inner_bound, int ld) { init(t, col0, inner_bound, ld); }
+    __device__ __forceinline__ void issue(float* lds, const float* base, int k_left, int wave) const {
+#pragma unroll
+        for (int s = 0; s < PASSES; s++)
+            dma_f4(base, lds + (s * NTHREADS + wave * 64) * 4, (krow + s * RPP < k_left) ? off[s] : OOB_OFFSET);
+    }
     __device__ __forceinline__ static const float* tile_base(const float* X, int col0, int k, int ld) {
         return X + (size_t)k * ld + col0;
     }
@@ -205,6 +259,84 @@ __device__ __forceinline__ void read_frag_kouter(float (&frag)[T][4], const floa
             frag[0][q] = v.x; frag[1][q] = v.y; frag[2][q] = v.z; frag[3][q] = v.w;
         }
     }
+}
+
+// ---------------------------------------------------------------------------
+// Epilogue shared by the kernels: predicated streaming stores of one tile's accumulators.
+// ---------------------------------------------------------------------------
+// MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
+// K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
+// BIAS: the bias row is added before the store (the lane's columns are the same for all of its
+// rows); "+ 0.0f" is the gamma term of the separate bias launch this replaces: it turns a -0 sum
+// into +0, so fused and unfused results share every bit.  A template parameter rather than a
+// run-time test, so the plain products carry none of it.
+template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
+                                           int col0, float* c_ptr, int wm, int wn, int r, int h) {
+    float bias_v[TN];
+    if constexpr (BIAS) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = col0 + wn * TN * 32 + (B_KIN ? (j * 32 + r) : (TN * r + j));
+            bias_v[j] = col < p.bias_width ? p.bias[col] : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int mrow = 8 * (e / 4) + 4 * h + (e % 4);
+            const int row = row0 + wm * TM * 32 + (A_KIN ? (i * 32 + mrow) : (TM * mrow + i));
+            if (row < p.rows) {
+                float* crow = c_ptr + (size_t)row * p.ldc;
+                float out[TN];
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    out[j] = acc[i][j][e];
+                    if constexpr (BIAS)
+                        if (row < p.bias_rows) out[j] = (out[j] + bias_v[j]) + 0.0f;
+                }
+                if constexpr (B_KIN) {
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const int col = col0 + wn * TN * 32 + j * 32 + r;
+                        if (col < p.cols) __builtin_nontemporal_store(out[j], crow + col);
+                    }
+                } else {
+                    const int col = col0 + wn * TN * 32 + TN * r;
+                    if (col < p.cols) {
+                        if constexpr (TN == 1) {
+                            __builtin_nontemporal_store(out[0], crow + col);
+                        } else if constexpr (TN == 2) {
+                            v2f v = {out[0], out[1]};
+                            __builtin_nontemporal_store(v, (v2f*)(crow + col));
+                        } else {
+                            v4f v = {out[0], out[1], out[2], out[3]};
+                            __builtin_nontemporal_store(v, (v4f*)(crow + col));
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// One group of 8 k: fragments from LDS, then 4 MFMA steps over the wave's TM x TN blocks.
+template <bool A_KIN, bool B_KIN, int TM, int TN, int BM, int BN, int KT>
+__device__ __forceinline__ void mma_group(v16f (&acc)[TM][TN], const float* as, const float* bs, int wm,
+                                          int wn, int g, int r, int h) {
+    float fa[TM][4], fb[TN][4];
+    if constexpr (A_KIN) read_frag_kinner<TM, KT>(fa, as, wm * TM * 32, g, r, h);
+    else                 read_frag_kouter<TM, BM>(fa, as, wm * TM * 32, g, r, h);
+    if constexpr (B_KIN) read_frag_kinner<TN, KT>(fb, bs, wn * TN * 32, g, r, h);
+    else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -352,21 +484,8 @@ void gemm_f32_mfma(const GemmParams p) {
             const float* as = As[buf];
             const float* bs = Bs[buf];
 #pragma unroll
-            for (int g = 0; g < KT / 8; g++) {
-                float fa[TM][4], fb[TN][4];
-                if constexpr (A_KIN) read_frag_kinner<TM, KT>(fa, as, wm * TM * 32, g, r, h);
-                else                 read_frag_kouter<TM, BM>(fa, as, wm * TM * 32, g, r, h);
-                if constexpr (B_KIN) read_frag_kinner<TN, KT>(fb, bs, wn * TN * 32, g, r, h);
-                else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
-#pragma unroll
-                for (int q = 0; q < 4; q++)
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int j = 0; j < TN; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q],
-                                                                             acc[i][j], 0, 0, 0);
-            }
+            for (int g = 0; g < KT / 8; g++)
+                mma_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(acc, as, bs, wm, wn, g, r, h);
             if (fetched) {
                 la.store(ra, As[buf ^ 1]);
                 lb.store(rb, Bs[buf ^ 1]);
@@ -379,63 +498,150 @@ void gemm_f32_mfma(const GemmParams p) {
         // here; they drain while the next tile computes) ----
         // MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
         // K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
-        // BIAS: the bias row is added before the store (the lane's columns are the same for all of
-        // its rows).  A template parameter rather than a run-time test, so the plain products carry
-        // none of it.
-        float bias_v[TN];
-        if constexpr (BIAS) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int col = cur.col0 + wn * TN * 32 + (B_KIN ? (j * 32 + r) : (TN * r + j));
-                bias_v[j] = col < p.bias_width ? p.bias[col] : 0.0f;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int mrow = 8 * (e / 4) + 4 * h + (e % 4);
-                const int row = cur.row0 + wm * TM * 32 + (A_KIN ? (i * 32 + mrow) : (TM * mrow + i));
-                if (row < p.rows) {
-                    float* crow = cur.c_ptr + (size_t)row * p.ldc;
-                    float out[TN];
-#pragma unroll
-                    for (int j = 0; j < TN; j++) {
-                        out[j] = acc[i][j][e];
-                        // "+ 0.0f" is the gamma term of the separate bias launch this replaces: it
-                        // turns a -0 sum into +0, so fused and unfused results share every bit
-                        if constexpr (BIAS)
-                            if (row < p.bias_rows) out[j] = (out[j] + bias_v[j]) + 0.0f;
-                    }
-                    if constexpr (B_KIN) {
-#pragma unroll
-                        for (int j = 0; j < TN; j++) {
-                            const int col = cur.col0 + wn * TN * 32 + j * 32 + r;
-                            if (col < p.cols) __builtin_nontemporal_store(out[j], crow + col);
-                        }
-                    } else {
-                        const int col = cur.col0 + wn * TN * 32 + TN * r;
-                        if (col < p.cols) {
-                            if constexpr (TN == 1) {
-                                __builtin_nontemporal_store(out[0], crow + col);
-                            } else if constexpr (TN == 2) {
-                                v2f v = {out[0], out[1]};
-                                __builtin_nontemporal_store(v, (v2f*)(crow + col));
-                            } else {
-                                v4f v = {out[0], out[1], out[2], out[3]};
-                                __builtin_nontemporal_store(v, (v4f*)(crow + col));
-                            }
-                        }
-                    }
-                }
-            }
-        }
+        store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc, p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
         if (!has_next) break;
         for (int i = 0; i < TM; i++)
             for (int j = 0; j < TN; j++) acc[i][j] = (v16f)(0.0f);
         cur = nxt;
         lid += G;
     }
+}
+
+// ---------------------------------------------------------------------------
+// The same product with the operands staged global -> LDS directly (buffer_load ... lds) through
+// NS stage buffers, NS-1 stages in flight ahead of the one being multiplied.  No staging
+// registers, no LDS stores by the waves, one barrier per stage.  The stream of stages runs across
+// tile boundaries: while the last stages of a tile are multiplied the first stages of the
+// workgroup's next tile are already on their way.
+//
+// Each stage buffer is its own __shared__ array and the buffer index is a compile-time constant
+// at every use (the stage loop is unrolled NS times): that is what lets the compiler tell which
+// in-flight transfer a fragment read depends on, instead of waiting for all of them.
+//
+// Synchronisation per stage: every wave waits until ITS OWN transfers of the stage have landed
+// (vmcnt; transfers complete in order, so "at most the (NS-2) younger stages outstanding" is
+// enough -- later stores only make the wait longer, never shorter), then the workgroup barrier
+// makes all four waves' parts visible and at the same time guarantees that everybody has
+// finished reading the buffer that the next transfer overwrites.  A stage slot with nothing
+// left to fetch still issues its transfers with every lane out of range (zeros, no memory
+// traffic) so that the count of younger transfers is the same constant everywhere.
+// ---------------------------------------------------------------------------
+template <bool A_KIN, bool B_KIN, int BM, int BN, int KT, int NS>
+constexpr int target_occupancy_dma() {
+    const int lds = NS * 4 * (BM * KT + BN * KT);
+    const int fit = (160 * 1024) / lds;
+    return fit > 4 ? 4 : (fit < 1 ? 1 : fit);
+}
+
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, bool BIAS>
+__global__ __launch_bounds__(NTHREADS, (target_occupancy_dma<A_KIN, B_KIN, WM * TM * 32, WN * TN * 32, KT, NS>()))
+void gemm_f32_mfma_dma(const GemmParams p) {
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    static_assert(NS >= 3 && NS <= 4, "stage buffers: 3 or 4");
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
+    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT>, KOuter<BN, KT>>::type;
+    constexpr int STAGE_FLOATS = LoadA::LDS_FLOATS + LoadB::LDS_FLOATS;
+    constexpr int XFERS = LoadA::PASSES + LoadB::PASSES;      // transfers per wave per stage
+    static_assert((NS - 2) * XFERS <= 63, "vmcnt holds 6 bits");
+
+    __shared__ __attribute__((aligned(16))) float S0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float S1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float S2[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float S3[NS > 3 ? STAGE_FLOATS : 4];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+    const size_t a_step = LoadA::k_advance(p.lda), b_step = LoadB::k_advance(p.ldb);
+
+    const int total = p.tiles_m * p.tiles_n * p.nz;
+    const int G = gridDim.x;
+    int lid = xcd_contiguous_id(blockIdx.x, G);   // G <= total, so lid is a valid tile
+
+    // ---- producer: the stage to fetch next ----
+    int f_lid = lid;
+    TileCtx ft = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, f_lid);
+    LoadA la;
+    LoadB lb;
+    la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+    lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+    const float* fa_ptr = ft.a_ptr;
+    const float* fb_ptr = ft.b_ptr;
+    int f_it = 0;
+    bool f_live = true;
+
+    auto fetch = [&](float* stage) {
+        const int k = ft.k0 + f_it * KT;
+        la.issue(stage, fa_ptr, f_live ? ft.ka_lim - k : 0, wave);
+        lb.issue(stage + LoadA::LDS_FLOATS, fb_ptr, f_live ? ft.kb_lim - k : 0, wave);
+        if (f_live) {
+            f_it++;
+            fa_ptr += a_step;
+            fb_ptr += b_step;
+            if (f_it == ft.nstage) {
+                f_lid += G;
+                if (f_lid < total) {
+                    ft = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, f_lid);
+                    la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+                    lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+                    fa_ptr = ft.a_ptr;
+                    fb_ptr = ft.b_ptr;
+                    f_it = 0;
+                } else {
+                    f_live = false;
+                }
+            }
+        }
+    };
+    auto stage_buf = [&](int s) -> float* { return s == 0 ? S0 : s == 1 ? S1 : s == 2 ? S2 : S3; };
+
+    // ---- consumer: the tile being multiplied ----
+    TileCtx cur = ft;
+    int it = 0;
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = (v16f)(0.0f);
+
+#pragma unroll
+    for (int s = 0; s < NS - 1; s++) fetch(stage_buf(s));
+
+    bool running = true;
+    while (running) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            if (!running) break;
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * XFERS));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            fetch(stage_buf((s + NS - 1) % NS));
+            __builtin_amdgcn_sched_barrier(0);
+            const float* as = stage_buf(s);
+            const float* bs = as + LoadA::LDS_FLOATS;
+#pragma unroll
+            for (int g = 0; g < KT / 8; g++)
+                mma_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(acc, as, bs, wm, wn, g, r, h);
+            if (++it == cur.nstage) {
+                store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc, p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
+                lid += G;
+                if (lid < total) {
+                    cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid);
+                    it = 0;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) acc[i][j] = (v16f)(0.0f);
+                } else {
+                    running = false;
+                }
+            }
+        }
+    }
+    // nothing of this wave may still be on its way into LDS when the wave ends
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 }
 
 // ---------------------------------------------------------------------------
@@ -502,6 +708,42 @@ static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stre
         case TILE_128x128_K64: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 64>(p, stream);
         case TILE_128x64_K64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 64>(p, stream);
         case TILE_64x128_K64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 64>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+
+template <bool A_KIN, bool B_KIN, bool BIAS, int WM, int WN, int TM, int TN, int KT, int NS>
+static hipError_t launch_cfg_dma(GemmParams p, hipStream_t stream) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    auto kernel = gemm_f32_mfma_dma<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, BIAS>;
+    p.tiles_m = (p.rows + BM - 1) / BM;
+    p.tiles_n = (p.cols + BN - 1) / BN;
+    const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
+    if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidValue;
+    static int resident_per_cu = 0;
+    if (resident_per_cu == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NTHREADS, 0) != hipSuccess || n < 1)
+            n = 1;
+        resident_per_cu = n;
+    }
+    const long long slots = (long long)device_num_cu() * resident_per_cu;
+    long long grid = total;
+    if (total > slots) {
+        const long long rounds = (total + slots - 1) / slots;
+        grid = (total + rounds - 1) / rounds;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <bool A_KIN, bool B_KIN, bool BIAS>
+static hipError_t launch_variant_dma(const GemmParams& p, int tile, hipStream_t stream) {
+    switch (tile) {
+        case TILE_DMA_128x128_S4:   return launch_cfg_dma<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, 4>(p, stream);
+        case TILE_DMA_64x64_S4:     return launch_cfg_dma<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, 4>(p, stream);
+        case TILE_DMA_64x64_K32_S4: return launch_cfg_dma<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, 4>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }

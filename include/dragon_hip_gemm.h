@@ -195,7 +195,9 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M);
  * and tests that sweep the kernel variants; not thread-safe against concurrent calls.
  * Shapes: 0 = 128x128, 1 = 64x64, 2 = 256x64, 3 = 64x256, 4 = 128x64, 5 = 64x128 (16 k per
  * LDS stage); 6 = 128x128, 7 = 64x64, 8 = 128x64, 9 = 64x128 with 32 k per stage; 10 = 64x64
- * with 64 k, 11 = 64x64 with 128 k, 12 = 128x128, 13 = 128x64, 14 = 64x128 with 64 k per stage. */
+ * with 64 k, 11 = 64x64 with 128 k, 12 = 128x128, 13 = 128x64, 14 = 64x128 with 64 k per stage;
+ * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
+ * directly through four stage buffers. */
 void dragon_gemm_force_tile(int32_t tile);
 
 #ifdef __cplusplus

@@ -58,7 +58,7 @@ SHAPES = [(1, 1, 1, 1), (3, 5, 6, 7), (5, 24, 21, 8), (15, 82, 96, 9), (4, 128, 
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("tile", list(range(-1, 18)))
 def test_batched_integer_inputs_bitwise(gpu, variant, tile):
     rng = np.random.default_rng(900 + variant * 10 + tile)
     gpu.force_tile(tile)

@@ -13,7 +13,9 @@ pytestmark = pytest.mark.gpu
 
 TILES = {-1: "auto", 0: "128x128", 1: "64x64", 2: "256x64", 3: "64x256", 4: "128x64", 5: "64x128",
          6: "128x128/k32", 7: "64x64/k32", 8: "128x64/k32", 9: "64x128/k32", 10: "64x64/k64",
-         11: "64x64/k128", 12: "128x128/k64", 13: "128x64/k64", 14: "64x128/k64"}
+         11: "64x64/k128", 12: "128x128/k64", 13: "128x64/k64", 14: "64x128/k64",
+         # direct global->LDS staging through 4 stage buffers
+         15: "dma 128x128", 16: "dma 64x64", 17: "dma 64x64/k32"}
 SHAPES = [(4, 4, 4), (8, 4, 12), (128, 128, 64), (64, 64, 16), (132, 260, 20), (100, 76, 36),
           (257, 129, 385), (512, 512, 512), (1000, 777, 1531), (31, 1023, 77), (1, 1, 1), (3, 2, 5)]
 
