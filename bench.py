@@ -83,9 +83,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias",
-                    help="which of the other workloads to time (default 3,4,5,bias): BASELINE configs "
-                         "3, 4, 5 and the biased fully-connected layer")
+    ap.add_argument("--configs", default="3,4,5,bias,transfer",
+                    help="which of the other workloads to time (default 3,4,5,bias,transfer): BASELINE "
+                         "configs 3, 4, 5, the biased fully-connected layer, tensor upload / download")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
                          "(the known-size copy that FETCH_SIZE / WRITE_SIZE are scaled by)")
@@ -331,6 +331,40 @@ def main():
             "pct_hbm_peak": round(100 * 8.0 * Nb * Mb / (ms * 1e-3) / 8e12, 1)}
         for x in (dX, dW, db, dY):
             x.free()
+
+    if "transfer" in extra:
+        # upload / download of a ragged tensor (8192 x 4093 floats, device rows of 4096) through a pinned
+        # staging buffer -- the device reads / writes the packed host data in place, chunks pipelined --
+        # against the reference's route (CPU re-layout in the staging buffer, one copy); host-clock time,
+        # GB/s of logical bytes.  Bound by the host link and the host's memcpy, not by the GPU.
+        log("tensor transfer ...")
+        Ht, Wt, St = 8192, 4093, 4096
+        Xh = np.random.default_rng(1).standard_normal((Ht, Wt)).astype(np.float32)
+        back = np.empty_like(Xh)
+        dT = Cuda.malloc(Ht * St * 4)
+        pinned = Cuda.mallocHost(Ht * St * 4)
+        pageable = np.empty(Ht * St, np.float32)
+        logical = Ht * Wt * 4.0
+
+        def host_time(fn, reps=5):
+            fn()
+            best = 1e9
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                fn()
+                best = min(best, time.perf_counter() - t0)
+            return best
+        for name, buf in (("pinned staging, device-side re-layout", pinned),
+                          ("pageable staging, CPU re-layout (the reference's route)", pageable.ctypes.data)):
+            up = host_time(lambda: Cuda.set2D_v2(stream, dT, Xh, buf, Ht, Wt, St))
+            dn = host_time(lambda: Cuda.get2D_v2(stream, dT, back, buf, Ht, Wt, St))
+            assert np.array_equal(back, Xh)
+            per_config["set2D 8192x4093 " + name] = {"ms": round(up * 1e3, 3),
+                                                     "GBps": round(logical / up / 1e9, 2)}
+            per_config["get2D 8192x4093 " + name] = {"ms": round(dn * 1e3, 3),
+                                                     "GBps": round(logical / dn / 1e9, 2)}
+        Cuda.free(dT)
+        Cuda.freeHost(pinned)
 
     Cuda.deleteStream(stream)
     out = {

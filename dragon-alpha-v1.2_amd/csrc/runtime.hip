@@ -9,15 +9,21 @@
 #include <atomic>
 #include <vector>
 #include "../../include/dragon_hip_runtime.h"
+#include "runtime_internal.h"
 
 namespace {
-
 std::atomic<int> g_last_error{0};
-
-inline int note(hipError_t e) {
+}
+namespace dragon_rt {
+int note(hipError_t e) {
     if (e != hipSuccess) g_last_error.store((int)e, std::memory_order_relaxed);
     return (int)e;
 }
+}  // namespace dragon_rt
+
+namespace {
+
+inline int note(hipError_t e) { return dragon_rt::note(e); }
 inline hipStream_t as_stream(int64_t s) { return (hipStream_t)(intptr_t)s; }
 inline hipEvent_t as_event(int64_t e) { return (hipEvent_t)(intptr_t)e; }
 inline void* as_ptr(int64_t a) { return (void*)(intptr_t)a; }
@@ -54,18 +60,6 @@ int launch_blocks(long long n, int threads) {
     if (b < 1) b = 1;
     if (b > 4096) b = 4096;
     return (int)b;
-}
-
-// host rows of `width` floats  ->  staging rows of `stride` floats, pad zeroed
-void expand_rows(float* dst, const float* src, int height, int width, int stride) {
-    for (int y = 0; y < height; y++) {
-        memcpy(dst + (size_t)y * stride, src + (size_t)y * width, sizeof(float) * (size_t)width);
-        for (int x = width; x < stride; x++) dst[(size_t)y * stride + x] = 0.0f;
-    }
-}
-void compact_rows(float* dst, const float* src, int height, int width, int stride) {
-    for (int y = 0; y < height; y++)
-        memcpy(dst + (size_t)y * width, src + (size_t)y * stride, sizeof(float) * (size_t)width);
 }
 
 }  // namespace
@@ -259,74 +253,6 @@ int dragon_Cuda_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t 
     hipLaunchKernelGGL(copy4_kernel, dim3(launch_blocks(n4, 256)), dim3(256), 0, as_stream(stream),
                        (v4f*)as_ptr(dst), (const v4f*)as_ptr(src), n4);
     return note(hipGetLastError());
-}
-
-static int d2h_sync(hipStream_t s, void* dst, const void* src, size_t bytes) {
-    int e = note(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
-    if (e) return e;
-    return note(hipStreamSynchronize(s));
-}
-static int h2d_sync(hipStream_t s, void* dst, const void* src, size_t bytes) {
-    int e = note(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
-    if (e) return e;
-    return note(hipStreamSynchronize(s));
-}
-
-int dragon_Cuda_get1D(int64_t stream, int64_t address, float* value, int32_t length) {
-    if (address == 0 || value == nullptr || length <= 0) return note(hipErrorInvalidValue);
-    return d2h_sync(as_stream(stream), value, as_ptr(address), sizeof(float) * (size_t)length);
-}
-int dragon_Cuda_get1D_v2(int64_t stream, int64_t address, float* value, int64_t buf,
-                         int32_t length) {
-    if (address == 0 || value == nullptr || buf == 0 || length <= 0) return note(hipErrorInvalidValue);
-    int e = d2h_sync(as_stream(stream), as_ptr(buf), as_ptr(address), sizeof(float) * (size_t)length);
-    if (e) return e;
-    memcpy(value, as_ptr(buf), sizeof(float) * (size_t)length);
-    return 0;
-}
-int dragon_Cuda_get2D_v2(int64_t stream, int64_t address, float* value, int64_t buf,
-                         int32_t height, int32_t width, int32_t stride) {
-    if (address == 0 || value == nullptr || buf == 0 || height <= 0 || width <= 0 || stride < width)
-        return note(hipErrorInvalidValue);
-    const size_t lengthv = (size_t)height * stride;
-    int e = d2h_sync(as_stream(stream), as_ptr(buf), as_ptr(address), sizeof(float) * lengthv);
-    if (e) return e;
-    compact_rows(value, (const float*)as_ptr(buf), height, width, stride);
-    return 0;
-}
-int dragon_Cuda_get2D(int64_t stream, int64_t address, float* value, int32_t height,
-                      int32_t width, int32_t stride) {
-    if (address == 0 || value == nullptr || height <= 0 || width <= 0 || stride < width)
-        return note(hipErrorInvalidValue);
-    std::vector<float> staging((size_t)height * stride);
-    return dragon_Cuda_get2D_v2(stream, address, value, (int64_t)(intptr_t)staging.data(), height,
-                                width, stride);
-}
-int dragon_Cuda_set1D(int64_t stream, int64_t address, const float* value, int32_t length) {
-    if (address == 0 || value == nullptr || length <= 0) return note(hipErrorInvalidValue);
-    return h2d_sync(as_stream(stream), as_ptr(address), value, sizeof(float) * (size_t)length);
-}
-int dragon_Cuda_set1D_v2(int64_t stream, int64_t address, const float* value, int64_t buf,
-                         int32_t length) {
-    if (address == 0 || value == nullptr || buf == 0 || length <= 0) return note(hipErrorInvalidValue);
-    memcpy(as_ptr(buf), value, sizeof(float) * (size_t)length);
-    return h2d_sync(as_stream(stream), as_ptr(address), as_ptr(buf), sizeof(float) * (size_t)length);
-}
-int dragon_Cuda_set2D_v2(int64_t stream, int64_t address, const float* value, int64_t buf,
-                         int32_t height, int32_t width, int32_t stride) {
-    if (address == 0 || value == nullptr || buf == 0 || height <= 0 || width <= 0 || stride < width)
-        return note(hipErrorInvalidValue);
-    expand_rows((float*)as_ptr(buf), value, height, width, stride);
-    return h2d_sync(as_stream(stream), as_ptr(address), as_ptr(buf),
-                    sizeof(float) * (size_t)height * stride);
-}
-int dragon_Cuda_set2D(int64_t stream, int64_t address, const float* value, int32_t height,
-                      int32_t width, int32_t stride) {
-    if (address == 0 || value == nullptr || height <= 0 || width <= 0 || stride < width)
-        return note(hipErrorInvalidValue);
-    std::vector<float> staging((size_t)height * stride);
-    return dragon_Cuda_set2D_v2(stream, address, value, (int64_t)(intptr_t)staging.data(), height,
-                                width, stride);
 }
 
 }  // extern "C"

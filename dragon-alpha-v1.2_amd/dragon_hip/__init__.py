@@ -194,6 +194,25 @@ class Cuda:
     def get2D(stream, address, value, height, width, stride):
         _check(lib.dragon_Cuda_get2D(stream, address, _host_ptr(value), height, width, stride))
 
+    # _v2: through a staging buffer of the caller's (an address from mallocHost, normally)
+    @staticmethod
+    def set1D_v2(stream, address, value, buf_address, length):
+        _check(lib.dragon_Cuda_set1D_v2(stream, address, _host_ptr(value), buf_address, length))
+
+    @staticmethod
+    def set2D_v2(stream, address, value, buf_address, height, width, stride):
+        _check(lib.dragon_Cuda_set2D_v2(stream, address, _host_ptr(value), buf_address, height, width,
+                                        stride))
+
+    @staticmethod
+    def get1D_v2(stream, address, value, buf_address, length):
+        _check(lib.dragon_Cuda_get1D_v2(stream, address, _host_ptr(value), buf_address, length))
+
+    @staticmethod
+    def get2D_v2(stream, address, value, buf_address, height, width, stride):
+        _check(lib.dragon_Cuda_get2D_v2(stream, address, _host_ptr(value), buf_address, height, width,
+                                        stride))
+
 
 class Cuda_matMul:
     """Natives and helpers of Cuda_matMul.java."""

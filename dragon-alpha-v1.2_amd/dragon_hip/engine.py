@@ -70,8 +70,12 @@ MATMUL, MATMUL_T1, MATMUL_T2, BMM, BMM_T1, BMM_T2 = range(6)
 class Engine:
     """alpha.engine.cuda_float32(deviceId, ...)"""
 
-    def __init__(self, device_id=0, stream_pool_size=32):
-        self._h = lib.dragon_engine_cuda_float32(device_id, stream_pool_size)
+    def __init__(self, device_id=0, stream_pool_size=32, max_trans_buf_size=0):
+        if max_trans_buf_size > 0:
+            self._h = lib.dragon_engine_cuda_float32_buffered(device_id, stream_pool_size,
+                                                              max_trans_buf_size)
+        else:
+            self._h = lib.dragon_engine_cuda_float32(device_id, stream_pool_size)
         if not self._h:
             msg = _last_code()
             code = lib.dragon_engine_last_cuda_code()
@@ -207,5 +211,5 @@ class Engine:
         return self.linear2_row(inplace, X1, X2, 1.0, 1.0, 0.0)
 
 
-def cuda_float32(device_id=0, stream_pool_size=32):
-    return Engine(device_id, stream_pool_size)
+def cuda_float32(device_id=0, stream_pool_size=32, max_trans_buf_size=0):
+    return Engine(device_id, stream_pool_size, max_trans_buf_size)

@@ -323,25 +323,101 @@ SyncerPtr CudaFloat32EngineBase::memset(int64_t address, int value, int64_t mems
     cu(dragon_Cuda_memsetAsync(stream, address, value, memsize));
     return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
 }
+// Transfers (:1197-1260): with a staging pool the _v2 natives, else the plain ones.
+namespace {
+struct StagingBlock {   // returns the block to the pool on every path out
+    PinnedMempool* pool;
+    PinnedMempool::Block b;
+    StagingBlock(PinnedMempool* p, int64_t bytes) : pool(p), b(p->malloc(bytes)) {}
+    ~StagingBlock() { pool->free(b.size, b.address); }
+};
+}  // namespace
 void CudaFloat32EngineBase::get1D(int64_t address, float* value, int length) {
     int64_t stream = streamPool_->getStream();
-    cu(dragon_Cuda_get1D(stream, address, value, length));
+    if (!bufPool_) cu(dragon_Cuda_get1D(stream, address, value, length));
+    else {
+        StagingBlock sb(bufPool_.get(), (int64_t)length << 2);
+        cu(dragon_Cuda_get1D_v2(stream, address, value, sb.b.address, length));
+    }
     streamPool_->returnStream(stream);
 }
 void CudaFloat32EngineBase::get2D(int64_t address, float* value, int height, int width, int stride) {
     int64_t stream = streamPool_->getStream();
-    cu(dragon_Cuda_get2D(stream, address, value, height, width, stride));
+    if (!bufPool_) cu(dragon_Cuda_get2D(stream, address, value, height, width, stride));
+    else {
+        StagingBlock sb(bufPool_.get(), ((int64_t)height * stride) << 2);
+        cu(dragon_Cuda_get2D_v2(stream, address, value, sb.b.address, height, width, stride));
+    }
     streamPool_->returnStream(stream);
 }
 void CudaFloat32EngineBase::set1D(int64_t address, const float* value, int length) {
     int64_t stream = streamPool_->getStream();
-    cu(dragon_Cuda_set1D(stream, address, value, length));
+    if (!bufPool_) cu(dragon_Cuda_set1D(stream, address, value, length));
+    else {
+        StagingBlock sb(bufPool_.get(), (int64_t)length << 2);
+        cu(dragon_Cuda_set1D_v2(stream, address, value, sb.b.address, length));
+    }
     streamPool_->returnStream(stream);
 }
 void CudaFloat32EngineBase::set2D(int64_t address, const float* value, int height, int width, int stride) {
     int64_t stream = streamPool_->getStream();
-    cu(dragon_Cuda_set2D(stream, address, value, height, width, stride));
+    if (!bufPool_) cu(dragon_Cuda_set2D(stream, address, value, height, width, stride));
+    else {
+        StagingBlock sb(bufPool_.get(), ((int64_t)height * stride) << 2);
+        cu(dragon_Cuda_set2D_v2(stream, address, value, sb.b.address, height, width, stride));
+    }
     streamPool_->returnStream(stream);
+}
+
+// ---- PinnedMempool (PinnedMempool.java:96-200) ---------------------------------------------------
+PinnedMempool::Block PinnedMempool::malloc(int64_t mem_size) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (mem_size <= 0) throw IllegalArgumentException("mem_size must be positive");
+    mem_size = (mem_size + 3) >> 2 << 2;
+    int64_t size = 0, address = 0;
+    auto it = pool_.lower_bound(mem_size);                       // remove_section(size, 1.5 * size)
+    if (it != pool_.end() && it->first <= (int64_t)((double)mem_size * 1.5)) {
+        size = it->first; address = it->second;
+        pool_.erase(it);
+    } else {
+        // the Java pool waits up to 10 s for another thread to free memory; this one fails at once
+        if (mem_size > max_mem_size_ - used_mem_size_)
+            throw std::runtime_error("[Error] Maximum Memory { " + std::to_string(max_mem_size_ >> 20) +
+                                     " } is insufficient. Try to alloc more");
+        while (mem_size > max_mem_size_ - total_mem_size_ && !pool_.empty()) {   // alloc_free: largest first
+            auto big = std::prev(pool_.end());
+            cu(dragon_Cuda_freeHost(big->second));
+            total_mem_size_ -= big->first;
+            blocks_.erase(big->second);
+            grave_.erase(big->second);
+            pool_.erase(big);
+        }
+        address = dragon_Cuda_mallocHost(mem_size);
+        if (address == 0)
+            throw std::runtime_error("Cuda_malloc_host: failed to alloc pinned-memory for [mem_size = " +
+                                     std::to_string(mem_size) + " ]");
+        size = mem_size;
+        total_mem_size_ += size;
+        blocks_[address] = size;
+    }
+    used_mem_size_ += size;
+    grave_.erase(address);
+    return Block{size >> 2, address};
+}
+bool PinnedMempool::free(int64_t size, int64_t address) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (address == 0 || grave_.count(address) || !blocks_.count(address)) return false;
+    const int64_t bytes = size << 2;
+    pool_.emplace(bytes, address);
+    grave_.insert(address);
+    used_mem_size_ -= bytes;
+    return true;
+}
+void PinnedMempool::clear() {
+    std::lock_guard<std::mutex> g(mu_);
+    for (auto& kv : blocks_) (void)dragon_Cuda_freeHost(kv.first);
+    blocks_.clear(); pool_.clear(); grave_.clear();
+    total_mem_size_ = used_mem_size_ = 0;
 }
 
 // Shared body of matMul / matMulT1 / matMulT2 (:1534-1589, :1751-1806, :1870-1925) and, with a
@@ -656,8 +732,10 @@ Tensor& Tensor::c() {
 }
 
 // ---- Engine ------------------------------------------------------------------------------------------------
-Engine::Engine(int deviceId, int streamPool_maxsize) {
+Engine::Engine(int deviceId, int streamPool_maxsize, int64_t max_trans_buf_size) {
     base_.reset(new CudaFloat32EngineBase(deviceId, streamPool_maxsize));
+    if (max_trans_buf_size > 0)
+        base_->buf_mempool(std::unique_ptr<PinnedMempool>(new PinnedMempool(max_trans_buf_size)));
     core_.reset(new EngineCore(base_.get(), true));
 }
 Engine::~Engine() {}

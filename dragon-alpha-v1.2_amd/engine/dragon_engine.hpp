@@ -10,13 +10,16 @@
 //   CudaFloat32EngineBase  z/dragon/engine/cuda/CudaFloat32EngineBase.java:70-92, 1148-1260, 1471-2020,
 //                          4517-4530 (linear2_2D_row)
 //   EngineCore             z/dragon/engine/EngineCore.java:693-811 (checks and x4 padding)
+//   PinnedMempool          z/dragon/engine/cuda/impl/PinnedMempool.java:96-200
 //   Tensor                 z/dragon/engine/Tensor.java:206-239 (length / lengthv / length_4x)
 //   Engine                 z/dragon/engine/Engine.java:522-551, 671-676, 824-837, 908-914, 955-1470,
 //                          4185-4207 (add_row / linear2_row)
 // (paths relative to source/alpha-Dragon-v1.2/src of the reference tree)
 #pragma once
 #include <stdint.h>
+#include <map>
 #include <memory>
+#include <set>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -63,6 +66,30 @@ private:
     std::mutex mu_;
 };
 
+// ---- pinned host staging buffers for tensor transfer (z/dragon/engine/cuda/impl/PinnedMempool.java)
+// Blocks are recycled by size: a request takes the smallest free block of [size, 1.5*size], else
+// allocates; when the budget is exhausted free blocks are released largest-first to make room.
+class PinnedMempool {
+public:
+    explicit PinnedMempool(int64_t maxMemorySize) : max_mem_size_(maxMemorySize) {}
+    ~PinnedMempool() { clear(); }
+    struct Block { int64_t size, address; };   // size in floats (bytes / 4), as the Java pool reports it
+    Block malloc(int64_t mem_size);            // mem_size in bytes
+    bool free(int64_t size, int64_t address);  // size as returned by malloc
+    void clear();
+    int64_t max_mem_size() const { return max_mem_size_; }
+    int64_t total_mem_size() const { return total_mem_size_; }
+    int64_t used_mem_size() const { return used_mem_size_; }
+    int physical_block_num() const { return (int)blocks_.size(); }
+    int buffered_block_num() const { return (int)pool_.size(); }
+private:
+    int64_t max_mem_size_, total_mem_size_ = 0, used_mem_size_ = 0;
+    std::multimap<int64_t, int64_t> pool_;     // free blocks: size in bytes -> address
+    std::map<int64_t, int64_t> blocks_;        // every block this pool owns: address -> size in bytes
+    std::set<int64_t> grave_;                  // addresses currently free (guards a double free)
+    std::mutex mu_;
+};
+
 // ---- completion handles ----------------------------------------------------------------------
 class Syncer {
 public:
@@ -93,6 +120,9 @@ public:
     CudaDevice& device() { return dev_; }
     CudaStreamPool& streamPool() { return *streamPool_; }
     void engineCore(EngineCore* core) { core_ = core; }
+    // staging pool for get / set; without one the transfers stage through pageable memory
+    PinnedMempool* buf_mempool() { return bufPool_.get(); }
+    void buf_mempool(std::unique_ptr<PinnedMempool> pool) { bufPool_ = std::move(pool); }
 
     // knobs (same names and defaults as the Java fields)
     int matMul_sk_threshold = 512, matMul_sk_maxPart = 16;
@@ -152,6 +182,7 @@ private:
                      int64_t Bias = 0, int lengthv = 0, int width = 0);
     CudaDevice dev_;
     std::unique_ptr<CudaStreamPool> streamPool_;
+    std::unique_ptr<PinnedMempool> bufPool_;
     EngineCore* core_ = nullptr;
 };
 
@@ -214,7 +245,8 @@ private:
 // ---- Engine: the tensor-level API ------------------------------------------------------------------------
 class Engine {
 public:
-    Engine(int deviceId, int streamPool_maxsize);
+    // max_trans_buf_size > 0 gives the engine a PinnedMempool of that many bytes (Alpha.java:770-790)
+    Engine(int deviceId, int streamPool_maxsize, int64_t max_trans_buf_size = 0);
     ~Engine();
     EngineCore& engineCore() { return *core_; }
     CudaFloat32EngineBase& engineBase() { return *base_; }

@@ -8,7 +8,7 @@
 
 using namespace dragon;
 
-struct dragon_engine { Engine eg; dragon_engine(int d, int p) : eg(d, p) {} };
+struct dragon_engine { Engine eg; dragon_engine(int d, int p, int64_t b = 0) : eg(d, p, b) {} };
 struct dragon_tensor { Tensor* ts; };
 
 namespace {
@@ -52,6 +52,12 @@ int32_t dragon_engine_last_cuda_code(void) { return g_cuda_code; }
 dragon_engine* dragon_engine_cuda_float32(int32_t device_id, int32_t stream_pool_size) {
     dragon_engine* e = nullptr;
     guard([&] { e = new dragon_engine(device_id, stream_pool_size); });
+    return e;
+}
+dragon_engine* dragon_engine_cuda_float32_buffered(int32_t device_id, int32_t stream_pool_size,
+                                                   int64_t max_trans_buf_size) {
+    dragon_engine* e = nullptr;
+    guard([&] { e = new dragon_engine(device_id, stream_pool_size, max_trans_buf_size); });
     return e;
 }
 void dragon_engine_delete(dragon_engine* eg) { delete eg; }
@@ -102,6 +108,10 @@ int32_t dragon_engine_get_param(dragon_engine* eg, const char* name) {
         else if (n == "last_stream_count") out = b.last_stream_count;
         else if (n == "live_blocks") out = (int32_t)eg->eg.engineCore().live_blocks();
         else if (n == "stream_pool_size") out = b.streamPool().total_stream_size();
+        else if (n == "buf_physical_blocks") out = b.buf_mempool() ? b.buf_mempool()->physical_block_num() : -1;
+        else if (n == "buf_buffered_blocks") out = b.buf_mempool() ? b.buf_mempool()->buffered_block_num() : -1;
+        else if (n == "buf_used_mem_size") out = b.buf_mempool() ? (int32_t)b.buf_mempool()->used_mem_size() : -1;
+        else if (n == "buf_total_mem_size_MB") out = b.buf_mempool() ? (int32_t)(b.buf_mempool()->total_mem_size() >> 20) : -1;
         else throw IllegalArgumentException("unknown parameter: " + n);
     });
     return out;

@@ -38,6 +38,11 @@ int32_t dragon_engine_last_cuda_code(void);
 /* alpha.engine.cuda_float32(deviceId, ...) with a stream pool of the given size (32 in the
  * reference's default constructor). */
 dragon_engine* dragon_engine_cuda_float32(int32_t device_id, int32_t stream_pool_size);
+/* the same with a pinned staging pool of max_trans_buf_size bytes for tensor upload / download
+ * (alpha.engine.cuda_float32(deviceId, streamPool, mempool, max_trans_buf_size, check),
+ * Alpha.java:770-790; PinnedMempool.java) */
+dragon_engine* dragon_engine_cuda_float32_buffered(int32_t device_id, int32_t stream_pool_size,
+                                                   int64_t max_trans_buf_size);
 void dragon_engine_delete(dragon_engine* eg);
 int dragon_engine_check(dragon_engine* eg, int32_t flag);   /* Engine.check(boolean) */
 int dragon_engine_sync(dragon_engine* eg, int32_t flag);    /* Engine.sync(boolean)  */
@@ -49,7 +54,9 @@ int dragon_engine_sync(dragon_engine* eg, int32_t flag);    /* Engine.sync(boole
  * count and recompute maxPart from it). */
 int dragon_engine_set_param(dragon_engine* eg, const char* name, int32_t value);
 int32_t dragon_engine_get_param(dragon_engine* eg, const char* name);   /* also "last_gridZ",
-    "last_stream_count", "live_blocks", "stream_pool_size" */
+    "last_stream_count", "live_blocks", "stream_pool_size", and of the staging pool
+    "buf_physical_blocks", "buf_buffered_blocks", "buf_used_mem_size", "buf_total_mem_size_MB"
+    (-1 without a pool) */
 
 /* split-K decision for padded dims; kind 0 matMul, 1 matMulT1, 2 matMulT2, 3 matMul_biased;
  * 1 = no split */
