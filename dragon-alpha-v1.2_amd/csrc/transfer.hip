@@ -9,7 +9,8 @@
 //   * the staging buffer holds the PACKED data and a kernel reads it (or writes it) in place over
 //     the host link: the pad never crosses the link, and the re-layout costs no CPU time;
 //   * the transfer is cut into chunks, so the CPU copy of chunk i+1 between the caller's array and
-//     the staging buffer overlaps the device's transfer of chunk i.  Every chunk has its own region
+//     the staging buffer overlaps the device's transfer of chunk i; long transfers share the CPU
+//     copies between the calling thread and one helper.  Every chunk has its own region
 //     of the staging buffer (it is as large as the whole tensor), so no region is reused and the
 //     only synchronisation is "chunk i has arrived" on the download side.
 // Device rows are written whole: the pad columns of an upload are zeroed by the device.
@@ -19,6 +20,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <string.h>
+#include <atomic>
+#include <thread>
 #include <vector>
 #include "../../include/dragon_hip_runtime.h"
 #include "runtime_internal.h"
@@ -121,6 +124,33 @@ struct Chunks {
 
 int sync(hipStream_t s) { return note(hipStreamSynchronize(s)); }
 
+// Runs body(i) for every chunk i, on the calling thread alone for short transfers and shared with
+// one helper thread for long ones (one core's memcpy is slower than the host link).  The chunks are
+// independent: each has its own region of the staging buffer and of the tensor.  Returns the first
+// failure; the helper works on the caller's device.
+template <typename F>
+int for_each_chunk(int count, F body) {
+    if (count < 4) {
+        for (int i = 0; i < count; i++)
+            if (int e = body(i)) return e;
+        return 0;
+    }
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::atomic<int> next{0}, err{0};
+    auto work = [&] {
+        for (;;) {
+            const int i = next.fetch_add(1);
+            if (i >= count || err.load()) return;
+            if (int e = body(i)) { err.store(e); return; }
+        }
+    };
+    std::thread helper([&] { if (hipSetDevice(dev) == hipSuccess) work(); });
+    work();
+    helper.join();
+    return err.load();
+}
+
 // ---- the reference's route: CPU re-layout in the staging buffer, one copy ----------------------
 void expand_rows(float* dst, const float* src, int height, int width, int stride) {
     for (int y = 0; y < height; y++) {
@@ -149,13 +179,13 @@ int download_staged(hipStream_t s, const float* dX, float* value, float* buf, in
 // ---- contiguous data through a pinned buffer, chunk by chunk --------------------------------------
 int upload_linear(hipStream_t s, float* dX, const float* value, float* buf, long long n) {
     const Chunks c(n);
-    for (int i = 0; i < c.count; i++) {
+    const int e = for_each_chunk(c.count, [&](int i) {
         const long long lo = c.lo(i), cnt = c.hi(i) - lo;
         memcpy(buf + lo, value + lo, sizeof(float) * (size_t)cnt);
-        int e = note(hipMemcpyAsync(dX + lo, buf + lo, sizeof(float) * (size_t)cnt, hipMemcpyHostToDevice, s));
-        if (e) { (void)hipStreamSynchronize(s); return e; }
-    }
-    return sync(s);
+        return note(hipMemcpyAsync(dX + lo, buf + lo, sizeof(float) * (size_t)cnt, hipMemcpyHostToDevice, s));
+    });
+    const int w = sync(s);     // also on failure: nothing may still read the buffer when we return
+    return e ? e : w;
 }
 
 struct EventList {
@@ -170,6 +200,18 @@ struct EventList {
     }
 };
 
+// chunk i has arrived in the staging buffer when its event has completed: copy it out
+int drain(hipStream_t s, const Chunks& c, EventList& done, float* value, const float* buf) {
+    const int e = for_each_chunk(c.count, [&](int i) {
+        if (int w = note(hipEventSynchronize(done.ev[i]))) return w;
+        const long long lo = c.lo(i);
+        memcpy(value + lo, buf + lo, sizeof(float) * (size_t)(c.hi(i) - lo));
+        return 0;
+    });
+    if (e) (void)hipStreamSynchronize(s);
+    return e;
+}
+
 int download_linear(hipStream_t s, const float* dX, float* value, float* buf, long long n) {
     const Chunks c(n);
     EventList done;
@@ -179,13 +221,7 @@ int download_linear(hipStream_t s, const float* dX, float* value, float* buf, lo
         if (!e) e = done.add(s);
         if (e) { (void)hipStreamSynchronize(s); return e; }
     }
-    for (int i = 0; i < c.count; i++) {
-        int e = note(hipEventSynchronize(done.ev[i]));
-        if (e) { (void)hipStreamSynchronize(s); return e; }
-        const long long lo = c.lo(i);
-        memcpy(value + lo, buf + lo, sizeof(float) * (size_t)(c.hi(i) - lo));
-    }
-    return 0;
+    return drain(s, c, done, value, buf);
 }
 
 // ---- strided rows through a pinned buffer that the device reads / writes in place ----------------
@@ -195,13 +231,13 @@ int upload_rows(hipStream_t s, float* dX, const float* value, float* buf, int he
     hipLaunchKernelGGL(zero_pad_kernel, dim3(blocks_for((long long)height * (stride - width), 256)), dim3(256),
                        0, s, dX, height, width, stride);
     int e = note(hipGetLastError());
-    for (int i = 0; i < c.count && !e; i++) {
+    if (!e) e = for_each_chunk(c.count, [&](int i) {
         const long long lo = c.lo(i), cnt = c.hi(i) - lo;
         memcpy(buf + lo, value + lo, sizeof(float) * (size_t)cnt);
         hipLaunchKernelGGL(spread_rows_kernel, dim3(blocks_for((cnt + 3) >> 2, 256)), dim3(256), 0, s,
                            (const float*)buf, dX, lo, cnt, n, width, stride);
-        e = note(hipGetLastError());
-    }
+        return note(hipGetLastError());
+    });
     const int w = sync(s);     // also on failure: nothing may still read the buffer when we return
     return e ? e : w;
 }
@@ -218,13 +254,7 @@ int download_rows(hipStream_t s, const float* dX, float* value, float* buf, int 
         if (!e) e = done.add(s);
     }
     if (e) { (void)hipStreamSynchronize(s); return e; }
-    for (int i = 0; i < c.count; i++) {
-        e = note(hipEventSynchronize(done.ev[i]));
-        if (e) { (void)hipStreamSynchronize(s); return e; }
-        const long long lo = c.lo(i);
-        memcpy(value + lo, buf + lo, sizeof(float) * (size_t)(c.hi(i) - lo));
-    }
-    return 0;
+    return drain(s, c, done, value, buf);
 }
 
 bool bad2d(int64_t address, const void* value, int height, int width, int stride) {
