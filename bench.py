@@ -83,9 +83,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias,transfer",
-                    help="which of the other workloads to time (default 3,4,5,bias,transfer): BASELINE "
-                         "configs 3, 4, 5, the biased fully-connected layer, tensor upload / download")
+    ap.add_argument("--configs", default="3,4,5,bias,transpose,transfer",
+                    help="which of the other workloads to time (default 3,4,5,bias,transpose,transfer): "
+                         "BASELINE configs 3, 4, 5, the biased fully-connected layer, dimension swaps, "
+                         "tensor upload / download")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
                          "(the known-size copy that FETCH_SIZE / WRITE_SIZE are scaled by)")
@@ -331,6 +332,27 @@ def main():
             "pct_hbm_peak": round(100 * 8.0 * Nb * Mb / (ms * 1e-3) / 8e12, 1)}
         for x in (dX, dW, db, dY):
             x.free()
+
+    if "transpose" in extra:
+        # the layout step of attention blocks: [B, S, H, D] <-> [B, H, S, D] (whole rows move) and the
+        # last-two-dimension swap K -> K^T per head (LDS-tiled); HBM-bound, read + write once
+        log("dimension swap ...")
+        E2 = dh.Cuda_expk2
+        Bq, Sq2, Hq, Dq = 32, 2048, 16, 64
+        nq = Bq * Sq2 * Hq * Dq                 # 64 Mi floats = 256 MiB: X and Y together exceed the 256 MB cache
+        dX2, dY2 = dh.DeviceArray(size=nq), dh.DeviceArray(size=nq)
+        for name, fn in (
+            ("transpose4D [32,2048,16,64] dims (1,2)", lambda: E2.transpose4D(
+                stream, dX2.address, dY2.address, Sq2, Hq, Dq, Hq, Sq2, Dq, 1, 2, Dq, Dq, nq)),
+            ("transpose4D [32,16,2048,64] dims (2,3)", lambda: E2.transpose4D(
+                stream, dX2.address, dY2.address, Hq, Sq2, Dq, Hq, Dq, Sq2, 2, 3, Dq, Sq2, nq)),
+            ("transpose2D [8192,8192]", lambda: E2.transpose2D(
+                stream, dX2.address, dY2.address, 8192, 8192, 8192, 8192, nq))):
+            ms = timer.per_launch_ms(fn, iters=50)
+            per_config[name + " (HBM-bound)"] = {
+                "ms": round(ms, 4), "alg_GBps": round(8.0 * nq / (ms * 1e-3) / 1e9, 1),
+                "pct_hbm_peak": round(100 * 8.0 * nq / (ms * 1e-3) / 8e12, 1)}
+        dX2.free(), dY2.free()
 
     if "transfer" in extra:
         # upload / download of a ragged tensor (8192 x 4093 floats, device rows of 4096) through a pinned

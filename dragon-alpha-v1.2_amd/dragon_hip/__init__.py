@@ -5,6 +5,7 @@ Thin, one-to-one wrappers over the C ABI (no compute happens in Python):
   Cuda             -- runtime natives of the reference's z.dragon.engine.cuda.impl.Cuda
   Cuda_matMul      -- natives + heuristics of ...impl.math.Cuda_matMul
   Cuda_batchMatMul -- natives + heuristics of ...impl.math.Cuda_batchMatMul
+  Cuda_expk2       -- transpose2D / 3D / 4D of ...impl.Cuda_expk2 (dimension swap)
   Cuda_function    -- linear_dual2D_row of ...impl.math.Cuda_function (the bias row)
   CudaException    -- the error type the reference's natives throw
 
@@ -285,6 +286,26 @@ class Cuda_function:
                           stride):
         _check(lib.dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta,
                                                           gamma, dY, lengthv, width, stride))
+
+
+class Cuda_expk2:
+    """The dimension-swap natives of Cuda_expk2.java."""
+
+    @staticmethod
+    def transpose2D(stream, dX, dY, Xdim1, Ydim1, strideX, strideY, length):
+        _check(lib.dragon_Cuda_expk2_transpose2D(stream, dX, dY, Xdim1, Ydim1, strideX, strideY, length))
+
+    @staticmethod
+    def transpose3D(stream, dX, dY, Xdim1, Xdim2, Ydim1, Ydim2, dimIndex1, dimIndex2, strideX, strideY,
+                    length):
+        _check(lib.dragon_Cuda_expk2_transpose3D(stream, dX, dY, Xdim1, Xdim2, Ydim1, Ydim2, dimIndex1,
+                                                 dimIndex2, strideX, strideY, length))
+
+    @staticmethod
+    def transpose4D(stream, dX, dY, Xdim1, Xdim2, Xdim3, Ydim1, Ydim2, Ydim3, dimIndex1, dimIndex2,
+                    strideX, strideY, length):
+        _check(lib.dragon_Cuda_expk2_transpose4D(stream, dX, dY, Xdim1, Xdim2, Xdim3, Ydim1, Ydim2, Ydim3,
+                                                 dimIndex1, dimIndex2, strideX, strideY, length))
 
 
 class Cuda_batchMatMul:

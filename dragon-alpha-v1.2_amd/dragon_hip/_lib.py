@@ -32,6 +32,9 @@ SIGNATURES = {
     "dragon_Cuda_matMul_SKbuf_summary": (i32, [i64, i64, i64, i32, i32]),
     "dragon_Cuda_function_linear_dual2D_row": (i32, [i64, i64, i64, i32, f32, f32, f32, i64, i32, i32, i32]),
     "dragon_Cuda_matMul_matMul_biased": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32]),
+    "dragon_Cuda_expk2_transpose2D": (i32, [i64, i64, i64, i32, i32, i32, i32, i32]),
+    "dragon_Cuda_expk2_transpose3D": (i32, [i64, i64, i64] + [i32] * 9),
+    "dragon_Cuda_expk2_transpose4D": (i32, [i64, i64, i64] + [i32] * 11),
     "dragon_Cuda_batchMatMul_batchMatMul": (i32, _BMM),
     "dragon_Cuda_batchMatMul_batchMatMul_texture": (i32, _BMM),
     "dragon_Cuda_batchMatMul_batchMatMulT1": (i32, _BMM),
@@ -125,6 +128,7 @@ SIGNATURES = {
     "dragon_engine_product_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
     "dragon_engine_fullconnect": (c_void_p, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
     "dragon_engine_fullconnect_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "dragon_engine_transpose": (c_void_p, [c_void_p, i32, c_void_p, i32, i32]),
     "dragon_engine_linear2_row": (c_void_p, [c_void_p, i32, c_void_p, c_void_p, f32, f32, f32]),
 }
 

@@ -207,6 +207,12 @@ class Engine:
             return X1
         return self._wrap(h)
 
+    def transpose(self, inplace, X, dimIdx1, dimIdx2):
+        h = lib.dragon_engine_transpose(self._h, int(inplace), X._h if X else None, dimIdx1, dimIdx2)
+        if h and X is not None and h == X._h:
+            return X
+        return self._wrap(h)
+
     def add_row(self, inplace, X1, X2):
         return self.linear2_row(inplace, X1, X2, 1.0, 1.0, 0.0)
 

@@ -516,6 +516,25 @@ SyncerPtr CudaFloat32EngineBase::linear2_2D_row(int64_t Y, int64_t X1, int64_t X
                                               lengthv, width, stride));
     return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
 }
+SyncerPtr CudaFloat32EngineBase::transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X,
+                                           const std::vector<int>& Xdim, int dimIndex1, int dimIndex2,
+                                           int strideX, int strideY, int length) {   // :1343-1375
+    int64_t stream = streamPool_->getStream();
+    if (Xdim.size() == 4)
+        cu(dragon_Cuda_expk2_transpose4D(stream, X, Y, Xdim[1], Xdim[2], Xdim[3], Ydim[1], Ydim[2], Ydim[3],
+                                         dimIndex1, dimIndex2, strideX, strideY, length));
+    else if (Xdim.size() == 3)
+        cu(dragon_Cuda_expk2_transpose3D(stream, X, Y, Xdim[1], Xdim[2], Ydim[1], Ydim[2], dimIndex1,
+                                         dimIndex2, strideX, strideY, length));
+    else
+        cu(dragon_Cuda_expk2_transpose2D(stream, X, Y, Xdim[1], Ydim[1], strideX, strideY, length));
+    return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
+}
+SyncerPtr CudaFloat32EngineBase::memcpy(int64_t dst, int64_t src, int64_t memsize) {   // :1173-1179
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_memcpyAsyncDeviceToDevice(stream, dst, src, memsize));
+    return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
+}
 SyncerPtr CudaFloat32EngineBase::matMulT1(int64_t C, int64_t A, int64_t B, int N, int M, int K) {
     return run_2d(1, matMulT1_gridZ(N, M, K), C, A, B, N, M, K);
 }
@@ -633,6 +652,32 @@ void EngineCore::matMul_check(int64_t C, int64_t A, int64_t B, int N, int M, int
     if (K <= 0) throw IllegalArgumentException(fmt("K { got %lld } must > 0", K));
 }
 
+SyncerPtr EngineCore::transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X,
+                                const std::vector<int>& Xdim, int dimIndex1, int dimIndex2, int widthX,
+                                int widthY, int length) {   // :582-613
+    if (check) {
+        auto s = [](int v) { return std::to_string(v); };
+        if (Y == 0) throw NullPointerException("Tensor Y is null");
+        if (X == 0) throw NullPointerException("Tensor X is null");
+        if (Ydim.size() < 2) throw IllegalArgumentException("Y.ndim { got " + s((int)Ydim.size()) + " } must >= 2");
+        if (Xdim.size() < 2) throw IllegalArgumentException("X.ndim { got " + s((int)Xdim.size()) + " } must >= 2");
+        if (widthX <= 0) throw IllegalArgumentException("widthX { got " + s(widthX) + " } <= 0");
+        if (length < widthX) throw IllegalArgumentException("length { got " + s(length) + " } < widthX { got " + s(widthX) + " }");
+        if (length % widthX != 0) throw IllegalArgumentException("lengthv { got " + s(length) + " } % widthX { got " + s(widthX) + " } != 0");
+        if (widthY <= 0) throw IllegalArgumentException("widthY { got " + s(widthY) + " } <= 0");
+        if (length < widthY) throw IllegalArgumentException("length { got " + s(length) + " } < widthY { got " + s(widthY) + " }");
+        if (length % widthY != 0) throw IllegalArgumentException("lengthv { got " + s(length) + " } % widthY { got " + s(widthY) + " } != 0");
+    }
+    return base_->transpose(Y, Ydim, X, Xdim, dimIndex1, dimIndex2, pad4(widthX), pad4(widthY), length);
+}
+SyncerPtr EngineCore::memcpy(int64_t dst, int64_t src, int length) {
+    if (check) {
+        if (dst == 0) throw NullPointerException("dst is null");
+        if (src == 0) throw NullPointerException("src is null");
+        if (length <= 0) throw IllegalArgumentException("length must be positive");
+    }
+    return base_->memcpy(dst, src, (int64_t)length << 2);
+}
 void EngineCore::func_param_check_row(int lengthv, int row_lengthv, int width, int stride) const {  // :1613-1622
     auto s = [](int v) { return std::to_string(v); };
     if (lengthv < row_lengthv)
@@ -1122,6 +1167,59 @@ Tensor* Engine::fullconnect_deltaW(Tensor* X, Tensor* deltaY) {   // deltaW = X^
     try { finish(deltaW, core_->matMulT1(deltaW->address, X->address, deltaY->address, XIW, YOW, GK)); }
     catch (...) { deleteTensor(deltaW); throw; }
     return deltaW;
+}
+
+// Engine.java:1797-1831.  The reference supports 2 to 4 dimensions (anything else falls through to
+// its 2-D native with the wrong shape); here more than 4 is refused.
+namespace {
+struct FreeAfter : Syncer {     // Syncer.dual(sc1, () -> core.free(old)): wait, then release the old memory
+    SyncerPtr first; EngineCore* core; int64_t size, address; bool done = false;
+    FreeAfter(SyncerPtr f, EngineCore* c, int64_t s, int64_t a) : first(std::move(f)), core(c), size(s), address(a) {}
+    ~FreeAfter() override { try { sync(); } catch (...) {} }
+    void sync() override {
+        if (done) return;
+        first->sync();
+        core->free(size, address);
+        done = true;
+    }
+};
+}  // namespace
+Tensor* Engine::copy(Tensor* X) {
+    require(X, "X");
+    Tensor* Y = &empty(X->dim)->c();
+    try { finish(Y, core_->memcpy(Y->address, X->address, X->length_4x)); }
+    catch (...) { deleteTensor(Y); throw; }
+    return Y;
+}
+Tensor* Engine::transpose(bool inplace, Tensor* X, int dimIdx1, int dimIdx2) {
+    require(X, "X");
+    const int nd = X->ndim();
+    if (dimIdx1 < 0) dimIdx1 += nd;
+    if (dimIdx2 < 0) dimIdx2 += nd;
+    if (dimIdx1 == dimIdx2) return inplace ? X : copy(X);
+    if (check_) {
+        must_greater_equal(nd, "X.ndim", 2);
+        if (nd > 4) throw IllegalArgumentException("X.ndim { got " + std::to_string(nd) + " } must <= 4");
+        if (dimIdx1 < 0 || dimIdx1 >= nd) throw IllegalArgumentException("dimIdx1 is out of range");
+        if (dimIdx2 < 0 || dimIdx2 >= nd) throw IllegalArgumentException("dimIdx2 is out of range");
+    }
+    X->c();
+    std::vector<int> Ydim = X->dim;
+    std::swap(Ydim[dimIdx1], Ydim[dimIdx2]);
+    Tensor* Y = &empty(Ydim)->c();
+    SyncerPtr sc1;
+    try {
+        sc1 = core_->transpose(Y->address, Ydim, X->address, X->dim, dimIdx1, dimIdx2, X->lastDim(),
+                               Y->lastDim(), X->length);
+    } catch (...) { deleteTensor(Y); throw; }
+    if (!inplace) { finish(Y, std::move(sc1)); return Y; }
+    // X takes over Y's shape and memory; the old memory goes back once the kernel has read it
+    const int64_t old_size = X->mem_size, old_addr = X->address;
+    X->dim = Y->dim; X->length = Y->length; X->lengthv = Y->lengthv; X->length_4x = Y->length_4x;
+    X->mem_size = Y->mem_size; X->address = Y->address;
+    delete Y;
+    finish(X, SyncerPtr(new FreeAfter(std::move(sc1), core_.get(), old_size, old_addr)));
+    return X;
 }
 
 // Engine.java:4185-4207, check_row :3781-3788

@@ -13,7 +13,7 @@
 //   PinnedMempool          z/dragon/engine/cuda/impl/PinnedMempool.java:96-200
 //   Tensor                 z/dragon/engine/Tensor.java:206-239 (length / lengthv / length_4x)
 //   Engine                 z/dragon/engine/Engine.java:522-551, 671-676, 824-837, 908-914, 955-1470,
-//                          4185-4207 (add_row / linear2_row)
+//                          4185-4207 (add_row / linear2_row), 1797-1831 (transpose)
 // (paths relative to source/alpha-Dragon-v1.2/src of the reference tree)
 #pragma once
 #include <stdint.h>
@@ -170,6 +170,9 @@ public:
     SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
     SyncerPtr linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                              float beta, float gamma, int lengthv, int width, int stride);
+    SyncerPtr transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X, const std::vector<int>& Xdim,
+                        int dimIndex1, int dimIndex2, int strideX, int strideY, int length);
+    SyncerPtr memcpy(int64_t dst, int64_t src, int64_t memsize);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int BK, int AK);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN, int AN, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int CM, int BM, int K);
@@ -212,6 +215,9 @@ public:
     SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
     SyncerPtr linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                              float beta, float gamma, int lengthv, int width);
+    SyncerPtr transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X, const std::vector<int>& Xdim,
+                        int dimIndex1, int dimIndex2, int widthX, int widthY, int length);
+    SyncerPtr memcpy(int64_t dst, int64_t src, int length);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
@@ -282,6 +288,11 @@ public:
     Tensor* fullconnect_biased(Tensor* Y, Tensor* X, Tensor* W, Tensor* Bias);
     Tensor* fullconnect_deltaX(Tensor* deltaY, Tensor* W);
     Tensor* fullconnect_deltaW(Tensor* X, Tensor* deltaY);
+
+    // exchange of two dimensions (negative indices count from the end); inplace gives X the new
+    // shape and memory and frees the old memory once the kernel is done
+    Tensor* transpose(bool inplace, Tensor* X, int dimIdx1, int dimIdx2);
+    Tensor* copy(Tensor* X);
 
     // Y = alpha*X1 + beta*X2 + gamma with the row vector X2 broadcast over the rows of X1
     Tensor* add_row(bool inplace, Tensor* X1, Tensor* X2) { return linear2_row(inplace, X1, X2, 1.0f, 1.0f, 0.0f); }

@@ -257,6 +257,16 @@ int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor*
         }
     });
 }
+dragon_tensor* dragon_engine_transpose(dragon_engine* eg, int32_t inplace, dragon_tensor* X,
+                                       int32_t dimIdx1, int32_t dimIdx2) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        t = eg->eg.transpose(inplace != 0, T(X), dimIdx1, dimIdx2);
+    });
+    if (!t) return nullptr;
+    return (X && t == X->ts) ? X : wrap(t);
+}
 dragon_tensor* dragon_engine_linear2_row(dragon_engine* eg, int32_t inplace, dragon_tensor* X1,
                                          dragon_tensor* X2, float alpha, float beta, float gamma) {
     Tensor* t = nullptr;

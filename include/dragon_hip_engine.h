@@ -103,6 +103,12 @@ dragon_tensor* dragon_engine_fullconnect(dragon_engine* eg, int32_t op, dragon_t
 int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor* Y,
                                    dragon_tensor* X, dragon_tensor* W, dragon_tensor* Bias);
 
+/* Engine.transpose(inplace, X, dimIdx1, dimIdx2) (Engine.java:1797-1831): exchange of two dimensions
+ * of a 2-D .. 4-D tensor, negative indices count from the end.  inplace != 0 gives X the new shape
+ * and memory and returns X itself; equal indices return X (inplace) or a copy. */
+dragon_tensor* dragon_engine_transpose(dragon_engine* eg, int32_t inplace, dragon_tensor* X,
+                                       int32_t dimIdx1, int32_t dimIdx2);
+
 /* linear2_row / add_row (Engine.java:4185-4207): Y = alpha*X1 + beta*X2 + gamma, the row vector
  * X2 broadcast over the rows of X1.  inplace != 0 writes into X1 and returns X1 itself. */
 dragon_tensor* dragon_engine_linear2_row(dragon_engine* eg, int32_t inplace, dragon_tensor* X1,

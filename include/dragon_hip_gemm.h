@@ -113,6 +113,28 @@ int dragon_Cuda_matMul_matMul_biased(const int64_t* streams, int32_t length,
                                      int32_t N, int32_t M, int32_t K,
                                      int32_t lengthv, int32_t width);
 
+/* ---- dimension swap (the layout step either side of the batched products) ---------
+ * Y = X with dimensions dimIndex1 and dimIndex2 exchanged.  Tensors are row-major with the last
+ * dimension stored at strideX / strideY floats (the width rounded up to 4, pad zero); `length` is
+ * the number of logical elements; Xdim0 = length / (the other X dims).  When the swap leaves the
+ * last dimension alone strideX == strideY and whole padded rows move; otherwise Y's pad columns
+ * are written as zeros.  X and Y must not overlap.  Issued on `stream`.
+ * Replace Java_z_dragon_engine_cuda_impl_Cuda_1expk2_transpose2D / 3D / 4D
+ * (engine-cuda-base/Cuda_expk2/Cuda_expk2/Cuda_transpose.cuh:13-75), called from
+ * CudaFloat32EngineBase.transpose (alpha-Dragon-v1.2/src/z/dragon/engine/cuda/CudaFloat32EngineBase.java:1343-1375). */
+int dragon_Cuda_expk2_transpose2D(int64_t stream, int64_t dX, int64_t dY,
+                                  int32_t Xdim1, int32_t Ydim1,
+                                  int32_t strideX, int32_t strideY, int32_t length);
+int dragon_Cuda_expk2_transpose3D(int64_t stream, int64_t dX, int64_t dY,
+                                  int32_t Xdim1, int32_t Xdim2, int32_t Ydim1, int32_t Ydim2,
+                                  int32_t dimIndex1, int32_t dimIndex2,
+                                  int32_t strideX, int32_t strideY, int32_t length);
+int dragon_Cuda_expk2_transpose4D(int64_t stream, int64_t dX, int64_t dY,
+                                  int32_t Xdim1, int32_t Xdim2, int32_t Xdim3,
+                                  int32_t Ydim1, int32_t Ydim2, int32_t Ydim3,
+                                  int32_t dimIndex1, int32_t dimIndex2,
+                                  int32_t strideX, int32_t strideY, int32_t length);
+
 /* ---- batched products (grid depth = Batch) --------------------------------------- */
 
 /* C[b][N,M] = A[b][N,AK] * B[b][BK,M], k < BK.  M and AK are multiples of 4, N and BK

@@ -419,6 +419,36 @@ void oracle_linear_dual2D_row(const float* X1, const float* X2, int row_lengthv,
 }
 
 /* ------------------------------------------------------------------------ */
+/* Dimension swap                                                            */
+/* ------------------------------------------------------------------------ */
+
+/* Y[x with entries i1 and i2 exchanged] = X[x] for every logical element, X taken as 4-D
+ * (leading dimensions 1 for fewer), the last dimension of X stored at strideX and of Y at
+ * strideY floats; Y is not touched outside its logical elements.  Index arithmetic of the
+ * reference's general kernel
+ * (engine-cuda-base/Cuda_expk2/Cuda_expk2/Cuda_transpose4D.cuh:91-120). */
+void oracle_transpose4D(const float* X, float* Y, const int* xdim, int i1, int i2, int strideX,
+                        int strideY) {
+    int ydim[4] = {xdim[0], xdim[1], xdim[2], xdim[3]};
+    ydim[i1] = xdim[i2]; ydim[i2] = xdim[i1];
+    const long long Xdim123 = (long long)xdim[1] * xdim[2] * xdim[3], Xdim23 = (long long)xdim[2] * xdim[3];
+    const long long length = Xdim123 * xdim[0];
+    for (long long index = 0; index < length; index++) {
+        int x[4];
+        long long res = index;
+        x[0] = (int)(res / Xdim123); res -= x[0] * Xdim123;
+        x[1] = (int)(res / Xdim23); res -= x[1] * Xdim23;
+        x[2] = (int)(res / xdim[3]);
+        x[3] = (int)(res - (long long)x[2] * xdim[3]);
+        int t = x[i1]; x[i1] = x[i2]; x[i2] = t;
+        long long yoffset = (((long long)x[0] * ydim[1] + x[1]) * ydim[2] + x[2]) * ydim[3] + x[3];
+        const long long xo = (index / xdim[3]) * strideX + (index % xdim[3]);
+        const long long yo = (yoffset / ydim[3]) * strideY + (yoffset % ydim[3]);
+        Y[yo] = X[xo];
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* Error metrics used by the parity tests                                    */
 /* ------------------------------------------------------------------------ */
 

@@ -48,6 +48,7 @@ for _name, _res, _args in [
     ("oracle_smooth_maxPart", c_int, [c_int]),
     ("oracle_gridZ", c_int, [c_int] * 6 + [c_float, c_float, c_int]),
     ("oracle_linear_dual2D_row", None, [_P, _P, c_int, c_float, c_float, c_float, _P, c_int, c_int, c_int]),
+    ("oracle_transpose4D", None, [_P, _P, POINTER(c_int), c_int, c_int, c_int, c_int]),
     ("oracle_samePercent_relative", c_float, [_P, _P, c_int, c_float]),
     ("oracle_num_threads", c_int, []),
 ]:
@@ -193,6 +194,26 @@ def linear_dual2D_row(X1, X2, alpha, beta, gamma, width):
     Y = np.empty_like(X1)
     _o.oracle_linear_dual2D_row(p1, p2, stride, alpha, beta, gamma, Y.ctypes.data_as(_P),
                                 rows * stride, width, stride)
+    return Y
+
+
+def transpose(Xp, dims, i1, i2):
+    """Xp: device-layout array [..., stride] of a tensor with logical dims `dims` (2 to 4 of them,
+    stride = last dim rounded up to 4).  Returns the device-layout array of the tensor with
+    dimensions i1 and i2 exchanged, pad zero."""
+    dims = list(dims)
+    nd = len(dims)
+    assert 2 <= nd <= 4
+    Xp, px = _f32(Xp)
+    d4 = [1] * (4 - nd) + dims
+    a, b = i1 + 4 - nd, i2 + 4 - nd
+    yd = list(dims)
+    yd[i1], yd[i2] = yd[i2], yd[i1]
+    sx, sy = (dims[-1] + 3) // 4 * 4, (yd[-1] + 3) // 4 * 4
+    assert Xp.size == int(np.prod(dims[:-1])) * sx
+    Y = np.zeros(yd[:-1] + [sy], np.float32)
+    arr = (c_int * 4)(*d4)
+    _o.oracle_transpose4D(px, Y.ctypes.data_as(_P), arr, a, b, sx, sy)
     return Y
 
 

@@ -332,6 +332,27 @@ def test_bias_row_general_coefficients_within_rounding_of_fp64():
     assert np.all(Y[:, width:] == 0)
 
 
+def _dev_layout(X):
+    s = (X.shape[-1] + 3) // 4 * 4
+    out = np.zeros(X.shape[:-1] + (s,), np.float32)
+    out[..., :X.shape[-1]] = X
+    return out
+
+
+@pytest.mark.parametrize("dims,i1,i2", [((5, 7), 0, 1), ((4, 8), 1, 0), ((2, 3, 5), 1, 2), ((2, 3, 5), 0, 2),
+                                        ((2, 3, 5), 0, 1), ((2, 3, 4, 6), 1, 2), ((2, 3, 4, 6), 0, 3),
+                                        ((2, 3, 4, 6), 2, 3), ((3, 1, 2, 9), 1, 3), ((1, 1), 0, 1)])
+def test_transpose_oracle_is_numpy_swapaxes_and_an_involution(dims, i1, i2):
+    X = RNG.standard_normal(dims).astype(np.float32)
+    Yp = oracle.transpose(_dev_layout(X), dims, i1, i2)
+    Y = np.swapaxes(X, i1, i2)
+    assert Yp.shape[:-1] == Y.shape[:-1] and Yp.shape[-1] == (Y.shape[-1] + 3) // 4 * 4
+    assert np.array_equal(Yp[..., :Y.shape[-1]], Y)        # every element where numpy puts it
+    assert not Yp[..., Y.shape[-1]:].any()                 # pad untouched (zero)
+    back = oracle.transpose(Yp, list(Y.shape), i1, i2)     # swapping twice restores the layout
+    assert np.array_equal(back, _dev_layout(X))
+
+
 def test_reference_micro_helpers_when_built():
     ref = oracle.load_ref()
     if ref is None:
