@@ -75,6 +75,7 @@ std::vector<int64_t> long_array(JNIEnv* env, jlongArray arr, jint length) {
 #define BMM(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1batchMatMul_##name
 #define RT(name) Java_z_dragon_engine_cuda_impl_Cuda_##name
 #define FN(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1function_##name
+#define EK(name) Java_z_dragon_engine_cuda_impl_Cuda_1expk2_##name
 
 extern "C" {
 
@@ -134,6 +135,25 @@ JNIEXPORT void JNICALL FN(linear_1dual2D_1row)(JNIEnv* env, jclass, jlong stream
                                                jint stride) {
     handle(env, dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta, gamma,
                                                        dY, lengthv, width, stride));
+}
+
+// ---- Cuda_expk2: dimension swap (reference: Cuda_expk2/Cuda_expk2/Cuda_transpose.cuh:13-75) ----
+JNIEXPORT void JNICALL EK(transpose2D)(JNIEnv* env, jclass, jlong stream, jlong dX, jlong dY, jint Xdim1,
+                                       jint Ydim1, jint strideX, jint strideY, jint length) {
+    handle(env, dragon_Cuda_expk2_transpose2D(stream, dX, dY, Xdim1, Ydim1, strideX, strideY, length));
+}
+JNIEXPORT void JNICALL EK(transpose3D)(JNIEnv* env, jclass, jlong stream, jlong dX, jlong dY, jint Xdim1,
+                                       jint Xdim2, jint Ydim1, jint Ydim2, jint dimIndex1, jint dimIndex2,
+                                       jint strideX, jint strideY, jint length) {
+    handle(env, dragon_Cuda_expk2_transpose3D(stream, dX, dY, Xdim1, Xdim2, Ydim1, Ydim2, dimIndex1,
+                                              dimIndex2, strideX, strideY, length));
+}
+JNIEXPORT void JNICALL EK(transpose4D)(JNIEnv* env, jclass, jlong stream, jlong dX, jlong dY, jint Xdim1,
+                                       jint Xdim2, jint Xdim3, jint Ydim1, jint Ydim2, jint Ydim3,
+                                       jint dimIndex1, jint dimIndex2, jint strideX, jint strideY,
+                                       jint length) {
+    handle(env, dragon_Cuda_expk2_transpose4D(stream, dX, dY, Xdim1, Xdim2, Xdim3, Ydim1, Ydim2, Ydim3,
+                                              dimIndex1, dimIndex2, strideX, strideY, length));
 }
 
 // ---- Cuda_batchMatMul -------------------------------------------------------------------------

@@ -67,7 +67,11 @@ __global__ __launch_bounds__(256) void transpose_last_kernel(const float* __rest
 
     // read: 16 lanes x 16 bytes along X's last dimension, 16 tile rows per pass.  Reading up to
     // the stride is safe and gives zeros beyond the width (the pad is zero).
-    const int lx = threadIdx.x & 15, ly = threadIdx.x >> 4;
+    // lane -> (16-byte column lx, row ly): each half-wave covers 8 columns x 4 rows, which with the
+    // row stride of 65 floats puts its 32 four-byte LDS accesses on 32 different banks, for the
+    // row-wise stores here and for the column-wise loads below alike
+    const int lx = (threadIdx.x & 7) | ((threadIdx.x >> 2) & 8);
+    const int ly = ((threadIdx.x >> 3) & 3) | ((threadIdx.x >> 4) & 12);
     x[3] = q0 + 4 * lx;
 #pragma unroll
     for (int i = 0; i < TP; i += 16) {

@@ -20,6 +20,7 @@ FILES = [
     "Cuda/Cuda/Cuda_Exception.cuh",
     "Cuda/Cuda/Cuda_float.cuh",
     "Cuda_function/Cuda_function/A.cu",
+    "Cuda_expk2/Cuda_expk2/Cuda_transpose.cuh",
 ]
 # of the element-wise library only the bias row belongs to the path
 ONLY = {"Cuda_function/Cuda_function/A.cu": {"Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear_1dual2D_1row"}}

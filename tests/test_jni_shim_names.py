@@ -12,13 +12,14 @@ GOLDEN = os.path.join(ROOT, "tests", "golden", "jni_symbols.txt")
 PREFIX = {"MM": "Java_z_dragon_engine_cuda_impl_math_Cuda_1matMul_",
           "BMM": "Java_z_dragon_engine_cuda_impl_math_Cuda_1batchMatMul_",
           "RT": "Java_z_dragon_engine_cuda_impl_Cuda_",
-          "FN": "Java_z_dragon_engine_cuda_impl_math_Cuda_1function_"}
+          "FN": "Java_z_dragon_engine_cuda_impl_math_Cuda_1function_",
+          "EK": "Java_z_dragon_engine_cuda_impl_Cuda_1expk2_"}
 
 
 def shim_names():
     text = open(SHIM).read()
     names = set()
-    for macro, arg in re.findall(r"JNICALL\s+(MM|BMM|RT|FN)\((\w+)\)\s*\(", text):
+    for macro, arg in re.findall(r"JNICALL\s+(MM|BMM|RT|FN|EK)\((\w+)\)\s*\(", text):
         names.add(PREFIX[macro] + arg)
     for kind, arg in re.findall(r"^DEF_(MM2D|MMSK|BMM|BMM_MMA)\((\w+),", text, flags=re.M):
         names.add(PREFIX["MM" if kind.startswith("MM") else "BMM"] + arg)
@@ -44,9 +45,16 @@ def test_bias_row_native_is_in_the_shim():
     assert rows <= s
 
 
+def test_dimension_swap_natives_are_in_the_shim():
+    g, s = golden(), shim_names()
+    swaps = {n for n, f in g.items() if "Cuda_transpose" in f}
+    assert swaps == {PREFIX["EK"] + n for n in ("transpose2D", "transpose3D", "transpose4D")}
+    assert swaps <= s
+
+
 def test_runtime_subset_names_exist_in_the_reference():
     g, s = golden(), shim_names()
-    runtime = {n for n in s if n.startswith(PREFIX["RT"])}
+    runtime = {n for n in s if n.startswith(PREFIX["RT"]) and not n.startswith(PREFIX["EK"])}
     assert len(runtime) >= 40
     unknown = sorted(n for n in runtime if n not in g)
     assert not unknown, "names the reference does not define: %s" % unknown
