@@ -279,13 +279,26 @@ class Cuda_matMul:
 
 
 class Cuda_function:
-    """The one native of Cuda_function.java the biased products use."""
+    """The natives of Cuda_function.java on the path: the bias row and the scalar linear map."""
+
+    @staticmethod
+    def linear2D(stream, alpha, dX, beta, dY, lengthv, width, stride):
+        _check(lib.dragon_Cuda_function_linear2D(stream, alpha, dX, beta, dY, lengthv, width, stride))
 
     @staticmethod
     def linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta, gamma, dY, lengthv, width,
                           stride):
         _check(lib.dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta,
                                                           gamma, dY, lengthv, width, stride))
+
+
+class Cuda_reduce:
+    """Row softmax in one launch (stands in for row_max + row_softmax + div2D_field)."""
+
+    @staticmethod
+    def softmax2D(stream, dX, dY, field_length, row_lengthv, width, stride, scale=1.0):
+        _check(lib.dragon_Cuda_reduce_softmax2D(stream, dX, dY, field_length, row_lengthv, width, stride,
+                                                scale))
 
 
 class Cuda_expk2:

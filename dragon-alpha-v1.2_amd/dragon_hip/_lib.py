@@ -32,6 +32,8 @@ SIGNATURES = {
     "dragon_Cuda_matMul_SKbuf_summary": (i32, [i64, i64, i64, i32, i32]),
     "dragon_Cuda_function_linear_dual2D_row": (i32, [i64, i64, i64, i32, f32, f32, f32, i64, i32, i32, i32]),
     "dragon_Cuda_matMul_matMul_biased": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32]),
+    "dragon_Cuda_function_linear2D": (i32, [i64, f32, i64, f32, i64, i32, i32, i32]),
+    "dragon_Cuda_reduce_softmax2D": (i32, [i64, i64, i64, i32, i32, i32, i32, f32]),
     "dragon_Cuda_expk2_transpose2D": (i32, [i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_expk2_transpose3D": (i32, [i64, i64, i64] + [i32] * 9),
     "dragon_Cuda_expk2_transpose4D": (i32, [i64, i64, i64] + [i32] * 11),
@@ -128,6 +130,8 @@ SIGNATURES = {
     "dragon_engine_product_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
     "dragon_engine_fullconnect": (c_void_p, [c_void_p, i32, c_void_p, c_void_p, c_void_p]),
     "dragon_engine_fullconnect_into": (i32, [c_void_p, i32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "dragon_engine_linear": (c_void_p, [c_void_p, i32, f32, c_void_p, f32]),
+    "dragon_engine_softmax": (c_void_p, [c_void_p, i32, c_void_p, i32, f32]),
     "dragon_engine_transpose": (c_void_p, [c_void_p, i32, c_void_p, i32, i32]),
     "dragon_engine_linear2_row": (c_void_p, [c_void_p, i32, c_void_p, c_void_p, f32, f32, f32]),
 }

@@ -207,6 +207,17 @@ class Engine:
             return X1
         return self._wrap(h)
 
+    def linear(self, inplace, alpha, X, beta):
+        h = lib.dragon_engine_linear(self._h, int(inplace), alpha, X._h if X else None, beta)
+        return X if (inplace and h) else self._wrap(h)
+
+    def sdiv(self, inplace, X, C):
+        return self.linear(inplace, 1.0 / C, X, 0.0)
+
+    def softmax(self, inplace, X, features=-1, scale=1.0):
+        h = lib.dragon_engine_softmax(self._h, int(inplace), X._h if X else None, features, scale)
+        return X if (inplace and h) else self._wrap(h)
+
     def transpose(self, inplace, X, dimIdx1, dimIdx2):
         h = lib.dragon_engine_transpose(self._h, int(inplace), X._h if X else None, dimIdx1, dimIdx2)
         if h and X is not None and h == X._h:

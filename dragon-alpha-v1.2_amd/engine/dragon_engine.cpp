@@ -530,6 +530,20 @@ SyncerPtr CudaFloat32EngineBase::transpose(int64_t Y, const std::vector<int>& Yd
         cu(dragon_Cuda_expk2_transpose2D(stream, X, Y, Xdim[1], Ydim[1], strideX, strideY, length));
     return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
 }
+SyncerPtr CudaFloat32EngineBase::linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv,
+                                          int width, int stride) {
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_function_linear2D(stream, alpha, X, beta, Y, lengthv, width, stride));
+    return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
+}
+// :5738-5774 issues row_max, row_softmax and div2D_field with two temporary blocks; one launch here
+SyncerPtr CudaFloat32EngineBase::softmax2D(int64_t Y, int64_t X, int field_length, int row_lengthv,
+                                           int lengthv, int width, int stride, float scale) {
+    (void)lengthv;
+    int64_t stream = streamPool_->getStream();
+    cu(dragon_Cuda_reduce_softmax2D(stream, X, Y, field_length, row_lengthv, width, stride, scale));
+    return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
+}
 SyncerPtr CudaFloat32EngineBase::memcpy(int64_t dst, int64_t src, int64_t memsize) {   // :1173-1179
     int64_t stream = streamPool_->getStream();
     cu(dragon_Cuda_memcpyAsyncDeviceToDevice(stream, dst, src, memsize));
@@ -669,6 +683,36 @@ SyncerPtr EngineCore::transpose(int64_t Y, const std::vector<int>& Ydim, int64_t
         if (length % widthY != 0) throw IllegalArgumentException("lengthv { got " + s(length) + " } % widthY { got " + s(widthY) + " } != 0");
     }
     return base_->transpose(Y, Ydim, X, Xdim, dimIndex1, dimIndex2, pad4(widthX), pad4(widthY), length);
+}
+SyncerPtr EngineCore::linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv, int width) {
+    const int stride = pad4(width);
+    if (check) {
+        if (Y == 0) throw NullPointerException("Tensor Y is null");
+        if (X == 0) throw NullPointerException("Tensor X is null");
+        auto s = [](int v) { return std::to_string(v); };
+        if (lengthv < width) throw IllegalArgumentException("lengthv { got " + s(lengthv) + " } < width { got " + s(width) + " }");
+        if (width <= 0) throw IllegalArgumentException("width { got " + s(width) + " } <= 0");
+        if (lengthv % stride != 0) throw IllegalArgumentException("lengthv { got " + s(lengthv) + " } % stride { got " + s(stride) + " } != 0");
+    }
+    return base_->linear2D(Y, alpha, X, beta, lengthv, width, stride);
+}
+SyncerPtr EngineCore::softmax2D(int64_t Y, int64_t X, int row_length, int lengthv, int width, float scale) {  // :3368-3384
+    const int stride = pad4(width);
+    if (check) {
+        if (X == 0) throw NullPointerException("Tensor X is NULL");
+        if (Y == 0) throw NullPointerException("Tensor Y is NULL");
+        auto s = [](int v) { return std::to_string(v); };
+        if (width <= 0) throw IllegalArgumentException("width { got " + s(width) + " } <= 0");   // :1646-1657
+        if (lengthv < row_length) throw IllegalArgumentException("lengthv { got " + s(lengthv) + " } < row_length { got " + s(row_length) + " }");
+        if (row_length < width) throw IllegalArgumentException("row_length { got " + s(row_length) + " } < width { got " + s(width) + " }");
+        if (row_length % width != 0) throw IllegalArgumentException("row_length { got " + s(row_length) + " } % width { got " + s(width) + " } != 0");
+    }
+    const int row_lengthv = row_length / width * stride;
+    if (check && lengthv % row_lengthv != 0)
+        throw IllegalArgumentException("lengthv { got " + std::to_string(lengthv) + " } % row_lengthv { got " +
+                                       std::to_string(row_lengthv) + " } != 0");
+    const int field_length = lengthv / row_lengthv;
+    return base_->softmax2D(Y, X, field_length, row_lengthv, lengthv, width, stride, scale);
 }
 SyncerPtr EngineCore::memcpy(int64_t dst, int64_t src, int length) {
     if (check) {
@@ -1220,6 +1264,30 @@ Tensor* Engine::transpose(bool inplace, Tensor* X, int dimIdx1, int dimIdx2) {
     delete Y;
     finish(X, SyncerPtr(new FreeAfter(std::move(sc1), core_.get(), old_size, old_addr)));
     return X;
+}
+
+// Engine.java:4002-4013
+Tensor* Engine::linear(bool inplace, float alpha, Tensor* X, float beta) {
+    require(X, "X");
+    Tensor* Y = inplace ? X : &empty(X->dim)->c();
+    try { finish(Y, core_->linear2D(Y->address, alpha, X->address, beta, X->lengthv, X->lastDim())); }
+    catch (...) { if (!inplace) deleteTensor(Y); throw; }
+    return Y;
+}
+// Engine.java:6082-6100
+Tensor* Engine::softmax_scaled(bool inplace, Tensor* X, float scale, int features) {
+    require(X, "X");
+    if (features == -1) features = X->lastDim();
+    if (check_) {
+        must_greater_equal(X->ndim(), "X.ndim", 2);
+        if (features <= 0 || X->length % features != 0)
+            throw IllegalArgumentException("X.length { got " + std::to_string(X->length) + " } % features { got " +
+                                           std::to_string(features) + " } != 0");
+    }
+    Tensor* Y = inplace ? X : &empty(X->dim)->c();
+    try { finish(Y, core_->softmax2D(Y->address, X->address, features, X->lengthv, X->lastDim(), scale)); }
+    catch (...) { if (!inplace) deleteTensor(Y); throw; }
+    return Y;
 }
 
 // Engine.java:4185-4207, check_row :3781-3788

@@ -13,7 +13,7 @@
 //   PinnedMempool          z/dragon/engine/cuda/impl/PinnedMempool.java:96-200
 //   Tensor                 z/dragon/engine/Tensor.java:206-239 (length / lengthv / length_4x)
 //   Engine                 z/dragon/engine/Engine.java:522-551, 671-676, 824-837, 908-914, 955-1470,
-//                          4185-4207 (add_row / linear2_row), 1797-1831 (transpose)
+//                          4185-4207 (add_row / linear2_row), 1797-1831 (transpose), 4002-4013 (linear / sdiv), 6082-6100 (softmax)
 // (paths relative to source/alpha-Dragon-v1.2/src of the reference tree)
 #pragma once
 #include <stdint.h>
@@ -172,6 +172,10 @@ public:
                              float beta, float gamma, int lengthv, int width, int stride);
     SyncerPtr transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X, const std::vector<int>& Xdim,
                         int dimIndex1, int dimIndex2, int strideX, int strideY, int length);
+    SyncerPtr linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv, int width, int stride);
+    // scale is not an argument of the Java method: 1 reproduces it, another value folds a preceding sdiv
+    SyncerPtr softmax2D(int64_t Y, int64_t X, int field_length, int row_lengthv, int lengthv, int width,
+                        int stride, float scale = 1.0f);
     SyncerPtr memcpy(int64_t dst, int64_t src, int64_t memsize);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int BK, int AK);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN, int AN, int M, int K);
@@ -217,6 +221,8 @@ public:
                              float beta, float gamma, int lengthv, int width);
     SyncerPtr transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X, const std::vector<int>& Xdim,
                         int dimIndex1, int dimIndex2, int widthX, int widthY, int length);
+    SyncerPtr linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv, int width);
+    SyncerPtr softmax2D(int64_t Y, int64_t X, int row_length, int lengthv, int width, float scale = 1.0f);
     SyncerPtr memcpy(int64_t dst, int64_t src, int length);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
@@ -293,6 +299,15 @@ public:
     // shape and memory and frees the old memory once the kernel is done
     Tensor* transpose(bool inplace, Tensor* X, int dimIdx1, int dimIdx2);
     Tensor* copy(Tensor* X);
+
+    // Y = alpha*X + beta; sdiv(X, C) = X / C = linear(1/C, X, 0)
+    Tensor* linear(bool inplace, float alpha, Tensor* X, float beta);
+    Tensor* sdiv(bool inplace, Tensor* X, float C) { return linear(inplace, 1.0f / C, X, 0.0f); }
+    // softmax over groups of `features` elements (-1: the last dimension).  softmax_scaled is
+    // softmax(scale * X) in the same launch: softmax(sdiv(X, C)) without the extra pass (not in the
+    // Java class).
+    Tensor* softmax(bool inplace, Tensor* X, int features = -1) { return softmax_scaled(inplace, X, 1.0f, features); }
+    Tensor* softmax_scaled(bool inplace, Tensor* X, float scale, int features = -1);
 
     // Y = alpha*X1 + beta*X2 + gamma with the row vector X2 broadcast over the rows of X1
     Tensor* add_row(bool inplace, Tensor* X1, Tensor* X2) { return linear2_row(inplace, X1, X2, 1.0f, 1.0f, 0.0f); }

@@ -257,6 +257,26 @@ int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor*
         }
     });
 }
+dragon_tensor* dragon_engine_linear(dragon_engine* eg, int32_t inplace, float alpha, dragon_tensor* X,
+                                    float beta) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        t = eg->eg.linear(inplace != 0, alpha, T(X), beta);
+    });
+    if (!t) return nullptr;
+    return inplace ? X : wrap(t);
+}
+dragon_tensor* dragon_engine_softmax(dragon_engine* eg, int32_t inplace, dragon_tensor* X, int32_t features,
+                                     float scale) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        t = eg->eg.softmax_scaled(inplace != 0, T(X), scale, features);
+    });
+    if (!t) return nullptr;
+    return inplace ? X : wrap(t);
+}
 dragon_tensor* dragon_engine_transpose(dragon_engine* eg, int32_t inplace, dragon_tensor* X,
                                        int32_t dimIdx1, int32_t dimIdx2) {
     Tensor* t = nullptr;

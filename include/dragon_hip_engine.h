@@ -103,6 +103,16 @@ dragon_tensor* dragon_engine_fullconnect(dragon_engine* eg, int32_t op, dragon_t
 int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor* Y,
                                    dragon_tensor* X, dragon_tensor* W, dragon_tensor* Bias);
 
+/* Engine.linear(inplace, alpha, X, beta): Y = alpha*X + beta (Engine.java:4005-4013); Engine.sdiv(X, C)
+ * is linear(1/C, X, 0).  inplace != 0 writes into X and returns X itself. */
+dragon_tensor* dragon_engine_linear(dragon_engine* eg, int32_t inplace, float alpha, dragon_tensor* X,
+                                    float beta);
+/* Engine.softmax(inplace, X, features) (Engine.java:6082-6100): softmax over groups of `features`
+ * elements, -1 = the last dimension.  scale = 1 is the Java method; another value computes
+ * softmax(scale * X) in the same launch. */
+dragon_tensor* dragon_engine_softmax(dragon_engine* eg, int32_t inplace, dragon_tensor* X, int32_t features,
+                                     float scale);
+
 /* Engine.transpose(inplace, X, dimIdx1, dimIdx2) (Engine.java:1797-1831): exchange of two dimensions
  * of a 2-D .. 4-D tensor, negative indices count from the end.  inplace != 0 gives X the new shape
  * and memory and returns X itself; equal indices return X (inplace) or a copy. */

@@ -135,6 +135,26 @@ int dragon_Cuda_expk2_transpose4D(int64_t stream, int64_t dX, int64_t dY,
                                   int32_t dimIndex1, int32_t dimIndex2,
                                   int32_t strideX, int32_t strideY, int32_t length);
 
+/* ---- between the two batched products of an attention block ------------------------ */
+
+/* Y[i] = alpha*X[i] + beta for i < lengthv, elements whose column (i % stride) is >= width
+ * multiplied by zero.  Y may alias X.  Engine.linear / Engine.sdiv (X / C = linear(1/C, X, 0)).
+ * Replaces Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear2D
+ * (engine-cuda-base/Cuda_function/Cuda_function/A.cu:170-183). */
+int dragon_Cuda_function_linear2D(int64_t stream, float alpha, int64_t dX, float beta, int64_t dY,
+                                  int32_t lengthv, int32_t width, int32_t stride);
+
+/* Y = softmax(scale * X) over each of the field_length fields of row_lengthv floats (a multiple
+ * of stride; only columns < width of every memory row take part, the pad of Y gets zeros):
+ * y = exp(s*x - max) / sum(exp(s*x - max)).  Y may alias X.  One launch; scale = 1 gives
+ * Engine.softmax, scale = 1/C folds the sdiv that precedes it in an attention block.
+ * No native of this shape in the reference, which runs Cuda_reduce.row_max, Cuda_reduce.row_softmax
+ * and Cuda_function.div2D_field with two temporary buffers
+ * (alpha-Dragon-v1.2/src/z/dragon/engine/cuda/CudaFloat32EngineBase.java:5738-5774); a host that owns
+ * that method calls this instead. */
+int dragon_Cuda_reduce_softmax2D(int64_t stream, int64_t dX, int64_t dY, int32_t field_length,
+                                 int32_t row_lengthv, int32_t width, int32_t stride, float scale);
+
 /* ---- batched products (grid depth = Batch) --------------------------------------- */
 
 /* C[b][N,M] = A[b][N,AK] * B[b][BK,M], k < BK.  M and AK are multiples of 4, N and BK

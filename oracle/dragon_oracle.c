@@ -419,6 +419,45 @@ void oracle_linear_dual2D_row(const float* X1, const float* X2, int row_lengthv,
 }
 
 /* ------------------------------------------------------------------------ */
+/* Scalar linear map and row softmax                                         */
+/* ------------------------------------------------------------------------ */
+
+/* Y[i] = alpha*X[i] + beta, pad columns (i % stride >= width) multiplied by zero
+ * (engine-cuda-base/Cuda_function/Cuda_function/type1_linear2D.cuh, within_width: micro.cuh:61-65);
+ * product and sum rounded separately. */
+void oracle_linear2D(float alpha, const float* X, float beta, float* Y, int lengthv, int width, int stride) {
+    for (int i = 0; i < lengthv; i++) {
+        float p = alpha * X[i];
+        float y = p + beta;
+        y *= ((i % stride) < width) ? 1.0f : 0.0f;
+        Y[i] = y;
+    }
+}
+
+/* Softmax of scale*X over each field of row_lengthv floats, logical elements only
+ * (column < width of every memory row), pad of Y zero: the result of the reference's sequence
+ * M = row_max(X); E = exp(X - M), V = row_sum(E); Y = E / V
+ * (alpha-Dragon-v1.2/src/z/dragon/engine/cuda/CudaFloat32EngineBase.java:5753-5771), every step in
+ * float, the sum taken left to right.  scale = 1 is Engine.softmax; another value is the sdiv
+ * (Engine.java:4002) applied first. */
+void oracle_softmax2D(const float* X, float* Y, int field_length, int row_lengthv, int width, int stride,
+                      float scale) {
+    for (int f = 0; f < field_length; f++) {
+        const float* x = X + (size_t)f * row_lengthv;
+        float* y = Y + (size_t)f * row_lengthv;
+        float m = -3.0e38f;
+        for (int i = 0; i < row_lengthv; i++)
+            if ((i % stride) < width) { float t = x[i] * scale; if (t > m) m = t; }
+        float sum = 0.0f;
+        for (int i = 0; i < row_lengthv; i++) {
+            if ((i % stride) < width) { float t = x[i] * scale; y[i] = expf(t - m); sum += y[i]; }
+            else y[i] = 0.0f;
+        }
+        for (int i = 0; i < row_lengthv; i++) y[i] = y[i] / sum;
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* Dimension swap                                                            */
 /* ------------------------------------------------------------------------ */
 

@@ -48,6 +48,8 @@ for _name, _res, _args in [
     ("oracle_smooth_maxPart", c_int, [c_int]),
     ("oracle_gridZ", c_int, [c_int] * 6 + [c_float, c_float, c_int]),
     ("oracle_linear_dual2D_row", None, [_P, _P, c_int, c_float, c_float, c_float, _P, c_int, c_int, c_int]),
+    ("oracle_linear2D", None, [c_float, _P, c_float, _P, c_int, c_int, c_int]),
+    ("oracle_softmax2D", None, [_P, _P, c_int, c_int, c_int, c_int, c_float]),
     ("oracle_transpose4D", None, [_P, _P, POINTER(c_int), c_int, c_int, c_int, c_int]),
     ("oracle_samePercent_relative", c_float, [_P, _P, c_int, c_float]),
     ("oracle_num_threads", c_int, []),
@@ -194,6 +196,28 @@ def linear_dual2D_row(X1, X2, alpha, beta, gamma, width):
     Y = np.empty_like(X1)
     _o.oracle_linear_dual2D_row(p1, p2, stride, alpha, beta, gamma, Y.ctypes.data_as(_P),
                                 rows * stride, width, stride)
+    return Y
+
+
+def linear2D(alpha, Xp, beta, width):
+    """Xp: device-layout [rows, stride].  alpha*X + beta with the pad columns times zero."""
+    Xp, px = _f32(Xp)
+    stride = Xp.shape[-1]
+    Y = np.empty_like(Xp)
+    _o.oracle_linear2D(alpha, px, beta, Y.ctypes.data_as(_P), Xp.size, width, stride)
+    return Y
+
+
+def softmax2D(Xp, width, features=None, scale=1.0):
+    """Xp: device-layout [rows, stride]; softmax of scale*X over groups of `features` logical
+    elements (a multiple of width; default one memory row).  Pad of the result is zero."""
+    Xp, px = _f32(Xp)
+    rows, stride = Xp.shape
+    features = width if features is None else features
+    assert features % width == 0 and rows % (features // width) == 0
+    row_lengthv = features // width * stride
+    Y = np.empty_like(Xp)
+    _o.oracle_softmax2D(px, Y.ctypes.data_as(_P), Xp.size // row_lengthv, row_lengthv, width, stride, scale)
     return Y
 
 
