@@ -43,7 +43,8 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-constexpr float NEG_BIG = -3.0e38f;
+// what pad elements and idle lanes hold: below every input, and exp(NEG_BIG - max) is an exact 0
+#define NEG_BIG (-__builtin_inff())
 
 // One wavefront per field; the field (at most 256*NV floats) stays in registers between the
 // three steps max -> exp and sum -> divide.  Four fields per workgroup.
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const float* __restri
     for (int s = 0; s < NV; s++) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            // pad elements hold NEG_BIG: exp gives an exact 0, which is also what the pad of Y gets
+            // pad elements hold -inf: exp gives an exact 0, which is also what the pad of Y gets
             v[s][j] = expf(v[s][j] - m);
             sum += v[s][j];
         }

@@ -445,7 +445,7 @@ void oracle_softmax2D(const float* X, float* Y, int field_length, int row_length
     for (int f = 0; f < field_length; f++) {
         const float* x = X + (size_t)f * row_lengthv;
         float* y = Y + (size_t)f * row_lengthv;
-        float m = -3.0e38f;
+        float m = -INFINITY;
         for (int i = 0; i < row_lengthv; i++)
             if ((i % stride) < width) { float t = x[i] * scale; if (t > m) m = t; }
         float sum = 0.0f;

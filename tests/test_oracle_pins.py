@@ -353,6 +353,44 @@ def test_transpose_oracle_is_numpy_swapaxes_and_an_involution(dims, i1, i2):
     assert np.array_equal(back, _dev_layout(X))
 
 
+def test_softmax_oracle_against_fp64_and_its_invariants():
+    rows, width, stride = 40, 37, 40
+    X = np.zeros((rows, stride), np.float32)
+    X[:, :width] = RNG.standard_normal((rows, width)).astype(np.float32) * 3
+    X[:, width:] = 50.0                                 # garbage in the pad must not take part
+    Y = oracle.softmax2D(X, width)
+    e = np.exp(X[:, :width].astype(np.float64) - X[:, :width].astype(np.float64).max(1, keepdims=True))
+    R = e / e.sum(1, keepdims=True)
+    # x - max rounded to float (an absolute error of up to 2^-25 |x - max| in the exponent), exp within an
+    # ulp, a float sum of 37 terms, one division
+    dist = np.abs(X[:, :width].astype(np.float64) - X[:, :width].astype(np.float64).max(1, keepdims=True))
+    assert np.all(np.abs(Y[:, :width] - R) <= 2.0 ** -24 * (dist + 8) * R + 1e-38)
+    assert not Y[:, width:].any()
+    assert np.allclose(Y.sum(1), 1.0, atol=3e-7)
+    # equal inputs over a power-of-two count give exactly 1/n; one element gives exactly 1
+    U = np.full((3, 8), 2.5, np.float32)
+    assert np.array_equal(oracle.softmax2D(U, 8), np.full((3, 8), 0.125, np.float32))
+    one = np.zeros((5, 4), np.float32); one[:, 0] = RNG.standard_normal(5)
+    assert np.array_equal(oracle.softmax2D(one, 1)[:, 0], np.ones(5, np.float32))
+    # a dominant element: exp underflows to an exact zero next to an exact one
+    D = np.zeros((1, 4), np.float32); D[0, :3] = [0.0, 200.0, -5.0]
+    assert np.array_equal(oracle.softmax2D(D, 3)[0, :3], np.array([0.0, 1.0, 0.0], np.float32))
+    # features spanning two memory rows: softmax over both rows' logical elements together
+    Y2 = oracle.softmax2D(X, width, features=2 * width)
+    e2 = np.exp(X[:, :width].astype(np.float64).reshape(rows // 2, 2 * width))
+    R2 = (e2 / e2.sum(1, keepdims=True)).reshape(rows, width)
+    assert np.all(np.abs(Y2[:, :width] - R2) <= 1e-6 * R2 + 1e-38)
+    # the scale is the same as scaling the input first (power of two: exact)
+    assert np.array_equal(oracle.softmax2D(X, width, scale=0.5), oracle.softmax2D(X * np.float32(0.5), width))
+
+
+def test_linear2D_oracle():
+    X = np.zeros((6, 8), np.float32); X[:, :7] = RNG.integers(-9, 9, (6, 7))
+    X[:, 7] = 3.0
+    Y = oracle.linear2D(2.0, X, -1.0, 7)
+    assert np.array_equal(Y[:, :7], 2 * X[:, :7] - 1) and not Y[:, 7].any()
+
+
 def test_reference_micro_helpers_when_built():
     ref = oracle.load_ref()
     if ref is None:
