@@ -83,9 +83,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias,transpose,transfer",
-                    help="which of the other workloads to time (default 3,4,5,bias,transpose,transfer): "
-                         "BASELINE configs 3, 4, 5, the biased fully-connected layer, dimension swaps, "
+    ap.add_argument("--configs", default="3,4,5,bias,attention,transpose,transfer",
+                    help="which of the other workloads to time (default 3,4,5,bias,attention,transpose,"
+                         "transfer): BASELINE configs 3, 4, 5, the biased fully-connected layer, the "
+                         "attention chain, dimension swaps, "
                          "tensor upload / download")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
@@ -331,6 +332,54 @@ def main():
             "ms": round(ms, 4), "alg_GBps": round(8.0 * Nb * Mb / (ms * 1e-3) / 1e9, 1),
             "pct_hbm_peak": round(100 * 8.0 * Nb * Mb / (ms * 1e-3) / 8e12, 1)}
         for x in (dX, dW, db, dY):
+            x.free()
+
+    if "attention" in extra:
+        # the chain between the inputs and the output of an attention block at the config-4 shape
+        # (batch 64 = 4 x 16 heads, 1024 tokens, 64 per head): P = softmax(Q.K^T / 8), Y = P.V
+        log("attention chain ...")
+        Bt, Sq, D = 64, 1024, 64
+        g = synthetic.stream_for(4)
+        dQ = dh.DeviceArray(g.normal((Bt, Sq, D), 0.0, 1.0))
+        dK = dh.DeviceArray(g.normal((Bt, Sq, D), 0.0, 1.0))
+        dV = dh.DeviceArray(g.normal((Bt, Sq, D), 0.0, 1.0))
+        dP = dh.DeviceArray(size=Bt * Sq * Sq)
+        dO = dh.DeviceArray(size=Bt * Sq * D)
+        RD, FN = dh.Cuda_reduce, dh.Cuda_function
+        nP = Bt * Sq * Sq
+
+        def qk():
+            BMM.batchMatMulT2_texture(S, 1, dQ.address, dK.address, dP.address, Bt, Sq, Sq, Sq, D)
+
+        def pv():
+            BMM.batchMatMul_texture(S, 1, dP.address, dV.address, dO.address, Bt, Sq, D, Sq, Sq)
+
+        def chain_fused_scale():
+            qk()
+            RD.softmax2D(stream, dP.address, dP.address, Bt * Sq, Sq, Sq, Sq, 0.125)
+            pv()
+
+        def chain_with_sdiv():
+            qk()
+            FN.linear2D(stream, 0.125, dP.address, 0.0, dP.address, nP, Sq, Sq)
+            RD.softmax2D(stream, dP.address, dP.address, Bt * Sq, Sq, Sq, Sq, 1.0)
+            pv()
+        ms = timer.per_launch_ms(lambda: RD.softmax2D(stream, dP.address, dP.address, Bt * Sq, Sq, Sq, Sq,
+                                                      0.125), iters=30)
+        per_config["softmax2D 65536 rows of 1024, in place (HBM-bound, 512 MiB)"] = {
+            "ms": round(ms, 4), "alg_GBps": round(8.0 * nP / (ms * 1e-3) / 1e9, 1),
+            "pct_hbm_peak": round(100 * 8.0 * nP / (ms * 1e-3) / 8e12, 1)}
+        ms = timer.per_launch_ms(lambda: FN.linear2D(stream, 0.125, dP.address, 0.0, dP.address, nP, Sq, Sq),
+                                 iters=30)
+        per_config["linear2D (sdiv) 64 Mi floats in place (HBM-bound, 512 MiB)"] = {
+            "ms": round(ms, 4), "alg_GBps": round(8.0 * nP / (ms * 1e-3) / 1e9, 1),
+            "pct_hbm_peak": round(100 * 8.0 * nP / (ms * 1e-3) / 8e12, 1)}
+        fl_chain = 2 * 2.0 * Bt * Sq * Sq * D
+        ms = timer.per_launch_ms(chain_fused_scale, iters=20)
+        record("attention chain Q.K^T -> softmax(x/8) -> P.V, batch 64 x 1024 x 64 (3 launches)", fl_chain, ms)
+        ms = timer.per_launch_ms(chain_with_sdiv, iters=20)
+        record("attention chain with a separate sdiv launch (4 launches)", fl_chain, ms)
+        for x in (dQ, dK, dV, dP, dO):
             x.free()
 
     if "transpose" in extra:
