@@ -270,9 +270,13 @@ __device__ __forceinline__ void read_frag_kouter(float (&frag)[T][4], const floa
 // rows); "+ 0.0f" is the gamma term of the separate bias launch this replaces: it turns a -0 sum
 // into +0, so fused and unfused results share every bit.  A template parameter rather than a
 // run-time test, so the plain products carry none of it.
+// The stores go through a buffer descriptor whose base is the tile's origin: a lane outside C gets
+// an out-of-range offset and the hardware drops its store, so the whole epilogue is straight-line
+// code -- no branch per store and 32-bit offset arithmetic only.
 template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS>
 __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
                                            int col0, float* c_ptr, int wm, int wn, int r, int h) {
+    constexpr int NT_STORE = 2;   // cache policy bit "nt": C is written once and not read back here
     float bias_v[TN];
     if constexpr (BIAS) {
 #pragma unroll
@@ -281,40 +285,52 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
             bias_v[j] = col < p.bias_width ? p.bias[col] : 0.0f;
         }
     }
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(c_ptr + (size_t)row0 * p.ldc + col0), 0, RSRC_RECORDS, RSRC_FLAGS);
+    const int ldc4 = p.ldc * 4;
+    // A store's address = tile origin (descriptor) + lane part (vector offset: the lane's first row
+    // and its column) + row part (scalar offset: a compile-time row count times the row pitch).
+    // Only the lane part is range-checked by the hardware, so "outside C" is expressed there.
+    const int lane_row = wm * TM * 32 + (A_KIN ? 4 * h : TM * 4 * h);
+    const int rows_left = p.rows - row0, cols_left = p.cols - col0;
+    constexpr int NCOL = B_KIN ? TN : 1;
+    int lane_off[NCOL];
+#pragma unroll
+    for (int j = 0; j < NCOL; j++) {
+        const int lcol = wn * TN * 32 + (B_KIN ? (j * 32 + r) : (TN * r));
+        lane_off[j] = (lcol < cols_left) ? lane_row * ldc4 + lcol * 4 : OOB_OFFSET;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-            const int mrow = 8 * (e / 4) + 4 * h + (e % 4);
-            const int row = row0 + wm * TM * 32 + (A_KIN ? (i * 32 + mrow) : (TM * mrow + i));
-            if (row < p.rows) {
-                float* crow = c_ptr + (size_t)row * p.ldc;
-                float out[TN];
+            const int crow = A_KIN ? (i * 32 + 8 * (e / 4) + (e % 4)) : (TM * (8 * (e / 4) + (e % 4)) + i);
+            const bool row_ok = lane_row < rows_left - crow;
+            const int row_soff = crow * ldc4;
+            float out[TN];
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    out[j] = acc[i][j][e];
-                    if constexpr (BIAS)
-                        if (row < p.bias_rows) out[j] = (out[j] + bias_v[j]) + 0.0f;
-                }
-                if constexpr (B_KIN) {
+            for (int j = 0; j < TN; j++) {
+                out[j] = acc[i][j][e];
+                if constexpr (BIAS)
+                    if (row0 + lane_row + crow < p.bias_rows) out[j] = (out[j] + bias_v[j]) + 0.0f;
+            }
+            if constexpr (B_KIN) {
 #pragma unroll
-                    for (int j = 0; j < TN; j++) {
-                        const int col = col0 + wn * TN * 32 + j * 32 + r;
-                        if (col < p.cols) __builtin_nontemporal_store(out[j], crow + col);
-                    }
+                for (int j = 0; j < TN; j++)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[j]), rsrc,
+                                                          row_ok ? lane_off[j] : OOB_OFFSET, row_soff, NT_STORE);
+            } else {
+                const int off = row_ok ? lane_off[0] : OOB_OFFSET;
+                if constexpr (TN == 1) {
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[0]), rsrc, off, row_soff,
+                                                          NT_STORE);
+                } else if constexpr (TN == 2) {
+                    typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+                    const v2f v = {out[0], out[1]};
+                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rsrc, off, row_soff, NT_STORE);
                 } else {
-                    const int col = col0 + wn * TN * 32 + TN * r;
-                    if (col < p.cols) {
-                        if constexpr (TN == 1) {
-                            __builtin_nontemporal_store(out[0], crow + col);
-                        } else if constexpr (TN == 2) {
-                            v2f v = {out[0], out[1]};
-                            __builtin_nontemporal_store(v, (v2f*)(crow + col));
-                        } else {
-                            v4f v = {out[0], out[1], out[2], out[3]};
-                            __builtin_nontemporal_store(v, (v4f*)(crow + col));
-                        }
-                    }
+                    const v4f v = {out[0], out[1], out[2], out[3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc, off, row_soff, NT_STORE);
                 }
             }
         }
