@@ -1,0 +1,163 @@
+// C ABI of the forward convolution (declared in include/dragon_hip_conv.h): argument checks and
+// the mapping of the convolution geometry onto the implicit-GEMM launch.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/dragon_hip_conv.h"
+#include "../../include/dragon_hip_gemm.h"
+#include "gemm_mfma.h"
+
+using namespace dragon;
+
+namespace {
+
+inline bool aligned16(int64_t a) { return (a & 15) == 0; }
+
+int num_compute_units() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    return n;
+}
+
+int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW, int64_t dW, int FH, int FW,
+                 int64_t dY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                 int64_t dBias = 0, int lengthv = 0, int width = 0) {
+    if (streams == nullptr || length < 1 || length > 10) return hipErrorInvalidValue;
+    if (dX == 0 || dW == 0 || dY == 0 || !aligned16(dX) || !aligned16(dW) || !aligned16(dY))
+        return hipErrorInvalidValue;
+    if (IH <= 0 || IW <= 0 || FH <= 0 || FW <= 0 || OH <= 0 || OW <= 0 || N <= 0 || IC <= 0 || OC <= 0 ||
+        sh <= 0 || sw <= 0 || ph < 0 || pw < 0 || (IC & 3) || (OC & 3))
+        return hipErrorInvalidValue;
+    const long long GM = (long long)N * OH * OW, GK = (long long)FH * FW * IC;
+    const long long sizeX = (long long)N * IH * IW * IC;
+    if (GM > 0x7fffffffLL || GK >= (1LL << 24) || sizeX >= (1LL << 29) || GM * OC > 0x7fffffffLL * 4LL)
+        return hipErrorInvalidValue;
+    GemmParams p = {};
+    p.A = (const float*)(intptr_t)dX;
+    p.B = (const float*)(intptr_t)dW;
+    p.C = (float*)(intptr_t)dY;
+    p.rows = (int)GM; p.cols = OC; p.k_total = (int)GK;
+    p.lda = (int)GK; p.a_outer = (int)GM; p.a_inner = (int)GK;     // A exists only as a gather
+    p.ldb = (int)GK; p.b_outer = OC; p.b_inner = (int)GK;
+    p.ldc = OC;
+    p.nz = 1;
+    p.cv_IH = IH; p.cv_IW = IW; p.cv_IC = IC; p.cv_FW = FW; p.cv_OH = OH; p.cv_OW = OW;
+    p.cv_sh = sh; p.cv_sw = sw; p.cv_ph = ph; p.cv_pw = pw;
+    p.cv_rcp_IC = 1.0f / (float)IC;
+    p.cv_rcp_FW = 1.0f / (float)FW;
+    if (dBias != 0) {
+        if (!aligned16(dBias) || width <= 0 || width > OC || lengthv <= 0 || lengthv % OC != 0 ||
+            lengthv / OC > GM)
+            return hipErrorInvalidValue;
+        p.bias = (const float*)(intptr_t)dBias;
+        p.bias_rows = lengthv / OC;
+        p.bias_width = width;
+    }
+    int tile = gemm_choose_tile(p.rows, p.cols, 1, p.k_total, num_compute_units());
+    if (tile >= TILE_COUNT) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape
+        tile = (tile == TILE_DMA_128x128_S4) ? TILE_128x128 : (tile == TILE_DMA_64x64_S4) ? TILE_64x64 : TILE_64x64_K32;
+    }
+    return gemm_launch_conv(p, tile, (hipStream_t)(intptr_t)streams[0]);
+}
+
+}  // namespace
+
+extern "C" {
+
+int dragon_Cuda_conv3D_conv3D(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW, int64_t dW,
+                              int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW, int32_t N, int32_t IC,
+                              int32_t OC, int32_t sh, int32_t sw, int32_t ph, int32_t pw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_conv3D_texture(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                      int64_t dW, int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW,
+                                      int32_t N, int32_t IC, int32_t OC, int32_t sh, int32_t sw, int32_t ph,
+                                      int32_t pw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_conv3D_np(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW, int64_t dW,
+                                 int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW, int32_t N,
+                                 int32_t IC, int32_t OC, int32_t sh, int32_t sw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, 0, 0);
+}
+int dragon_Cuda_conv3D_conv3D_W1(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW, int64_t dW,
+                                 int64_t dY, int32_t N, int32_t IC, int32_t OC) {
+    return conv_forward(s, n, dX, IH, IW, dW, 1, 1, dY, IH, IW, N, IC, OC, 1, 1, 0, 0);
+}
+int dragon_Cuda_conv3D_conv3DV2(int32_t, const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                int64_t dW, int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW,
+                                int32_t N, int32_t IC, int32_t OC, int32_t sh, int32_t sw, int32_t ph,
+                                int32_t pw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_kernel_remode(int64_t stream, int64_t dW, int64_t dCW, int32_t FH, int32_t FW,
+                                     int32_t OC, int32_t IC) {
+    if (FH <= 0 || FW <= 0 || OC <= 0 || IC <= 0 || (IC & 3) || (OC & 3)) return hipErrorInvalidValue;
+    const long long GK = (long long)FH * FW * IC;
+    if (GK * OC > 0x7fffffffLL) return hipErrorInvalidValue;
+    // W[OC][GK] -> CW[GK][OC]: a 2-D transpose, both row lengths multiples of 4
+    return dragon_Cuda_expk2_transpose2D(stream, dW, dCW, (int32_t)GK, OC, (int32_t)GK, OC, (int32_t)(GK * OC));
+}
+int dragon_Cuda_conv3D_conv3D_GemmR(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW, int64_t dW,
+                                    int64_t, int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW,
+                                    int32_t N, int32_t IC, int32_t OC, int32_t sh, int32_t sw, int32_t ph,
+                                    int32_t pw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_conv3D_GemmR_SGM(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                        int64_t dW, int64_t, int32_t FH, int32_t FW, int64_t dY, int32_t OH,
+                                        int32_t OW, int32_t N, int32_t IC, int32_t OC, int32_t sh, int32_t sw,
+                                        int32_t ph, int32_t pw, int32_t) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_conv3D_GemmR_texture(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                            int64_t dW, int64_t, int32_t FH, int32_t FW, int64_t dY, int32_t OH,
+                                            int32_t OW, int32_t N, int32_t IC, int32_t OC, int32_t sh,
+                                            int32_t sw, int32_t ph, int32_t pw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_conv3D_GemmR_texture_SGM(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                                int64_t dW, int64_t, int32_t FH, int32_t FW, int64_t dY,
+                                                int32_t OH, int32_t OW, int32_t N, int32_t IC, int32_t OC,
+                                                int32_t sh, int32_t sw, int32_t ph, int32_t pw, int32_t) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int dragon_Cuda_conv3D_conv3D_GemmR_W1(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                       int64_t dW, int64_t, int64_t dY, int32_t N, int32_t IC, int32_t OC) {
+    return conv_forward(s, n, dX, IH, IW, dW, 1, 1, dY, IH, IW, N, IC, OC, 1, 1, 0, 0);
+}
+int dragon_Cuda_conv3D_conv3D_GemmR_W1_SGM(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                           int64_t dW, int64_t, int64_t dY, int32_t N, int32_t IC, int32_t OC,
+                                           int32_t) {
+    return conv_forward(s, n, dX, IH, IW, dW, 1, 1, dY, IH, IW, N, IC, OC, 1, 1, 0, 0);
+}
+int dragon_Cuda_conv3D_conv3D_GemmV2R(int32_t, const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW,
+                                      int64_t dW, int64_t, int32_t FH, int32_t FW, int64_t dY, int32_t OH,
+                                      int32_t OW, int32_t N, int32_t IC, int32_t OC, int32_t sh, int32_t sw,
+                                      int32_t ph, int32_t pw) {
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+#define DRAGON_WINOGRAD(name, extra_decl)                                                                     \
+    int name(int32_t, const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW, int64_t dW, int64_t,    \
+             int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW, int32_t N, int32_t IC, int32_t OC,     \
+             int32_t ph, int32_t pw extra_decl) {                                                              \
+        const int e = conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, 1, 1, ph, pw);          \
+        return e ? -e : 1;                                                                                     \
+    }
+#define DRAGON_COMMA_INT , int32_t
+DRAGON_WINOGRAD(dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s8_R_texture, )
+DRAGON_WINOGRAD(dragon_Cuda_conv3D_conv3D_Im2col_WinogradR_s8_texture_SGM, DRAGON_COMMA_INT)
+DRAGON_WINOGRAD(dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s16_R_texture, )
+DRAGON_WINOGRAD(dragon_Cuda_conv3D_conv3D_Im2col_WinogradR_s16_texture_SGM, DRAGON_COMMA_INT)
+#undef DRAGON_WINOGRAD
+#undef DRAGON_COMMA_INT
+
+int dragon_Cuda_conv3D_conv3D_biased(const int64_t* s, int32_t n, int64_t dX, int32_t IH, int32_t IW, int64_t dW,
+                                     int32_t FH, int32_t FW, int64_t dY, int32_t OH, int32_t OW, int32_t N,
+                                     int32_t IC, int32_t OC, int32_t sh, int32_t sw, int32_t ph, int32_t pw,
+                                     int64_t dBias, int32_t lengthv, int32_t width) {
+    if (dBias == 0) return hipErrorInvalidValue;
+    return conv_forward(s, n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw, dBias, lengthv, width);
+}
+
+}  // extern "C"

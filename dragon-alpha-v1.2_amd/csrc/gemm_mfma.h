@@ -51,6 +51,10 @@ struct GemmParams {
     int split;              // non-zero selects split-K
     int k_slice;            // slice z covers [z*k_slice, (z+1)*k_slice), the last runs to k_total
     long long sizeC;        // floats per split-K partial
+    // implicit-GEMM convolution (gemm_launch_conv): A is gathered from X[N, IH, IW, IC]; rows = N*OH*OW,
+    // k_total = FH*FW*IC, B = W[OC, FH*FW*IC], C = Y[N*OH*OW, OC]
+    int cv_IH, cv_IW, cv_IC, cv_FW, cv_OH, cv_OW, cv_sh, cv_sw, cv_ph, cv_pw;
+    float cv_rcp_IC, cv_rcp_FW;
     const float* bias;      // optional row vector added to C[i][j] for i < bias_rows, j < bias_width
     int bias_rows, bias_width;
     int tiles_m, tiles_n;   // filled by the launcher
@@ -61,6 +65,9 @@ void gemm_force_tile(int tile);
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
 hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);
+// Y = conv(X, W) [+ bias row over OC] as an implicit GEMM (the A * B^T kernel with a gathered A);
+// classic tile ids only
+hipError_t gemm_launch_conv(const GemmParams& p, int tile, hipStream_t stream);
 // the GEMM_NN product with p.bias added in the epilogue (what gemm_launch forwards to when p.bias is set)
 hipError_t gemm_launch_nn_biased(const GemmParams& p, int tile, hipStream_t stream);
 

@@ -226,6 +226,77 @@ struct KOuter {
     __device__ __forceinline__ static size_t k_advance(int ld) { return (size_t)KT * ld; }
 };
 
+// Implicit-GEMM convolution: the A operand of Y[GM, OC] = A[GM, GK] * W[OC, GK]^T is never
+// materialised.  Row m = (n, oh, ow) and column k = (fh, fw, ic) of A is X[n, oh*sh - ph + fh,
+// ow*sw - pw + fw, ic], or zero when that pixel lies in the padding.  IC is a multiple of 4, so a
+// 16-byte chunk of 4 consecutive k stays inside one pixel; the chunk's address is
+// row part (fixed per tile) + k part (changes per stage), and "in the padding" / "row outside" /
+// "k beyond GK" all become the out-of-range offset that makes the load return zeros.
+// Same LDS layout and swizzle as KInner, so the fragment reads do not know the difference.
+template <int R, int KT>
+struct ConvInner {
+    static constexpr int CPR = KT / 4;
+    static constexpr int RPP = NTHREADS / CPR;
+    static constexpr int PASSES = R / RPP;
+    static constexpr int LDS_STRIDE = KT;
+    static constexpr int LDS_FLOATS = R * LDS_STRIDE;
+    static_assert(R % RPP == 0 && PASSES >= 1, "tile does not divide over the workgroup");
+
+    int base[PASSES];   // element offset of pixel (n, oh*sh - ph, ow*sw - pw), channel 0
+    int ih0[PASSES];    // oh*sh - ph, or far below zero for a row outside the matrix
+    int iw0[PASSES];
+    int kcol, row_first, chunk;
+
+    __device__ __forceinline__ void init_conv(int t, int row0, int gm, const GemmParams& p) {
+        const int c = t % CPR, r0 = t / CPR;
+        kcol = c * 4;
+        row_first = r0;
+        chunk = c;
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const int m = row0 + r0 + s * RPP;
+            const int q = m / p.cv_OW, ow = m - q * p.cv_OW;
+            const int n = q / p.cv_OH, oh = q - n * p.cv_OH;
+            const int ih = oh * p.cv_sh - p.cv_ph, iw = ow * p.cv_sw - p.cv_pw;
+            ih0[s] = (m < gm) ? ih : -(1 << 30);
+            iw0[s] = iw;
+            base[s] = ((n * p.cv_IH + ih) * p.cv_IW + iw) * p.cv_IC;
+        }
+    }
+    // k = first k of the stage; k_left = GK - k
+    __device__ __forceinline__ void load_conv(v4f (&reg)[PASSES], const float* X, int k_left, int k,
+                                              const GemmParams& p) const {
+        const int kk = k + kcol;                     // < 2^24, checked by the host
+        // kk = (fh * FW + fw) * IC + ic by float reciprocals with an exact integer correction
+        int pix = (int)((float)kk * p.cv_rcp_IC);
+        int ic = kk - pix * p.cv_IC;
+        if (ic < 0) { pix--; ic += p.cv_IC; }
+        if (ic >= p.cv_IC) { pix++; ic -= p.cv_IC; }
+        int fh = (int)((float)pix * p.cv_rcp_FW);
+        int fw = pix - fh * p.cv_FW;
+        if (fw < 0) { fh--; fw += p.cv_FW; }
+        if (fw >= p.cv_FW) { fh++; fw -= p.cv_FW; }
+        const int koff = (fh * p.cv_IW + fw) * p.cv_IC + ic;
+        const bool kok = kcol < k_left;
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const bool ok = kok && (unsigned)(ih0[s] + fh) < (unsigned)p.cv_IH &&
+                            (unsigned)(iw0[s] + fw) < (unsigned)p.cv_IW;
+            reg[s] = buffer_load_f4(X, ok ? (base[s] + koff) * 4 : OOB_OFFSET);
+        }
+    }
+    __device__ __forceinline__ void store(const v4f (&reg)[PASSES], float* lds) const {
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const int r = row_first + s * RPP;
+            *(v4f*)(lds + r * LDS_STRIDE + 4 * (chunk ^ kin_swizzle<KT>(r))) = reg[s];
+        }
+    }
+    // the descriptor's base is X itself: every offset is absolute (X holds fewer than 2^29 floats)
+    __device__ __forceinline__ static const float* tile_base(const float* X, int, int, int) { return X; }
+    __device__ __forceinline__ static size_t k_advance(int) { return 0; }
+};
+
 // ---------------------------------------------------------------------------
 // Fragment reads: LDS -> MFMA operands for one group of 8 k
 //   frag[b][q]: operand of block b for MFMA step q (k = 8*g + 4*h + q)
@@ -428,12 +499,15 @@ constexpr int target_occupancy() {
     return fit > 4 ? 4 : (fit < 1 ? 1 : fit);
 }
 
-template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, bool BIAS>
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, bool BIAS, bool CONV = false>
 __global__ __launch_bounds__(NTHREADS, (target_occupancy<A_KIN, B_KIN, WM * TM * 32, WN * TN * 32, KT>()))
 void gemm_f32_mfma(const GemmParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    static_assert(!CONV || (A_KIN && B_KIN), "the convolution is the A * B^T form with a gathered A");
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
+    using LoadA = typename std::conditional<
+        CONV, ConvInner<BM, KT>,
+        typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type>::type;
     using LoadB = typename std::conditional<B_KIN, KInner<BN, KT>, KOuter<BN, KT>>::type;
 
     __shared__ __attribute__((aligned(16))) float As[2][LoadA::LDS_FLOATS];
@@ -452,7 +526,8 @@ void gemm_f32_mfma(const GemmParams p) {
     TileCtx cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid);
     LoadA la;
     LoadB lb;
-    la.init(t, cur.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+    if constexpr (CONV) la.init_conv(t, cur.row0, p.a_outer, p);
+    else la.init(t, cur.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
     lb.init(t, cur.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
 
     v16f acc[TM][TN];
@@ -464,7 +539,8 @@ void gemm_f32_mfma(const GemmParams p) {
     v4f ra[LoadA::PASSES], rb[LoadB::PASSES];
 
     // stage 0 of the first tile
-    la.load(ra, cur.a_ptr, cur.ka_lim - cur.k0);
+    if constexpr (CONV) la.load_conv(ra, cur.a_ptr, cur.ka_lim - cur.k0, cur.k0, p);
+    else la.load(ra, cur.a_ptr, cur.ka_lim - cur.k0);
     lb.load(rb, cur.b_ptr, cur.kb_lim - cur.k0);
     la.store(ra, As[0]);
     lb.store(rb, Bs[0]);
@@ -483,14 +559,17 @@ void gemm_f32_mfma(const GemmParams p) {
                 a_ptr += a_step;
                 b_ptr += b_step;
                 const int knext = cur.k0 + (it + 1) * KT;
-                la.load(ra, a_ptr, cur.ka_lim - knext);
+                if constexpr (CONV) la.load_conv(ra, a_ptr, cur.ka_lim - knext, knext, p);
+                else la.load(ra, a_ptr, cur.ka_lim - knext);
                 lb.load(rb, b_ptr, cur.kb_lim - knext);
                 fetched = true;
             } else if (has_next) {       // first stage of the next tile -> registers
                 nxt = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid + G);
-                la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+                if constexpr (CONV) la.init_conv(t, nxt.row0, p.a_outer, p);
+                else la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
                 lb.init(t, nxt.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
-                la.load(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0);
+                if constexpr (CONV) la.load_conv(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0, nxt.k0, p);
+                else la.load(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0);
                 lb.load(rb, nxt.b_ptr, nxt.kb_lim - nxt.k0);
                 fetched = true;
             }
@@ -678,10 +757,10 @@ static int device_num_cu() {
     return cached[dev];
 }
 
-template <bool A_KIN, bool B_KIN, bool BIAS, int WM, int WN, int TM, int TN, int KT>
+template <bool A_KIN, bool B_KIN, bool BIAS, int WM, int WN, int TM, int TN, int KT, bool CONV = false>
 static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    auto kernel = gemm_f32_mfma<A_KIN, B_KIN, WM, WN, TM, TN, KT, BIAS>;
+    auto kernel = gemm_f32_mfma<A_KIN, B_KIN, WM, WN, TM, TN, KT, BIAS, CONV>;
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
@@ -706,24 +785,24 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <bool A_KIN, bool B_KIN, bool BIAS>
+template <bool A_KIN, bool B_KIN, bool BIAS, bool CONV = false>
 static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stream) {
     switch (tile) {
-        case TILE_128x128: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16>(p, stream);
-        case TILE_64x64:   return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16>(p, stream);
-        case TILE_256x64:  return launch_cfg<A_KIN, B_KIN, BIAS, 4, 1, 2, 2, 16>(p, stream);
-        case TILE_64x256:  return launch_cfg<A_KIN, B_KIN, BIAS, 1, 4, 2, 2, 16>(p, stream);
-        case TILE_128x64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 16>(p, stream);
-        case TILE_64x128:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 16>(p, stream);
-        case TILE_128x128_K32: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 32>(p, stream);
-        case TILE_64x64_K32:   return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32>(p, stream);
-        case TILE_128x64_K32:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 32>(p, stream);
-        case TILE_64x128_K32:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 32>(p, stream);
-        case TILE_64x64_K64:   return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 64>(p, stream);
-        case TILE_64x64_K128:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 128>(p, stream);
-        case TILE_128x128_K64: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 64>(p, stream);
-        case TILE_128x64_K64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 64>(p, stream);
-        case TILE_64x128_K64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 64>(p, stream);
+        case TILE_128x128: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV>(p, stream);
+        case TILE_64x64:   return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, CONV>(p, stream);
+        case TILE_256x64:  return launch_cfg<A_KIN, B_KIN, BIAS, 4, 1, 2, 2, 16, CONV>(p, stream);
+        case TILE_64x256:  return launch_cfg<A_KIN, B_KIN, BIAS, 1, 4, 2, 2, 16, CONV>(p, stream);
+        case TILE_128x64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 16, CONV>(p, stream);
+        case TILE_64x128:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 16, CONV>(p, stream);
+        case TILE_128x128_K32: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 32, CONV>(p, stream);
+        case TILE_64x64_K32:   return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, CONV>(p, stream);
+        case TILE_128x64_K32:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 32, CONV>(p, stream);
+        case TILE_64x128_K32:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 32, CONV>(p, stream);
+        case TILE_64x64_K64:   return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 64, CONV>(p, stream);
+        case TILE_64x64_K128:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 128, CONV>(p, stream);
+        case TILE_128x128_K64: return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 64, CONV>(p, stream);
+        case TILE_128x64_K64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 64, CONV>(p, stream);
+        case TILE_64x128_K64:  return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 64, CONV>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -5,6 +5,7 @@ Thin, one-to-one wrappers over the C ABI (no compute happens in Python):
   Cuda             -- runtime natives of the reference's z.dragon.engine.cuda.impl.Cuda
   Cuda_matMul      -- natives + heuristics of ...impl.math.Cuda_matMul
   Cuda_batchMatMul -- natives + heuristics of ...impl.math.Cuda_batchMatMul
+  Cuda_conv3D      -- forward-convolution natives of ...impl.math.Cuda_conv3D
   Cuda_expk2       -- transpose2D / 3D / 4D of ...impl.Cuda_expk2 (dimension swap)
   Cuda_function    -- linear_dual2D_row of ...impl.math.Cuda_function (the bias row)
   CudaException    -- the error type the reference's natives throw
@@ -290,6 +291,76 @@ class Cuda_function:
                           stride):
         _check(lib.dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta,
                                                           gamma, dY, lengthv, width, stride))
+
+
+class Cuda_conv3D:
+    """Forward-convolution natives of Cuda_conv3D.java (every family runs the same implicit-GEMM kernel)."""
+
+    @staticmethod
+    def output_feature_dim(IH, IW, FH, FW, N, OC, sh, sw, ph, pw):
+        return [N, (IH - FH + 2 * ph) // sh + 1, (IW - FW + 2 * pw) // sw + 1, OC]
+
+    @staticmethod
+    def conv3D(streams, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D(arr, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh,
+                                             sw, ph, pw))
+
+    @staticmethod
+    def conv3D_texture(streams, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D_texture(arr, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC,
+                                                     OC, sh, sw, ph, pw))
+
+    @staticmethod
+    def conv3D_np(streams, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D_np(arr, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC,
+                                                sh, sw))
+
+    @staticmethod
+    def conv3D_W1(streams, length, dX, IH, IW, dW, dY, N, IC, OC):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D_W1(arr, length, dX, IH, IW, dW, dY, N, IC, OC))
+
+    @staticmethod
+    def conv3DV2(useTexture, streams, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3DV2(int(useTexture), arr, length, dX, IH, IW, dW, FH, FW, dY, OH,
+                                               OW, N, IC, OC, sh, sw, ph, pw))
+
+    @staticmethod
+    def kernel_remode(stream, dW, dCW, FH, FW, OC, IC):
+        _check(lib.dragon_Cuda_conv3D_kernel_remode(stream, dW, dCW, FH, FW, OC, IC))
+
+    @staticmethod
+    def conv3D_GemmR(streams, length, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D_GemmR(arr, length, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC,
+                                                   OC, sh, sw, ph, pw))
+
+    @staticmethod
+    def conv3D_GemmR_W1(streams, length, dX, IH, IW, dW, dCW, dY, N, IC, OC):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D_GemmR_W1(arr, length, dX, IH, IW, dW, dCW, dY, N, IC, OC))
+
+    @staticmethod
+    def conv3D_Im2col_Winograd_s8_R_texture(useTexture, streams, length, dX, IH, IW, dW, dCW, FH, FW, dY, OH,
+                                            OW, N, IC, OC, ph, pw):
+        arr, _ = _stream_array(streams)
+        rc = lib.dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s8_R_texture(
+            int(useTexture), arr, length, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC, OC, ph, pw)
+        if rc < 0:
+            raise CudaException(-rc)
+        return rc == 1
+
+    @staticmethod
+    def conv3D_biased(streams, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw, dBias,
+                      lengthv, width):
+        """Convolution and bias row in one launch; no native of this name in the reference."""
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_conv3D_conv3D_biased(arr, length, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC,
+                                                    sh, sw, ph, pw, dBias, lengthv, width))
 
 
 class Cuda_reduce:

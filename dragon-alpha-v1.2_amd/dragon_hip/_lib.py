@@ -21,6 +21,9 @@ p_i32 = POINTER(c_int32)
 _MM2D = [p_i64, i32, i64, i64, i64, i32, i32, i32]
 _MMSK = [p_i64, i32, i32, i64, i64, i64, i64, i32, i32, i32]
 _BMM = [p_i64, i32, i64, i64, i64, i32, i32, i32, i32, i32]
+# streams, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw  (and with CW after W)
+_CONV = [p_i64, i32, i64, i32, i32, i64, i32, i32, i64, i32, i32, i32, i32, i32, i32, i32, i32, i32]
+_CONVR = [p_i64, i32, i64, i32, i32, i64, i64, i32, i32, i64, i32, i32, i32, i32, i32, i32, i32, i32, i32]
 SIGNATURES = {
     # include/dragon_hip_gemm.h
     "dragon_Cuda_matMul_matMul": (i32, _MM2D),
@@ -37,6 +40,25 @@ SIGNATURES = {
     "dragon_Cuda_expk2_transpose2D": (i32, [i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_expk2_transpose3D": (i32, [i64, i64, i64] + [i32] * 9),
     "dragon_Cuda_expk2_transpose4D": (i32, [i64, i64, i64] + [i32] * 11),
+    # include/dragon_hip_conv.h
+    "dragon_Cuda_conv3D_conv3D": (i32, _CONV),
+    "dragon_Cuda_conv3D_conv3D_texture": (i32, _CONV),
+    "dragon_Cuda_conv3D_conv3D_np": (i32, _CONV[:-2]),
+    "dragon_Cuda_conv3D_conv3D_W1": (i32, [p_i64, i32, i64, i32, i32, i64, i64, i32, i32, i32]),
+    "dragon_Cuda_conv3D_conv3DV2": (i32, [i32] + _CONV),
+    "dragon_Cuda_conv3D_kernel_remode": (i32, [i64, i64, i64, i32, i32, i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_GemmR": (i32, _CONVR),
+    "dragon_Cuda_conv3D_conv3D_GemmR_SGM": (i32, _CONVR + [i32]),
+    "dragon_Cuda_conv3D_conv3D_GemmR_texture": (i32, _CONVR),
+    "dragon_Cuda_conv3D_conv3D_GemmR_texture_SGM": (i32, _CONVR + [i32]),
+    "dragon_Cuda_conv3D_conv3D_GemmR_W1": (i32, [p_i64, i32, i64, i32, i32, i64, i64, i64, i32, i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_GemmR_W1_SGM": (i32, [p_i64, i32, i64, i32, i32, i64, i64, i64, i32, i32, i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_GemmV2R": (i32, [i32] + _CONVR),
+    "dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s8_R_texture": (i32, [i32] + _CONVR[:-4] + [i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_Im2col_WinogradR_s8_texture_SGM": (i32, [i32] + _CONVR[:-4] + [i32, i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s16_R_texture": (i32, [i32] + _CONVR[:-4] + [i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_Im2col_WinogradR_s16_texture_SGM": (i32, [i32] + _CONVR[:-4] + [i32, i32, i32]),
+    "dragon_Cuda_conv3D_conv3D_biased": (i32, _CONV + [i64, i32, i32]),
     "dragon_Cuda_batchMatMul_batchMatMul": (i32, _BMM),
     "dragon_Cuda_batchMatMul_batchMatMul_texture": (i32, _BMM),
     "dragon_Cuda_batchMatMul_batchMatMulT1": (i32, _BMM),

@@ -458,6 +458,40 @@ void oracle_softmax2D(const float* X, float* Y, int field_length, int row_length
 }
 
 /* ------------------------------------------------------------------------ */
+/* Forward convolution                                                       */
+/* ------------------------------------------------------------------------ */
+
+/* Y[n][oh][ow][oc] = sum over fh, fw, ic of X[n][oh*sh-ph+fh][ow*sw-pw+fw][ic] * W[oc][fh][fw][ic],
+ * pixels in the padding skipped; logical (unpadded) row-major arrays.  The loop nest and the
+ * double-precision accumulator with a final cast to float of the reference's CPU check
+ * (ZUTIL-STD-1.2/src/z/util/math/vector/Tense.java:141-171, used by
+ * alpha-Dragon-v1.2/test/test/cuda/conv3D/Cuda_conv3D_test.java).  acc32 != 0 accumulates in float,
+ * fh, fw, ic ascending, instead: the order-exact twin for integer-valued inputs. */
+void oracle_conv3D(const float* X, int IH, int IW, const float* W, int FH, int FW, float* Y, int OH, int OW,
+                   int N, int IC, int OC, int sh, int sw, int ph, int pw, int acc32) {
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++)
+        for (int oc = 0; oc < OC; oc++)
+            for (int oh = 0; oh < OH; oh++)
+                for (int ow = 0; ow < OW; ow++) {
+                    const int ih_s = oh * sh - ph, iw_s = ow * sw - pw;
+                    double v = 0;
+                    float vf = 0.0f;
+                    for (int fh = 0; fh < FH; fh++)
+                        for (int fw = 0; fw < FW; fw++)
+                            for (int ic = 0; ic < IC; ic++) {
+                                const int ih = ih_s + fh, iw = iw_s + fw;
+                                if (ih < 0 || iw < 0 || ih >= IH || iw >= IW) continue;
+                                const float x = X[(((size_t)n * IH + ih) * IW + iw) * IC + ic];
+                                const float w = W[(((size_t)oc * FH + fh) * FW + fw) * IC + ic];
+                                if (acc32) { float pr = x * w; vf = vf + pr; }
+                                else v += (double)x * (double)w;
+                            }
+                    Y[(((size_t)n * OH + oh) * OW + ow) * OC + oc] = acc32 ? vf : (float)v;
+                }
+}
+
+/* ------------------------------------------------------------------------ */
 /* Dimension swap                                                            */
 /* ------------------------------------------------------------------------ */
 

@@ -50,6 +50,7 @@ for _name, _res, _args in [
     ("oracle_linear_dual2D_row", None, [_P, _P, c_int, c_float, c_float, c_float, _P, c_int, c_int, c_int]),
     ("oracle_linear2D", None, [c_float, _P, c_float, _P, c_int, c_int, c_int]),
     ("oracle_softmax2D", None, [_P, _P, c_int, c_int, c_int, c_int, c_float]),
+    ("oracle_conv3D", None, [_P, c_int, c_int, _P, c_int, c_int, _P] + [c_int] * 10),
     ("oracle_transpose4D", None, [_P, _P, POINTER(c_int), c_int, c_int, c_int, c_int]),
     ("oracle_samePercent_relative", c_float, [_P, _P, c_int, c_float]),
     ("oracle_num_threads", c_int, []),
@@ -218,6 +219,21 @@ def softmax2D(Xp, width, features=None, scale=1.0):
     row_lengthv = features // width * stride
     Y = np.empty_like(Xp)
     _o.oracle_softmax2D(px, Y.ctypes.data_as(_P), Xp.size // row_lengthv, row_lengthv, width, stride, scale)
+    return Y
+
+
+def conv3D(X, W, sh, sw, ph, pw, OH=None, OW=None, acc32=False):
+    """X[N, IH, IW, IC], W[OC, FH, FW, IC] logical arrays -> Y[N, OH, OW, OC]."""
+    X, px = _f32(X)
+    W, pw_ = _f32(W)
+    N, IH, IW, IC = X.shape
+    OC, FH, FW, IC2 = W.shape
+    assert IC == IC2
+    OH = (IH - FH + 2 * ph) // sh + 1 if OH is None else OH
+    OW = (IW - FW + 2 * pw) // sw + 1 if OW is None else OW
+    Y = np.zeros((N, OH, OW, OC), np.float32)
+    _o.oracle_conv3D(px, IH, IW, pw_, FH, FW, Y.ctypes.data_as(_P), OH, OW, N, IC, OC, sh, sw, ph, pw,
+                     1 if acc32 else 0)
     return Y
 
 

@@ -11,7 +11,7 @@ import pytest
 from oracle import oracle
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("dragon_hip_gemm.h", "dragon_hip_runtime.h", "dragon_hip_engine.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("dragon_hip_gemm.h", "dragon_hip_conv.h", "dragon_hip_runtime.h", "dragon_hip_engine.h")]
 INVALID_VALUE = 1   # hipErrorInvalidValue
 
 

@@ -1,0 +1,169 @@
+"""Forward convolution as an implicit GEMM on the GPU, through the C ABI, against the CPU oracle
+(the reference's naive loops with an FP64 accumulator).  Tolerances as for the products, with
+K = FH*FW*IC: relative Frobenius error <= 1e-5, per-element |err| <= 1e-4*sqrt(K)*max|X|*max|W|;
+integer-valued inputs must match bit for bit (every summation order is exact there); and the
+reference's own acceptance rule (samePercent_relative at 1e-5 >= 0.999, test/cuda/conv3D/
+Cuda_conv3D_test.java:76-86) is evaluated as well."""
+import numpy as np
+import pytest
+
+from oracle import oracle
+from helpers import assert_within_tolerance
+
+pytestmark = pytest.mark.gpu
+
+
+def pad_last(x, first_to4=False):
+    s = (x.shape[-1] + 3) // 4 * 4
+    n0 = (x.shape[0] + 3) // 4 * 4 if first_to4 else x.shape[0]
+    out = np.zeros((n0,) + x.shape[1:-1] + (s,), np.float32)
+    out[:x.shape[0], ..., :x.shape[-1]] = x
+    return out
+
+
+def run_conv(dh, X, W, sh, sw, ph, pw, entry="conv3D", bias=None, fill=7.0):
+    """Logical X[N,IH,IW,IC], W[OC,FH,FW,IC] -> logical Y plus the full padded device array."""
+    CV = dh.Cuda_conv3D
+    N, IH, IW, IC = X.shape
+    OC, FH, FW, _ = W.shape
+    OH, OW = (IH - FH + 2 * ph) // sh + 1, (IW - FW + 2 * pw) // sw + 1
+    Xp, Wp = pad_last(X, first_to4=True), pad_last(W, first_to4=True)    # the engine pads N, IC, OC to x4
+    Wp = Wp[:(OC + 3) // 4 * 4]
+    N4, IC4, OC4 = Xp.shape[0], Xp.shape[-1], Wp.shape[0]
+    dX, dW = dh.DeviceArray(Xp), dh.DeviceArray(Wp)
+    dY = dh.DeviceArray(size=N4 * OH * OW * OC4 + 16)
+    dY.fill(fill)
+    s = [0]
+    if entry == "conv3D":
+        CV.conv3D(s, 1, dX.address, IH, IW, dW.address, FH, FW, dY.address, OH, OW, N4, IC4, OC4, sh, sw, ph, pw)
+    elif entry == "texture":
+        CV.conv3D_texture(s, 1, dX.address, IH, IW, dW.address, FH, FW, dY.address, OH, OW, N4, IC4, OC4, sh, sw, ph, pw)
+    elif entry == "V2":
+        CV.conv3DV2(True, s, 1, dX.address, IH, IW, dW.address, FH, FW, dY.address, OH, OW, N4, IC4, OC4, sh, sw, ph, pw)
+    elif entry == "np":
+        assert ph == 0 and pw == 0
+        CV.conv3D_np(s, 1, dX.address, IH, IW, dW.address, FH, FW, dY.address, OH, OW, N4, IC4, OC4, sh, sw)
+    elif entry == "W1":
+        assert FH == 1 and FW == 1 and sh == 1 and sw == 1 and ph == 0 and pw == 0
+        CV.conv3D_W1(s, 1, dX.address, IH, IW, dW.address, dY.address, N4, IC4, OC4)
+    elif entry in ("GemmR", "GemmR_W1", "winograd"):
+        dCW = dh.DeviceArray(size=Wp.size)
+        CV.kernel_remode(0, dW.address, dCW.address, FH, FW, OC4, IC4)
+        if entry == "GemmR":
+            CV.conv3D_GemmR(s, 1, dX.address, IH, IW, dW.address, dCW.address, FH, FW, dY.address, OH, OW, N4, IC4,
+                            OC4, sh, sw, ph, pw)
+        elif entry == "GemmR_W1":
+            CV.conv3D_GemmR_W1(s, 1, dX.address, IH, IW, dW.address, dCW.address, dY.address, N4, IC4, OC4)
+        else:
+            assert sh == 1 and sw == 1
+            assert CV.conv3D_Im2col_Winograd_s8_R_texture(True, s, 1, dX.address, IH, IW, dW.address, dCW.address,
+                                                          FH, FW, dY.address, OH, OW, N4, IC4, OC4, ph, pw)
+        dh.Cuda.streamSynchronize(0)
+        CW = dCW.get((FH, FW, IC4, OC4))
+        assert np.array_equal(CW, np.transpose(Wp.reshape(OC4, FH, FW, IC4), (1, 2, 3, 0)))   # the re-ordered filter
+        dCW.free()
+    elif entry == "biased":
+        bp = np.zeros(OC4, np.float32); bp[:OC] = bias
+        db = dh.DeviceArray(bp)
+        CV.conv3D_biased(s, 1, dX.address, IH, IW, dW.address, FH, FW, dY.address, OH, OW, N4, IC4, OC4, sh, sw, ph,
+                         pw, db.address, N * OH * OW * OC4, OC)
+        dh.Cuda.streamSynchronize(0)
+        db.free()
+    else:
+        raise ValueError(entry)
+    dh.Cuda.streamSynchronize(0)
+    raw = dY.get()
+    for d in (dX, dW, dY):
+        d.free()
+    assert np.all(raw[N4 * OH * OW * OC4:] == fill)                 # nothing written past Y
+    Yp = raw[:N4 * OH * OW * OC4].reshape(N4, OH, OW, OC4)
+    return Yp[:N, :, :, :OC], Yp
+
+
+# IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw: the shapes of the reference's test sweep in small, ragged
+# channel counts, strides, paddings up to FH-1, windows hanging over the border, 1x1, tall filters
+GEOMS = [(5, 5, 3, 3, 2, 3, 5, 1, 1, 1, 1), (8, 7, 3, 3, 3, 4, 8, 2, 2, 1, 1), (33, 33, 4, 4, 4, 16, 33, 1, 1, 1, 1),
+         (32, 32, 3, 3, 4, 16, 64, 2, 2, 1, 1), (6, 6, 1, 1, 5, 7, 9, 1, 1, 0, 0), (7, 9, 3, 2, 2, 5, 6, 2, 1, 0, 0),
+         (4, 4, 4, 4, 1, 2, 3, 1, 1, 3, 3), (10, 6, 5, 3, 2, 8, 130, 3, 2, 2, 1), (16, 16, 3, 3, 8, 64, 128, 1, 1, 1, 1),
+         (12, 12, 7, 7, 2, 3, 20, 2, 2, 3, 3), (1, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0), (9, 5, 2, 5, 3, 130, 4, 1, 1, 1, 2)]
+
+
+@pytest.mark.parametrize("geom", GEOMS)
+def test_conv3D_matches_oracle(dh, gpu, geom):
+    IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw = geom
+    rng = np.random.default_rng(sum(geom))
+    X = rng.uniform(-1, 1, (N, IH, IW, IC)).astype(np.float32)
+    W = rng.uniform(-1, 1, (OC, FH, FW, IC)).astype(np.float32)
+    Y, Yp = run_conv(dh, X, W, sh, sw, ph, pw)
+    R = oracle.conv3D(X, W, sh, sw, ph, pw)
+    assert Y.shape == R.shape
+    assert_within_tolerance(Y, R, FH * FW * IC, X, W, "conv3D %s" % (geom,))
+    assert oracle.samePercent_relative(R, Y, 1e-5) >= 0.99
+    assert not Yp[N:].any() and not Yp[..., OC:].any()              # pad images and pad channels are zeros
+    # integer-valued inputs: bit for bit
+    Xi = rng.integers(-3, 4, X.shape).astype(np.float32)
+    Wi = rng.integers(-3, 4, W.shape).astype(np.float32)
+    Yi, _ = run_conv(dh, Xi, Wi, sh, sw, ph, pw)
+    assert np.array_equal(Yi, oracle.conv3D(Xi, Wi, sh, sw, ph, pw))
+
+
+@pytest.mark.parametrize("tile", list(range(-1, 18)))
+def test_conv3D_every_tile_shape(dh, gpu, tile):
+    rng = np.random.default_rng(300 + tile)
+    X = rng.integers(-3, 4, (3, 11, 9, 12)).astype(np.float32)
+    W = rng.integers(-3, 4, (70, 3, 3, 12)).astype(np.float32)
+    dh.force_tile(tile)
+    try:
+        Y, _ = run_conv(dh, X, W, 2, 1, 1, 1)
+    finally:
+        dh.force_tile(-1)
+    assert np.array_equal(Y, oracle.conv3D(X, W, 2, 1, 1, 1))
+
+
+@pytest.mark.parametrize("entry", ["texture", "V2", "np", "W1", "GemmR", "GemmR_W1", "winograd"])
+def test_every_native_family_computes_the_same_convolution(dh, gpu, entry):
+    rng = np.random.default_rng(len(entry))
+    if entry in ("W1", "GemmR_W1"):
+        g = (9, 7, 1, 1, 3, 10, 21, 1, 1, 0, 0)
+    elif entry == "np":
+        g = (11, 9, 3, 4, 3, 6, 21, 2, 1, 0, 0)
+    elif entry == "winograd":
+        g = (12, 10, 3, 3, 3, 8, 40, 1, 1, 1, 1)
+    else:
+        g = (12, 10, 3, 5, 3, 6, 40, 2, 2, 1, 2)
+    IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw = g
+    X = rng.integers(-3, 4, (N, IH, IW, IC)).astype(np.float32)
+    W = rng.integers(-3, 4, (OC, FH, FW, IC)).astype(np.float32)
+    Y, _ = run_conv(dh, X, W, sh, sw, ph, pw, entry=entry)
+    assert np.array_equal(Y, oracle.conv3D(X, W, sh, sw, ph, pw))
+
+
+def test_conv3D_biased_equals_two_launches(dh, gpu):
+    rng = np.random.default_rng(9)
+    X = rng.uniform(-1, 1, (3, 10, 9, 7)).astype(np.float32)
+    W = rng.uniform(-1, 1, (37, 3, 3, 7)).astype(np.float32)
+    bias = rng.uniform(-2, 2, 37).astype(np.float32)
+    Yb, Ypb = run_conv(dh, X, W, 1, 2, 1, 1, entry="biased", bias=bias)
+    Y, _ = run_conv(dh, X, W, 1, 2, 1, 1)
+    assert np.array_equal(Yb.view(np.uint32), ((Y + bias) + np.float32(0)).view(np.uint32))   # an exact float add
+    assert not Ypb[3:].any() and not Ypb[..., 37:].any()
+
+
+def test_conv3D_argument_errors(dh, gpu):
+    CV = dh.Cuda_conv3D
+    d = dh.DeviceArray(size=4096)
+    a = d.address
+    ok = dict(dX=a, IH=4, IW=4, dW=a + 2048, FH=3, FW=3, dY=a + 8192, OH=4, OW=4, N=4, IC=4, OC=4, sh=1, sw=1, ph=1, pw=1)
+
+    def call(**kw):
+        g = dict(ok); g.update(kw)
+        CV.conv3D([0], 1, g["dX"], g["IH"], g["IW"], g["dW"], g["FH"], g["FW"], g["dY"], g["OH"], g["OW"], g["N"],
+                  g["IC"], g["OC"], g["sh"], g["sw"], g["ph"], g["pw"])
+    call()
+    for bad in (dict(dX=0), dict(dW=0), dict(dY=0), dict(IC=3), dict(OC=6), dict(sh=0), dict(ph=-1), dict(FH=0),
+                dict(OH=0), dict(N=0), dict(dX=a + 4), dict(IC=1 << 22, FH=3, FW=3)):
+        with pytest.raises(dh.CudaException) as e:
+            call(**bad)
+        assert e.value.code == 1, bad
+    dh.Cuda.streamSynchronize(0)
+    d.free()

@@ -391,6 +391,54 @@ def test_linear2D_oracle():
     assert np.array_equal(Y[:, :7], 2 * X[:, :7] - 1) and not Y[:, 7].any()
 
 
+def _conv_numpy(X, W, sh, sw, ph, pw):
+    """Independent restatement: zero-pad, gather windows with stride tricks, contract with einsum in FP64."""
+    N, IH, IW, IC = X.shape
+    OC, FH, FW, _ = W.shape
+    Xp = np.zeros((N, IH + 2 * ph, IW + 2 * pw, IC), np.float64)
+    Xp[:, ph:ph + IH, pw:pw + IW] = X
+    OH, OW = (IH - FH + 2 * ph) // sh + 1, (IW - FW + 2 * pw) // sw + 1
+    win = np.lib.stride_tricks.sliding_window_view(Xp, (FH, FW), axis=(1, 2))[:, ::sh, ::sw][:, :OH, :OW]
+    return np.einsum("nhwcij,oijc->nhwo", win, W.astype(np.float64))
+
+
+@pytest.mark.parametrize("geom", [(5, 5, 3, 3, 1, 1, 1, 1), (8, 7, 3, 3, 2, 2, 1, 1), (9, 9, 4, 4, 1, 1, 1, 1),
+                                  (6, 6, 1, 1, 1, 1, 0, 0), (7, 9, 3, 2, 2, 1, 0, 0), (4, 4, 4, 4, 1, 1, 3, 3),
+                                  (10, 6, 5, 3, 3, 2, 2, 1)])
+def test_conv_oracle_against_an_independent_formulation(geom):
+    IH, IW, FH, FW, sh, sw, ph, pw = geom
+    N, IC, OC = 2, 3, 5
+    X = RNG.standard_normal((N, IH, IW, IC)).astype(np.float32)
+    W = RNG.standard_normal((OC, FH, FW, IC)).astype(np.float32)
+    Y = oracle.conv3D(X, W, sh, sw, ph, pw)
+    R = _conv_numpy(X, W, sh, sw, ph, pw)
+    assert Y.shape == R.shape
+    assert np.array_equal(Y, R.astype(np.float32))          # FP64 accumulation rounded once: same floats
+    # integer inputs: the float accumulator variant is exact too
+    Xi = RNG.integers(-3, 4, X.shape).astype(np.float32)
+    Wi = RNG.integers(-3, 4, W.shape).astype(np.float32)
+    assert np.array_equal(oracle.conv3D(Xi, Wi, sh, sw, ph, pw, acc32=True), _conv_numpy(Xi, Wi, sh, sw, ph, pw))
+
+
+def test_conv_oracle_special_cases():
+    # a 1x1 filter is a matrix product over the channels
+    X = RNG.standard_normal((2, 4, 5, 6)).astype(np.float32)
+    W = RNG.standard_normal((7, 1, 1, 6)).astype(np.float32)
+    Y = oracle.conv3D(X, W, 1, 1, 0, 0)
+    assert np.allclose(Y.reshape(-1, 7), X.reshape(-1, 6).astype(np.float64) @ W.reshape(7, 6).T.astype(np.float64),
+                       rtol=1e-6, atol=1e-6)
+    # a one-hot filter copies a shifted channel; the border comes from the zero padding
+    W1 = np.zeros((1, 3, 3, 6), np.float32); W1[0, 0, 2, 4] = 1.0        # picks X[ih-1, iw+1, channel 4]
+    Y1 = oracle.conv3D(X, W1, 1, 1, 1, 1)[..., 0]
+    exp = np.zeros_like(Y1); exp[:, 1:, :-1] = X[:, :-1, 1:, 4]
+    assert np.array_equal(Y1, exp)
+    # linear in W
+    Wa = RNG.standard_normal((3, 3, 3, 6)).astype(np.float32)
+    Wb = RNG.standard_normal((3, 3, 3, 6)).astype(np.float32)
+    ya, yb = oracle.conv3D(X, Wa, 2, 1, 1, 0), oracle.conv3D(X, Wb, 2, 1, 1, 0)
+    assert np.allclose(oracle.conv3D(X, Wa + Wb, 2, 1, 1, 0), ya + yb, rtol=1e-5, atol=1e-5)
+
+
 def test_reference_micro_helpers_when_built():
     ref = oracle.load_ref()
     if ref is None:
