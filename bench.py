@@ -83,11 +83,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias,attention,transpose,transfer",
-                    help="which of the other workloads to time (default 3,4,5,bias,attention,transpose,"
-                         "transfer): BASELINE configs 3, 4, 5, the biased fully-connected layer, the "
-                         "attention chain, dimension swaps, "
-                         "tensor upload / download")
+    ap.add_argument("--configs", default="3,4,5,bias,attention,conv,transpose,transfer",
+                    help="which of the other workloads to time (default all): BASELINE configs 3, 4, 5, "
+                         "the biased fully-connected layer, the attention chain, the forward convolution, "
+                         "dimension swaps, tensor upload / download")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
                          "(the known-size copy that FETCH_SIZE / WRITE_SIZE are scaled by)")
@@ -381,6 +380,34 @@ def main():
         record("attention chain with a separate sdiv launch (4 launches)", fl_chain, ms)
         for x in (dQ, dK, dV, dP, dO):
             x.free()
+
+    if "conv" in extra:
+        # forward convolution as an implicit GEMM: the shape of the reference's own speed test
+        # (test/cuda/conv3D/Cuda_conv3D_test.java main: 64x64 images, batch 64, 64 -> 64 channels, 7x7) and
+        # the 3x3 layers its commented alternatives list; flops = 2 * GN * GM * GK as that test counts them
+        log("convolution ...")
+        CV = dh.Cuda_conv3D
+        g = synthetic.stream_for(7)
+        for (IH, IW, Nc, IC, OC, FH, FW, st, pd) in ((64, 64, 64, 64, 64, 7, 7, 1, 3), (32, 32, 128, 128, 128, 3, 3, 1, 1),
+                                                     (16, 16, 128, 256, 256, 3, 3, 1, 1), (8, 8, 128, 512, 512, 3, 3, 1, 1),
+                                                     (64, 64, 128, 64, 128, 3, 3, 2, 1), (32, 32, 128, 256, 256, 1, 1, 1, 0)):
+            OH, OW = (IH - FH + 2 * pd) // st + 1, (IW - FW + 2 * pd) // st + 1
+            dXc = dh.DeviceArray(g.normal((Nc * IH * IW * IC,), 0.0, 1.0))
+            dWc = dh.DeviceArray(g.normal((OC * FH * FW * IC,), 0.0, 0.05))
+            dbc = dh.DeviceArray(g.normal((OC,), 0.0, 1.0))
+            dYc = dh.DeviceArray(size=Nc * OH * OW * OC)
+            flc = 2.0 * OC * (Nc * OH * OW) * (FH * FW * IC)
+            name = "conv3D X[%d,%d,%d,%d] W[%d,%d,%d,%d] s%d p%d" % (Nc, IH, IW, IC, OC, FH, FW, IC, st, pd)
+            ms = timer.per_launch_ms(lambda: CV.conv3D(
+                S, 1, dXc.address, IH, IW, dWc.address, FH, FW, dYc.address, OH, OW, Nc, IC, OC, st, st, pd, pd),
+                iters=20)
+            record(name, flc, ms)
+            ms = timer.per_launch_ms(lambda: CV.conv3D_biased(
+                S, 1, dXc.address, IH, IW, dWc.address, FH, FW, dYc.address, OH, OW, Nc, IC, OC, st, st, pd, pd,
+                dbc.address, Nc * OH * OW * OC, OC), iters=20)
+            record(name + " + bias", flc, ms)
+            for x in (dXc, dWc, dbc, dYc):
+                x.free()
 
     if "transpose" in extra:
         # the layout step of attention blocks: [B, S, H, D] <-> [B, H, S, D] (whole rows move) and the

@@ -200,6 +200,33 @@ class Engine:
     def matMul_biased(self, *t):
         return self._fullconnect(4, t, 3)
 
+    # ---- forward convolution over NHWC tensors (Engine.java:2076-2204) ----
+    def conv3D(self, *a, Bias=None):
+        """conv3D(Y, X, W, sh, sw[, ph, pw]) writes into Y (padding derived from the shapes when omitted);
+        conv3D(X, W, sh, sw, ph, pw) or conv3D(X, W, OH, OW, sh, sw, ph, pw) creates Y."""
+        n_t = sum(1 for x in a if isinstance(x, Tensor) or x is None)
+        ts, num = a[:n_t], [int(v) for v in a[n_t:]]
+        hs = [x._h if x is not None else None for x in ts]
+        hb = Bias._h if Bias is not None else None
+        if n_t == 3:
+            sh, sw, ph, pw = num if len(num) == 4 else (num[0], num[1], -1, -1)
+            rc = lib.dragon_engine_conv3D_into(self._h, hs[0], hs[1], hs[2], sh, sw, ph, pw, hb)
+            if rc:
+                _raise(rc)
+            return ts[0]
+        OH, OW, sh, sw, ph, pw = num if len(num) == 6 else [-1, -1] + num
+        return self._wrap(lib.dragon_engine_conv3D(self._h, hs[0], hs[1], OH, OW, sh, sw, ph, pw, hb))
+
+    @staticmethod
+    def conv3D_GEMM_nstream(GM, OC):
+        return lib.dragon_policy_conv3D_GEMM_nstream(GM, OC)
+
+    def conv3D_biased(self, *a):
+        """The argument lists of conv3D with the Bias tensor last."""
+        if a[-1] is None:
+            raise NullPointerException("Bias is null")
+        return self.conv3D(*a[:-1], Bias=a[-1])
+
     def linear2_row(self, inplace, X1, X2, alpha, beta, gamma):
         h = lib.dragon_engine_linear2_row(self._h, int(inplace), X1._h if X1 else None,
                                           X2._h if X2 else None, alpha, beta, gamma)

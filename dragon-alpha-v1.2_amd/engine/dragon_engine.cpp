@@ -4,6 +4,7 @@
 
 #include <string.h>
 
+#include "../../include/dragon_hip_conv.h"
 #include "../../include/dragon_hip_gemm.h"
 #include "../../include/dragon_hip_runtime.h"
 
@@ -122,6 +123,18 @@ private:
     CudaStreamPool* pool_;
     int64_t stream_, event_ = 0;
     bool called_ = false;
+};
+
+struct FreeAfter : Syncer {     // Syncer.dual(sc1, () -> core.free(old)): wait, then release the old memory
+    SyncerPtr first; EngineCore* core; int64_t size, address; bool done = false;
+    FreeAfter(SyncerPtr f, EngineCore* c, int64_t s, int64_t a) : first(std::move(f)), core(c), size(s), address(a) {}
+    ~FreeAfter() override { try { sync(); } catch (...) {} }
+    void sync() override {
+        if (done) return;
+        first->sync();
+        core->free(size, address);
+        done = true;
+    }
 };
 
 std::mutex g_cuda_class_lock;  // the reference serialises setDevice+malloc/free on Cuda.class
@@ -294,6 +307,28 @@ int CudaFloat32EngineBase::matMul_gridZ(int N, int M, int K) const {
     SplitKKnobs k = {matMul_sk_threshold, matMul_sk_maxPart, matMul_sk_minBlock_perSM, matMul_sk_maxBlock_perSM};
     return policy_matMul_gridZ(N, M, K, dev_.multiProcessorCount(), k);
 }
+// Cuda_conv3D.java:264-327: one stream per power-of-two piece of each extent, ten at most
+static int conv_pieces(int G) {
+    if ((G & (G - 1)) == 0) return 1;
+    int s = 0;
+    for (int bit = 128; bit >= 4; bit >>= 1) {
+        if (G >= bit) s++;
+        G &= bit - 1;
+        if (G == 0) break;
+    }
+    return s;
+}
+int policy_conv3D_GEMM_nstream(int GM, int OC) {
+    const int size = conv_pieces(OC) * conv_pieces(GM);
+    return size < 10 ? size : 10;
+}
+int policy_conv3D_GEMMV2_nstream(int N, int OC) { return policy_conv3D_GEMM_nstream(N, OC); }
+float policy_conv3D_psu(int IH, int IW, int OH, int OW, int FH, int FW, int sh, int sw) {   // :18-22
+    const int input_size = IH * IW;
+    const int pad_size = ((OH - 1) * sh + FH) * ((OW - 1) * sw + FW);
+    return 1.0f * pad_size / input_size;
+}
+
 int CudaFloat32EngineBase::matMul_biased_gridZ(int N, int M, int K) const {
     SplitKKnobs k = {matMul_sk_threshold, matMul_sk_maxPart, matMul_sk_minBlock_perSM, matMul_sk_maxBlock_perSM};
     return policy_matMul_biased_gridZ(N, M, K, dev_.multiProcessorCount(), k);
@@ -515,6 +550,110 @@ SyncerPtr CudaFloat32EngineBase::linear2_2D_row(int64_t Y, int64_t X1, int64_t X
     cu(dragon_Cuda_function_linear_dual2D_row(stream, X1, X2, row_lengthv, alpha, beta, gamma, Y,
                                               lengthv, width, stride));
     return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
+}
+// CudaFloat32EngineBase.java:2258-2383 (conv3D), :2386-2545 (conv3D_biased).  The reference chooses among
+// kernel families; every family is the same MFMA kernel here, so what remains of the dispatch is which
+// native is called (it documents the shape class) and the stream / event protocol.
+SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W,
+                                          int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph,
+                                          int pw, int64_t Bias, int lengthv, int width) {
+    const int GM = N * OH * OW;
+    const bool w1 = (FH == 1) && (FW == 1) && (sh == 1) && (sw == 1) && (ph == 0) && (pw == 0);
+    if (conv3D_remode && (OC > 31) && (GM > 31)) {
+        // stage 1: W -> CW on its own stream; stage 2 waits for it
+        const int GK = FH * FW * IC;
+        EngineCore::Block block = core_->malloc(GK * OC);
+        int64_t stream = 0;
+        std::vector<int64_t> s;
+        try {
+            stream = streamPool_->getStream();
+            cu(dragon_Cuda_conv3D_kernel_remode(stream, W, block.address, FH, FW, OC, IC));
+            int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+            cu(dragon_Cuda_eventRecord(event, stream));
+            s = streamPool_->getStreamArray(policy_conv3D_GEMM_nstream(GM, OC));
+            const int n = (int)s.size();
+            last_gridZ = 1; last_stream_count = n;
+            cu(dragon_Cuda_streamsWaitEvent_default(s.data(), n, event));
+            if (w1)
+                cu(dragon_Cuda_conv3D_conv3D_GemmR_W1(s.data(), n, X, IH, IW, W, block.address, Y, N, IC, OC));
+            else if (conv3D_Gemm_useTexture)
+                cu(dragon_Cuda_conv3D_conv3D_GemmR_texture(s.data(), n, X, IH, IW, W, block.address, FH, FW, Y,
+                                                           OH, OW, N, IC, OC, sh, sw, ph, pw));
+            else
+                cu(dragon_Cuda_conv3D_conv3D_GemmR(s.data(), n, X, IH, IW, W, block.address, FH, FW, Y, OH, OW,
+                                                   N, IC, OC, sh, sw, ph, pw));
+            cu(dragon_Cuda_deleteEvent(event));
+            if (Bias) {   // stage 3 on the first stream, after stage 2
+                int64_t event2 = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+                cu(dragon_Cuda_eventRecord_streams(event2, s.data(), n));
+                cu(dragon_Cuda_streamWaitEvent_default(stream, event2));
+                cu(dragon_Cuda_function_linear_dual2D_row(stream, Y, Bias, OC, 1.0f, 1.0f, 0.0f, Y, lengthv,
+                                                          width, OC));
+                cu(dragon_Cuda_deleteEvent(event2));
+            }
+        } catch (...) {
+            if (stream) {   // the block may be in use by what was issued: drain before it goes back
+                dragon_Cuda_streamSynchronize(stream);
+                streamPool_->returnStream(stream);
+            }
+            if (!s.empty()) {
+                for (int64_t q : s) dragon_Cuda_streamSynchronize(q);
+                streamPool_->returnStreamArray(s);
+            }
+            core_->free(block.size, block.address);
+            throw;
+        }
+        s.insert(s.begin(), stream);   // Vector.append(stream, streamArray): the syncer waits for all of them
+        return SyncerPtr(new FreeAfter(SyncerPtr(new StreamArraySyncer(streamPool_.get(), s)), core_,
+                                       block.size, block.address));
+    }
+    const bool V2 = (N > 127) && (OC > 127) &&
+                    policy_conv3D_psu(IH, IW, OH, OW, FH, FW, sh, sw) >= conv3D_GemmV2_Q;
+    std::vector<int64_t> s = streamPool_->getStreamArray(V2 ? policy_conv3D_GEMMV2_nstream(N, OC)
+                                                            : policy_conv3D_GEMM_nstream(GM, OC));
+    const int n = (int)s.size();
+    last_gridZ = 1; last_stream_count = n;
+    const bool useTexture = conv3D_Gemm_useTexture && (OC > 15);
+    try {
+        if (Bias && conv3D_biased_fused)
+            cu(dragon_Cuda_conv3D_conv3D_biased(s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh,
+                                                sw, ph, pw, Bias, lengthv, width));
+        else {
+            if (w1)
+                cu(dragon_Cuda_conv3D_conv3D_W1(s.data(), n, X, IH, IW, W, Y, N, IC, OC));
+            else if ((ph == 0) && (pw == 0))
+                cu(dragon_Cuda_conv3D_conv3D_np(s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw));
+            else if (V2)
+                cu(dragon_Cuda_conv3D_conv3DV2(useTexture, s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC,
+                                               OC, sh, sw, ph, pw));
+            else if (useTexture)
+                cu(dragon_Cuda_conv3D_conv3D_texture(s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC,
+                                                     sh, sw, ph, pw));
+            else
+                cu(dragon_Cuda_conv3D_conv3D(s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw,
+                                             ph, pw));
+            if (Bias) {   // the second launch, on streams[0] after every stream of the first
+                int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+                cu(dragon_Cuda_eventRecord_streams(event, s.data(), n));
+                cu(dragon_Cuda_streamWaitEvent_default(s[0], event));
+                cu(dragon_Cuda_function_linear_dual2D_row(s[0], Y, Bias, OC, 1.0f, 1.0f, 0.0f, Y, lengthv,
+                                                          width, OC));
+                cu(dragon_Cuda_deleteEvent(event));
+            }
+        }
+    } catch (...) { streamPool_->returnStreamArray(s); throw; }
+    return SyncerPtr(new StreamArraySyncer(streamPool_.get(), s));
+}
+SyncerPtr CudaFloat32EngineBase::conv3D(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W,
+                                        int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph,
+                                        int pw) {
+    return run_conv(Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, 0, 0, 0);
+}
+SyncerPtr CudaFloat32EngineBase::conv3D_biased(int64_t Y, int OH, int OW, int64_t X, int IH, int IW,
+                                               int64_t W, int FH, int FW, int N, int IC, int OC, int sh,
+                                               int sw, int ph, int pw, int64_t Bias, int lengthv, int width) {
+    if (Bias == 0) throw NullPointerException("Tensor Bias is null");
+    return run_conv(Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, Bias, lengthv, width);
 }
 SyncerPtr CudaFloat32EngineBase::transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X,
                                            const std::vector<int>& Xdim, int dimIndex1, int dimIndex2,
@@ -742,6 +881,53 @@ SyncerPtr EngineCore::matMul_biased(int64_t C, int64_t A, int64_t B, int N, int 
     }
     return base_->matMul_biased(C, A, B, pad4(N), M_4x, pad4(K), Bias, lengthv, M);
 }
+// EngineCore.java:816-845
+void EngineCore::conv3D_param_check(int OH, int OW, int IH, int IW, int FH, int FW, int N, int IC, int OC,
+                                    int sh, int sw, int ph, int pw) const {
+    auto s = [](long long v) { return std::to_string(v); };
+    if (OH <= 0) throw IllegalArgumentException("OH { got " + s(OH) + " } must > 0");
+    if (OW <= 0) throw IllegalArgumentException("OW { got " + s(OW) + " } must > 0");
+    if (N <= 0) throw IllegalArgumentException("N  { got " + s(N) + " } must > 0");
+    if (IC <= 0) throw IllegalArgumentException("IC { got " + s(IC) + " } must > 0");
+    if (OC <= 0) throw IllegalArgumentException("OC { got " + s(OC) + " } must > 0");
+    if (sh <= 0) throw IllegalArgumentException("sh { got " + s(sh) + " } must > 0");
+    if (sw <= 0) throw IllegalArgumentException("sw { got " + s(sw) + " } must > 0");
+    if (ph < 0) throw IllegalArgumentException("ph { got " + s(ph) + " } must >= 0");
+    if (pw < 0) throw IllegalArgumentException("pw { got " + s(pw) + " } must >= 0");
+    if (FH <= ph) throw IllegalArgumentException("FH { got " + s(FH) + " } <= ph { got " + s(ph) + " }");
+    if (FW <= pw) throw IllegalArgumentException("FW { got " + s(FW) + " } <= pw { got " + s(pw) + " }");
+    if (FH < sh) throw IllegalArgumentException("FH { got " + s(FH) + " } < sh { got " + s(sh) + " }");
+    if (FW < sw) throw IllegalArgumentException("FW { got " + s(FW) + " } < sw { got " + s(sw) + " }");
+    if (FH > IH + (ph << 1))
+        throw IllegalArgumentException("FH { got " + s(FH) + " } > IH { got " + s(IH) + " } + 2 * ph { " + s(ph) + " }");
+    if (FW > IW + (pw << 1))
+        throw IllegalArgumentException("FW { got " + s(FW) + " } > IW { got " + s(IW) + " } + 2 * pw { " + s(pw) + " }");
+}
+SyncerPtr EngineCore::conv3D(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH, int FW,
+                             int N, int IC, int OC, int sh, int sw, int ph, int pw) {   // :848-869
+    if (check) {
+        if (Y == 0) throw NullPointerException("Tensor Y is null");
+        if (X == 0) throw NullPointerException("Tensor X is null");
+        if (W == 0) throw NullPointerException("Tensor W is null");
+        conv3D_param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw);
+    }
+    return base_->conv3D(Y, OH, OW, X, IH, IW, W, FH, FW, pad4(N), pad4(IC), pad4(OC), sh, sw, ph, pw);
+}
+SyncerPtr EngineCore::conv3D_biased(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH,
+                                    int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                    int64_t Bias, int lengthv) {   // :871-898
+    const int OC_4x = pad4(OC);
+    if (check) {
+        if (Y == 0) throw NullPointerException("Tensor Y is null");
+        if (X == 0) throw NullPointerException("Tensor X is null");
+        if (W == 0) throw NullPointerException("Tensor W is null");
+        conv3D_param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw);
+        if (Bias == 0) throw NullPointerException("Tensor Bias is null");
+        func_param_check_row(lengthv, OC_4x, OC, OC_4x);
+    }
+    return base_->conv3D_biased(Y, OH, OW, X, IH, IW, W, FH, FW, pad4(N), pad4(IC), OC_4x, sh, sw, ph, pw,
+                                Bias, lengthv, OC);
+}
 SyncerPtr EngineCore::linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                                      float beta, float gamma, int lengthv, int width) {   // :1965-1983
     const int stride = pad4(width);
@@ -966,6 +1152,59 @@ Tensor* Engine::matMul_biased(Tensor* C, Tensor* A, Tensor* B, Tensor* Bias) {
     finish(C, core_->matMul_biased(C->address, A->address, B->address, A->dim[0], B->dim[1], A->dimAt(1),
                                    Bias->address, C->lengthv));
     return C;
+}
+// Engine.java:2076-2204.  Y given: the padding defaults are derived from the shapes, rounded up.
+Tensor* Engine::conv3D(Tensor* Y, Tensor* X, Tensor* W, int sh, int sw, int ph, int pw) {
+    return conv3D_biased(Y, X, W, sh, sw, ph, pw, nullptr);
+}
+Tensor* Engine::conv3D_biased(Tensor* Y, Tensor* X, Tensor* W, int sh, int sw, int ph, int pw, Tensor* Bias) {
+    require(Y, "Y"); require(X, "X"); require(W, "W");
+    if (check_) {
+        equals(Y->ndim(), "Y.ndim", 4, "4"); equals(X->ndim(), "X.ndim", 4, "4"); equals(W->ndim(), "W.ndim", 4, "4");
+        equals(Y->dimAt(0), "Y.batch", X->dimAt(0), "X.batch");
+        equals(W->dimAt(0), "W.OC", Y->dimAt(3), "Y.OC");
+        equals(W->dimAt(3), "W.IC", X->dimAt(3), "X.IC");
+        if (Bias) equals(Bias->lastDim(), "Bias.lastDim", W->dimAt(0), "W.OC");
+    }
+    const int OH = Y->dim[1], OW = Y->dim[2];
+    const int XN = X->dim[0], IH = X->dim[1], IW = X->dim[2];
+    const int WOC = W->dim[0], FH = W->dim[1], FW = W->dim[2], WIC = W->dim[3];
+    if (ph == -1) ph = ((OH - 1) * sh + FH - IH + 1) >> 1;
+    if (pw == -1) pw = ((OW - 1) * sw + FW - IW + 1) >> 1;
+    finish(Y, Bias ? core_->conv3D_biased(Y->address, OH, OW, X->address, IH, IW, W->address, FH, FW, XN, WIC, WOC,
+                                          sh, sw, ph, pw, Bias->address, Y->lengthv)
+                   : core_->conv3D(Y->address, OH, OW, X->address, IH, IW, W->address, FH, FW, XN, WIC, WOC, sh,
+                                   sw, ph, pw));
+    return Y;
+}
+// Y created: the output size defaults are derived from the padding, rounded down
+Tensor* Engine::conv3D(Tensor* X, Tensor* W, int OH, int OW, int sh, int sw, int ph, int pw) {
+    return conv3D_biased(X, W, OH, OW, sh, sw, ph, pw, nullptr);
+}
+Tensor* Engine::conv3D_biased(Tensor* X, Tensor* W, int OH, int OW, int sh, int sw, int ph, int pw,
+                              Tensor* Bias) {
+    require(X, "X"); require(W, "W");
+    if (check_) {
+        equals(X->ndim(), "X.ndim", 4, "4"); equals(W->ndim(), "W.ndim", 4, "4");
+        equals(W->dimAt(3), "W.IC", X->dimAt(3), "X.IC");
+        if (Bias) equals(Bias->lastDim(), "Bias.lastDim", W->dimAt(0), "W.OC");
+        if (sh <= 0 || sw <= 0) throw IllegalArgumentException("sh, sw must > 0");
+    }
+    const int XN = X->dim[0], IH = X->dim[1], IW = X->dim[2];
+    const int WOC = W->dim[0], FH = W->dim[1], FW = W->dim[2], WIC = W->dim[3];
+    if (OH == -1) OH = (IH - FH + (ph << 1)) / sh + 1;
+    if (OW == -1) OW = (IW - FW + (pw << 1)) / sw + 1;
+    if (check_ && (OH <= 0 || OW <= 0))
+        throw IllegalArgumentException("OH { got " + std::to_string(OH) + " }, OW { got " + std::to_string(OW) +
+                                       " } must > 0");
+    Tensor* Y = &empty({XN, OH, OW, WOC})->c();
+    try {
+        finish(Y, Bias ? core_->conv3D_biased(Y->address, OH, OW, X->address, IH, IW, W->address, FH, FW, XN, WIC,
+                                              WOC, sh, sw, ph, pw, Bias->address, Y->lengthv)
+                       : core_->conv3D(Y->address, OH, OW, X->address, IH, IW, W->address, FH, FW, XN, WIC, WOC,
+                                       sh, sw, ph, pw));
+    } catch (...) { deleteTensor(Y); throw; }
+    return Y;
 }
 Tensor* Engine::matMulT1(Tensor* A, Tensor* B) {
     require(A, "A"); require(B, "B");
@@ -1216,17 +1455,6 @@ Tensor* Engine::fullconnect_deltaW(Tensor* X, Tensor* deltaY) {   // deltaW = X^
 // Engine.java:1797-1831.  The reference supports 2 to 4 dimensions (anything else falls through to
 // its 2-D native with the wrong shape); here more than 4 is refused.
 namespace {
-struct FreeAfter : Syncer {     // Syncer.dual(sc1, () -> core.free(old)): wait, then release the old memory
-    SyncerPtr first; EngineCore* core; int64_t size, address; bool done = false;
-    FreeAfter(SyncerPtr f, EngineCore* c, int64_t s, int64_t a) : first(std::move(f)), core(c), size(s), address(a) {}
-    ~FreeAfter() override { try { sync(); } catch (...) {} }
-    void sync() override {
-        if (done) return;
-        first->sync();
-        core->free(size, address);
-        done = true;
-    }
-};
 }  // namespace
 Tensor* Engine::copy(Tensor* X) {
     require(X, "X");

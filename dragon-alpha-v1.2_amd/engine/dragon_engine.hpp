@@ -112,6 +112,10 @@ int policy_matMul_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
 int policy_matMul_biased_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
 int policy_matMulT1_gridZ(int N, int M, int K, int SM, const SplitKKnobs& k);
 int policy_matMulT2_gridZ(int N, int M, int K, int SM, const SplitKKnobs& t2, const SplitKKnobs& mm);
+// stream counts and the "padding scale up" ratio of the convolution natives (Cuda_conv3D.java:18-28, 264-327)
+int policy_conv3D_GEMM_nstream(int GM, int OC);
+int policy_conv3D_GEMMV2_nstream(int N, int OC);
+float policy_conv3D_psu(int IH, int IW, int OH, int OW, int FH, int FW, int sh, int sw);
 
 // ---- the engine "plugin": split-K policy, stream checkout, event protocol -----------------------
 class CudaFloat32EngineBase {
@@ -137,6 +141,16 @@ public:
     // Not a field of the Java class: when set (the default) an unsplit matMul_biased adds the bias
     // row inside the product's launch; when cleared it issues the reference's two launches.
     bool matMul_biased_fused = true;
+    // Convolution knobs.  conv3D_remode is the Java field (CudaFloat32EngineBase.java:2025): re-order W to
+    // CW[FH, FW, IC, OC] in a temporary block and call the GemmR natives.  The Java default is true because
+    // its CUDA kernels read CW faster; the MFMA kernel reads W as stored and never touches CW, so the
+    // default here is false (one launch, no temporary block).  Set it to get the reference's sequence.
+    bool conv3D_remode = false;
+    bool conv3D_Gemm_useTexture = true;
+    float conv3D_GemmV2_Q = 1.25f;
+    // Not a Java field: conv3D_biased adds the bias inside the convolution's launch (default) or issues the
+    // reference's second launch linear_dual2D_row.
+    bool conv3D_biased_fused = true;
 
     void matMul_splitK_threshold(int threshold);     // must be a positive power of two
     void matMul_splitK_maxPart(int maxPart);         // must be >= 4
@@ -170,6 +184,12 @@ public:
     SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
     SyncerPtr linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                              float beta, float gamma, int lengthv, int width, int stride);
+    // forward convolution; Bias = 0 for the plain form.  N, IC, OC arrive padded by EngineCore
+    SyncerPtr conv3D(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH, int FW,
+                     int N, int IC, int OC, int sh, int sw, int ph, int pw);
+    SyncerPtr conv3D_biased(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH, int FW,
+                            int N, int IC, int OC, int sh, int sw, int ph, int pw, int64_t Bias,
+                            int lengthv, int width);
     SyncerPtr transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X, const std::vector<int>& Xdim,
                         int dimIndex1, int dimIndex2, int strideX, int strideY, int length);
     SyncerPtr linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv, int width, int stride);
@@ -187,6 +207,9 @@ public:
 private:
     SyncerPtr run_2d(int variant, int gridZ, int64_t C, int64_t A, int64_t B, int N, int M, int K,
                      int64_t Bias = 0, int lengthv = 0, int width = 0);
+    SyncerPtr run_conv(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH, int FW,
+                       int N, int IC, int OC, int sh, int sw, int ph, int pw, int64_t Bias, int lengthv,
+                       int width);
     CudaDevice dev_;
     std::unique_ptr<CudaStreamPool> streamPool_;
     std::unique_ptr<PinnedMempool> bufPool_;
@@ -219,6 +242,10 @@ public:
     SyncerPtr matMulT2(int64_t C, int64_t A, int64_t B, int N, int M, int K);
     SyncerPtr linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                              float beta, float gamma, int lengthv, int width);
+    SyncerPtr conv3D(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH, int FW,
+                     int N, int IC, int OC, int sh, int sw, int ph, int pw);
+    SyncerPtr conv3D_biased(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W, int FH, int FW,
+                            int N, int IC, int OC, int sh, int sw, int ph, int pw, int64_t Bias, int lengthv);
     SyncerPtr transpose(int64_t Y, const std::vector<int>& Ydim, int64_t X, const std::vector<int>& Xdim,
                         int dimIndex1, int dimIndex2, int widthX, int widthY, int length);
     SyncerPtr linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv, int width);
@@ -231,6 +258,8 @@ public:
 private:
     void matMul_check(int64_t C, int64_t A, int64_t B, int N, int M, int K) const;
     void func_param_check_row(int lengthv, int row_lengthv, int width, int stride) const;
+    void conv3D_param_check(int OH, int OW, int IH, int IW, int FH, int FW, int N, int IC, int OC, int sh,
+                            int sw, int ph, int pw) const;
     CudaFloat32EngineBase* base_;
     int64_t live_blocks_ = 0;
     std::mutex mu_;
@@ -294,6 +323,14 @@ public:
     Tensor* fullconnect_biased(Tensor* Y, Tensor* X, Tensor* W, Tensor* Bias);
     Tensor* fullconnect_deltaX(Tensor* deltaY, Tensor* W);
     Tensor* fullconnect_deltaW(Tensor* X, Tensor* deltaY);
+
+    // forward convolution over NHWC tensors: X[N, IH, IW, IC], W[OC, FH, FW, IC] -> Y[N, OH, OW, OC].
+    // With Y given, ph / pw = -1 derive the padding from the shapes (rounded up); without Y, OH / OW = -1
+    // derive the output size from the padding (rounded down).  Bias[OC] is added to every output pixel.
+    Tensor* conv3D(Tensor* Y, Tensor* X, Tensor* W, int sh, int sw, int ph = -1, int pw = -1);
+    Tensor* conv3D(Tensor* X, Tensor* W, int OH, int OW, int sh, int sw, int ph, int pw);
+    Tensor* conv3D_biased(Tensor* Y, Tensor* X, Tensor* W, int sh, int sw, int ph, int pw, Tensor* Bias);
+    Tensor* conv3D_biased(Tensor* X, Tensor* W, int OH, int OW, int sh, int sw, int ph, int pw, Tensor* Bias);
 
     // exchange of two dimensions (negative indices count from the end); inplace gives X the new
     // shape and memory and frees the old memory once the kernel is done

@@ -81,6 +81,9 @@ int dragon_engine_set_param(dragon_engine* eg, const char* name, int32_t v) {
         else if (n == "matMulT2_splitK_maxPart") b.matMulT2_splitK_maxPart(v);
         else if (n == "tf32") b.tf32(v != 0);
         else if (n == "matMul_biased_fused") b.matMul_biased_fused = (v != 0);
+        else if (n == "conv3D_remode") b.conv3D_remode = (v != 0);
+        else if (n == "conv3D_Gemm_useTexture") b.conv3D_Gemm_useTexture = (v != 0);
+        else if (n == "conv3D_biased_fused") b.conv3D_biased_fused = (v != 0);
         else if (n == "batchMatMul_useTexture") b.batchMatMul_useTexture = (v != 0);
         else if (n == "batchMatMulT2_useTexture") b.batchMatMulT2_useTexture = (v != 0);
         else if (n == "multiProcessorCount") {
@@ -103,6 +106,8 @@ int32_t dragon_engine_get_param(dragon_engine* eg, const char* name) {
         else if (n == "matMulT2_splitK_threshold") out = b.matMulT2_sk_threshold;
         else if (n == "matMulT2_splitK_maxPart") out = b.matMulT2_sk_maxPart;
         else if (n == "matMul_biased_fused") out = b.matMul_biased_fused ? 1 : 0;
+        else if (n == "conv3D_remode") out = b.conv3D_remode ? 1 : 0;
+        else if (n == "conv3D_biased_fused") out = b.conv3D_biased_fused ? 1 : 0;
         else if (n == "multiProcessorCount") out = b.device().multiProcessorCount();
         else if (n == "last_gridZ") out = b.last_gridZ;
         else if (n == "last_stream_count") out = b.last_stream_count;
@@ -257,6 +262,23 @@ int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor*
         }
     });
 }
+dragon_tensor* dragon_engine_conv3D(dragon_engine* eg, dragon_tensor* X, dragon_tensor* W, int32_t OH, int32_t OW,
+                                    int32_t sh, int32_t sw, int32_t ph, int32_t pw, dragon_tensor* Bias) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        t = eg->eg.conv3D_biased(T(X), T(W), OH, OW, sh, sw, ph, pw, Bias ? T(Bias) : nullptr);
+    });
+    return t ? wrap(t) : nullptr;
+}
+int dragon_engine_conv3D_into(dragon_engine* eg, dragon_tensor* Y, dragon_tensor* X, dragon_tensor* W, int32_t sh,
+                              int32_t sw, int32_t ph, int32_t pw, dragon_tensor* Bias) {
+    return guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        eg->eg.conv3D_biased(T(Y), T(X), T(W), sh, sw, ph, pw, Bias ? T(Bias) : nullptr);
+    });
+}
+int32_t dragon_policy_conv3D_GEMM_nstream(int32_t GM, int32_t OC) { return policy_conv3D_GEMM_nstream(GM, OC); }
 dragon_tensor* dragon_engine_linear(dragon_engine* eg, int32_t inplace, float alpha, dragon_tensor* X,
                                     float beta) {
     Tensor* t = nullptr;

@@ -103,6 +103,20 @@ dragon_tensor* dragon_engine_fullconnect(dragon_engine* eg, int32_t op, dragon_t
 int dragon_engine_fullconnect_into(dragon_engine* eg, int32_t op, dragon_tensor* Y,
                                    dragon_tensor* X, dragon_tensor* W, dragon_tensor* Bias);
 
+/* Engine.conv3D / conv3D_biased (Engine.java:2076-2204) over NHWC tensors X[N, IH, IW, IC],
+ * W[OC, FH, FW, IC] -> Y[N, OH, OW, OC]; Bias (NULL = none) is added to every output pixel.
+ * dragon_engine_conv3D creates Y: OH / OW = -1 derive the output size from the padding (rounded down).
+ * dragon_engine_conv3D_into writes into Y: ph / pw = -1 derive the padding from the shapes (rounded up).
+ * Parameters "conv3D_remode" (default 0 here; the Java default is 1) and "conv3D_biased_fused" (default
+ * 1; not a Java field) choose between one launch and the reference's launch sequences. */
+dragon_tensor* dragon_engine_conv3D(dragon_engine* eg, dragon_tensor* X, dragon_tensor* W, int32_t OH,
+                                    int32_t OW, int32_t sh, int32_t sw, int32_t ph, int32_t pw,
+                                    dragon_tensor* Bias);
+int dragon_engine_conv3D_into(dragon_engine* eg, dragon_tensor* Y, dragon_tensor* X, dragon_tensor* W,
+                              int32_t sh, int32_t sw, int32_t ph, int32_t pw, dragon_tensor* Bias);
+/* Cuda_conv3D.GEMM_nstream(GM, OC) (Cuda_conv3D.java:264-285): how many streams the engine checks out */
+int32_t dragon_policy_conv3D_GEMM_nstream(int32_t GM, int32_t OC);
+
 /* Engine.linear(inplace, alpha, X, beta): Y = alpha*X + beta (Engine.java:4005-4013); Engine.sdiv(X, C)
  * is linear(1/C, X, 0).  inplace != 0 writes into X and returns X itself. */
 dragon_tensor* dragon_engine_linear(dragon_engine* eg, int32_t inplace, float alpha, dragon_tensor* X,

@@ -170,3 +170,104 @@ def test_conv3D_argument_errors(dh, gpu):
         assert e.value.code == 1, bad
     dh.Cuda.streamSynchronize(0)
     d.free()
+
+
+# ---- engine level -----------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def eg(gpu):
+    from dragon_hip import engine
+    e = engine.cuda_float32(0, 32)
+    yield e
+    e.close()
+
+
+def check_conv(eg, rng, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw):
+    """testCorrect of test/cuda/conv3D/Cuda_conv3D_test.java:42-105: both forms of eg.conv3D against the
+    CPU loops by samePercent_relative at 1e-5, plus conv3D_biased == conv3D then add_row, exactly."""
+    OH, OW = (IH - FH + 2 * ph) // sh + 1, (IW - FW + 2 * pw) // sw + 1
+    X = rng.random(N * IH * IW * IC, dtype=np.float32)
+    W = rng.random(OC * FH * FW * IC, dtype=np.float32)
+    Bv = rng.random(OC, dtype=np.float32)
+    tX, tW, tB = eg.tensor(X, N, IH, IW, IC), eg.tensor(W, OC, FH, FW, IC), eg.tensor(Bv, OC)
+    tY1 = eg.conv3D(tX, tW, sh, sw, ph, pw)
+    tY2 = eg.conv3D(eg.empty(N, OH, OW, OC).c(), tX, tW, sh, sw)
+    assert tY1.dim == [N, OH, OW, OC]
+    Y1 = oracle.conv3D(X.reshape(N, IH, IW, IC), W.reshape(OC, FH, FW, IC), sh, sw, ph, pw).reshape(-1)
+    Y2, Y3 = eg.valueOf(tY1), eg.valueOf(tY2)
+    assert oracle.samePercent_relative(Y1, Y2, 1e-5) >= 0.999
+    if ((OH - 1) * sh + FH - IH + 1) >> 1 == ph and ((OW - 1) * sw + FW - IW + 1) >> 1 == pw:
+        assert np.array_equal(Y2, Y3)                          # the derived padding is the one given
+    tY4 = eg.conv3D_biased(tX, tW, sh, sw, ph, pw, tB)
+    tY5 = eg.add_row(True, eg.conv3D(tX, tW, OH, OW, sh, sw, ph, pw), tB)
+    assert np.array_equal(eg.valueOf(tY4), eg.valueOf(tY5))
+    tY6 = eg.conv3D_biased(eg.zeros(N, OH, OW, OC).c(), tX, tW, sh, sw, ph, pw, tB)
+    assert np.array_equal(eg.valueOf(tY4), eg.valueOf(tY6))
+    # pads of Y stay zero: images beyond N, channels beyond OC
+    from dragon_hip import Cuda
+    raw = np.empty(tY4.length_4x, np.float32)
+    Cuda.get1D(0, tY4.address, raw, tY4.length_4x)
+    raw = raw.reshape((N + 3) // 4 * 4, OH, OW, (OC + 3) // 4 * 4)
+    assert not raw[N:].any() and not raw[..., OC:].any()
+    eg.delete(tX, tW, tB, tY1, tY2, tY4, tY5, tY6)
+
+
+SHAPES = [(8, 8, 3, 3, 4, 16, 32, 1, 1, 1, 1), (9, 7, 3, 3, 3, 5, 33, 2, 2, 1, 1), (16, 16, 7, 7, 2, 8, 64, 1, 1, 3, 3),
+          (12, 12, 1, 1, 5, 128, 37, 1, 1, 0, 0), (33, 33, 5, 5, 4, 16, 19, 2, 2, 0, 0), (6, 10, 1, 7, 2, 6, 40, 1, 1, 0, 3),
+          (2, 2, 3, 3, 16, 32, 48, 2, 2, 1, 1)]
+
+
+@pytest.mark.parametrize("remode,fused", [(0, 1), (1, 1), (0, 0), (1, 0)])
+def test_engine_conv3D_like_the_reference(eg, remode, fused):
+    rng = np.random.default_rng(40 + 2 * remode + fused)
+    base = eg.get_param("live_blocks")
+    eg.set_param("conv3D_remode", remode)
+    eg.set_param("conv3D_biased_fused", fused)
+    try:
+        for g in SHAPES:
+            check_conv(eg, rng, *g)
+    finally:
+        eg.set_param("conv3D_remode", 0)
+        eg.set_param("conv3D_biased_fused", 1)
+    assert eg.get_param("live_blocks") == base                 # the re-ordered filter's block went back
+
+
+def test_engine_conv3D_async_and_stream_counts(eg):
+    rng = np.random.default_rng(50)
+    N, IH, IW, IC, OC = 4, 10, 10, 8, 36
+    X = rng.integers(-2, 3, (N, IH, IW, IC)).astype(np.float32)
+    W = rng.integers(-2, 3, (OC, 3, 3, IC)).astype(np.float32)
+    tX, tW = eg.tensor(X, N, IH, IW, IC), eg.tensor(W, OC, 3, 3, IC)
+    eg.sync(False)
+    try:
+        outs = [eg.conv3D(tX, tW, 1, 1, 1, 1) for _ in range(6)]
+        assert eg.get_param("last_stream_count") == eg.conv3D_GEMM_nstream(N * IH * IW, OC)
+        R = oracle.conv3D(X, W, 1, 1, 1, 1).reshape(-1)
+        for t in outs:
+            assert np.array_equal(eg.valueOf(t.c()), R)
+    finally:
+        eg.sync(True)
+    eg.delete(tX, tW, *outs)
+
+
+def test_engine_conv3D_error_behaviour(eg):
+    from dragon_hip.engine import IllegalArgumentException, NullPointerException
+    tX, tW = eg.zeros(2, 6, 6, 4), eg.zeros(8, 3, 3, 4)
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D(tX, eg.zeros(8, 3, 3, 5), 1, 1, 1, 1)        # W.IC != X.IC
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D(tX, tW, 1, 1, 3, 1)                          # FH <= ph
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D(tX, tW, 4, 1, 1, 1)                          # FH < sh
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D(tX, tW, 0, 1, 1, 1)
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D(eg.zeros(2, 2, 2, 4), eg.zeros(8, 5, 5, 4), 1, 1, 1, 1)   # FH > IH + 2 ph
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D(eg.zeros(2, 6, 6, 7), tX, tW, 1, 1)          # Y.OC != W.OC
+    with pytest.raises(IllegalArgumentException):
+        eg.conv3D_biased(tX, tW, 1, 1, 1, 1, eg.zeros(9))      # Bias.lastDim != OC
+    with pytest.raises(NullPointerException):
+        eg.conv3D(None, tW, 1, 1, 1, 1)
+    assert eg.conv3D_GEMM_nstream(64, 64) == 1 and eg.conv3D_GEMM_nstream(196, 36) == 6
+    assert eg.conv3D_GEMM_nstream(255 * 4, 252) == 10
