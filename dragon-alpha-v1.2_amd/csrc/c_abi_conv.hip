@@ -45,6 +45,7 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     p.cv_sh = sh; p.cv_sw = sw; p.cv_ph = ph; p.cv_pw = pw;
     p.cv_rcp_IC = 1.0f / (float)IC;
     p.cv_rcp_FW = 1.0f / (float)FW;
+    p.cv_walk = 1;
     if (dBias != 0) {
         if (!aligned16(dBias) || width <= 0 || width > OC || lengthv <= 0 || lengthv % OC != 0 ||
             lengthv / OC > GM)

@@ -55,6 +55,7 @@ struct GemmParams {
     // k_total = FH*FW*IC, B = W[OC, FH*FW*IC], C = Y[N*OH*OW, OC]
     int cv_IH, cv_IW, cv_IC, cv_FW, cv_OH, cv_OW, cv_sh, cv_sw, cv_ph, cv_pw;
     float cv_rcp_IC, cv_rcp_FW;
+    int cv_walk;          // 1: visit the K chunks filter-column fastest (see the kernel), 0: in storage order
     const float* bias;      // optional row vector added to C[i][j] for i < bias_rows, j < bias_width
     int bias_rows, bias_width;
     int tiles_m, tiles_n;   // filled by the launcher

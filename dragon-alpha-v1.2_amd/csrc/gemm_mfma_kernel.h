@@ -547,18 +547,43 @@ void gemm_f32_mfma(const GemmParams p) {
     __syncthreads();
     int buf = 0;
 
+    // Convolution: the order in which the K chunks of a tile are visited.  In storage order
+    // (filter row, filter column, channel) two uses of the same input element are IC/KT stages
+    // apart, and by then the other workgroups of the XCD have pushed it out of the L2.  With the
+    // filter column running fastest, consecutive stages read the same pixels shifted by one, so
+    // all but 1/OW of a stage's input is what the previous stage fetched.  Any order gives the
+    // same sum up to rounding; whole chunks only, so IC must be a multiple of KT.
+    const int cv_nic = CONV ? p.cv_IC / KT : 0;
+    const bool cv_walk = CONV && p.cv_walk && (p.cv_IC % KT == 0) && cv_nic > 1 && p.cv_FW > 1;
+    int cv_fw = 0, cv_ic = 0, cv_k = 0;
+
     for (;;) {
         const bool has_next = lid + G < total;
         TileCtx nxt = cur;
         const float* a_ptr = cur.a_ptr;
         const float* b_ptr = cur.b_ptr;
+        if constexpr (CONV) { cv_fw = 0; cv_ic = 0; cv_k = 0; }
         for (int it = 0; it < cur.nstage; it++) {
             const bool last = (it + 1 == cur.nstage);
             bool fetched = false;
             if (!last) {                 // next stage of this tile -> registers
                 a_ptr += a_step;
-                b_ptr += b_step;
-                const int knext = cur.k0 + (it + 1) * KT;
+                int knext;
+                if constexpr (CONV) {
+                    if (cv_walk) {       // next filter column; then next channel chunk; then next filter row
+                        cv_k += p.cv_IC;
+                        if (++cv_fw == p.cv_FW) {
+                            cv_fw = 0;
+                            cv_k += KT - p.cv_FW * p.cv_IC;
+                            if (++cv_ic == cv_nic) { cv_ic = 0; cv_k += (p.cv_FW - 1) * p.cv_IC; }
+                        }
+                    } else cv_k += KT;
+                    knext = cv_k;
+                    b_ptr = cur.b_ptr + cv_k;
+                } else {
+                    b_ptr += b_step;
+                    knext = cur.k0 + (it + 1) * KT;
+                }
                 if constexpr (CONV) la.load_conv(ra, a_ptr, cur.ka_lim - knext, knext, p);
                 else la.load(ra, a_ptr, cur.ka_lim - knext);
                 lb.load(rb, b_ptr, cur.kb_lim - knext);
