@@ -1,6 +1,7 @@
 // JNI shim: the exact symbols the reference's Java classes bind
 //   z.dragon.engine.cuda.impl.math.Cuda_matMul        (reference: Cuda_matMul/Cuda_matMul/A.cu:20-178)
 //   z.dragon.engine.cuda.impl.math.Cuda_batchMatMul   (reference: Cuda_batchMatMul/Cuda_batchMatMul/A.cu:20-143)
+//   z.dragon.engine.cuda.impl.math.Cuda_conv3D        (reference: Cuda_conv3D/Cuda_conv3D/A.cu:18-600)
 //   z.dragon.engine.cuda.impl.Cuda (the subset this path uses; reference: Cuda/Cuda/Cuda_memory.cuh,
 //   Cuda_Stream.cuh, Cuda_Event.cuh, Cuda_Device.cuh, Cuda_float.cuh)
 // each forwarding to the C ABI of include/dragon_hip_gemm.h / dragon_hip_runtime.h and turning a
@@ -16,6 +17,7 @@
 
 #include <vector>
 
+#include "../../../include/dragon_hip_conv.h"
 #include "../../../include/dragon_hip_gemm.h"
 #include "../../../include/dragon_hip_runtime.h"
 
@@ -76,6 +78,7 @@ std::vector<int64_t> long_array(JNIEnv* env, jlongArray arr, jint length) {
 #define RT(name) Java_z_dragon_engine_cuda_impl_Cuda_##name
 #define FN(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1function_##name
 #define EK(name) Java_z_dragon_engine_cuda_impl_Cuda_1expk2_##name
+#define CV(name) Java_z_dragon_engine_cuda_impl_math_Cuda_1conv3D_##name
 
 extern "C" {
 
@@ -135,6 +138,143 @@ JNIEXPORT void JNICALL FN(linear_1dual2D_1row)(JNIEnv* env, jclass, jlong stream
                                                jint stride) {
     handle(env, dragon_Cuda_function_linear_dual2D_row(stream, dX1, dX2, row_lengthv, alpha, beta, gamma,
                                                        dY, lengthv, width, stride));
+}
+
+// Y = alpha*X + beta (reference: Cuda_function/Cuda_function/A.cu:170-185)
+JNIEXPORT void JNICALL FN(linear2D)(JNIEnv* env, jclass, jlong stream, jfloat alpha, jlong dX, jfloat beta,
+                                    jlong dY, jint lengthv, jint width, jint stride) {
+    handle(env, dragon_Cuda_function_linear2D(stream, alpha, dX, beta, dY, lengthv, width, stride));
+}
+
+// ---- Cuda_conv3D: forward convolution (reference: Cuda_conv3D/Cuda_conv3D/A.cu:18-600) ----------
+JNIEXPORT void JNICALL CV(kernel_1remode)(JNIEnv* env, jclass, jlong stream, jlong dW, jlong dCW, jint FH,
+                                          jint FW, jint OC, jint IC) {
+    handle(env, dragon_Cuda_conv3D_kernel_remode(stream, dW, dCW, FH, FW, OC, IC));
+}
+#define DEF_CV(jname, cname)                                                                            \
+    JNIEXPORT void JNICALL CV(jname)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dX, \
+                                     jint IH, jint IW, jlong dW, jint FH, jint FW, jlong dY, jint OH,    \
+                                     jint OW, jint N, jint IC, jint OC, jint sh, jint sw, jint ph,       \
+                                     jint pw) {                                                          \
+        Streams st(env, streamArray, length);                                                            \
+        if (!st.ok) return;                                                                              \
+        handle(env, cname(st.s, st.n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph, pw));   \
+    }
+DEF_CV(conv3D, dragon_Cuda_conv3D_conv3D)
+DEF_CV(conv3D_1texture, dragon_Cuda_conv3D_conv3D_texture)
+JNIEXPORT void JNICALL CV(conv3DV2)(JNIEnv* env, jclass, jboolean useTexture, jlongArray streamArray,
+                                    jint length, jlong dX, jint IH, jint IW, jlong dW, jint FH, jint FW,
+                                    jlong dY, jint OH, jint OW, jint N, jint IC, jint OC, jint sh, jint sw,
+                                    jint ph, jint pw) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3DV2(useTexture, st.s, st.n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC,
+                                            OC, sh, sw, ph, pw));
+}
+JNIEXPORT void JNICALL CV(conv3D_1np)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dX,
+                                      jint IH, jint IW, jlong dW, jint FH, jint FW, jlong dY, jint OH, jint OW,
+                                      jint N, jint IC, jint OC, jint sh, jint sw) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3D_np(st.s, st.n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw));
+}
+JNIEXPORT void JNICALL CV(conv3D_1W1)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dX,
+                                      jint IH, jint IW, jlong dW, jlong dY, jint N, jint IC, jint OC) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3D_W1(st.s, st.n, dX, IH, IW, dW, dY, N, IC, OC));
+}
+#define DEF_CVR(jname, cname)                                                                           \
+    JNIEXPORT void JNICALL CV(jname)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dX, \
+                                     jint IH, jint IW, jlong dW, jlong dCW, jint FH, jint FW, jlong dY,  \
+                                     jint OH, jint OW, jint N, jint IC, jint OC, jint sh, jint sw,       \
+                                     jint ph, jint pw) {                                                 \
+        Streams st(env, streamArray, length);                                                            \
+        if (!st.ok) return;                                                                              \
+        handle(env, cname(st.s, st.n, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph,    \
+                          pw));                                                                          \
+    }
+DEF_CVR(conv3D_1GemmR, dragon_Cuda_conv3D_conv3D_GemmR)
+DEF_CVR(conv3D_1GemmR_1texture, dragon_Cuda_conv3D_conv3D_GemmR_texture)
+#define DEF_CVR_SGM(jname, cname)                                                                       \
+    JNIEXPORT void JNICALL CV(jname)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dX, \
+                                     jint IH, jint IW, jlong dW, jlong dCW, jint FH, jint FW, jlong dY,  \
+                                     jint OH, jint OW, jint N, jint IC, jint OC, jint sh, jint sw,       \
+                                     jint ph, jint pw, jint GM_slice) {                                  \
+        Streams st(env, streamArray, length);                                                            \
+        if (!st.ok) return;                                                                              \
+        handle(env, cname(st.s, st.n, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw, ph,    \
+                          pw, GM_slice));                                                                \
+    }
+DEF_CVR_SGM(conv3D_1GemmR_1SGM, dragon_Cuda_conv3D_conv3D_GemmR_SGM)
+DEF_CVR_SGM(conv3D_1GemmR_1texture_1SGM, dragon_Cuda_conv3D_conv3D_GemmR_texture_SGM)
+JNIEXPORT void JNICALL CV(conv3D_1GemmR_1W1)(JNIEnv* env, jclass, jlongArray streamArray, jint length,
+                                             jlong dX, jint IH, jint IW, jlong dW, jlong dCW, jlong dY, jint N,
+                                             jint IC, jint OC) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3D_GemmR_W1(st.s, st.n, dX, IH, IW, dW, dCW, dY, N, IC, OC));
+}
+JNIEXPORT void JNICALL CV(conv3D_1GemmR_1W1_1SGM)(JNIEnv* env, jclass, jlongArray streamArray, jint length,
+                                                  jlong dX, jint IH, jint IW, jlong dW, jlong dCW, jlong dY,
+                                                  jint N, jint IC, jint OC, jint GM_slice) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3D_GemmR_W1_SGM(st.s, st.n, dX, IH, IW, dW, dCW, dY, N, IC, OC, GM_slice));
+}
+JNIEXPORT void JNICALL CV(conv3D_1GemmV2R)(JNIEnv* env, jclass, jboolean useTexture, jlongArray streamArray,
+                                           jint length, jlong dX, jint IH, jint IW, jlong dW, jlong dCW,
+                                           jint FH, jint FW, jlong dY, jint OH, jint OW, jint N, jint IC,
+                                           jint OC, jint sh, jint sw, jint ph, jint pw) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3D_GemmV2R(useTexture, st.s, st.n, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW,
+                                                  N, IC, OC, sh, sw, ph, pw));
+}
+// the im2col-Winograd natives answer "handled" (true) or leave the work to the caller's next branch
+#define DEF_CVW(jname, cname)                                                                           \
+    JNIEXPORT jboolean JNICALL CV(jname)(JNIEnv* env, jclass, jboolean useTexture,                       \
+                                         jlongArray streamArray, jint length, jlong dX, jint IH,         \
+                                         jint IW, jlong dW, jlong dCW, jint FH, jint FW, jlong dY,       \
+                                         jint OH, jint OW, jint N, jint IC, jint OC, jint ph, jint pw) { \
+        Streams st(env, streamArray, length);                                                            \
+        if (!st.ok) return JNI_FALSE;                                                                    \
+        const int rc = cname(useTexture, st.s, st.n, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC, OC, \
+                             ph, pw);                                                                    \
+        if (rc < 0) { throwCudaException(env, -rc); return JNI_FALSE; }                                  \
+        return rc ? JNI_TRUE : JNI_FALSE;                                                                \
+    }
+DEF_CVW(conv3D_1Im2col_1Winograd_1s8_1R_1texture, dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s8_R_texture)
+DEF_CVW(conv3D_1Im2col_1Winograd_1s16_1R_1texture, dragon_Cuda_conv3D_conv3D_Im2col_Winograd_s16_R_texture)
+#define DEF_CVW_SGM(jname, cname)                                                                       \
+    JNIEXPORT jboolean JNICALL CV(jname)(JNIEnv* env, jclass, jboolean useTexture,                       \
+                                         jlongArray streamArray, jint length, jlong dX, jint IH,         \
+                                         jint IW, jlong dW, jlong dCW, jint FH, jint FW, jlong dY,       \
+                                         jint OH, jint OW, jint N, jint IC, jint OC, jint ph, jint pw,   \
+                                         jint GM_slice) {                                                \
+        Streams st(env, streamArray, length);                                                            \
+        if (!st.ok) return JNI_FALSE;                                                                    \
+        const int rc = cname(useTexture, st.s, st.n, dX, IH, IW, dW, dCW, FH, FW, dY, OH, OW, N, IC, OC, \
+                             ph, pw, GM_slice);                                                          \
+        if (rc < 0) { throwCudaException(env, -rc); return JNI_FALSE; }                                  \
+        return rc ? JNI_TRUE : JNI_FALSE;                                                                \
+    }
+DEF_CVW_SGM(conv3D_1Im2col_1WinogradR_1s8_1texture_1SGM, dragon_Cuda_conv3D_conv3D_Im2col_WinogradR_s8_texture_SGM)
+DEF_CVW_SGM(conv3D_1Im2col_1WinogradR_1s16_1texture_1SGM, dragon_Cuda_conv3D_conv3D_Im2col_WinogradR_s16_texture_SGM)
+
+// One launch for the convolution + bias row.  The reference has no such native: a maintainer who wants it
+// declares `public static native void conv3D_biased(long[] streamArray, int length, long dX_address, int IH,
+// int IW, long dW_address, int FH, int FW, long dY_address, int OH, int OW, int N, int IC, int OC, int sh,
+// int sw, int ph, int pw, long dBias_address, int lengthv, int width)` in Cuda_conv3D.java and calls it from
+// CudaFloat32EngineBase.conv3D_biased in place of the convolution native and linear_dual2D_row.
+JNIEXPORT void JNICALL CV(conv3D_1biased)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dX,
+                                          jint IH, jint IW, jlong dW, jint FH, jint FW, jlong dY, jint OH,
+                                          jint OW, jint N, jint IC, jint OC, jint sh, jint sw, jint ph, jint pw,
+                                          jlong dBias, jint lengthv, jint width) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_conv3D_conv3D_biased(st.s, st.n, dX, IH, IW, dW, FH, FW, dY, OH, OW, N, IC, OC, sh, sw,
+                                                 ph, pw, dBias, lengthv, width));
 }
 
 // ---- Cuda_expk2: dimension swap (reference: Cuda_expk2/Cuda_expk2/Cuda_transpose.cuh:13-75) ----

@@ -21,9 +21,11 @@ FILES = [
     "Cuda/Cuda/Cuda_float.cuh",
     "Cuda_function/Cuda_function/A.cu",
     "Cuda_expk2/Cuda_expk2/Cuda_transpose.cuh",
+    "Cuda_conv3D/Cuda_conv3D/A.cu",
 ]
-# of the element-wise library only the bias row belongs to the path
-ONLY = {"Cuda_function/Cuda_function/A.cu": {"Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear_1dual2D_1row"}}
+# of the element-wise library only the bias row and the scalar linear map belong to the path
+ONLY = {"Cuda_function/Cuda_function/A.cu": {"Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear_1dual2D_1row",
+                                             "Java_z_dragon_engine_cuda_impl_math_Cuda_1function_linear2D"}}
 out = []
 for f in FILES:
     text = open(os.path.join(CU, f), encoding="utf-8", errors="replace").read()

@@ -13,16 +13,20 @@ PREFIX = {"MM": "Java_z_dragon_engine_cuda_impl_math_Cuda_1matMul_",
           "BMM": "Java_z_dragon_engine_cuda_impl_math_Cuda_1batchMatMul_",
           "RT": "Java_z_dragon_engine_cuda_impl_Cuda_",
           "FN": "Java_z_dragon_engine_cuda_impl_math_Cuda_1function_",
-          "EK": "Java_z_dragon_engine_cuda_impl_Cuda_1expk2_"}
+          "EK": "Java_z_dragon_engine_cuda_impl_Cuda_1expk2_",
+          "CV": "Java_z_dragon_engine_cuda_impl_math_Cuda_1conv3D_"}
 
 
 def shim_names():
     text = open(SHIM).read()
     names = set()
-    for macro, arg in re.findall(r"JNICALL\s+(MM|BMM|RT|FN|EK)\((\w+)\)\s*\(", text):
-        names.add(PREFIX[macro] + arg)
+    for macro, arg in re.findall(r"JNICALL\s+(MM|BMM|RT|FN|EK|CV)\((\w+)\)\s*\(", text):
+        if arg != "jname":           # the macro bodies
+            names.add(PREFIX[macro] + arg)
     for kind, arg in re.findall(r"^DEF_(MM2D|MMSK|BMM|BMM_MMA)\((\w+),", text, flags=re.M):
         names.add(PREFIX["MM" if kind.startswith("MM") else "BMM"] + arg)
+    for arg in re.findall(r"^DEF_CV\w*\((\w+),", text, flags=re.M):
+        names.add(PREFIX["CV"] + arg)
     return names
 
 
@@ -41,8 +45,16 @@ def test_every_matmul_native_of_the_reference_is_in_the_shim():
 def test_bias_row_native_is_in_the_shim():
     g, s = golden(), shim_names()
     rows = {n for n, f in g.items() if "Cuda_function" in f}
-    assert rows == {PREFIX["FN"] + "linear_1dual2D_1row"}
+    assert rows == {PREFIX["FN"] + "linear_1dual2D_1row", PREFIX["FN"] + "linear2D"}
     assert rows <= s
+
+
+def test_every_convolution_native_of_the_reference_is_in_the_shim():
+    g, s = golden(), shim_names()
+    conv = {n for n, f in g.items() if "Cuda_conv3D" in f}
+    assert len(conv) == 17           # kernel_remode, 5 plain, 7 with the re-ordered filter, 4 im2col-Winograd
+    assert conv <= s, sorted(conv - s)
+    assert {n for n in s if n.startswith(PREFIX["CV"])} - conv == {PREFIX["CV"] + "conv3D_1biased"}
 
 
 def test_dimension_swap_natives_are_in_the_shim():
