@@ -1,0 +1,244 @@
+// Attention block in one launch on the FP32 matrix cores of gfx950:
+//     Y[b, i, :] = sum_j softmax_j(scale * <Q[b, i, :], K[b, j, :]>) * V[b, j, :]
+// which the reference computes as batchMatMulT2 -> sdiv -> softmax -> batchMatMul, with a
+// transpose(1, 2) on every tensor around them (nn/unit/complex/block/ChannelMHA.java:66-83 of
+// alpha-Dragon-v1.2/src/z/dragon).  Here the score matrix never reaches memory: a workgroup owns 128
+// queries of one (image, head), walks over the keys 32 at a time and keeps a running maximum, a
+// running sum and the un-normalised output per query ("online softmax").  Row strides are
+// arguments, so the [N, L, head, d] tensors of the layer are read and written where they lie and
+// the four transposes disappear as well.
+//
+// Both products are computed transposed, S^T = K.Q^T and Y^T = V^T.P^T, with
+// v_mfma_f32_32x32x2_f32.  In that instruction's result layout lane (c, h) holds column c, and a
+// column is a query in both S^T and Y^T: the maximum, the sum and the rescaling factor of a query
+// live in the lane that needs them (the two halves h of a wavefront exchange one value per step),
+// and the probabilities P^T come out of the first product exactly in the register layout the
+// second product wants for its B operand -- no trip through LDS between the two.
+//
+//   S^T = K.Q^T :  A = K tile from LDS, [key][d] in 16-byte chunks, chunk swizzled like every
+//                  K-inner tile of the matrix products (one ds_read_b128 feeds 4 MFMA steps);
+//                  B = Q, 4 consecutive d per lane and group, loaded once into registers.
+//   Y^T = V^T.P^T: A = V tile from LDS, [key][d], lane r reads column r of the d-block (a
+//                  ds_read_b32 over 32 consecutive floats); B = P^T in place.
+//   MFMA step v of the second product consumes key 8*(v/4) + 4*h + v%4 from lane half h, which
+//   is the row the first product's result register v holds.
+//
+// K and V tiles are fetched one step ahead into registers (buffer loads, rows beyond the key
+// count and chunks beyond the head dimension read as zero) and stored to the other LDS buffer
+// after the step's matrix work; one barrier per step.
+#include "gemm_mfma_kernel.h"
+#include "runtime_internal.h"
+#include "../../include/dragon_hip_gemm.h"
+
+namespace dragon {
+namespace {
+
+constexpr int AQ = 128;   // queries per workgroup: 32 per wavefront
+constexpr int AK = 32;    // keys per step
+
+struct AttnParams {
+    const float* Q; const float* K; const float* V; float* Y;
+    int head, nq, nk;            // heads per image, queries, keys
+    int dk4, dv4;                // head dimension of Q / K and of V / Y, multiples of 4
+    int qtiles;                  // workgroups per (image, head)
+    long long q_n, q_h; int q_l; // element strides: image, head, row
+    long long k_n, k_h; int k_l;
+    long long v_n, v_h; int v_l;
+    long long y_n, y_h; int y_l;
+    float c;                     // scale * log2(e): the exponentials are base 2
+};
+
+__device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
+
+// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32) or 2 (d <= 64)
+template <int DB>
+__global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnParams p) {
+    constexpr int DW = DB * 32;            // tile width in floats
+    constexpr int CPR = DW / 4;            // 16-byte chunks per tile row
+    constexpr int RPP = NTHREADS / CPR;    // tile rows staged per pass
+    constexpr int PASSES = AK / RPP;       // = DB
+    constexpr int NG = DW / 8;             // groups of 8 d (4 MFMA steps each)
+    static_assert(PASSES * RPP == AK, "the key tile divides over the workgroup");
+
+    __shared__ __attribute__((aligned(16))) float Ks[2][AK * DW];
+    __shared__ __attribute__((aligned(16))) float Vs[2][AK * DW];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int r = lane & 31, h = lane >> 5;
+
+    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);   // one XCD's L2 serves whole heads
+    const int bh = lid / p.qtiles, qt = lid - bh * p.qtiles;
+    const int n = bh / p.head, hd = bh - n * p.head;
+    const float* Qb = p.Q + n * p.q_n + hd * p.q_h;
+    const float* Kb = p.K + n * p.k_n + hd * p.k_h;
+    const float* Vb = p.V + n * p.v_n + hd * p.v_h;
+    float* Yb = p.Y + n * p.y_n + hd * p.y_h;
+
+    // ---- this lane's query: row r of the wavefront's 32, d = 8g + 4h .. +3 per group ----
+    const int q = qt * AQ + wave * 32 + r;
+    v4f qf[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int d = 8 * g + 4 * h;
+        qf[g] = buffer_load_f4(Qb, (q < p.nq && d < p.dk4) ? (q * p.q_l + d) * 4 : OOB_OFFSET);
+    }
+
+    // ---- staging of the K / V tiles ----
+    const int s_chunk = t % CPR, s_row = t / CPR;
+    v4f kreg[PASSES], vreg[PASSES];
+    auto fetch = [&](int key0) {
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const int key = key0 + s_row + s * RPP;
+            const bool in = key < p.nk;
+            kreg[s] = buffer_load_f4(Kb, (in && s_chunk * 4 < p.dk4) ? (key * p.k_l + s_chunk * 4) * 4 : OOB_OFFSET);
+            vreg[s] = buffer_load_f4(Vb, (in && s_chunk * 4 < p.dv4) ? (key * p.v_l + s_chunk * 4) * 4 : OOB_OFFSET);
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const int row = s_row + s * RPP;
+            *(v4f*)(&Ks[buf][row * DW + 4 * (s_chunk ^ kin_swizzle<DW>(row))]) = kreg[s];
+            *(v4f*)(&Vs[buf][row * DW + 4 * s_chunk]) = vreg[s];
+        }
+    };
+
+    v16f o[DB];
+#pragma unroll
+    for (int b = 0; b < DB; b++) o[b] = (v16f)(0.0f);
+    float m = -__builtin_inff(), l = 0.0f;      // running maximum (shared by the halves), this half's sum
+
+    const int steps = (p.nk + AK - 1) / AK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    for (int it = 0; it < steps; it++) {
+        const bool more = it + 1 < steps;
+        if (more) fetch((it + 1) * AK);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- S^T[key][query] for this step's 32 keys ----
+        v16f s = (v16f)(0.0f);
+        const float* ks = Ks[buf];
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            const v4f kf = *(const v4f*)(ks + r * DW + 4 * ((2 * g + h) ^ kin_swizzle<DW>(r)));
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[g].x, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[g].y, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[g].z, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[g].w, s, 0, 0, 0);
+        }
+
+        // ---- online softmax, per lane = per query; register v is key 8*(v/4) + 4h + v%4 ----
+#pragma unroll
+        for (int v = 0; v < 16; v++) s[v] *= p.c;
+        if (!more && (p.nk & (AK - 1))) {           // the last step of a ragged key count
+            const int left = p.nk - it * AK;
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (8 * (v / 4) + 4 * h + (v % 4) >= left) s[v] = -__builtin_inff();
+        }
+        float mt = s[0];
+#pragma unroll
+        for (int v = 1; v < 16; v++) mt = fmaxf(mt, s[v]);
+        mt = fmaxf(mt, xhalf(mt));
+        const float m_new = fmaxf(m, mt);
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);   // 0 on the first step (m = -inf)
+        m = m_new;
+        float sum = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            s[v] = __builtin_amdgcn_exp2f(s[v] - m_new);
+            sum += s[v];
+        }
+        l = l * alpha + sum;
+#pragma unroll
+        for (int b = 0; b < DB; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) o[b][v] *= alpha;
+
+        // ---- Y^T[d][query] += V^T[d][key] * P^T[key][query] ----
+        const float* vs = Vs[buf];
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int key = 8 * (v / 4) + 4 * h + (v % 4);
+#pragma unroll
+            for (int b = 0; b < DB; b++)
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * DW + b * 32 + r], s[v], o[b], 0, 0, 0);
+        }
+
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // ---- normalise and store: register v of block b is d = 32b + 8*(v/4) + 4h + v%4 ----
+    l += xhalf(l);
+    const float inv = 1.0f / l;
+    if (q < p.nq) {
+        float* yrow = Yb + (size_t)q * p.y_l;
+#pragma unroll
+        for (int b = 0; b < DB; b++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = 32 * b + 8 * g + 4 * h;
+                if (d < p.dv4) {
+                    v4f y = {o[b][4 * g] * inv, o[b][4 * g + 1] * inv, o[b][4 * g + 2] * inv, o[b][4 * g + 3] * inv};
+                    *(v4f*)(yrow + d) = y;
+                }
+            }
+    }
+}
+
+inline bool aligned16(int64_t a) { return (a & 15) == 0; }
+
+}  // namespace
+}  // namespace dragon
+
+using namespace dragon;
+
+extern "C" {
+
+int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
+                                  int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL, int32_t dK4,
+                                  int32_t dV4, int32_t head_inner, float scale) {
+    if (streams == nullptr || length < 1 || length > 10) return hipErrorInvalidValue;
+    if (dQ == 0 || dK == 0 || dV == 0 || dY == 0 || !aligned16(dQ) || !aligned16(dK) || !aligned16(dV) ||
+        !aligned16(dY))
+        return hipErrorInvalidValue;
+    if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 64 ||
+        dV4 > 64 || !(scale == scale))
+        return hipErrorInvalidValue;
+    // offsets inside one (image, head) slice travel as 32-bit byte offsets
+    const long long rowK = head_inner ? (long long)head * dK4 : dK4, rowV = head_inner ? (long long)head * dV4 : dV4;
+    const long long maxL = QL > VL ? QL : VL, maxRow = rowK > rowV ? rowK : rowV;
+    if ((maxL + AQ) * maxRow * 4 >= 0x7ffffff0LL || (long long)N * head > 0x7fffffffLL / ((QL + AQ - 1) / AQ))
+        return hipErrorInvalidValue;
+    AttnParams p;
+    p.Q = (const float*)(intptr_t)dQ; p.K = (const float*)(intptr_t)dK; p.V = (const float*)(intptr_t)dV;
+    p.Y = (float*)(intptr_t)dY;
+    p.head = head; p.nq = QL; p.nk = VL; p.dk4 = dK4; p.dv4 = dV4;
+    p.qtiles = (QL + AQ - 1) / AQ;
+    if (head_inner) {   // [N, L, head, d]: a row of a head lies head*d apart from the next
+        p.q_l = p.k_l = (int)rowK; p.v_l = p.y_l = (int)rowV;
+        p.q_h = p.k_h = dK4; p.v_h = p.y_h = dV4;
+        p.q_n = (long long)QL * rowK; p.k_n = (long long)VL * rowK;
+        p.v_n = (long long)VL * rowV; p.y_n = (long long)QL * rowV;
+    } else {            // [N, head, L, d]
+        p.q_l = p.k_l = dK4; p.v_l = p.y_l = dV4;
+        p.q_h = (long long)QL * dK4; p.k_h = (long long)VL * dK4;
+        p.v_h = (long long)VL * dV4; p.y_h = (long long)QL * dV4;
+        p.q_n = p.q_h * head; p.k_n = p.k_h * head; p.v_n = p.v_h * head; p.y_n = p.y_h * head;
+    }
+    p.c = scale * 1.44269504088896340736f;
+    hipStream_t s = (hipStream_t)(intptr_t)streams[0];
+    const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);
+    if (dK4 <= 32 && dV4 <= 32) hipLaunchKernelGGL(attention_f32_mfma<1>, grid, block, 0, s, p);
+    else hipLaunchKernelGGL(attention_f32_mfma<2>, grid, block, 0, s, p);
+    return hipGetLastError();
+}
+
+}  // extern "C"

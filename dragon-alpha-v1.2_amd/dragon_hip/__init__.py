@@ -372,6 +372,16 @@ class Cuda_reduce:
                                                 scale))
 
 
+class Cuda_attention:
+    """softmax(scale * Q.K^T).V in one launch (stands in for the chain of ChannelMHA.java:66-83)."""
+
+    @staticmethod
+    def forward(streams, length, dQ, dK, dV, dY, N, head, QL, VL, dK4, dV4, head_inner, scale):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_attention_forward(arr, length, dQ, dK, dV, dY, N, head, QL, VL, dK4, dV4,
+                                                 int(head_inner), scale))
+
+
 class Cuda_expk2:
     """The dimension-swap natives of Cuda_expk2.java."""
 

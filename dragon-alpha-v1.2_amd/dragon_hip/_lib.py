@@ -37,6 +37,7 @@ SIGNATURES = {
     "dragon_Cuda_matMul_matMul_biased": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_function_linear2D": (i32, [i64, f32, i64, f32, i64, i32, i32, i32]),
     "dragon_Cuda_reduce_softmax2D": (i32, [i64, i64, i64, i32, i32, i32, i32, f32]),
+    "dragon_Cuda_attention_forward": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32, i32, i32, f32]),
     "dragon_Cuda_expk2_transpose2D": (i32, [i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_expk2_transpose3D": (i32, [i64, i64, i64] + [i32] * 9),
     "dragon_Cuda_expk2_transpose4D": (i32, [i64, i64, i64] + [i32] * 11),

@@ -155,6 +155,23 @@ int dragon_Cuda_function_linear2D(int64_t stream, float alpha, int64_t dX, float
 int dragon_Cuda_reduce_softmax2D(int64_t stream, int64_t dX, int64_t dY, int32_t field_length,
                                  int32_t row_lengthv, int32_t width, int32_t stride, float scale);
 
+/* The attention block in one launch: per (image n, head h)
+ *     Y[n, h, i, :] = sum_j softmax_j(scale * <Q[n, h, i, :], K[n, h, j, :]>) * V[n, h, j, :]
+ * for QL queries and VL keys, head dimensions dK4 (Q, K) and dV4 (V, Y), both multiples of 4 and at
+ * most 64 (pad columns of Q, K, V zero, as everywhere; the pad columns of Y get zeros).
+ * head_inner = 0: tensors laid out [N, head, L, d4] -- the operands of the reference's
+ *                 batchMatMulT2 / batchMatMul after its transpose(1, 2);
+ * head_inner = 1: tensors laid out [N, L, head, d4] (= [N, L, head*d4]) -- as the layer holds them
+ *                 before that transpose; Y comes out in the layout the block returns, so the four
+ *                 transposes of the block are not needed either.
+ * The score matrix is never stored.  No native of this shape in the reference, which runs
+ * batchMatMulT2, linear2D (sdiv), row_max, row_softmax, div2D_field, batchMatMul and four transposes
+ * (alpha-Dragon-v1.2/src/z/dragon/nn/unit/complex/block/ChannelMHA.java:66-83); a host that owns that
+ * block calls this instead when no mask is set and the head dimensions fit.  Work goes to streams[0]. */
+int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
+                                  int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL, int32_t dK4,
+                                  int32_t dV4, int32_t head_inner, float scale);
+
 /* ---- batched products (grid depth = Batch) --------------------------------------- */
 
 /* C[b][N,M] = A[b][N,AK] * B[b][BK,M], k < BK.  M and AK are multiples of 4, N and BK

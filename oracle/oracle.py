@@ -222,6 +222,26 @@ def softmax2D(Xp, width, features=None, scale=1.0):
     return Y
 
 
+def attention(Q, K, V, alpha):
+    """Y = softmax(alpha * Q.K^T).V per batch entry, as the reference chains its operators
+    (nn/unit/complex/block/ChannelMHA.java:74-78: batchMatMulT2, sdiv, softmax, batchMatMul).
+    Logical float32 arrays Q[B, QL, dk], K[B, VL, dk], V[B, VL, dv] -> Y[B, QL, dv]."""
+    def pad_last(x):
+        s = (x.shape[-1] + 3) // 4 * 4
+        out = np.zeros(x.shape[:-1] + (s,), np.float32)
+        out[..., :x.shape[-1]] = x
+        return out
+    B, QL, dk = Q.shape
+    VL, dv = V.shape[1], V.shape[2]
+    Qp, Kp, Vp = pad_last(Q), pad_last(K), pad_last(V)
+    VL4, dk4, dv4 = (VL + 3) // 4 * 4, Qp.shape[-1], Vp.shape[-1]
+    P = bmm(T2, Qp, Kp, B, QL, VL4, VL, dk4)                       # [B, QL, VL4], columns >= VL zero
+    P = linear2D(alpha, P.reshape(B * QL, VL4), 0.0, VL)           # sdiv(C, P) = linear(1/C, P, 0)
+    P = softmax2D(P, VL)
+    Y = bmm(NN, P.reshape(B, QL, VL4), Vp, B, QL, dv4, VL, VL4)    # [B, QL, dv4]
+    return Y[:, :, :dv]
+
+
 def conv3D(X, W, sh, sw, ph, pw, OH=None, OW=None, acc32=False):
     """X[N, IH, IW, IC], W[OC, FH, FW, IC] logical arrays -> Y[N, OH, OW, OC]."""
     X, px = _f32(X)

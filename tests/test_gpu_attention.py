@@ -1,0 +1,151 @@
+"""The attention block in one launch (softmax(scale * Q.K^T).V without the score matrix in memory)
+against the reference's operator chain restated on the CPU (oracle.attention: batchMatMulT2, sdiv,
+softmax, batchMatMul in float, nn/unit/complex/block/ChannelMHA.java:74-78) and against the same
+mathematics in FP64.
+
+Tolerance.  Y is a convex combination of the rows of V, so |Y| <= max|V|; the float chain and the
+fused kernel both carry the rounding of the scores (K = d products), of the exponentials and of a
+sum over VL terms.  Gate: relative Frobenius error <= 1e-5 and per-element
+|err| <= 1e-4 * sqrt(d) * max|V| * (1 + |scale| * max|Q| * max|K|) against FP64 (the second factor is
+the sensitivity of the softmax to the rounding of its scores), and the fused result must be at least as
+close to FP64 as twice the float chain's own distance plus 1e-6."""
+import numpy as np
+import pytest
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def pad_last(x):
+    s = (x.shape[-1] + 3) // 4 * 4
+    out = np.zeros(x.shape[:-1] + (s,), np.float32)
+    out[..., :x.shape[-1]] = x
+    return out
+
+
+def attention_f64(Q, K, V, scale):
+    """[N, head, L, d] logical arrays."""
+    S = np.einsum("nhqd,nhkd->nhqk", Q.astype(np.float64), K.astype(np.float64)) * np.float64(np.float32(scale))
+    P = np.exp(S - S.max(-1, keepdims=True))
+    P /= P.sum(-1, keepdims=True)
+    return np.einsum("nhqk,nhkd->nhqd", P, V.astype(np.float64))
+
+
+def run_attention(dh, Q, K, V, scale, head_inner, fill=7.0):
+    """Q[N, head, QL, dk], K[N, head, VL, dk], V[N, head, VL, dv] logical; returns Y[N, head, QL, dv] and the
+    raw padded device array.  With head_inner the device tensors are [N, L, head, d4]."""
+    N, H, QL, dk = Q.shape
+    VL, dv = V.shape[2], V.shape[3]
+    Qp, Kp, Vp = pad_last(Q), pad_last(K), pad_last(V)
+    dk4, dv4 = Qp.shape[-1], Vp.shape[-1]
+    if head_inner:
+        Qp, Kp, Vp = (np.ascontiguousarray(x.transpose(0, 2, 1, 3)) for x in (Qp, Kp, Vp))
+    dQ, dK, dV = dh.DeviceArray(Qp), dh.DeviceArray(Kp), dh.DeviceArray(Vp)
+    ny = N * H * QL * dv4
+    dY = dh.DeviceArray(size=ny + 16)
+    dY.fill(fill)
+    dh.Cuda_attention.forward([0], 1, dQ.address, dK.address, dV.address, dY.address, N, H, QL, VL, dk4, dv4,
+                              head_inner, scale)
+    dh.Cuda.streamSynchronize(0)
+    raw = dY.get()
+    for d in (dQ, dK, dV, dY):
+        d.free()
+    assert np.all(raw[ny:] == fill)
+    Yp = raw[:ny].reshape((N, QL, H, dv4) if head_inner else (N, H, QL, dv4))
+    if head_inner:
+        Yp = Yp.transpose(0, 2, 1, 3)
+    assert not Yp[..., dv:].any()                        # the pad columns of Y are zeros
+    return Yp[..., :dv]
+
+
+def check(dh, rng, N, H, QL, VL, dk, dv, scale, head_inner, amp=1.0):
+    Q = rng.uniform(-amp, amp, (N, H, QL, dk)).astype(np.float32)
+    K = rng.uniform(-amp, amp, (N, H, VL, dk)).astype(np.float32)
+    V = rng.uniform(-1, 1, (N, H, VL, dv)).astype(np.float32)
+    Y = run_attention(dh, Q, K, V, scale, head_inner)
+    R64 = attention_f64(Q, K, V, scale)
+    R32 = oracle.attention(Q.reshape(N * H, QL, dk), K.reshape(N * H, VL, dk), V.reshape(N * H, VL, dv),
+                           scale).reshape(N, H, QL, dv)
+    assert np.isfinite(Y).all()
+    e_dev, e_ref = np.abs(Y - R64).max(), np.abs(R32 - R64).max()
+    bound = 1e-4 * np.sqrt(dk) * np.abs(V).max() * (1 + abs(scale) * np.abs(Q).max() * np.abs(K).max())
+    assert np.linalg.norm(Y - R64) <= 1e-5 * np.linalg.norm(R64), (N, H, QL, VL, dk, dv)
+    assert e_dev <= bound, (e_dev, bound)
+    assert e_dev <= 2 * e_ref + 1e-6, (e_dev, e_ref)
+    return Y
+
+
+SHAPES = [  # N, head, QL, VL, dk, dv
+    (1, 1, 1, 1, 4, 4), (2, 3, 37, 29, 20, 20), (1, 2, 128, 128, 64, 64), (2, 2, 130, 257, 64, 64),
+    (1, 4, 300, 31, 32, 32), (1, 1, 64, 1000, 61, 64), (3, 1, 5, 33, 7, 40), (1, 2, 129, 64, 40, 12),
+    (1, 1, 255, 96, 64, 8)]
+
+
+@pytest.mark.parametrize("head_inner", [0, 1])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_attention_matches_the_chain_and_fp64(dh, gpu, shape, head_inner):
+    N, H, QL, VL, dk, dv = shape
+    rng = np.random.default_rng(sum(shape) + head_inner)
+    check(dh, rng, N, H, QL, VL, dk, dv, 1.0 / np.sqrt(H * dk), head_inner)
+
+
+def test_attention_scale_variants_and_sharp_rows(dh, gpu):
+    rng = np.random.default_rng(77)
+    for scale, amp in ((1.0, 1.0), (-0.5, 1.0), (0.0, 1.0), (4.0, 3.0)):
+        check(dh, rng, 1, 2, 70, 90, 24, 24, scale, 0, amp)
+    # one key dominates: Y equals that key's row of V to float accuracy
+    Q = np.zeros((1, 1, 40, 8), np.float32); Q[..., 0] = 50.0
+    K = np.zeros((1, 1, 70, 8), np.float32); K[0, 0, 41, 0] = 1.0
+    V = rng.uniform(-1, 1, (1, 1, 70, 16)).astype(np.float32)
+    Y = run_attention(dh, Q, K, V, 1.0, 0)
+    assert np.abs(Y - V[0, 0, 41]).max() <= 1e-6
+    # equal scores: Y is the plain mean of V
+    Y = run_attention(dh, np.zeros_like(Q), K, V, 1.0, 0)
+    assert np.abs(Y - V.astype(np.float64).mean(2)).max() <= 1e-6
+    # a value far above the float range of exp stays finite (the maximum is subtracted first)
+    Q[..., 0] = 3e4
+    K[0, 0, :, 0] = rng.uniform(-3e4, 3e4, 70).astype(np.float32)
+    Y = run_attention(dh, Q, K, V, 1.0, 0)
+    assert np.isfinite(Y).all() and np.abs(Y - V[0, 0, np.argmax(K[0, 0, :, 0])]).max() <= 1e-6
+
+
+def test_attention_equals_the_device_chain(dh, gpu):
+    # the same block through the three launches it replaces
+    rng = np.random.default_rng(5)
+    B, QL, VL, d = 8, 200, 168, 64
+    Q = rng.standard_normal((1, B, QL, d)).astype(np.float32)
+    K = rng.standard_normal((1, B, VL, d)).astype(np.float32)
+    V = rng.standard_normal((1, B, VL, d)).astype(np.float32)
+    Y = run_attention(dh, Q, K, V, 0.125, 0)
+    dQ, dK, dV = dh.DeviceArray(Q), dh.DeviceArray(K), dh.DeviceArray(V)
+    dP, dO = dh.DeviceArray(size=B * QL * VL), dh.DeviceArray(size=B * QL * d)
+    BMM = dh.Cuda_batchMatMul
+    BMM.batchMatMulT2([0], 1, dQ.address, dK.address, dP.address, B, QL, VL, VL, d)
+    dh.Cuda_reduce.softmax2D(0, dP.address, dP.address, B * QL, VL, VL, VL, 0.125)
+    BMM.batchMatMul([0], 1, dP.address, dV.address, dO.address, B, QL, d, VL, VL)
+    dh.Cuda.streamSynchronize(0)
+    O = dO.get()[:B * QL * d].reshape(1, B, QL, d)
+    for x in (dQ, dK, dV, dP, dO):
+        x.free()
+    assert np.abs(Y - O).max() <= 2e-6 * max(1.0, np.abs(V).max())
+
+
+def test_attention_argument_errors(dh, gpu):
+    d = dh.DeviceArray(size=65536)
+    a = d.address
+    ok = dict(dQ=a, dK=a + 4096, dV=a + 8192, dY=a + 16384, N=1, head=2, QL=8, VL=8, dK4=8, dV4=8, hi=0, scale=1.0)
+
+    def call(**kw):
+        g = dict(ok); g.update(kw)
+        dh.Cuda_attention.forward([0], kw.get("length", 1), g["dQ"], g["dK"], g["dV"], g["dY"], g["N"], g["head"],
+                                  g["QL"], g["VL"], g["dK4"], g["dV4"], g["hi"], g["scale"])
+    call()
+    for bad in (dict(dQ=0), dict(dK=0), dict(dV=0), dict(dY=0), dict(dQ=a + 4), dict(N=0), dict(head=0), dict(QL=0),
+                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=68), dict(dV4=128), dict(scale=float("nan")),
+                dict(length=0), dict(length=11)):
+        with pytest.raises(dh.CudaException) as e:
+            call(**bad)
+        assert e.value.code == 1, bad
+    dh.Cuda.streamSynchronize(0)
+    d.free()
