@@ -378,7 +378,31 @@ def main():
         record("attention chain Q.K^T -> softmax(x/8) -> P.V, batch 64 x 1024 x 64 (3 launches)", fl_chain, ms)
         ms = timer.per_launch_ms(chain_with_sdiv, iters=20)
         record("attention chain with a separate sdiv launch (4 launches)", fl_chain, ms)
-        for x in (dQ, dK, dV, dP, dO):
+        # the same block in one launch (score matrix never stored), on [N, head, L, d] operands and on the
+        # layer's own [N, L, head, d] tensors; and what the reference's block runs around the chain:
+        # transpose(1, 2) of Q, K, V before and of Y after
+        AT, E2 = dh.Cuda_attention, dh.Cuda_expk2
+        Nn, Hh = 4, 16
+        ms = timer.per_launch_ms(lambda: AT.forward(S, 1, dQ.address, dK.address, dV.address, dO.address, Nn, Hh,
+                                                    Sq, Sq, D, D, 0, 0.125), iters=20)
+        record("attention block in one launch, [N, head, L, d] operands", fl_chain, ms)
+        ms = timer.per_launch_ms(lambda: AT.forward(S, 1, dQ.address, dK.address, dV.address, dO.address, Nn, Hh,
+                                                    Sq, Sq, D, D, 1, 0.125), iters=20)
+        record("attention block in one launch, [N, L, head, d] tensors as the layer holds them", fl_chain, ms)
+        dT = [dh.DeviceArray(size=Bt * Sq * D) for _ in range(4)]
+        nT = Bt * Sq * D
+
+        def block_as_the_reference_runs_it():
+            for src, dst in ((dQ, dT[0]), (dK, dT[1]), (dV, dT[2])):
+                E2.transpose4D(stream, src.address, dst.address, Sq, Hh, D, Hh, Sq, D, 1, 2, D, D, nT)
+            BMM.batchMatMulT2_texture(S, 1, dT[0].address, dT[1].address, dP.address, Bt, Sq, Sq, Sq, D)
+            FN.linear2D(stream, 0.125, dP.address, 0.0, dP.address, nP, Sq, Sq)
+            RD.softmax2D(stream, dP.address, dP.address, Bt * Sq, Sq, Sq, Sq, 1.0)
+            BMM.batchMatMul_texture(S, 1, dP.address, dT[2].address, dT[3].address, Bt, Sq, D, Sq, Sq)
+            E2.transpose4D(stream, dT[3].address, dO.address, Hh, Sq, D, Sq, Hh, D, 1, 2, D, D, nT)
+        ms = timer.per_launch_ms(block_as_the_reference_runs_it, iters=20)
+        record("attention block as the reference issues it: 4 transposes + product, sdiv, softmax, product", fl_chain, ms)
+        for x in [dQ, dK, dV, dP, dO] + dT:
             x.free()
 
     if "conv" in extra:
