@@ -156,6 +156,7 @@ SIGNATURES = {
     "dragon_engine_conv3D": (c_void_p, [c_void_p, c_void_p, c_void_p, i32, i32, i32, i32, i32, i32, c_void_p]),
     "dragon_engine_conv3D_into": (i32, [c_void_p, c_void_p, c_void_p, c_void_p, i32, i32, i32, i32, c_void_p]),
     "dragon_policy_conv3D_GEMM_nstream": (i32, [i32, i32]),
+    "dragon_engine_attention": (c_void_p, [c_void_p, c_void_p, c_void_p, c_void_p, i32, f32]),
     "dragon_engine_linear": (c_void_p, [c_void_p, i32, f32, c_void_p, f32]),
     "dragon_engine_softmax": (c_void_p, [c_void_p, i32, c_void_p, i32, f32]),
     "dragon_engine_transpose": (c_void_p, [c_void_p, i32, c_void_p, i32, i32]),

@@ -2,6 +2,7 @@
 // action goes through the C ABI (dragon_Cuda_* entry points); no HIP call is made here.
 #include "dragon_engine.hpp"
 
+#include <math.h>
 #include <string.h>
 
 #include "../../include/dragon_hip_conv.h"
@@ -683,6 +684,16 @@ SyncerPtr CudaFloat32EngineBase::softmax2D(int64_t Y, int64_t X, int field_lengt
     cu(dragon_Cuda_reduce_softmax2D(stream, X, Y, field_length, row_lengthv, width, stride, scale));
     return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
 }
+SyncerPtr CudaFloat32EngineBase::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL,
+                                           int VL, int dK4, int dV4, bool head_inner, float scale) {
+    std::vector<int64_t> s = streamPool_->getStreamArray(1);
+    last_gridZ = 1; last_stream_count = (int)s.size();
+    try {
+        cu(dragon_Cuda_attention_forward(s.data(), (int)s.size(), Q, K, V, Y, N, head, QL, VL, dK4, dV4,
+                                         head_inner ? 1 : 0, scale));
+    } catch (...) { streamPool_->returnStreamArray(s); throw; }
+    return SyncerPtr(new StreamArraySyncer(streamPool_.get(), s));
+}
 SyncerPtr CudaFloat32EngineBase::memcpy(int64_t dst, int64_t src, int64_t memsize) {   // :1173-1179
     int64_t stream = streamPool_->getStream();
     cu(dragon_Cuda_memcpyAsyncDeviceToDevice(stream, dst, src, memsize));
@@ -927,6 +938,27 @@ SyncerPtr EngineCore::conv3D_biased(int64_t Y, int OH, int OW, int64_t X, int IH
     }
     return base_->conv3D_biased(Y, OH, OW, X, IH, IW, W, FH, FW, pad4(N), pad4(IC), OC_4x, sh, sw, ph, pw,
                                 Bias, lengthv, OC);
+}
+SyncerPtr EngineCore::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL, int VL,
+                                int dK, int dV, bool head_inner, float scale) {
+    if (check) {
+        if (Y == 0) throw NullPointerException("Tensor Y is null");
+        if (Q == 0) throw NullPointerException("Tensor Q is null");
+        if (K == 0) throw NullPointerException("Tensor K is null");
+        if (V == 0) throw NullPointerException("Tensor V is null");
+        auto s = [](long long v) { return std::to_string(v); };
+        if (N <= 0) throw IllegalArgumentException("N { got " + s(N) + " } must > 0");
+        if (head <= 0) throw IllegalArgumentException("head { got " + s(head) + " } must > 0");
+        if (QL <= 0) throw IllegalArgumentException("Q.seq_len { got " + s(QL) + " } must > 0");
+        if (VL <= 0) throw IllegalArgumentException("V.seq_len { got " + s(VL) + " } must > 0");
+        if (dK <= 0 || dV <= 0) throw IllegalArgumentException("head dimensions must > 0");
+        if (head > 1 && ((dK & 3) || (dV & 3)))
+            throw IllegalArgumentException("with several heads the head dimensions { got " + s(dK) + ", " + s(dV) +
+                                           " } must be multiples of 4");
+        if (pad4(dK) > 64 || pad4(dV) > 64)
+            throw IllegalArgumentException("head dimensions { got " + s(dK) + ", " + s(dV) + " } must <= 64");
+    }
+    return base_->attention(Y, Q, K, V, N, head, QL, VL, pad4(dK), pad4(dV), head_inner, scale);
 }
 SyncerPtr EngineCore::linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                                      float beta, float gamma, int lengthv, int width) {   // :1965-1983
@@ -1492,6 +1524,36 @@ Tensor* Engine::transpose(bool inplace, Tensor* X, int dimIdx1, int dimIdx2) {
     delete Y;
     finish(X, SyncerPtr(new FreeAfter(std::move(sc1), core_.get(), old_size, old_addr)));
     return X;
+}
+
+Tensor* Engine::attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale) {
+    require(Q, "Q"); require(K, "K"); require(V, "V");
+    if (check_) {    // ChannelMHA.java:45-63
+        must_greater_equal(Q->ndim(), "Q.ndim", 2); must_greater_equal(K->ndim(), "K.ndim", 2);
+        must_greater_equal(V->ndim(), "V.ndim", 2);
+        equals(Q->dimAt(0), "Q.batch", K->dimAt(0), "K.batch");
+        equals(Q->dimAt(0), "Q.batch", V->dimAt(0), "V.batch");
+        equals(Q->lastDim(), "Q.seq_dim", K->lastDim(), "K.seq_dim");
+        if (head <= 0) throw IllegalArgumentException("head { got " + std::to_string(head) + " } must > 0");
+        if (Q->lastDim() % head != 0 || V->lastDim() % head != 0)
+            throw IllegalArgumentException("seq_dim { got " + std::to_string(Q->lastDim()) + ", " +
+                                           std::to_string(V->lastDim()) + " } mod head { got " +
+                                           std::to_string(head) + " } != 0");
+    }
+    const int N = Q->dim[0], KC = Q->lastDim(), VC = V->lastDim();
+    const int QL = Q->length / (N * KC), KL = K->length / (N * KC), VL = V->length / (N * VC);
+    if (check_ && KL != VL)
+        throw IllegalArgumentException("K.seq_len { got " + std::to_string(KL) + " } != V.seq_len { got " +
+                                       std::to_string(VL) + " }");
+    if (scale == 0.0f) scale = 1.0f / sqrtf((float)KC);
+    std::vector<int> Ydim = Q->dim;
+    Ydim.back() = VC;
+    Tensor* Y = &empty(Ydim)->c();
+    try {
+        finish(Y, core_->attention(Y->address, Q->address, K->address, V->address, N, head, QL, VL, KC / head,
+                                   VC / head, true, scale));
+    } catch (...) { deleteTensor(Y); throw; }
+    return Y;
 }
 
 // Engine.java:4002-4013

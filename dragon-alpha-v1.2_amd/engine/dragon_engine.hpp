@@ -197,6 +197,10 @@ public:
     SyncerPtr softmax2D(int64_t Y, int64_t X, int field_length, int row_lengthv, int lengthv, int width,
                         int stride, float scale = 1.0f);
     SyncerPtr memcpy(int64_t dst, int64_t src, int64_t memsize);
+    // softmax(scale * Q.K^T).V per (image, head) in one launch; not a Java method (the reference's block
+    // issues transposes, batchMatMulT2, sdiv, softmax, batchMatMul: nn/unit/complex/block/ChannelMHA.java:66-83)
+    SyncerPtr attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL, int VL, int dK4,
+                        int dV4, bool head_inner, float scale);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int BK, int AK);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN, int AN, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int CM, int BM, int K);
@@ -251,6 +255,9 @@ public:
     SyncerPtr linear2D(int64_t Y, float alpha, int64_t X, float beta, int lengthv, int width);
     SyncerPtr softmax2D(int64_t Y, int64_t X, int row_length, int lengthv, int width, float scale = 1.0f);
     SyncerPtr memcpy(int64_t dst, int64_t src, int length);
+    // head dimensions arrive unpadded; with more than one head they must be multiples of 4 already
+    SyncerPtr attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL, int VL, int dK,
+                        int dV, bool head_inner, float scale);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
@@ -345,6 +352,13 @@ public:
     // Java class).
     Tensor* softmax(bool inplace, Tensor* X, int features = -1) { return softmax_scaled(inplace, X, 1.0f, features); }
     Tensor* softmax_scaled(bool inplace, Tensor* X, float scale, int features = -1);
+
+    // The attention block of ChannelMHA (nn/unit/complex/block/ChannelMHA.java:66-83) in one launch:
+    // Q[N, QL, KC], K[N, VL, KC], V[N, VL, VC] hold `head` heads side by side in their last dimension;
+    // Y[N, QL, VC] = per head softmax(scale * Q.K^T).V.  scale = 0 means the block's own 1/sqrt(KC).
+    // Needs KC/head and VC/head <= 64 (and multiples of 4 when head > 1); other shapes take the operator
+    // chain (transpose, batchMatMulT2, softmax_scaled, batchMatMul, transpose).  Not a Java method.
+    Tensor* attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale = 0.0f);
 
     // Y = alpha*X1 + beta*X2 + gamma with the row vector X2 broadcast over the rows of X1
     Tensor* add_row(bool inplace, Tensor* X1, Tensor* X2) { return linear2_row(inplace, X1, X2, 1.0f, 1.0f, 0.0f); }

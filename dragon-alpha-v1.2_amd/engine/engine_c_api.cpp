@@ -299,6 +299,15 @@ dragon_tensor* dragon_engine_softmax(dragon_engine* eg, int32_t inplace, dragon_
     if (!t) return nullptr;
     return inplace ? X : wrap(t);
 }
+dragon_tensor* dragon_engine_attention(dragon_engine* eg, dragon_tensor* Q, dragon_tensor* K, dragon_tensor* V,
+                                       int32_t head, float scale) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        t = eg->eg.attention(T(Q), T(K), T(V), head, scale);
+    });
+    return t ? wrap(t) : nullptr;
+}
 dragon_tensor* dragon_engine_transpose(dragon_engine* eg, int32_t inplace, dragon_tensor* X,
                                        int32_t dimIdx1, int32_t dimIdx2) {
     Tensor* t = nullptr;

@@ -117,6 +117,14 @@ int dragon_engine_conv3D_into(dragon_engine* eg, dragon_tensor* Y, dragon_tensor
 /* Cuda_conv3D.GEMM_nstream(GM, OC) (Cuda_conv3D.java:264-285): how many streams the engine checks out */
 int32_t dragon_policy_conv3D_GEMM_nstream(int32_t GM, int32_t OC);
 
+/* The attention block of nn/unit/complex/block/ChannelMHA.java:66-83 in one launch: Q[N, QL, KC],
+ * K[N, VL, KC], V[N, VL, VC] with `head` heads side by side in the last dimension ->
+ * Y[N, QL, VC] = per head softmax(scale * Q.K^T).V; scale = 0 selects the block's 1/sqrt(KC).
+ * KC/head and VC/head must be <= 64 and, with several heads, multiples of 4 (IllegalArgumentException
+ * otherwise: such shapes take the operator chain).  Not a Java method. */
+dragon_tensor* dragon_engine_attention(dragon_engine* eg, dragon_tensor* Q, dragon_tensor* K, dragon_tensor* V,
+                                       int32_t head, float scale);
+
 /* Engine.linear(inplace, alpha, X, beta): Y = alpha*X + beta (Engine.java:4005-4013); Engine.sdiv(X, C)
  * is linear(1/C, X, 0).  inplace != 0 writes into X and returns X itself. */
 dragon_tensor* dragon_engine_linear(dragon_engine* eg, int32_t inplace, float alpha, dragon_tensor* X,

@@ -149,3 +149,60 @@ def test_attention_argument_errors(dh, gpu):
         assert e.value.code == 1, bad
     dh.Cuda.streamSynchronize(0)
     d.free()
+
+
+# ---- engine level -----------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def eg(gpu):
+    from dragon_hip import engine
+    e = engine.cuda_float32(0, 32)
+    yield e
+    e.close()
+
+
+@pytest.mark.parametrize("shape", [(2, 37, 29, 4, 20, 20), (1, 130, 130, 2, 64, 32), (3, 16, 50, 1, 7, 9),
+                                   (2, 64, 64, 8, 8, 8)])
+def test_engine_attention_equals_the_block_of_the_reference(eg, shape):
+    # ChannelMHA.java:66-83 through the engine mirror, operator by operator, against the one-launch form
+    N, QL, VL, head, dk, dv = shape
+    rng = np.random.default_rng(sum(shape))
+    KC, VC = head * dk, head * dv
+    Q = rng.uniform(-1, 1, (N, QL, KC)).astype(np.float32)
+    K = rng.uniform(-1, 1, (N, VL, KC)).astype(np.float32)
+    V = rng.uniform(-1, 1, (N, VL, VC)).astype(np.float32)
+    base = eg.get_param("live_blocks")
+    tQ, tK, tV = (eg.tensor(x, *x.shape) for x in (Q, K, V))
+    tY = eg.attention(tQ, tK, tV, head)
+    assert tY.dim == [N, QL, VC]
+    Y = eg.valueOf(tY).reshape(N, QL, head, dv)
+    # the chain on [N, L, head, d] views
+    t4 = [eg.tensor(x.reshape(N, -1, head, d), N, x.shape[1], head, d) for x, d in ((Q, dk), (K, dk), (V, dv))]
+    tQt, tKt, tVt = (eg.transpose(False, t, 1, 2) for t in t4)
+    tP = eg.softmax(True, eg.batchMatMulT2(tQt, tKt), scale=float(1 / np.sqrt(KC)))
+    tO = eg.transpose(True, eg.batchMatMul(tP, tVt), 1, 2)
+    O = eg.valueOf(tO).reshape(N, QL, head, dv)
+    assert np.abs(Y - O).max() <= 2e-6
+    R = attention_f64(Q.reshape(N, QL, head, dk).transpose(0, 2, 1, 3), K.reshape(N, VL, head, dk).transpose(0, 2, 1, 3),
+                      V.reshape(N, VL, head, dv).transpose(0, 2, 1, 3), 1 / np.sqrt(KC)).transpose(0, 2, 1, 3)
+    assert np.linalg.norm(Y - R) <= 1e-5 * np.linalg.norm(R)
+    eg.delete(tQ, tK, tV, tY, tQt, tKt, tVt, tP, tO, *t4)
+    assert eg.get_param("live_blocks") == base
+
+
+def test_engine_attention_error_behaviour(eg):
+    from dragon_hip.engine import IllegalArgumentException, NullPointerException
+    tQ, tK, tV = eg.zeros(2, 8, 24), eg.zeros(2, 9, 24), eg.zeros(2, 9, 24)
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(tQ, tK, tV, 5)                            # seq_dim mod head
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(tQ, tK, tV, 4)                            # head dimension 6 is no multiple of 4
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(tQ, eg.zeros(2, 9, 20), tV, 1)            # K.seq_dim != Q.seq_dim
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(tQ, tK, eg.zeros(2, 10, 24), 1)           # K.seq_len != V.seq_len
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(eg.zeros(2, 8, 72), eg.zeros(2, 9, 72), tV, 1)   # head dimension above 64
+    with pytest.raises(NullPointerException):
+        eg.attention(None, tK, tV, 1)
+    assert eg.attention(tQ, tK, tV, 2).dim == [2, 8, 24]
