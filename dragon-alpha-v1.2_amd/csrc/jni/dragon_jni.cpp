@@ -312,6 +312,19 @@ DEF_BMM(batchMatMulT1_1mma, dragon_Cuda_batchMatMul_batchMatMulT1_mma)
 DEF_BMM(batchMatMulT2, dragon_Cuda_batchMatMul_batchMatMulT2)
 DEF_BMM(batchMatMulT2_1texture, dragon_Cuda_batchMatMul_batchMatMulT2_texture)
 
+// The attention block in one launch.  The reference has no such native: a maintainer who wants it declares
+// `public static native void attention(long[] streamArray, int length, long dQ_address, long dK_address,
+// long dV_address, long dY_address, int N, int head, int QL, int VL, int dK4, int dV4, boolean head_inner,
+// float scale)` in Cuda_batchMatMul.java and calls it from ChannelMHA.__forward__ when mask == null.
+JNIEXPORT void JNICALL BMM(attention)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dQ,
+                                      jlong dK, jlong dV, jlong dY, jint N, jint head, jint QL, jint VL,
+                                      jint dK4, jint dV4, jboolean head_inner, jfloat scale) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_attention_forward(st.s, st.n, dQ, dK, dV, dY, N, head, QL, VL, dK4, dV4,
+                                              head_inner ? 1 : 0, scale));
+}
+
 #define DEF_BMM_MMA(jname, cname)                                                                \
     JNIEXPORT void JNICALL BMM(jname)(JNIEnv* env, jclass, jboolean useTexture,                  \
                                       jlongArray streamArray, jint length, jlong dA, jlong dB,   \
