@@ -3,7 +3,7 @@
 // which the reference computes as batchMatMulT2 -> sdiv -> softmax -> batchMatMul, with a
 // transpose(1, 2) on every tensor around them (nn/unit/complex/block/ChannelMHA.java:66-83 of
 // alpha-Dragon-v1.2/src/z/dragon).  Here the score matrix never reaches memory: a workgroup owns 128
-// queries of one (image, head), walks over the keys 32 at a time and keeps a running maximum, a
+// queries of one (image, head), walks over the keys 64 at a time and keeps a reference maximum, a
 // running sum and the un-normalised output per query ("online softmax").  Row strides are
 // arguments, so the [N, L, head, d] tensors of the layer are read and written where they lie and
 // the four transposes disappear as well.
@@ -26,6 +26,14 @@
 // K and V tiles are fetched one step ahead into registers (buffer loads, rows beyond the key
 // count and chunks beyond the head dimension read as zero) and stored to the other LDS buffer
 // after the step's matrix work; one barrier per step.
+//
+// The vector instructions of the softmax are not hidden behind the matrix work (taking them out
+// shortens the kernel by exactly their issue time), so there are as few as possible: the scale
+// is folded into Q when it is loaded; and the reference maximum that the exponentials subtract
+// is only raised -- which costs a rescaling of the 32 output registers -- when some query's
+// scores exceed it by more than 2^8.  Any reference gives the same result after the final
+// division by the sum; letting it lag keeps every term below 2^8 and skips the rescaling in
+// almost every step.
 #include "gemm_mfma_kernel.h"
 #include "runtime_internal.h"
 #include "../../include/dragon_hip_gemm.h"
@@ -34,7 +42,7 @@ namespace dragon {
 namespace {
 
 constexpr int AQ = 128;   // queries per workgroup: 32 per wavefront
-constexpr int AK = 32;    // keys per step
+constexpr int LAG = 8;    // the reference maximum may lag the true one by 2^LAG
 
 struct AttnParams {
     const float* Q; const float* K; const float* V; float* Y;
@@ -50,13 +58,15 @@ struct AttnParams {
 
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
-// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32) or 2 (d <= 64)
-template <int DB>
+// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32) or 2 (d <= 64);
+// KB = 32-key blocks per step
+template <int DB, int KB>
 __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnParams p) {
+    constexpr int AK = KB * 32;            // keys per step
     constexpr int DW = DB * 32;            // tile width in floats
     constexpr int CPR = DW / 4;            // 16-byte chunks per tile row
     constexpr int RPP = NTHREADS / CPR;    // tile rows staged per pass
-    constexpr int PASSES = AK / RPP;       // = DB
+    constexpr int PASSES = AK / RPP;       // = DB * KB
     constexpr int NG = DW / 8;             // groups of 8 d (4 MFMA steps each)
     static_assert(PASSES * RPP == AK, "the key tile divides over the workgroup");
 
@@ -82,6 +92,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
     for (int g = 0; g < NG; g++) {
         const int d = 8 * g + 4 * h;
         qf[g] = buffer_load_f4(Qb, (q < p.nq && d < p.dk4) ? (q * p.q_l + d) * 4 : OOB_OFFSET);
+        qf[g] *= p.c;                       // scores come out in units of log2: scale * log2(e) * <q, k>
     }
 
     // ---- staging of the K / V tiles ----
@@ -108,7 +119,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
     v16f o[DB];
 #pragma unroll
     for (int b = 0; b < DB; b++) o[b] = (v16f)(0.0f);
-    float m = -__builtin_inff(), l = 0.0f;      // running maximum (shared by the halves), this half's sum
+    float m = -__builtin_inff(), l = 0.0f;      // reference maximum (shared by the halves), this half's sum
 
     const int steps = (p.nk + AK - 1) / AK;
     fetch(0);
@@ -120,55 +131,68 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
         if (more) fetch((it + 1) * AK);
         __builtin_amdgcn_sched_barrier(0);
 
-        // ---- S^T[key][query] for this step's 32 keys ----
-        v16f s = (v16f)(0.0f);
+        // ---- S^T[key][query] for this step's keys, one 32-key block after the other ----
+        v16f s[KB];
         const float* ks = Ks[buf];
 #pragma unroll
-        for (int g = 0; g < NG; g++) {
-            const v4f kf = *(const v4f*)(ks + r * DW + 4 * ((2 * g + h) ^ kin_swizzle<DW>(r)));
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[g].x, s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[g].y, s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[g].z, s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[g].w, s, 0, 0, 0);
+        for (int kb = 0; kb < KB; kb++) {
+            s[kb] = (v16f)(0.0f);
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                const v4f kf = *(const v4f*)(ks + (kb * 32 + r) * DW + 4 * ((2 * g + h) ^ kin_swizzle<DW>(r)));
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[g].x, s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[g].y, s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[g].z, s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[g].w, s[kb], 0, 0, 0);
+            }
         }
 
-        // ---- online softmax, per lane = per query; register v is key 8*(v/4) + 4h + v%4 ----
-#pragma unroll
-        for (int v = 0; v < 16; v++) s[v] *= p.c;
+        // ---- online softmax, per lane = per query; register v of block kb is key 32kb + 8*(v/4) + 4h + v%4 ----
         if (!more && (p.nk & (AK - 1))) {           // the last step of a ragged key count
             const int left = p.nk - it * AK;
 #pragma unroll
-            for (int v = 0; v < 16; v++)
-                if (8 * (v / 4) + 4 * h + (v % 4) >= left) s[v] = -__builtin_inff();
-        }
-        float mt = s[0];
+            for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-        for (int v = 1; v < 16; v++) mt = fmaxf(mt, s[v]);
+                for (int v = 0; v < 16; v++)
+                    if (32 * kb + 8 * (v / 4) + 4 * h + (v % 4) >= left) s[kb][v] = -__builtin_inff();
+        }
+        float mt = s[0][0];
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int v = (kb == 0); v < 16; v++) mt = fmaxf(mt, s[kb][v]);
         mt = fmaxf(mt, xhalf(mt));
-        const float m_new = fmaxf(m, mt);
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);   // 0 on the first step (m = -inf)
-        m = m_new;
+        if (__builtin_amdgcn_ballot_w64(mt > m + (float)LAG) != 0) {   // same decision for the whole wavefront
+            const float m_new = fmaxf(m, mt);
+            const float alpha = __builtin_amdgcn_exp2f(m - m_new);     // 0 on the first step (m = -inf)
+            m = m_new;
+            l *= alpha;
+#pragma unroll
+            for (int b = 0; b < DB; b++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) o[b][v] *= alpha;
+        }
         float sum = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            s[v] = __builtin_amdgcn_exp2f(s[v] - m_new);
-            sum += s[v];
-        }
-        l = l * alpha + sum;
+        for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-        for (int b = 0; b < DB; b++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) o[b][v] *= alpha;
+            for (int v = 0; v < 16; v++) {
+                s[kb][v] = __builtin_amdgcn_exp2f(s[kb][v] - m);
+                sum += s[kb][v];
+            }
+        l += sum;
 
         // ---- Y^T[d][query] += V^T[d][key] * P^T[key][query] ----
         const float* vs = Vs[buf];
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int key = 8 * (v / 4) + 4 * h + (v % 4);
+        for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-            for (int b = 0; b < DB; b++)
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * DW + b * 32 + r], s[v], o[b], 0, 0, 0);
-        }
+            for (int v = 0; v < 16; v++) {
+                const int key = 32 * kb + 8 * (v / 4) + 4 * h + (v % 4);
+#pragma unroll
+                for (int b = 0; b < DB; b++)
+                    o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * DW + b * 32 + r], s[kb][v], o[b], 0, 0, 0);
+            }
 
         if (more) stage(buf ^ 1);
         __syncthreads();
@@ -236,8 +260,8 @@ int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_
     p.c = scale * 1.44269504088896340736f;
     hipStream_t s = (hipStream_t)(intptr_t)streams[0];
     const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);
-    if (dK4 <= 32 && dV4 <= 32) hipLaunchKernelGGL(attention_f32_mfma<1>, grid, block, 0, s, p);
-    else hipLaunchKernelGGL(attention_f32_mfma<2>, grid, block, 0, s, p);
+    if (dK4 <= 32 && dV4 <= 32) hipLaunchKernelGGL((attention_f32_mfma<1, 2>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((attention_f32_mfma<2, 2>), grid, block, 0, s, p);
     return hipGetLastError();
 }
 

@@ -110,6 +110,30 @@ def test_attention_scale_variants_and_sharp_rows(dh, gpu):
     assert np.isfinite(Y).all() and np.abs(Y - V[0, 0, np.argmax(K[0, 0, :, 0])]).max() <= 1e-6
 
 
+@pytest.mark.parametrize("step", [0.02, 0.3, 2.0, 9.0, -0.3])
+def test_attention_with_scores_that_keep_rising(dh, gpu, step):
+    # The kernel lets its reference maximum lag behind the true running maximum (it is raised only when a
+    # score exceeds it by 2^8).  Scores that climb a little with every key never trigger the raise for
+    # long stretches, scores that climb fast trigger it every step, falling scores never after the first:
+    # all must give the FP64 result.
+    rng = np.random.default_rng(31)
+    VL, d = 700, 16
+    Q = np.zeros((1, 1, 70, d), np.float32); Q[..., 0] = 1.0
+    Q[0, 0, :, 1] = rng.uniform(-1, 1, 70)
+    K = np.zeros((1, 1, VL, d), np.float32)
+    K[0, 0, :, 0] = (step * np.arange(VL)).astype(np.float32)
+    K[0, 0, :, 1] = rng.uniform(-1, 1, VL)
+    V = rng.uniform(-1, 1, (1, 1, VL, d)).astype(np.float32)
+    Y = run_attention(dh, Q, K, V, 1.0, 0)
+    R = attention_f64(Q, K, V, 1.0)
+    assert np.isfinite(Y).all()
+    # a score of size |s| carries a rounding error of 2^-24 |s|, which the exponential turns into a relative one
+    smax = np.abs(np.einsum("nhqd,nhkd->nhqk", Q.astype(np.float64), K.astype(np.float64))).max()
+    assert np.abs(Y - R).max() <= 2e-6 + 2.0 ** -23 * smax, (np.abs(Y - R).max(), smax)
+    R32 = oracle.attention(Q[0], K[0], V[0], 1.0)
+    assert np.abs(Y - R).max() <= 2 * np.abs(R32 - R[0]).max() + 2e-6       # no worse than the float chain
+
+
 def test_attention_equals_the_device_chain(dh, gpu):
     # the same block through the three launches it replaces
     rng = np.random.default_rng(5)
