@@ -58,7 +58,7 @@ struct AttnParams {
 
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
-// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32) or 2 (d <= 64);
+// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32), 2 (d <= 64) or 4 (d <= 128);
 // KB = 32-key blocks per step
 template <int DB, int KB>
 __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnParams p) {
@@ -233,8 +233,8 @@ int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_
     if (dQ == 0 || dK == 0 || dV == 0 || dY == 0 || !aligned16(dQ) || !aligned16(dK) || !aligned16(dV) ||
         !aligned16(dY))
         return hipErrorInvalidValue;
-    if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 64 ||
-        dV4 > 64 || !(scale == scale))
+    if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 128 ||
+        dV4 > 128 || !(scale == scale))
         return hipErrorInvalidValue;
     // offsets inside one (image, head) slice travel as 32-bit byte offsets
     const long long rowK = head_inner ? (long long)head * dK4 : dK4, rowV = head_inner ? (long long)head * dV4 : dV4;
@@ -261,7 +261,8 @@ int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_
     hipStream_t s = (hipStream_t)(intptr_t)streams[0];
     const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);
     if (dK4 <= 32 && dV4 <= 32) hipLaunchKernelGGL((attention_f32_mfma<1, 2>), grid, block, 0, s, p);
-    else hipLaunchKernelGGL((attention_f32_mfma<2, 2>), grid, block, 0, s, p);
+    else if (dK4 <= 64 && dV4 <= 64) hipLaunchKernelGGL((attention_f32_mfma<2, 2>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((attention_f32_mfma<4, 1>), grid, block, 0, s, p);
     return hipGetLastError();
 }
 

@@ -30,7 +30,7 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
         return hipErrorInvalidValue;
     const long long GM = (long long)N * OH * OW, GK = (long long)FH * FW * IC;
     const long long sizeX = (long long)N * IH * IW * IC;
-    if (GM > 0x7fffffffLL || GK >= (1LL << 24) || sizeX >= (1LL << 29) || GM * OC > 0x7fffffffLL * 4LL)
+    if (GM > 0x7fffffffLL || GK >= (1LL << 24) || sizeX >= (1LL << 29) || GM * OC > 0x7fffffffLL)
         return hipErrorInvalidValue;
     GemmParams p = {};
     p.A = (const float*)(intptr_t)dX;

@@ -955,8 +955,8 @@ SyncerPtr EngineCore::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int 
         if (head > 1 && ((dK & 3) || (dV & 3)))
             throw IllegalArgumentException("with several heads the head dimensions { got " + s(dK) + ", " + s(dV) +
                                            " } must be multiples of 4");
-        if (pad4(dK) > 64 || pad4(dV) > 64)
-            throw IllegalArgumentException("head dimensions { got " + s(dK) + ", " + s(dV) + " } must <= 64");
+        if (pad4(dK) > 128 || pad4(dV) > 128)
+            throw IllegalArgumentException("head dimensions { got " + s(dK) + ", " + s(dV) + " } must <= 128");
     }
     return base_->attention(Y, Q, K, V, N, head, QL, VL, pad4(dK), pad4(dV), head_inner, scale);
 }

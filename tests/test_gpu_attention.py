@@ -79,7 +79,8 @@ def check(dh, rng, N, H, QL, VL, dk, dv, scale, head_inner, amp=1.0):
 SHAPES = [  # N, head, QL, VL, dk, dv
     (1, 1, 1, 1, 4, 4), (2, 3, 37, 29, 20, 20), (1, 2, 128, 128, 64, 64), (2, 2, 130, 257, 64, 64),
     (1, 4, 300, 31, 32, 32), (1, 1, 64, 1000, 61, 64), (3, 1, 5, 33, 7, 40), (1, 2, 129, 64, 40, 12),
-    (1, 1, 255, 96, 64, 8)]
+    (1, 1, 255, 96, 64, 8), (1, 2, 100, 150, 128, 128), (1, 1, 70, 90, 96, 72), (2, 1, 33, 65, 100, 128),
+    (1, 1, 129, 40, 16, 125)]
 
 
 @pytest.mark.parametrize("head_inner", [0, 1])
@@ -166,7 +167,7 @@ def test_attention_argument_errors(dh, gpu):
                                   g["QL"], g["VL"], g["dK4"], g["dV4"], g["hi"], g["scale"])
     call()
     for bad in (dict(dQ=0), dict(dK=0), dict(dV=0), dict(dY=0), dict(dQ=a + 4), dict(N=0), dict(head=0), dict(QL=0),
-                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=68), dict(dV4=128), dict(scale=float("nan")),
+                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=132), dict(dV4=256), dict(scale=float("nan")),
                 dict(length=0), dict(length=11)):
         with pytest.raises(dh.CudaException) as e:
             call(**bad)
@@ -186,7 +187,7 @@ def eg(gpu):
 
 
 @pytest.mark.parametrize("shape", [(2, 37, 29, 4, 20, 20), (1, 130, 130, 2, 64, 32), (3, 16, 50, 1, 7, 9),
-                                   (2, 64, 64, 8, 8, 8)])
+                                   (2, 64, 64, 8, 8, 8), (1, 140, 70, 2, 128, 96)])
 def test_engine_attention_equals_the_block_of_the_reference(eg, shape):
     # ChannelMHA.java:66-83 through the engine mirror, operator by operator, against the one-launch form
     N, QL, VL, head, dk, dv = shape
@@ -226,7 +227,7 @@ def test_engine_attention_error_behaviour(eg):
     with pytest.raises(IllegalArgumentException):
         eg.attention(tQ, tK, eg.zeros(2, 10, 24), 1)           # K.seq_len != V.seq_len
     with pytest.raises(IllegalArgumentException):
-        eg.attention(eg.zeros(2, 8, 72), eg.zeros(2, 9, 72), tV, 1)   # head dimension above 64
+        eg.attention(eg.zeros(2, 8, 136), eg.zeros(2, 9, 136), tV, 1)   # head dimension above 128
     with pytest.raises(NullPointerException):
         eg.attention(None, tK, tV, 1)
     assert eg.attention(tQ, tK, tV, 2).dim == [2, 8, 24]
