@@ -242,7 +242,7 @@ struct ConvInner {
     static constexpr int LDS_FLOATS = R * LDS_STRIDE;
     static_assert(R % RPP == 0 && PASSES >= 1, "tile does not divide over the workgroup");
 
-    int base[PASSES];   // element offset of pixel (n, oh*sh - ph, ow*sw - pw), channel 0
+    int base[PASSES];   // element offset of pixel (n, oh*sh - ph, ow*sw - pw), channel kcol
     int ih0[PASSES];    // oh*sh - ph, or far below zero for a row outside the matrix
     int iw0[PASSES];
     int kcol, row_first, chunk;
@@ -260,7 +260,7 @@ struct ConvInner {
             const int ih = oh * p.cv_sh - p.cv_ph, iw = ow * p.cv_sw - p.cv_pw;
             ih0[s] = (m < gm) ? ih : -(1 << 30);
             iw0[s] = iw;
-            base[s] = ((n * p.cv_IH + ih) * p.cv_IW + iw) * p.cv_IC;
+            base[s] = ((n * p.cv_IH + ih) * p.cv_IW + iw) * p.cv_IC + kcol;
         }
     }
     // k = first k of the stage; k_left = GK - k
@@ -276,13 +276,26 @@ struct ConvInner {
         int fw = pix - fh * p.cv_FW;
         if (fw < 0) { fh--; fw += p.cv_FW; }
         if (fw >= p.cv_FW) { fh++; fw -= p.cv_FW; }
-        const int koff = (fh * p.cv_IW + fw) * p.cv_IC + ic;
+        const int koff = (fh * p.cv_IW + fw) * p.cv_IC + ic - kcol;
         const bool kok = kcol < k_left;
 #pragma unroll
         for (int s = 0; s < PASSES; s++) {
             const bool ok = kok && (unsigned)(ih0[s] + fh) < (unsigned)p.cv_IH &&
                             (unsigned)(iw0[s] + fw) < (unsigned)p.cv_IW;
             reg[s] = buffer_load_f4(X, ok ? (base[s] + koff) * 4 : OOB_OFFSET);
+        }
+    }
+    // The same for a stage that lies inside one filter tap (IC a multiple of KT): the tap (fh, fw)
+    // and the stage's first channel ic0 are the same for every lane, so the caller keeps them in
+    // scalar registers and the lanes are left with two compares and one add per row.
+    __device__ __forceinline__ void load_conv_tap(v4f (&reg)[PASSES], const float* X, int fh, int fw, int ic0,
+                                                  const GemmParams& p) const {
+        const int koff4 = ((fh * p.cv_IW + fw) * p.cv_IC + ic0) * 4;
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const bool ok = (unsigned)(ih0[s] + fh) < (unsigned)p.cv_IH &&
+                            (unsigned)(iw0[s] + fw) < (unsigned)p.cv_IW;
+            reg[s] = buffer_load_f4(X, ok ? base[s] * 4 + koff4 : OOB_OFFSET);
         }
     }
     __device__ __forceinline__ void store(const v4f (&reg)[PASSES], float* lds) const {
@@ -538,31 +551,34 @@ void gemm_f32_mfma(const GemmParams p) {
 
     v4f ra[LoadA::PASSES], rb[LoadB::PASSES];
 
+    // Convolution: the order in which the K chunks of a tile are visited.  In storage order
+    // (filter row, filter column, channel) two uses of the same input element are IC/KT stages
+    // apart, and by then the other workgroups of the XCD have pushed it out of the L2.  With the
+    // filter column running fastest, consecutive stages read the same pixels shifted by one, so
+    // all but 1/OW of a stage's input is what the previous stage fetched.  Any order gives the
+    // same sum up to rounding; whole chunks only, so IC must be a multiple of KT -- and then a
+    // stage lies inside one filter tap, which the scalar unit tracks (cv_fh, cv_fw, cv_ic).
+    const int cv_nic = CONV ? p.cv_IC / KT : 0;
+    const bool cv_walk = CONV && p.cv_walk && (p.cv_IC % KT == 0);
+    int cv_fh = 0, cv_fw = 0, cv_ic = 0, cv_k = 0;
+
     // stage 0 of the first tile
-    if constexpr (CONV) la.load_conv(ra, cur.a_ptr, cur.ka_lim - cur.k0, cur.k0, p);
-    else la.load(ra, cur.a_ptr, cur.ka_lim - cur.k0);
+    if constexpr (CONV) {
+        if (cv_walk) la.load_conv_tap(ra, cur.a_ptr, 0, 0, 0, p);
+        else la.load_conv(ra, cur.a_ptr, cur.ka_lim - cur.k0, cur.k0, p);
+    } else la.load(ra, cur.a_ptr, cur.ka_lim - cur.k0);
     lb.load(rb, cur.b_ptr, cur.kb_lim - cur.k0);
     la.store(ra, As[0]);
     lb.store(rb, Bs[0]);
     __syncthreads();
     int buf = 0;
 
-    // Convolution: the order in which the K chunks of a tile are visited.  In storage order
-    // (filter row, filter column, channel) two uses of the same input element are IC/KT stages
-    // apart, and by then the other workgroups of the XCD have pushed it out of the L2.  With the
-    // filter column running fastest, consecutive stages read the same pixels shifted by one, so
-    // all but 1/OW of a stage's input is what the previous stage fetched.  Any order gives the
-    // same sum up to rounding; whole chunks only, so IC must be a multiple of KT.
-    const int cv_nic = CONV ? p.cv_IC / KT : 0;
-    const bool cv_walk = CONV && p.cv_walk && (p.cv_IC % KT == 0) && cv_nic > 1 && p.cv_FW > 1;
-    int cv_fw = 0, cv_ic = 0, cv_k = 0;
-
     for (;;) {
         const bool has_next = lid + G < total;
         TileCtx nxt = cur;
         const float* a_ptr = cur.a_ptr;
         const float* b_ptr = cur.b_ptr;
-        if constexpr (CONV) { cv_fw = 0; cv_ic = 0; cv_k = 0; }
+        if constexpr (CONV) { cv_fh = 0; cv_fw = 0; cv_ic = 0; cv_k = 0; }
         for (int it = 0; it < cur.nstage; it++) {
             const bool last = (it + 1 == cur.nstage);
             bool fetched = false;
@@ -575,7 +591,7 @@ void gemm_f32_mfma(const GemmParams p) {
                         if (++cv_fw == p.cv_FW) {
                             cv_fw = 0;
                             cv_k += KT - p.cv_FW * p.cv_IC;
-                            if (++cv_ic == cv_nic) { cv_ic = 0; cv_k += (p.cv_FW - 1) * p.cv_IC; }
+                            if (++cv_ic == cv_nic) { cv_ic = 0; cv_fh++; cv_k += (p.cv_FW - 1) * p.cv_IC; }
                         }
                     } else cv_k += KT;
                     knext = cv_k;
@@ -584,8 +600,10 @@ void gemm_f32_mfma(const GemmParams p) {
                     b_ptr += b_step;
                     knext = cur.k0 + (it + 1) * KT;
                 }
-                if constexpr (CONV) la.load_conv(ra, a_ptr, cur.ka_lim - knext, knext, p);
-                else la.load(ra, a_ptr, cur.ka_lim - knext);
+                if constexpr (CONV) {
+                    if (cv_walk) la.load_conv_tap(ra, a_ptr, cv_fh, cv_fw, cv_ic * KT, p);
+                    else la.load_conv(ra, a_ptr, cur.ka_lim - knext, knext, p);
+                } else la.load(ra, a_ptr, cur.ka_lim - knext);
                 lb.load(rb, b_ptr, cur.kb_lim - knext);
                 fetched = true;
             } else if (has_next) {       // first stage of the next tile -> registers
@@ -593,8 +611,10 @@ void gemm_f32_mfma(const GemmParams p) {
                 if constexpr (CONV) la.init_conv(t, nxt.row0, p.a_outer, p);
                 else la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
                 lb.init(t, nxt.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
-                if constexpr (CONV) la.load_conv(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0, nxt.k0, p);
-                else la.load(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0);
+                if constexpr (CONV) {
+                    if (cv_walk) la.load_conv_tap(ra, nxt.a_ptr, 0, 0, 0, p);
+                    else la.load_conv(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0, nxt.k0, p);
+                } else la.load(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0);
                 lb.load(rb, nxt.b_ptr, nxt.kb_lim - nxt.k0);
                 fetched = true;
             }
