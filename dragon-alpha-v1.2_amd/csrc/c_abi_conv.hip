@@ -58,6 +58,9 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     if (tile >= TILE_COUNT) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape
         tile = (tile == TILE_DMA_128x128_S4) ? TILE_128x128 : (tile == TILE_DMA_64x64_S4) ? TILE_64x64 : TILE_64x64_K32;
     }
+    // 256 gathered rows per workgroup cost the loader four rows' worth of registers per lane and the
+    // kernel spills; 128 x 64 measures the same or better on every layer tried
+    if (tile == TILE_256x64) tile = TILE_128x64;
     return gemm_launch_conv(p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
