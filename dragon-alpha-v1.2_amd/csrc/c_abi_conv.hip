@@ -54,13 +54,29 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
         p.bias_rows = lengthv / OC;
         p.bias_width = width;
     }
-    int tile = gemm_choose_tile(p.rows, p.cols, 1, p.k_total, num_compute_units());
+    const int num_cu = num_compute_units();
+    int tile = gemm_choose_tile(p.rows, p.cols, 1, p.k_total, num_cu);
     if (tile >= TILE_COUNT) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape
         tile = (tile == TILE_DMA_128x128_S4) ? TILE_128x128 : (tile == TILE_DMA_64x64_S4) ? TILE_64x64 : TILE_64x64_K32;
     }
     // 256 gathered rows per workgroup cost the loader four rows' worth of registers per lane and the
     // kernel spills; 128 x 64 measures the same or better on every layer tried
-    if (tile == TILE_256x64) tile = TILE_128x64;
+    const bool free_choice = gemm_forced_tile() == TILE_AUTO;   // a forced shape (tests, sweeps) is taken as it is
+    if (free_choice && tile == TILE_256x64) tile = TILE_128x64;
+    // a gathered row of A costs the loader more than a row of W: of the two 8192-element shapes take the
+    // one with fewer A rows when the filters fill it
+    if (free_choice && tile == TILE_128x64 && OC > 64) tile = TILE_64x128;
+    // 32 k per stage halve the per-stage instructions; worth it while the larger LDS footprint does not
+    // cost co-resident workgroups (2 of 128x128, 3 of the 8192-element shapes fit a compute unit)
+    if (free_choice && (IC & 31) == 0) {
+        const int bm = (tile == TILE_128x128 || tile == TILE_128x64) ? 128 : 64;
+        const int bn = (tile == TILE_128x128 || tile == TILE_64x128) ? 128 : 64;
+        const long long tiles = ((GM + bm - 1) / bm) * ((OC + bn - 1) / bn);
+        const long long per_cu = (tiles + num_cu - 1) / num_cu;
+        if (tile == TILE_128x128 && per_cu <= 2) tile = TILE_128x128_K32;
+        else if (tile == TILE_64x128 && per_cu <= 3) tile = TILE_64x128_K32;
+        else if (tile == TILE_128x64 && per_cu <= 3) tile = TILE_128x64_K32;
+    }
     return gemm_launch_conv(p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 

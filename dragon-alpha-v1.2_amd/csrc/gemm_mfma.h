@@ -63,6 +63,7 @@ struct GemmParams {
 
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu);
 void gemm_force_tile(int tile);
+int gemm_forced_tile();   // TILE_AUTO when the choice is left to gemm_choose_tile
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
 hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);

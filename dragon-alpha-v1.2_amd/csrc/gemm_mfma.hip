@@ -6,6 +6,7 @@ namespace dragon {
 
 static int g_forced_tile = TILE_AUTO;
 void gemm_force_tile(int tile) { g_forced_tile = tile; }
+int gemm_forced_tile() { return g_forced_tile; }
 
 // What the tile shapes are worth, measured on MI355X (fractions of a compute unit's
 // FP32 matrix peak): `alone` is what one resident workgroup sustains by itself (its
