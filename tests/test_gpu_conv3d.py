@@ -123,6 +123,21 @@ def test_conv3D_every_tile_shape(dh, gpu, tile):
     assert np.array_equal(Y, oracle.conv3D(X, W, 2, 1, 1, 1))
 
 
+@pytest.mark.parametrize("tile", list(range(-1, 15)))
+def test_conv3D_every_tile_shape_with_whole_channel_stages(dh, gpu, tile):
+    # 128 channels: every stage depth (16 ... 128 k) divides them, so every shape takes the loader that keeps
+    # the filter tap in scalar registers and visits the filter columns fastest
+    rng = np.random.default_rng(400 + tile)
+    X = rng.integers(-3, 4, (2, 9, 8, 128)).astype(np.float32)
+    W = rng.integers(-3, 4, (40, 3, 3, 128)).astype(np.float32)
+    dh.force_tile(tile)
+    try:
+        Y, _ = run_conv(dh, X, W, 1, 2, 1, 1)
+    finally:
+        dh.force_tile(-1)
+    assert np.array_equal(Y, oracle.conv3D(X, W, 1, 2, 1, 1))
+
+
 @pytest.mark.parametrize("entry", ["texture", "V2", "np", "W1", "GemmR", "GemmR_W1", "winograd"])
 def test_every_native_family_computes_the_same_convolution(dh, gpu, entry):
     rng = np.random.default_rng(len(entry))
