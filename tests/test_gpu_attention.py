@@ -156,6 +156,37 @@ def test_attention_equals_the_device_chain(dh, gpu):
     assert np.abs(Y - O).max() <= 2e-6 * max(1.0, np.abs(V).max())
 
 
+def test_attention_at_the_full_batched_workload_shape(dh, gpu):
+    # 4 images x 16 heads, 1024 queries and keys, 64 per head (the shape of the batched benchmark workload):
+    # the one-launch block against the three launches it replaces, both layouts, plus two properties that do
+    # not depend on the size: rows of V all equal -> Y equals that row; Y lies within the range of V
+    rng = np.random.default_rng(64)
+    N, H, L, d = 4, 16, 1024, 64
+    Q = (rng.standard_normal((N, H, L, d)) * 0.5).astype(np.float32)
+    K = (rng.standard_normal((N, H, L, d)) * 0.5).astype(np.float32)
+    V = rng.standard_normal((N, H, L, d)).astype(np.float32)
+    Y0 = run_attention(dh, Q, K, V, 0.125, 0)
+    Y1 = run_attention(dh, Q, K, V, 0.125, 1)
+    assert np.array_equal(Y0, Y1)                        # the layout changes addresses, not arithmetic
+    dQ, dK, dV = dh.DeviceArray(Q), dh.DeviceArray(K), dh.DeviceArray(V)
+    B = N * H
+    dP, dO = dh.DeviceArray(size=B * L * L), dh.DeviceArray(size=B * L * d)
+    BMM = dh.Cuda_batchMatMul
+    BMM.batchMatMulT2([0], 1, dQ.address, dK.address, dP.address, B, L, L, L, d)
+    dh.Cuda_reduce.softmax2D(0, dP.address, dP.address, B * L, L, L, L, 0.125)
+    BMM.batchMatMul([0], 1, dP.address, dV.address, dO.address, B, L, d, L, L)
+    dh.Cuda.streamSynchronize(0)
+    O = dO.get().reshape(N, H, L, d)
+    for x in (dQ, dK, dV, dP, dO):
+        x.free()
+    assert np.abs(Y0 - O).max() <= 4e-6 * np.abs(V).max()
+    assert np.linalg.norm(Y0 - O) <= 1e-5 * np.linalg.norm(O)
+    assert Y0.max() <= V.max() and Y0.min() >= V.min()
+    Vc = np.broadcast_to(V[:, :, :1, :], V.shape).copy()
+    Yc = run_attention(dh, Q, K, Vc, 0.125, 0)
+    assert np.abs(Yc - Vc[:, :, :1, :]).max() <= 2e-6 * np.abs(V).max()
+
+
 def test_attention_argument_errors(dh, gpu):
     d = dh.DeviceArray(size=65536)
     a = d.address
