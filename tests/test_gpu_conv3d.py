@@ -156,6 +156,33 @@ def test_every_native_family_computes_the_same_convolution(dh, gpu, entry):
     assert np.array_equal(Y, oracle.conv3D(X, W, sh, sw, ph, pw))
 
 
+def test_conv3D_at_the_reference_speed_test_shape(dh, gpu):
+    # 64 images of 64x64, 64 -> 64 channels, 7x7, padding 3 (test/cuda/conv3D/Cuda_conv3D_test.java main):
+    # too large for the CPU loops, so (a) a one-hot filter must copy a shifted channel bit for bit, and
+    # (b) 4000 randomly chosen outputs are recomputed in FP64 from their 3136-term definition
+    rng = np.random.default_rng(7)
+    N, IH, IW, IC, OC, F, P = 64, 64, 64, 64, 64, 7, 3
+    X = rng.uniform(-1, 1, (N, IH, IW, IC)).astype(np.float32)
+    W = np.zeros((OC, F, F, IC), np.float32)
+    for oc in range(OC):
+        W[oc, oc % F, (oc // F) % F, (oc * 5) % IC] = 1.0
+    Y, _ = run_conv(dh, X, W, 1, 1, P, P)
+    Xp = np.zeros((N, IH + 2 * P, IW + 2 * P, IC), np.float32)
+    Xp[:, P:P + IH, P:P + IW] = X
+    for oc in (0, 1, 13, 48, 63):
+        fh, fw, ic = oc % F, (oc // F) % F, (oc * 5) % IC
+        assert np.array_equal(Y[..., oc], Xp[:, fh:fh + IH, fw:fw + IW, ic]), oc
+    W = rng.uniform(-1, 1, (OC, F, F, IC)).astype(np.float32)
+    Y, _ = run_conv(dh, X, W, 1, 1, P, P)
+    idx = np.stack([rng.integers(0, N, 4000), rng.integers(0, IH, 4000), rng.integers(0, IW, 4000),
+                    rng.integers(0, OC, 4000)], 1)
+    Xd, Wd = Xp.astype(np.float64), W.astype(np.float64)
+    ref = np.array([np.vdot(Xd[n, oh:oh + F, ow:ow + F, :], Wd[oc]) for n, oh, ow, oc in idx])
+    got = Y[idx[:, 0], idx[:, 1], idx[:, 2], idx[:, 3]]
+    assert np.abs(got - ref).max() <= 1e-4 * np.sqrt(F * F * IC)
+    assert np.linalg.norm(got - ref) <= 1e-5 * np.linalg.norm(ref)
+
+
 def test_conv3D_biased_equals_two_launches(dh, gpu):
     rng = np.random.default_rng(9)
     X = rng.uniform(-1, 1, (3, 10, 9, 7)).astype(np.float32)
