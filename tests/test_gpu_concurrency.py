@@ -59,6 +59,77 @@ def test_host_threads_on_their_own_streams(dh, gpu):
     assert not errors, errors
 
 
+def test_host_threads_convolution_and_attention(dh, gpu):
+    # the same for the forward convolution (integer data: exact) and the one-launch attention block (every
+    # launch must give the bits of the first, single-threaded one)
+    from oracle import oracle
+    Cuda, CV, AT = dh.Cuda, dh.Cuda_conv3D, dh.Cuda_attention
+    rng = np.random.default_rng(1)
+    conv_cases, attn_cases = [], []
+    for (N, IH, IW, IC, OC, F, s, p_) in [(4, 9, 8, 16, 20, 3, 1, 1), (8, 12, 12, 4, 36, 5, 2, 2), (4, 6, 6, 64, 128, 1, 1, 0)]:
+        X = rng.integers(-3, 4, (N, IH, IW, IC)).astype(np.float32)
+        W = rng.integers(-3, 4, (OC, F, F, IC)).astype(np.float32)
+        conv_cases.append((X, W, s, p_, oracle.conv3D(X, W, s, s, p_, p_)))
+    for (B, QL, VL, d) in [(6, 70, 90, 32), (3, 200, 130, 64), (2, 33, 257, 128)]:
+        Q, K, V = (rng.uniform(-1, 1, (B, L, d)).astype(np.float32) for L in (QL, VL, VL))
+        dQ, dK, dV, dO = dh.DeviceArray(Q), dh.DeviceArray(K), dh.DeviceArray(V), dh.DeviceArray(size=B * QL * d)
+        AT.forward([0], 1, dQ.address, dK.address, dV.address, dO.address, 1, B, QL, VL, d, d, 0, 0.2)
+        Cuda.streamSynchronize(0)
+        attn_cases.append((Q, K, V, dO.get((B, QL, d))))
+        for x in (dQ, dK, dV, dO):
+            x.free()
+    errors = []
+
+    def conv_worker(idx):
+        try:
+            X, W, s, p_, R = conv_cases[idx]
+            N, IH, IW, IC = X.shape
+            OC, F = W.shape[0], W.shape[1]
+            OH, OW = R.shape[1], R.shape[2]
+            stream = Cuda.newStream_NonBlocking()
+            dX, dW, dY = dh.DeviceArray(X), dh.DeviceArray(W), dh.DeviceArray(size=R.size)
+            for it in range(20):
+                CV.conv3D([stream], 1, dX.address, IH, IW, dW.address, F, F, dY.address, OH, OW, N, IC, OC, s, s, p_, p_)
+                Cuda.streamSynchronize(stream)
+                out = np.empty(R.size, np.float32)
+                Cuda.get1D(stream, dY.address, out, R.size)
+                if not np.array_equal(out.reshape(R.shape), R):
+                    errors.append(("conv", idx, it))
+            for x in (dX, dW, dY):
+                x.free()
+            Cuda.deleteStream(stream)
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append(("conv", idx, repr(e)))
+
+    def attn_worker(idx):
+        try:
+            Q, K, V, R = attn_cases[idx]
+            B, QL, d = Q.shape
+            VL = K.shape[1]
+            stream = Cuda.newStream_NonBlocking()
+            dQ, dK, dV, dO = dh.DeviceArray(Q), dh.DeviceArray(K), dh.DeviceArray(V), dh.DeviceArray(size=R.size)
+            for it in range(20):
+                AT.forward([stream], 1, dQ.address, dK.address, dV.address, dO.address, 1, B, QL, VL, d, d, 0, 0.2)
+                Cuda.streamSynchronize(stream)
+                out = np.empty(R.size, np.float32)
+                Cuda.get1D(stream, dO.address, out, R.size)
+                if not np.array_equal(out.reshape(R.shape), R):
+                    errors.append(("attention", idx, it))
+            for x in (dQ, dK, dV, dO):
+                x.free()
+            Cuda.deleteStream(stream)
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append(("attention", idx, repr(e)))
+
+    threads = [threading.Thread(target=conv_worker, args=(i,)) for i in range(3)]
+    threads += [threading.Thread(target=attn_worker, args=(i,)) for i in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_launches_replay_from_a_hip_graph(gpu):
     # Graph capture goes through torch (its stream and graph objects), and torch has to be imported
     # before the library: both bring a HIP runtime of the same name and the process keeps the first.
