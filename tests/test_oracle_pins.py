@@ -439,6 +439,29 @@ def test_conv_oracle_special_cases():
     assert np.allclose(oracle.conv3D(X, Wa + Wb, 2, 1, 1, 0), ya + yb, rtol=1e-5, atol=1e-5)
 
 
+def test_attention_oracle_is_the_chain_and_matches_fp64():
+    # oracle.attention composes the pinned batched products, linear2D and softmax2D the way the reference's
+    # block does; against the same mathematics in FP64, and on cases with a known answer
+    for (B, QL, VL, dk, dv, alpha) in [(3, 5, 9, 7, 6, 0.3), (2, 33, 65, 20, 12, 0.125), (1, 1, 1, 1, 1, 2.0),
+                                       (2, 17, 40, 64, 64, -0.5)]:
+        Q = RNG.standard_normal((B, QL, dk)).astype(np.float32)
+        K = RNG.standard_normal((B, VL, dk)).astype(np.float32)
+        V = RNG.standard_normal((B, VL, dv)).astype(np.float32)
+        Y = oracle.attention(Q, K, V, alpha)
+        S = np.einsum("bqd,bkd->bqk", Q.astype(np.float64), K.astype(np.float64)) * np.float64(np.float32(alpha))
+        P = np.exp(S - S.max(-1, keepdims=True))
+        P /= P.sum(-1, keepdims=True)
+        R = np.einsum("bqk,bkd->bqd", P, V.astype(np.float64))
+        assert Y.shape == R.shape
+        assert np.abs(Y - R).max() <= 1e-5 * max(1.0, np.abs(V).max()), (B, QL, VL)
+    V = RNG.standard_normal((1, 9, 4)).astype(np.float32)
+    Y = oracle.attention(np.zeros((1, 3, 5), np.float32), RNG.standard_normal((1, 9, 5)).astype(np.float32), V, 1.0)
+    assert np.abs(Y - V.astype(np.float64).mean(1)).max() <= 1e-6          # equal scores: the mean of V
+    Q = np.zeros((1, 2, 4), np.float32); Q[..., 0] = 60.0
+    K = np.zeros((1, 9, 4), np.float32); K[0, 6, 0] = 1.0
+    assert np.abs(oracle.attention(Q, K, V, 1.0) - V[0, 6]).max() <= 1e-6   # one key dominates: its row of V
+
+
 def test_reference_micro_helpers_when_built():
     ref = oracle.load_ref()
     if ref is None:
