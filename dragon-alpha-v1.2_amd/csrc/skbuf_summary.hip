@@ -46,8 +46,15 @@ __global__ __launch_bounds__(256) void skbuf_summary_kernel(const float* __restr
 #pragma unroll
             for (int u = 0; u < AHEAD; u++) kahan_step(v, c, b[u]);
         }
-        for (; p < part; p++)
-            kahan_step(v, c, __builtin_nontemporal_load((const V*)(src + (size_t)p * sizeC)));
+        if (p < part) {      // the remainder: its loads go out together as well
+            V b[AHEAD - 1];
+#pragma unroll
+            for (int u = 0; u < AHEAD - 1; u++)
+                if (p + u < part) b[u] = __builtin_nontemporal_load((const V*)(src + (size_t)(p + u) * sizeC));
+#pragma unroll
+            for (int u = 0; u < AHEAD - 1; u++)
+                if (p + u < part) kahan_step(v, c, b[u]);
+        }
         *(V*)(C + at) = v;
     }
 }
