@@ -62,8 +62,10 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     // 256 gathered rows per workgroup cost the loader four rows' worth of registers per lane and the
     // kernel spills; 128 x 64 measures the same or better on every layer tried
     const bool free_choice = gemm_forced_tile() == TILE_AUTO;   // a forced shape (tests, sweeps) is taken as it is
-    // stages of 32 k only where they are whole channel groups (the loader's cheap path)
-    if (free_choice && tile == TILE_128x128_K32 && (IC & 31) != 0) tile = TILE_128x128;
+    // the stage depth is decided below, where the channel count is known: back to the 16-k shapes first
+    if (free_choice)
+        tile = tile == TILE_128x128_K32 ? TILE_128x128 : tile == TILE_128x64_K32 ? TILE_128x64
+             : tile == TILE_64x128_K32 ? TILE_64x128 : tile;
     if (free_choice && tile == TILE_256x64) tile = TILE_128x64;
     // a gathered row of A costs the loader more than a row of W: of the two 8192-element shapes take the
     // one with fewer A rows when the filters fill it

@@ -81,7 +81,7 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
         p.sizeC = (long long)N * M;
         p.split = 1;  // a zero K_slice leaves every slice but the last empty: they write zeros
     }
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units());
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), variant);
     return gemm_launch(variant, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -170,7 +170,7 @@ int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length, 
     p.ldc = M;
     p.sA = (long long)N * AK; p.sB = (long long)BK * M; p.sC = (long long)N * M;
     p.nz = Batch;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units());
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), GEMM_NN);
     return gemm_launch(GEMM_NN, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -197,7 +197,7 @@ int dragon_Cuda_batchMatMul_batchMatMulT1(const int64_t* streams, int32_t length
     p.ldc = M;
     p.sA = (long long)K * AN; p.sB = (long long)K * M; p.sC = (long long)CN * M;
     p.nz = Batch;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units());
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), GEMM_T1);
     return gemm_launch(GEMM_T1, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -218,7 +218,7 @@ int dragon_Cuda_batchMatMul_batchMatMulT2(const int64_t* streams, int32_t length
     p.ldc = CM;
     p.sA = (long long)N * K; p.sB = (long long)BM * K; p.sC = (long long)N * CM;
     p.nz = Batch;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units());
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), GEMM_T2);
     return gemm_launch(GEMM_T2, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 

@@ -61,7 +61,7 @@ struct GemmParams {
     int tiles_m, tiles_n;   // filled by the launcher
 };
 
-int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu);
+int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant = -1);   // variant: GEMM_* or -1
 void gemm_force_tile(int tile);
 int gemm_forced_tile();   // TILE_AUTO when the choice is left to gemm_choose_tile
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);

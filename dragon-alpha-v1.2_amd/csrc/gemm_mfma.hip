@@ -39,7 +39,7 @@ static const TileTraits kTiles[TILE_ALL_COUNT] = {
 // Pick the tile shape with the lowest estimated time: the matrix work of the busiest
 // compute unit (padded tiles, k rounded up to the stage), divided by what that unit
 // sustains with the workgroups it gets.
-int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu) {
+int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant) {
     if (g_forced_tile != TILE_AUTO) return g_forced_tile;
     int best = TILE_128x128;
     double best_cost = 1e300;
@@ -62,6 +62,14 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu) {
     if (best == TILE_128x128 && k >= 256) {
         const long long total = (long long)((rows + 127) / 128) * ((cols + 127) / 128) * nz;
         if ((total + num_cu - 1) / num_cu <= 2) best = TILE_128x128_K32;
+    }
+    // The same for the 8192-element shapes, of which three workgroups with 32-k stages fit a unit: 2-4 %
+    // faster up to three tiles per unit -- except 64 x 128 with both operands K-outer (A^T * B), where the
+    // 32-k stages lose.
+    if ((best == TILE_128x64 || (best == TILE_64x128 && variant != GEMM_T1)) && k >= 256) {
+        const int bm = best == TILE_128x64 ? 128 : 64, bn = best == TILE_128x64 ? 64 : 128;
+        const long long total = (long long)((rows + bm - 1) / bm) * ((cols + bn - 1) / bn) * nz;
+        if ((total + num_cu - 1) / num_cu <= 3) best = best == TILE_128x64 ? TILE_128x64_K32 : TILE_64x128_K32;
     }
     return best;
 }
