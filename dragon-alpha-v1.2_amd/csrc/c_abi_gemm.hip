@@ -290,5 +290,9 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M) {
 }
 
 void dragon_gemm_force_tile(int32_t tile) { gemm_force_tile(tile); }
+int32_t dragon_gemm_choose_tile(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu) {
+    if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
+    return gemm_choose_tile(rows, cols, nz, k, num_cu, variant);
+}
 
 }  // extern "C"

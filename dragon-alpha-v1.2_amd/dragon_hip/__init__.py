@@ -440,6 +440,11 @@ def force_tile(tile):
     lib.dragon_gemm_force_tile(int(tile))
 
 
+def choose_tile(variant, rows, cols, nz, k, num_cu=256):
+    """The tile shape the automatic choice takes (host arithmetic only)."""
+    return lib.dragon_gemm_choose_tile(variant, rows, cols, nz, k, num_cu)
+
+
 class DeviceArray:
     """A float32 device allocation filled from / read back into a numpy array.
 

@@ -258,6 +258,11 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M);
  * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
  * directly through four stage buffers. */
 void dragon_gemm_force_tile(int32_t tile);
+/* The shape the automatic choice takes for a product of `rows` x `cols` outputs, depth `nz` (batch or
+ * K slices), `k` per output, on `num_cu` compute units; variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, -1 = unknown.
+ * Pure host arithmetic (no device needed); returns the forced shape while one is forced, -1 on bad
+ * arguments.  For inspection and tests; no counterpart in the reference. */
+int32_t dragon_gemm_choose_tile(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu);
 
 #ifdef __cplusplus
 }
