@@ -121,7 +121,7 @@ def test_synthetic_generator_is_the_documented_stream(dh):
 
 def test_tile_choice_on_the_documented_shapes(dh):
     # host arithmetic only.  Shape ids: 0 = 128x128, 4 = 128x64, 5 = 64x128 with 16 k per stage; 6, 8, 9 the same
-    # with 32 k; 1 = 64x64; 15-17 staged directly into LDS.
+    # with 32 k; 1 = 64x64, 7 = 64x64 with 32 k; 15-17 staged directly into LDS.
     NN, T1, T2 = 0, 1, 2
     ct = dh.choose_tile
     dh.force_tile(-1)
@@ -129,6 +129,7 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 4096, 4096, 1, 4096) == 0                  # four tiles per compute unit: 16-k stages
         assert ct(v, 2816, 2816, 1, 4096) == 6                  # two per unit: 32-k stages cost no co-residency
         assert ct(v, 2048, 2048, 1, 2048) == 8                  # 128x64, two per unit: 32-k stages
+        assert ct(v, 1536, 1536, 1, 1536) == 7                  # 64x64, three per unit: 32-k stages
     assert ct(T1, 256, 256, 128, 1024) == 6                     # the split-K weight gradient (GridZ 128 slices of 1024)
     assert ct(NN, 1024, 64, 64, 1024) == 8                      # scores x V of the attention-shaped batch
     assert ct(T2, 1024, 1024, 64, 64) == 0 and ct(T1, 1024, 1024, 64, 64) == 0
