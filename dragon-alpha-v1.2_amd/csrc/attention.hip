@@ -234,7 +234,7 @@ int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_
         !aligned16(dY))
         return hipErrorInvalidValue;
     if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 128 ||
-        dV4 > 128 || !(scale == scale))
+        dV4 > 128 || !(scale - scale == 0.0f))   // NaN and the infinities fail the last test
         return hipErrorInvalidValue;
     // offsets inside one (image, head) slice travel as 32-bit byte offsets
     const long long rowK = head_inner ? (long long)head * dK4 : dK4, rowV = head_inner ? (long long)head * dV4 : dV4;

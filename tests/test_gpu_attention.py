@@ -198,7 +198,7 @@ def test_attention_argument_errors(dh, gpu):
                                   g["QL"], g["VL"], g["dK4"], g["dV4"], g["hi"], g["scale"])
     call()
     for bad in (dict(dQ=0), dict(dK=0), dict(dV=0), dict(dY=0), dict(dQ=a + 4), dict(N=0), dict(head=0), dict(QL=0),
-                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=132), dict(dV4=256), dict(scale=float("nan")),
+                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=132), dict(dV4=256), dict(scale=float("nan")), dict(scale=float("inf")),
                 dict(length=0), dict(length=11)):
         with pytest.raises(dh.CudaException) as e:
             call(**bad)
