@@ -32,12 +32,20 @@ std::string fmt(const char* f, long long a = 0, long long b = 0) {
     return buf;
 }
 
+// an event that is deleted when the scope ends, also when an exception leaves it
+struct ScopedEvent {
+    int64_t handle;
+    ScopedEvent() : handle(cu_handle(dragon_Cuda_newEvent_DisableTiming())) {}
+    ~ScopedEvent() { if (handle) dragon_Cuda_deleteEvent(handle); }
+    ScopedEvent(const ScopedEvent&) = delete;
+    ScopedEvent& operator=(const ScopedEvent&) = delete;
+};
+
 // streams -> streams[0]  (CudaFloat32EngineBase.java:649-654)
 void sync_streamArray_2_stream0(const std::vector<int64_t>& streams) {
-    int64_t event1 = cu_handle(dragon_Cuda_newEvent_DisableTiming());
-    cu(dragon_Cuda_eventRecord_streams(event1, streams.data(), (int)streams.size()));
-    cu(dragon_Cuda_streamWaitEvent_default(streams[0], event1));
-    cu(dragon_Cuda_deleteEvent(event1));
+    ScopedEvent event1;
+    cu(dragon_Cuda_eventRecord_streams(event1.handle, streams.data(), (int)streams.size()));
+    cu(dragon_Cuda_streamWaitEvent_default(streams[0], event1.handle));
 }
 
 // CudaFloat32EngineBase.java:657-694
@@ -476,12 +484,11 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
             } else {
                 cu(mma ? dragon_Cuda_matMul_matMul_mma(streamArray.data(), n, A, B, C, N, M, K)
                        : dragon_Cuda_matMul_matMul(streamArray.data(), n, A, B, C, N, M, K));
-                int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
-                cu(dragon_Cuda_eventRecord_streams(event, streamArray.data(), n));
-                cu(dragon_Cuda_streamWaitEvent_default(streamArray[0], event));
+                ScopedEvent event;
+                cu(dragon_Cuda_eventRecord_streams(event.handle, streamArray.data(), n));
+                cu(dragon_Cuda_streamWaitEvent_default(streamArray[0], event.handle));
                 cu(dragon_Cuda_function_linear_dual2D_row(streamArray[0], C, Bias, M, 1.0f, 1.0f, 0.0f,
                                                           C, lengthv, width, M));
-                cu(dragon_Cuda_deleteEvent(event));
             }
             // the reference's BiasedForwardSyncer (:924-956) waits on streams[0] alone, where the
             // bias row ran; the stream-array syncer joins the idle streams first, same result
@@ -519,12 +526,13 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
             rc = dragon_Cuda_matMul_matMulT2SK(streamArray.data(), n, GridZ, A, B, C, Cbuf, N, M, K);
         cu(rc);
         // stage 2: global reduction on streams[0] once every stream has finished stage 1
-        int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
-        cu(dragon_Cuda_eventRecord_streams(event, streamArray.data(), n));
         const int64_t stream = streamArray[0];
-        cu(dragon_Cuda_streamWaitEvent_default(stream, event));
+        {
+            ScopedEvent event;
+            cu(dragon_Cuda_eventRecord_streams(event.handle, streamArray.data(), n));
+            cu(dragon_Cuda_streamWaitEvent_default(stream, event.handle));
+        }
         cu(dragon_Cuda_matMul_SKbuf_summary(stream, Cbuf, C, part, sizeC));
-        cu(dragon_Cuda_deleteEvent(event));
         // stage 3 of matMul_biased: the bias row, after the reduction
         if (Bias != 0)
             cu(dragon_Cuda_function_linear_dual2D_row(stream, C, Bias, M, 1.0f, 1.0f, 0.0f, C, lengthv,
@@ -558,6 +566,8 @@ SyncerPtr CudaFloat32EngineBase::linear2_2D_row(int64_t Y, int64_t X1, int64_t X
 SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, int IH, int IW, int64_t W,
                                           int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph,
                                           int pw, int64_t Bias, int lengthv, int width) {
+    if ((long long)N * OH * OW > 0x7fffffffLL || (long long)FH * FW * IC * OC > 0x7fffffffLL)
+        throw IllegalArgumentException("the convolution is too large: N*OH*OW and FH*FW*IC*OC must fit 31 bits");
     const int GM = N * OH * OW;
     const bool w1 = (FH == 1) && (FW == 1) && (sh == 1) && (sw == 1) && (ph == 0) && (pw == 0);
     if (conv3D_remode && (OC > 31) && (GM > 31)) {
@@ -569,12 +579,12 @@ SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, 
         try {
             stream = streamPool_->getStream();
             cu(dragon_Cuda_conv3D_kernel_remode(stream, W, block.address, FH, FW, OC, IC));
-            int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
-            cu(dragon_Cuda_eventRecord(event, stream));
+            ScopedEvent event;
+            cu(dragon_Cuda_eventRecord(event.handle, stream));
             s = streamPool_->getStreamArray(policy_conv3D_GEMM_nstream(GM, OC));
             const int n = (int)s.size();
             last_gridZ = 1; last_stream_count = n;
-            cu(dragon_Cuda_streamsWaitEvent_default(s.data(), n, event));
+            cu(dragon_Cuda_streamsWaitEvent_default(s.data(), n, event.handle));
             if (w1)
                 cu(dragon_Cuda_conv3D_conv3D_GemmR_W1(s.data(), n, X, IH, IW, W, block.address, Y, N, IC, OC));
             else if (conv3D_Gemm_useTexture)
@@ -583,14 +593,12 @@ SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, 
             else
                 cu(dragon_Cuda_conv3D_conv3D_GemmR(s.data(), n, X, IH, IW, W, block.address, FH, FW, Y, OH, OW,
                                                    N, IC, OC, sh, sw, ph, pw));
-            cu(dragon_Cuda_deleteEvent(event));
             if (Bias) {   // stage 3 on the first stream, after stage 2
-                int64_t event2 = cu_handle(dragon_Cuda_newEvent_DisableTiming());
-                cu(dragon_Cuda_eventRecord_streams(event2, s.data(), n));
-                cu(dragon_Cuda_streamWaitEvent_default(stream, event2));
+                ScopedEvent event2;
+                cu(dragon_Cuda_eventRecord_streams(event2.handle, s.data(), n));
+                cu(dragon_Cuda_streamWaitEvent_default(stream, event2.handle));
                 cu(dragon_Cuda_function_linear_dual2D_row(stream, Y, Bias, OC, 1.0f, 1.0f, 0.0f, Y, lengthv,
                                                           width, OC));
-                cu(dragon_Cuda_deleteEvent(event2));
             }
         } catch (...) {
             if (stream) {   // the block may be in use by what was issued: drain before it goes back
@@ -634,13 +642,12 @@ SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, 
                 cu(dragon_Cuda_conv3D_conv3D(s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw,
                                              ph, pw));
             if (Bias) {   // the second launch, on streams[0] after every stream of the first
-                int64_t event = cu_handle(dragon_Cuda_newEvent_DisableTiming());
-                cu(dragon_Cuda_eventRecord_streams(event, s.data(), n));
-                cu(dragon_Cuda_streamWaitEvent_default(s[0], event));
+                ScopedEvent event;
+                cu(dragon_Cuda_eventRecord_streams(event.handle, s.data(), n));
+                cu(dragon_Cuda_streamWaitEvent_default(s[0], event.handle));
                 cu(dragon_Cuda_function_linear_dual2D_row(s[0], Y, Bias, OC, 1.0f, 1.0f, 0.0f, Y, lengthv,
                                                           width, OC));
-                cu(dragon_Cuda_deleteEvent(event));
-            }
+                }
         }
     } catch (...) { streamPool_->returnStreamArray(s); throw; }
     return SyncerPtr(new StreamArraySyncer(streamPool_.get(), s));
