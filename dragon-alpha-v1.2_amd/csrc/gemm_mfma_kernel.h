@@ -24,7 +24,9 @@
 //                    position c ^ swizzle(r) so that both the staging stores (lanes
 //                    walk along a row) and the fragment reads (lanes walk down the
 //                    rows) touch every bank once; a lane reads 4 consecutive k with
-//                    one ds_read_b128 and feeds 4 MFMA steps.
+//                    one ds_read_b128 and feeds 4 MFMA steps.  As the B operand its
+//                    rows are staged interleaved (LDS row 32*b + r = tile row T*r + b),
+//                    which gives the lane the same T adjacent columns as below.
 //   K-outer tile  -> LDS [k][row]; a lane reads T consecutive rows with one
 //                    ds_read, and those T values belong to T different MFMA
 //                    blocks (block b of a wave holds rows {T*p + b}).  The
@@ -115,8 +117,20 @@ __device__ __forceinline__ int kin_swizzle(int row) {
     return (KT == 16) ? ((row >> 2) & 3) : (KT == 32) ? ((row >> 1) & 7) : (row & 15);
 }
 
+// Which tile row an LDS row of a K-inner operand holds.  IL == 1: the same row.  IL > 1 (the B
+// operand, IL = the wavefront's MFMA blocks along the columns): inside each run of IL*32 rows, LDS row
+// 32*j + r holds tile row IL*r + j, so that lane r's IL blocks are IL CONSECUTIVE columns of C and leave
+// in one vector store, as they do for a K-outer operand.  Only the global side of the staging sees
+// this; the LDS layout, its swizzle and the fragment reads are the same for every IL.
+template <int IL>
+__device__ __forceinline__ int kin_tile_row(int lds_row) {
+    if constexpr (IL == 1) return lds_row;
+    const int local = lds_row % (IL * 32);
+    return lds_row - local + IL * (local % 32) + local / 32;
+}
+
 // K-inner operand: R rows of KT consecutive k.  LDS row stride KT floats, chunks swizzled.
-template <int R, int KT>
+template <int R, int KT, int IL = 1>
 struct KInner {
     static constexpr int CPR = KT / 4;            // float4 chunks per row
     static constexpr int RPP = NTHREADS / CPR;    // rows per pass
@@ -137,7 +151,7 @@ struct KInner {
         chunk = c;
 #pragma unroll
         for (int s = 0; s < PASSES; s++) {
-            const int r = r0 + s * RPP;
+            const int r = kin_tile_row<IL>(r0 + s * RPP);
             off[s] = (row0 + r < outer_bound) ? (r * ld + c * 4) * 4 : OOB_OFFSET;
         }
     }
@@ -162,8 +176,8 @@ struct KInner {
         const int slot = t % CPR, r0 = t / CPR;
 #pragma unroll
         for (int s = 0; s < PASSES; s++) {
-            const int r = r0 + s * RPP;
-            const int c = slot ^ kin_swizzle<KT>(r);
+            const int c = slot ^ kin_swizzle<KT>(r0 + s * RPP);
+            const int r = kin_tile_row<IL>(r0 + s * RPP);
             dma_kcol[s] = c * 4;
             off[s] = (row0 + r < outer_bound) ? (r * ld + c * 4) * 4 : OOB_OFFSET;
         }
@@ -349,7 +363,9 @@ __device__ __forceinline__ void read_frag_kouter(float (&frag)[T][4], const floa
 // Epilogue shared by the kernels: predicated streaming stores of one tile's accumulators.
 // ---------------------------------------------------------------------------
 // MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
-// K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
+// A operand, K-inner: block b covers 32 consecutive rows; K-outer: rows {TM*x + b}.  B operand, either
+// layout: block b of lane r is column TN*r + b (the K-inner staging interleaves its rows for this), so a
+// lane's TN values of one row are consecutive columns and leave in one vector store.
 // BIAS: the bias row is added before the store (the lane's columns are the same for all of its
 // rows); "+ 0.0f" is the gamma term of the separate bias launch this replaces: it turns a -0 sum
 // into +0, so fused and unfused results share every bit.  A template parameter rather than a
@@ -365,7 +381,7 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
     if constexpr (BIAS) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const int col = col0 + wn * TN * 32 + (B_KIN ? (j * 32 + r) : (TN * r + j));
+            const int col = col0 + wn * TN * 32 + TN * r + j;
             bias_v[j] = col < p.bias_width ? p.bias[col] : 0.0f;
         }
     }
@@ -377,13 +393,8 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
     // Only the lane part is range-checked by the hardware, so "outside C" is expressed there.
     const int lane_row = wm * TM * 32 + (A_KIN ? 4 * h : TM * 4 * h);
     const int rows_left = p.rows - row0, cols_left = p.cols - col0;
-    constexpr int NCOL = B_KIN ? TN : 1;
-    int lane_off[NCOL];
-#pragma unroll
-    for (int j = 0; j < NCOL; j++) {
-        const int lcol = wn * TN * 32 + (B_KIN ? (j * 32 + r) : (TN * r));
-        lane_off[j] = (lcol < cols_left) ? lane_row * ldc4 + lcol * 4 : OOB_OFFSET;
-    }
+    const int lcol = wn * TN * 32 + TN * r;
+    const int lane_off = (lcol < cols_left) ? lane_row * ldc4 + lcol * 4 : OOB_OFFSET;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -398,24 +409,17 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
                 if constexpr (BIAS)
                     if (row0 + lane_row + crow < p.bias_rows) out[j] = (out[j] + bias_v[j]) + 0.0f;
             }
-            if constexpr (B_KIN) {
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[j]), rsrc,
-                                                          row_ok ? lane_off[j] : OOB_OFFSET, row_soff, NT_STORE);
+            const int off = row_ok ? lane_off : OOB_OFFSET;
+            if constexpr (TN == 1) {
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[0]), rsrc, off, row_soff,
+                                                      NT_STORE);
+            } else if constexpr (TN == 2) {
+                typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+                const v2f v = {out[0], out[1]};
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rsrc, off, row_soff, NT_STORE);
             } else {
-                const int off = row_ok ? lane_off[0] : OOB_OFFSET;
-                if constexpr (TN == 1) {
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[0]), rsrc, off, row_soff,
-                                                          NT_STORE);
-                } else if constexpr (TN == 2) {
-                    typedef unsigned int v2u __attribute__((ext_vector_type(2)));
-                    const v2f v = {out[0], out[1]};
-                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rsrc, off, row_soff, NT_STORE);
-                } else {
-                    const v4f v = {out[0], out[1], out[2], out[3]};
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc, off, row_soff, NT_STORE);
-                }
+                const v4f v = {out[0], out[1], out[2], out[3]};
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc, off, row_soff, NT_STORE);
             }
         }
     }
@@ -521,7 +525,7 @@ void gemm_f32_mfma(const GemmParams p) {
     using LoadA = typename std::conditional<
         CONV, ConvInner<BM, KT>,
         typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type>::type;
-    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT>, KOuter<BN, KT>>::type;
+    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT, TN>, KOuter<BN, KT>>::type;
 
     __shared__ __attribute__((aligned(16))) float As[2][LoadA::LDS_FLOATS];
     __shared__ __attribute__((aligned(16))) float Bs[2][LoadB::LDS_FLOATS];
@@ -637,7 +641,9 @@ void gemm_f32_mfma(const GemmParams p) {
         // ---- epilogue: predicated streaming stores (C is written once and never read back
         // here; they drain while the next tile computes) ----
         // MFMA block element e of lane (r,h): block row = 8*(e/4) + 4*h + e%4, block col = r.
-        // K-inner operand: block b covers 32 consecutive outputs; K-outer: outputs {T*x + b}.
+        // A operand, K-inner: block b covers 32 consecutive rows; K-outer: rows {TM*x + b}.  B operand, either
+// layout: block b of lane r is column TN*r + b (the K-inner staging interleaves its rows for this), so a
+// lane's TN values of one row are consecutive columns and leave in one vector store.
         store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc, p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
         if (!has_next) break;
         for (int i = 0; i < TM; i++)
@@ -680,7 +686,7 @@ void gemm_f32_mfma_dma(const GemmParams p) {
     static_assert(NS >= 3 && NS <= 4, "stage buffers: 3 or 4");
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
-    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT>, KOuter<BN, KT>>::type;
+    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT, TN>, KOuter<BN, KT>>::type;
     constexpr int STAGE_FLOATS = LoadA::LDS_FLOATS + LoadB::LDS_FLOATS;
     constexpr int XFERS = LoadA::PASSES + LoadB::PASSES;      // transfers per wave per stage
     static_assert((NS - 2) * XFERS <= 63, "vmcnt holds 6 bits");
