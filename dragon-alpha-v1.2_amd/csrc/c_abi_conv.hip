@@ -12,13 +12,6 @@ namespace {
 
 inline bool aligned16(int64_t a) { return (a & 15) == 0; }
 
-int num_compute_units() {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 256;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
-    return n;
-}
-
 int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW, int64_t dW, int FH, int FW,
                  int64_t dY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                  int64_t dBias = 0, int lengthv = 0, int width = 0) {
@@ -54,7 +47,7 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
         p.bias_rows = lengthv / OC;
         p.bias_width = width;
     }
-    const int num_cu = num_compute_units();
+    const int num_cu = gemm_device_num_cu();
     int tile = gemm_choose_tile(p.rows, p.cols, 1, p.k_total, num_cu);
     if (tile >= TILE_COUNT) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape
         tile = (tile == TILE_DMA_128x128_S4) ? TILE_128x128 : (tile == TILE_DMA_64x64_S4) ? TILE_64x64 : TILE_64x64_K32;

@@ -16,20 +16,6 @@ constexpr int MAX_STREAMS = 10;  // the reference copies the handles into jlong 
 inline bool aligned16(int64_t a) { return (a & 15) == 0; }
 inline bool x4(int v) { return (v & 3) == 0; }
 
-int num_compute_units() {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            n <= 0)
-            n = 256;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
 int check_common(const int64_t* streams, int length, int64_t dA, int64_t dB, int64_t dC) {
     if (streams == nullptr || length < 1 || length > MAX_STREAMS) return hipErrorInvalidValue;
     if (dA == 0 || dB == 0 || dC == 0) return hipErrorInvalidValue;
@@ -81,7 +67,8 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
         p.sizeC = (long long)N * M;
         p.split = 1;  // a zero K_slice leaves every slice but the last empty: they write zeros
     }
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), variant);
+    if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, gemm_device_num_cu(), variant);
     return gemm_launch(variant, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -170,7 +157,8 @@ int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length, 
     p.ldc = M;
     p.sA = (long long)N * AK; p.sB = (long long)BK * M; p.sC = (long long)N * M;
     p.nz = Batch;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), GEMM_NN);
+    if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, gemm_device_num_cu(), GEMM_NN);
     return gemm_launch(GEMM_NN, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -197,7 +185,8 @@ int dragon_Cuda_batchMatMul_batchMatMulT1(const int64_t* streams, int32_t length
     p.ldc = M;
     p.sA = (long long)K * AN; p.sB = (long long)K * M; p.sC = (long long)CN * M;
     p.nz = Batch;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), GEMM_T1);
+    if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, gemm_device_num_cu(), GEMM_T1);
     return gemm_launch(GEMM_T1, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -218,7 +207,8 @@ int dragon_Cuda_batchMatMul_batchMatMulT2(const int64_t* streams, int32_t length
     p.ldc = CM;
     p.sA = (long long)N * K; p.sB = (long long)BM * K; p.sC = (long long)N * CM;
     p.nz = Batch;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, num_compute_units(), GEMM_T2);
+    if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, gemm_device_num_cu(), GEMM_T2);
     return gemm_launch(GEMM_T2, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 

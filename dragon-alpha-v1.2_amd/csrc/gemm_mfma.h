@@ -61,6 +61,11 @@ struct GemmParams {
     int tiles_m, tiles_n;   // filled by the launcher
 };
 
+// Compute units of the current device (256 when no device answers), cached per device.
+int gemm_device_num_cu();
+// The kernels address an operand tile with 32-bit byte offsets from the tile's origin: up to 256 rows
+// (or k) of pitch.  False when a leading stride is too long for that; the entry points reject such calls.
+bool gemm_pitches_addressable(const GemmParams& p);
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant = -1);   // variant: GEMM_* or -1
 void gemm_force_tile(int tile);
 int gemm_forced_tile();   // TILE_AUTO when the choice is left to gemm_choose_tile

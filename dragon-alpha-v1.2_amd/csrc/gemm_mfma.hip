@@ -1,12 +1,32 @@
 // Tile choice and dispatch of the FP32 GEMM kernel (gemm_mfma_kernel.h); instantiates the
 // plain products C = A*B, A^T*B, A*B^T in every tile shape.
 #include "gemm_mfma_kernel.h"
+#include <atomic>
 
 namespace dragon {
 
-static int g_forced_tile = TILE_AUTO;
-void gemm_force_tile(int tile) { g_forced_tile = tile; }
-int gemm_forced_tile() { return g_forced_tile; }
+int gemm_device_num_cu() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+bool gemm_pitches_addressable(const GemmParams& p) {
+    constexpr long long MAX_PITCH = (OOB_OFFSET / 4 - 256) / 256;   // floats
+    return p.lda <= MAX_PITCH && p.ldb <= MAX_PITCH && p.ldc <= MAX_PITCH;
+}
+
+// a test and tuning hook: one setting for the whole process
+static std::atomic<int> g_forced_tile{TILE_AUTO};
+void gemm_force_tile(int tile) { g_forced_tile.store(tile, std::memory_order_relaxed); }
+int gemm_forced_tile() { return g_forced_tile.load(std::memory_order_relaxed); }
 
 // What the tile shapes are worth, measured on MI355X (fractions of a compute unit's
 // FP32 matrix peak): `alone` is what one resident workgroup sustains by itself (its
@@ -40,7 +60,8 @@ static const TileTraits kTiles[TILE_ALL_COUNT] = {
 // compute unit (padded tiles, k rounded up to the stage), divided by what that unit
 // sustains with the workgroups it gets.
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant) {
-    if (g_forced_tile != TILE_AUTO) return g_forced_tile;
+    const int forced = gemm_forced_tile();
+    if (forced != TILE_AUTO) return forced;
     int best = TILE_128x128;
     double best_cost = 1e300;
     for (int tile = 0; tile < TILE_ALL_COUNT; tile++) {
@@ -80,6 +101,7 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant)
 }
 
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream) {
+    if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     if (p.bias != nullptr)   // the bias row exists for the forward product only
         return variant == GEMM_NN ? gemm_launch_nn_biased(p, tile, stream) : hipErrorInvalidValue;
     if (tile >= TILE_COUNT) return gemm_launch_dma(variant, p, tile, stream);

@@ -40,6 +40,7 @@
 // translation units so that they compile side by side).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <type_traits>
 #include <stdint.h>
 #include "gemm_mfma.h"
@@ -793,19 +794,16 @@ void gemm_f32_mfma_dma(const GemmParams p) {
 // ---------------------------------------------------------------------------
 // Host side: tile choice and launch
 // ---------------------------------------------------------------------------
-struct DeviceInfo { int num_cu; };
-
-static int device_num_cu() {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cached[dev] = n;
+// Workgroups of `kernel` a compute unit keeps resident, asked of the runtime once per instantiation
+// (concurrent first calls store the same value).
+template <typename Kernel>
+static int resident_workgroups(std::atomic<int>& cache, Kernel kernel) {
+    int n = cache.load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NTHREADS, 0) != hipSuccess || n < 1) n = 1;
+        cache.store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 template <bool A_KIN, bool B_KIN, bool BIAS, int WM, int WN, int TM, int TN, int KT, bool CONV = false>
@@ -817,16 +815,11 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
     if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidValue;
     // workgroups the device keeps resident: one persistent workgroup per slot
-    static int resident_per_cu = 0;   // per instantiation; a benign race fills it with the same value
-    if (resident_per_cu == 0) {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NTHREADS, 0) != hipSuccess || n < 1)
-            n = 1;
-        resident_per_cu = n;
-    }
+    static std::atomic<int> resident_cache{0};   // per instantiation
+    const int resident_per_cu = resident_workgroups(resident_cache, kernel);
     // One persistent workgroup per resident slot, trimmed so that every workgroup gets the
     // same number of tiles (+-1): a static schedule has no tail to balance a ragged last round.
-    const long long slots = (long long)device_num_cu() * resident_per_cu;
+    const long long slots = (long long)gemm_device_num_cu() * resident_per_cu;
     long long grid = total;
     if (total > slots) {
         const long long rounds = (total + slots - 1) / slots;
@@ -867,14 +860,9 @@ static hipError_t launch_cfg_dma(GemmParams p, hipStream_t stream) {
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
     if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidValue;
-    static int resident_per_cu = 0;
-    if (resident_per_cu == 0) {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, NTHREADS, 0) != hipSuccess || n < 1)
-            n = 1;
-        resident_per_cu = n;
-    }
-    const long long slots = (long long)device_num_cu() * resident_per_cu;
+    static std::atomic<int> resident_cache{0};   // per instantiation
+    const int resident_per_cu = resident_workgroups(resident_cache, kernel);
+    const long long slots = (long long)gemm_device_num_cu() * resident_per_cu;
     long long grid = total;
     if (total > slots) {
         const long long rounds = (total + slots - 1) / slots;

@@ -26,7 +26,11 @@
  *   - Callable from any host thread; no host-side global state is modified.
  *   - Errors: hipErrorInvalidValue (1) for a null address, a non-positive dimension, a
  *     stream count outside 1..10, a dimension that violates the x4 padding contract, or
- *     a misaligned address; otherwise the launch status.
+ *     a misaligned address, or a size beyond the limits below; otherwise the launch
+ *     status.
+ *   - Limits: a 2-D C holds at most 2^31-1 floats, and no row pitch (K, M, N, AK, AN,
+ *     CM as the layout has them) exceeds 2 097 150 floats: inside a tile the kernels
+ *     address with 32-bit byte offsets, 256 rows of pitch at most.
  */
 #ifndef DRAGON_HIP_GEMM_H
 #define DRAGON_HIP_GEMM_H

@@ -94,6 +94,13 @@ def test_argument_validation_rejects_before_touching_the_device(dh):
     t2 = lib.dragon_Cuda_batchMatMul_batchMatMulT2
     assert t2(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 5, 8, 9, 4) == INVALID_VALUE     # BM > CM
     assert t2(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 5, 8, 7, 6) == INVALID_VALUE     # K not x4
+    # a row pitch beyond what 32-bit tile-local byte offsets reach (256 rows of it) is refused, not wrapped
+    too_long = 1 << 21
+    assert f(s, 1, ok_ptr, ok_ptr, ok_ptr, 4, 4, too_long) == INVALID_VALUE            # A's pitch = K
+    assert lib.dragon_Cuda_matMul_matMulT2(s, 1, ok_ptr, ok_ptr, ok_ptr, 4, 4, too_long) == INVALID_VALUE
+    assert lib.dragon_Cuda_matMul_matMulT1(s, 1, ok_ptr, ok_ptr, ok_ptr, too_long, 4, 4) == INVALID_VALUE
+    assert b(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 4, 4, too_long, too_long) == INVALID_VALUE
+    assert t2(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 4, 4, 4, too_long) == INVALID_VALUE
 
 
 def test_python_wrapper_raises_the_exception_type(dh):
