@@ -49,16 +49,17 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     }
     const int num_cu = gemm_device_num_cu();
     int tile = gemm_choose_tile(p.rows, p.cols, 1, p.k_total, num_cu);
-    if (tile >= TILE_COUNT) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape
+    const bool free_choice = gemm_forced_tile() == TILE_AUTO;   // a forced shape (tests, sweeps) is taken as it is
+    if (free_choice) tile &= ~TILE_PAIRED;   // decided below, on the convolution's own measurements
+    if (gemm_tile_is_dma(tile)) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape
         tile = (tile == TILE_DMA_128x128_S4) ? TILE_128x128 : (tile == TILE_DMA_64x64_S4) ? TILE_64x64 : TILE_64x64_K32;
     }
-    // 256 gathered rows per workgroup cost the loader four rows' worth of registers per lane and the
-    // kernel spills; 128 x 64 measures the same or better on every layer tried
-    const bool free_choice = gemm_forced_tile() == TILE_AUTO;   // a forced shape (tests, sweeps) is taken as it is
     // the stage depth is decided below, where the channel count is known: back to the 16-k shapes first
     if (free_choice)
         tile = tile == TILE_128x128_K32 ? TILE_128x128 : tile == TILE_128x64_K32 ? TILE_128x64
              : tile == TILE_64x128_K32 ? TILE_64x128 : tile;
+    // 256 gathered rows per workgroup cost the loader four rows' worth of registers per lane and the
+    // kernel spills; 128 x 64 measures the same or better on every layer tried
     if (free_choice && tile == TILE_256x64) tile = TILE_128x64;
     // a gathered row of A costs the loader more than a row of W: of the two 8192-element shapes take the
     // one with fewer A rows when the filters fill it
@@ -74,6 +75,9 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
         else if (tile == TILE_64x128 && per_cu <= 3) tile = TILE_64x128_K32;
         else if (tile == TILE_128x64 && per_cu <= 3) tile = TILE_128x64_K32;
     }
+    // the paired-stage form pays later here than in the plain products (the gathering loader needs the
+    // registers): 3-5 % faster on 7x7x64 and 3x3x512 filters, 4-8 % slower on 3x3x64 and 1x1x256
+    if (free_choice && GK >= 3072 && tile != TILE_256x64 && tile != TILE_64x256) tile |= TILE_PAIRED;
     return gemm_launch_conv(p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 

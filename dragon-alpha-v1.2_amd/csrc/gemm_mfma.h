@@ -28,8 +28,13 @@ enum GemmTile {
     TILE_DMA_128x128_S4 = 15,
     TILE_DMA_64x64_S4 = 16,
     TILE_DMA_64x64_K32_S4 = 17,
-    TILE_ALL_COUNT = 18
+    TILE_ALL_COUNT = 18,
+    // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
+    // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
+    // short K; gemm_choose_tile sets it.
+    TILE_PAIRED = 0x100
 };
+inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
 //   K-inner operand (k contiguous): outer bound = number of rows that exist (exact),

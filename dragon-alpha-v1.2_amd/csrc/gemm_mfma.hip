@@ -84,6 +84,7 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant)
         const long long total = (long long)((rows + 127) / 128) * ((cols + 127) / 128) * nz;
         if ((total + num_cu - 1) / num_cu <= 2) best = TILE_128x128_K32;
     }
+
     // The same for the 8192-element shapes, of which three workgroups with 32-k stages fit a unit: 2-4 %
     // faster up to three tiles per unit -- except 64 x 128 with both operands K-outer (A^T * B), where the
     // 32-k stages lose.
@@ -97,6 +98,11 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant)
         const long long total = (long long)((rows + 63) / 64) * ((cols + 63) / 64) * nz;
         if ((total + num_cu - 1) / num_cu <= 5) best = TILE_64x64_K32;
     }
+    // The paired-stage form of the kernel, measured over 2048..4096 x 2048..4096 x K in all layouts: equal
+    // at K = 256, 2-5 % faster at 512..1024, 3.5-8 % at 4096; slower on a short K (8 % at K = 64).  The two
+    // 256-row shapes spill in it and gain only from K = 2048 on.
+    if (best <= TILE_64x128_K32 && k >= ((best == TILE_256x64 || best == TILE_64x256) ? 2048 : 512))
+        best |= TILE_PAIRED;
     return best;
 }
 
@@ -104,7 +110,7 @@ hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t s
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     if (p.bias != nullptr)   // the bias row exists for the forward product only
         return variant == GEMM_NN ? gemm_launch_nn_biased(p, tile, stream) : hipErrorInvalidValue;
-    if (tile >= TILE_COUNT) return gemm_launch_dma(variant, p, tile, stream);
+    if (gemm_tile_is_dma(tile)) return gemm_launch_dma(variant, p, tile, stream);
     switch (variant) {
         case GEMM_NN: return launch_variant<true, false, false>(p, tile, stream);
         case GEMM_T1: return launch_variant<false, false, false>(p, tile, stream);

@@ -5,7 +5,7 @@
 namespace dragon {
 
 hipError_t gemm_launch_nn_biased(const GemmParams& p, int tile, hipStream_t stream) {
-    if (tile >= TILE_COUNT) return launch_variant_dma<true, false, true>(p, tile, stream);
+    if (gemm_tile_is_dma(tile)) return launch_variant_dma<true, false, true>(p, tile, stream);
     return launch_variant<true, false, true>(p, tile, stream);
 }
 

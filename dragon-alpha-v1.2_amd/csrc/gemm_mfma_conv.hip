@@ -5,7 +5,7 @@
 namespace dragon {
 
 hipError_t gemm_launch_conv(const GemmParams& p, int tile, hipStream_t stream) {
-    if (tile < 0 || tile >= TILE_COUNT) return hipErrorInvalidValue;
+    if (tile < 0 || gemm_tile_is_dma(tile & ~TILE_PAIRED)) return hipErrorInvalidValue;
     if (p.bias != nullptr) return launch_variant<true, true, true, true>(p, tile, stream);
     return launch_variant<true, true, false, true>(p, tile, stream);
 }

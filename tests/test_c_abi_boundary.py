@@ -128,24 +128,27 @@ def test_synthetic_generator_is_the_documented_stream(dh):
 
 def test_tile_choice_on_the_documented_shapes(dh):
     # host arithmetic only.  Shape ids: 0 = 128x128, 4 = 128x64, 5 = 64x128 with 16 k per stage; 6, 8, 9 the same
-    # with 32 k; 1 = 64x64, 7 = 64x64 with 32 k; 15-17 staged directly into LDS.
+    # with 32 k; 1 = 64x64, 7 = 64x64 with 32 k; 15-17 staged directly into LDS; + P: the paired-stage form,
+    # taken from K = 512 on.
     NN, T1, T2 = 0, 1, 2
+    P = 256
     ct = dh.choose_tile
     dh.force_tile(-1)
     for v in (NN, T1, T2):
-        assert ct(v, 4096, 4096, 1, 4096) == 0                  # four tiles per compute unit: 16-k stages
-        assert ct(v, 2816, 2816, 1, 4096) == 6                  # two per unit: 32-k stages cost no co-residency
-        assert ct(v, 2048, 2048, 1, 2048) == 8                  # 128x64, two per unit: 32-k stages
-        assert ct(v, 1536, 1536, 1, 1536) == 7                  # 64x64, three per unit: 32-k stages
-    assert ct(T1, 256, 256, 128, 1024) == 6                     # the split-K weight gradient (GridZ 128 slices of 1024)
-    assert ct(NN, 1024, 64, 64, 1024) == 8                      # scores x V of the attention-shaped batch
+        assert ct(v, 4096, 4096, 1, 4096) == 0 + P                # four tiles per compute unit: 16-k stages
+        assert ct(v, 2816, 2816, 1, 4096) == 6 + P                # two per unit: 32-k stages cost no co-residency
+        assert ct(v, 2048, 2048, 1, 2048) == 8 + P                # 128x64, two per unit: 32-k stages
+        assert ct(v, 1536, 1536, 1, 1536) == 7 + P                # 64x64, three per unit: 32-k stages
+    assert ct(T1, 256, 256, 128, 1024) == 6 + P                   # the split-K weight gradient (GridZ 128 slices of 1024)
+    assert ct(NN, 1024, 64, 64, 1024) == 8 + P                    # scores x V of the attention-shaped batch
     assert ct(T2, 1024, 1024, 64, 64) == 0 and ct(T1, 1024, 1024, 64, 64) == 0
     assert ct(NN, 1000, 780, 1, 1532) in (16, 17)               # fewer tiles than units: direct-to-LDS 64x64
     assert ct(NN, 257, 388, 36, 129) == 1                       # batch of small ragged products: 64x64
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
-    if ct(NN, *shape) in (5, 9):
-        assert ct(NN, *shape) == 9 and ct(T2, *shape) == 9 and ct(T1, *shape) == 5
+    if ct(NN, *shape) in (5 + P, 9 + P):
+        assert ct(NN, *shape) == 9 + P and ct(T2, *shape) == 9 + P and ct(T1, *shape) == 5 + P
+    assert ct(NN, 4096, 4096, 1, 256) == 0 and ct(NN, 4096, 4096, 1, 512) == P    # a short K keeps the plain form
     dh.force_tile(7)
     assert ct(NN, 4096, 4096, 1, 4096) == 7                     # a forced shape is reported as it is
     dh.force_tile(-1)

@@ -137,7 +137,7 @@ def _biased_both_ways(dh, A, B, bias, tile):
     return C1, C2
 
 
-@pytest.mark.parametrize("tile", list(range(-1, 18)))
+@pytest.mark.parametrize("tile", list(range(-1, 18)) + list(range(256, 266)))
 def test_fused_bias_equals_two_launches_bitwise(dh, gpu, tile):
     rng = np.random.default_rng(1000 + tile)
     for (N, M, K) in [(130, 203, 77), (1, 5, 300), (257, 64, 129)]:

@@ -110,7 +110,7 @@ def test_conv3D_matches_oracle(dh, gpu, geom):
     assert np.array_equal(Yi, oracle.conv3D(Xi, Wi, sh, sw, ph, pw))
 
 
-@pytest.mark.parametrize("tile", list(range(-1, 18)))
+@pytest.mark.parametrize("tile", list(range(-1, 18)) + list(range(256, 266)))
 def test_conv3D_every_tile_shape(dh, gpu, tile):
     rng = np.random.default_rng(300 + tile)
     X = rng.integers(-3, 4, (3, 11, 9, 12)).astype(np.float32)
@@ -123,7 +123,7 @@ def test_conv3D_every_tile_shape(dh, gpu, tile):
     assert np.array_equal(Y, oracle.conv3D(X, W, 2, 1, 1, 1))
 
 
-@pytest.mark.parametrize("tile", list(range(-1, 15)))
+@pytest.mark.parametrize("tile", list(range(-1, 15)) + list(range(256, 266)))
 def test_conv3D_every_tile_shape_with_whole_channel_stages(dh, gpu, tile):
     # 128 channels: every stage depth (16 ... 128 k) divides them, so every shape takes the loader that keeps
     # the filter tap in scalar registers and visits the filter columns fastest

@@ -16,6 +16,9 @@ TILES = {-1: "auto", 0: "128x128", 1: "64x64", 2: "256x64", 3: "64x256", 4: "128
          11: "64x64/k128", 12: "128x128/k64", 13: "128x64/k64", 14: "64x128/k64",
          # direct global->LDS staging through 4 stage buffers
          15: "dma 128x128", 16: "dma 64x64", 17: "dma 64x64/k32"}
+# + 256: the paired-stage form of the shapes 0..9 (what the automatic choice takes for a long K)
+PAIRED = 256
+TILES.update({PAIRED + t: TILES[t] + " paired" for t in range(10)})
 SHAPES = [(4, 4, 4), (8, 4, 12), (128, 128, 64), (64, 64, 16), (132, 260, 20), (100, 76, 36),
           (257, 129, 385), (512, 512, 512), (1000, 777, 1531), (31, 1023, 77), (1, 1, 1), (3, 2, 5)]
 
@@ -38,6 +41,22 @@ def test_integer_inputs_bitwise(gpu, variant, tile):
         assert np.array_equal(C, R), "%s tile %s shape %s" % (VARIANT_NAMES[variant], TILES[tile], (N, M, K))
         # padded rows / columns of C are written as exact zeros (C was pre-filled with 123)
         assert np.count_nonzero(Cp[N:, :]) == 0 and np.count_nonzero(Cp[:, M:]) == 0
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("tile,K", [(PAIRED + 0, 112), (PAIRED + 1, 112), (PAIRED + 4, 80), (PAIRED + 5, 176),
+                                    (PAIRED + 6, 156), (PAIRED + 7, 156), (PAIRED + 9, 100), (0, 112)])
+def test_paired_stages_across_tile_boundaries(gpu, variant, tile, K):
+    """More tiles than resident workgroups and an odd number of stages: a workgroup's second tile starts
+    on the odd LDS buffer (one single stage, then pairs), the last stage of K is partial for some."""
+    rng = np.random.default_rng(4000 + tile + variant)
+    N = M = 4224 if tile in (PAIRED, 0) else 3100     # 33 x 33 tiles of 128 x 128; 49 x 49 of 64 x 64
+    gpu.force_tile(tile)
+    A, B = logical_operands(variant, rng, N, M, K, dist="int")
+    C, Cp = gpu_matmul_2d(gpu, variant, A, B, fill=123.0)
+    R = oracle.matmul_f64(variant, A, B).astype(np.float32)    # small integers: every order is exact
+    assert np.array_equal(C, R), "%s tile %s" % (VARIANT_NAMES[variant], TILES[tile])
+    assert np.count_nonzero(Cp[N:, :]) == 0 and np.count_nonzero(Cp[:, M:]) == 0
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])

@@ -83,7 +83,7 @@ def test_split_k_equals_unsplit_within_tolerance(gpu, variant):
         assert rel_fro(C, oracle.SKbuf_summary(Cb0, C0, GZ - 1)) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [1, 6, 7, 9, 10, 11, 12, 14, 15, 16, 17])
+@pytest.mark.parametrize("tile", [1, 6, 7, 9, 10, 11, 12, 14, 15, 16, 17, 256, 257, 262, 263, 265])
 def test_split_k_with_every_stage_depth(gpu, tile):
     # K slices that are not multiples of the k stage (16 or 32), on forced tile shapes
     rng = np.random.default_rng(50 + tile)
