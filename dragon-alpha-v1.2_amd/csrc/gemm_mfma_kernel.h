@@ -58,10 +58,12 @@ static constexpr int OOB_OFFSET = 0x7ffffff0; // >= num_records: the load return
 static constexpr int RSRC_RECORDS = 0x7ffffff0;
 static constexpr int RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format
 
-__device__ __forceinline__ v4f buffer_load_f4(const float* base, int byte_offset) {
+// byte_offset is the lane's part (range-checked by the hardware), scalar_offset a wave-uniform part
+// added to it unchecked
+__device__ __forceinline__ v4f buffer_load_f4(const float* base, int byte_offset, int scalar_offset = 0) {
     __amdgpu_buffer_rsrc_t r =
         __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, RSRC_RECORDS, RSRC_FLAGS);
-    v4u x = __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, 0);
+    v4u x = __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, scalar_offset, 0);
     return __builtin_bit_cast(v4f, x);
 }
 
@@ -159,11 +161,12 @@ struct KInner {
     // base points at (row0, k) of the operand; k_left = k_limit - k
     // GUARD false: the caller knows that the whole stage lies inside K (k_left >= KT), and the per-lane
     // test, which costs vector instructions between the MFMAs, is left out
+    // soff: a wave-uniform byte offset on top of base (the stage's distance from the tile's first one)
     template <bool GUARD = true>
-    __device__ __forceinline__ void load(v4f (&reg)[PASSES], const float* base, int k_left) const {
+    __device__ __forceinline__ void load(v4f (&reg)[PASSES], const float* base, int k_left, int soff = 0) const {
         const bool kok = !GUARD || kcol < k_left;
 #pragma unroll
-        for (int s = 0; s < PASSES; s++) reg[s] = buffer_load_f4(base, kok ? off[s] : OOB_OFFSET);
+        for (int s = 0; s < PASSES; s++) reg[s] = buffer_load_f4(base, kok ? off[s] : OOB_OFFSET, soff);
     }
     __device__ __forceinline__ void store(const v4f (&reg)[PASSES], float* lds) const {
 #pragma unroll
@@ -223,10 +226,10 @@ struct KOuter {
         }
     }
     template <bool GUARD = true>
-    __device__ __forceinline__ void load(v4f (&reg)[PASSES], const float* base, int k_left) const {
+    __device__ __forceinline__ void load(v4f (&reg)[PASSES], const float* base, int k_left, int soff = 0) const {
 #pragma unroll
         for (int s = 0; s < PASSES; s++)
-            reg[s] = buffer_load_f4(base, (!GUARD || krow + s * RPP < k_left) ? off[s] : OOB_OFFSET);
+            reg[s] = buffer_load_f4(base, (!GUARD || krow + s * RPP < k_left) ? off[s] : OOB_OFFSET, soff);
     }
     __device__ __forceinline__ void store(const v4f (&reg)[PASSES], float* lds) const {
 #pragma unroll
@@ -541,6 +544,8 @@ void gemm_f32_mfma(const GemmParams p) {
     const int r = lane & 31, h = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
     const size_t a_step = LoadA::k_advance(p.lda), b_step = LoadB::k_advance(p.ldb);
+    // the same in bytes, for the paired form (whose launcher checks that K times this fits 32 bits)
+    const int a_step4 = (int)(a_step * 4), b_step4 = (int)(b_step * 4);
 
     const int total = p.tiles_m * p.tiles_n * p.nz;
     const int G = gridDim.x;
@@ -601,7 +606,19 @@ void gemm_f32_mfma(const GemmParams p) {
             const int b = b_sel;
             const bool last = !INNER && (it + 1 == cur.nstage);
             bool fetched = false;
-            if (!last) {                 // next stage of this tile -> registers
+            constexpr bool BY_OFFSET = INNER && !CONV;
+            if constexpr (!CONV) {
+                if constexpr (INNER) {
+                    // next stage of this tile -> registers; the stage's distance from the tile's first
+                    // stage travels as the loads' scalar offset (one scalar add per operand and stage,
+                    // where an advancing pointer has the descriptor rebuilt from it each time)
+                    la.template load<false>(ra, cur.a_ptr, KT, (it + 1) * a_step4);
+                    lb.template load<false>(rb, cur.b_ptr, KT, (it + 1) * b_step4);
+                    fetched = true;
+                }
+            }
+            if (BY_OFFSET) {
+            } else if (!last) {          // next stage of this tile -> registers
                 a_ptr += a_step;
                 int knext;
                 if constexpr (CONV) {
@@ -646,6 +663,9 @@ void gemm_f32_mfma(const GemmParams p) {
             for (int g = 0; g < KT / 8; g++)
                 mma_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(acc, as, bs, wm, wn, g, r, h);
             if (fetched) {
+                // one wait for all of the stage's loads (issued a whole stage of matrix work ago) instead
+                // of one per staging register: vmcnt(0), the other counters left alone
+                if constexpr (INNER) __builtin_amdgcn_s_waitcnt(0x0F70);
                 la.store(ra, As[b ^ 1]);
                 lb.store(rb, Bs[b ^ 1]);
             }
@@ -673,6 +693,10 @@ void gemm_f32_mfma(const GemmParams p) {
                     stage(it, std::integral_constant<int, 0>(), std::true_type());
                     stage(it + 1, std::integral_constant<int, 1>(), std::true_type());
                 }
+            if constexpr (!CONV) {   // the inner stages left the pointers alone
+                a_ptr = cur.a_ptr + (size_t)it * a_step;
+                b_ptr = cur.b_ptr + (size_t)it * b_step;
+            }
         }
         for (; it < cur.nstage; it++) {
             stage(it, buf, std::false_type());
@@ -868,7 +892,16 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
 
 template <bool A_KIN, bool B_KIN, bool BIAS, bool CONV = false>
 static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stream) {
-    const bool paired = (tile & TILE_PAIRED) != 0;
+    // The paired form addresses a tile's stages by 32-bit scalar byte offsets from its first stage:
+    // K-inner operands advance 4 bytes per k, K-outer ones a whole row.  Where the longest K range
+    // of a tile would not fit, the plain form (advancing 64-bit pointers) runs instead.
+    long long kext = p.k_total;
+    if (p.split) {
+        const long long last = (long long)p.k_total - (long long)(p.nz - 1) * p.k_slice;
+        kext = last > p.k_slice ? last : p.k_slice;
+    }
+    const long long a_span = kext * 4 * (A_KIN ? 1 : p.lda), b_span = kext * 4 * (B_KIN ? 1 : p.ldb);
+    const bool paired = (tile & TILE_PAIRED) != 0 && a_span < 0x7fffffffLL && b_span < 0x7fffffffLL;
     switch (tile & ~TILE_PAIRED) {
         case TILE_128x128: return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV, true>(p, stream)
                                          : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV>(p, stream);
