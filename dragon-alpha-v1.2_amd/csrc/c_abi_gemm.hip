@@ -280,6 +280,17 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M) {
 }
 
 void dragon_gemm_force_tile(int32_t tile) { gemm_force_tile(tile); }
+int32_t dragon_gemm_paired_form_fits(int32_t variant, int32_t GridZ, int32_t N, int32_t M, int32_t K) {
+    if (variant < GEMM_NN || variant > GEMM_T2 || GridZ < 1 || N <= 0 || M <= 0 || K <= 0) return -1;
+    GemmParams p = {};
+    p.k_total = K;
+    p.lda = variant == GEMM_T1 ? N : K;
+    p.ldb = variant == GEMM_T2 ? K : M;
+    p.nz = GridZ;
+    p.split = GridZ > 1;
+    p.k_slice = ((K / GridZ) >> 3) << 3;
+    return gemm_paired_form_fits(variant != GEMM_T1, variant == GEMM_T2, p) ? 1 : 0;
+}
 int32_t dragon_gemm_choose_tile(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu) {
     if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
     return gemm_choose_tile(rows, cols, nz, k, num_cu, variant);

@@ -71,6 +71,10 @@ int gemm_device_num_cu();
 // The kernels address an operand tile with 32-bit byte offsets from the tile's origin: up to 256 rows
 // (or k) of pitch.  False when a leading stride is too long for that; the entry points reject such calls.
 bool gemm_pitches_addressable(const GemmParams& p);
+// The paired form addresses a tile's stages by 32-bit scalar byte offsets from its first stage: K-inner
+// operands advance 4 bytes per k, K-outer ones a whole row.  False where the longest K range of a tile
+// does not fit 31 bits; the launcher then runs the plain form (advancing 64-bit pointers) instead.
+bool gemm_paired_form_fits(bool a_k_inner, bool b_k_inner, const GemmParams& p);
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant = -1);   // variant: GEMM_* or -1
 void gemm_force_tile(int tile);
 int gemm_forced_tile();   // TILE_AUTO when the choice is left to gemm_choose_tile

@@ -23,6 +23,16 @@ bool gemm_pitches_addressable(const GemmParams& p) {
     return p.lda <= MAX_PITCH && p.ldb <= MAX_PITCH && p.ldc <= MAX_PITCH;
 }
 
+bool gemm_paired_form_fits(bool a_k_inner, bool b_k_inner, const GemmParams& p) {
+    long long kext = p.k_total;
+    if (p.split) {   // the last slice takes the remainder
+        const long long last = (long long)p.k_total - (long long)(p.nz - 1) * p.k_slice;
+        kext = last > p.k_slice ? last : p.k_slice;
+    }
+    const long long a_span = kext * 4 * (a_k_inner ? 1 : p.lda), b_span = kext * 4 * (b_k_inner ? 1 : p.ldb);
+    return a_span < 0x7fffffffLL && b_span < 0x7fffffffLL;
+}
+
 // a test and tuning hook: one setting for the whole process
 static std::atomic<int> g_forced_tile{TILE_AUTO};
 void gemm_force_tile(int tile) { g_forced_tile.store(tile, std::memory_order_relaxed); }

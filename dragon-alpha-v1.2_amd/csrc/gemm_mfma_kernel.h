@@ -892,16 +892,7 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
 
 template <bool A_KIN, bool B_KIN, bool BIAS, bool CONV = false>
 static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stream) {
-    // The paired form addresses a tile's stages by 32-bit scalar byte offsets from its first stage:
-    // K-inner operands advance 4 bytes per k, K-outer ones a whole row.  Where the longest K range
-    // of a tile would not fit, the plain form (advancing 64-bit pointers) runs instead.
-    long long kext = p.k_total;
-    if (p.split) {
-        const long long last = (long long)p.k_total - (long long)(p.nz - 1) * p.k_slice;
-        kext = last > p.k_slice ? last : p.k_slice;
-    }
-    const long long a_span = kext * 4 * (A_KIN ? 1 : p.lda), b_span = kext * 4 * (B_KIN ? 1 : p.ldb);
-    const bool paired = (tile & TILE_PAIRED) != 0 && a_span < 0x7fffffffLL && b_span < 0x7fffffffLL;
+    const bool paired = (tile & TILE_PAIRED) != 0 && gemm_paired_form_fits(A_KIN, B_KIN, p);
     switch (tile & ~TILE_PAIRED) {
         case TILE_128x128: return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV, true>(p, stream)
                                          : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV>(p, stream);

@@ -260,8 +260,15 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M);
  * LDS stage); 6 = 128x128, 7 = 64x64, 8 = 128x64, 9 = 64x128 with 32 k per stage; 10 = 64x64
  * with 64 k, 11 = 64x64 with 128 k, 12 = 128x128, 13 = 128x64, 14 = 64x128 with 64 k per stage;
  * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
- * directly through four stage buffers. */
+ * directly through four stage buffers.  Adding 256 to a shape 0..9 selects its paired-stage form
+ * (stages run two by two with compile-time LDS buffers; what the automatic choice takes from
+ * K = 512 on). */
 void dragon_gemm_force_tile(int32_t tile);
+/* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
+ * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the
+ * operand's advance per k (4 bytes, or a row of a K-outer operand) must stay below 2^31; 0 if not (the
+ * launch then runs the plain form), -1 on bad arguments.  Host arithmetic only; for tests. */
+int32_t dragon_gemm_paired_form_fits(int32_t variant, int32_t GridZ, int32_t N, int32_t M, int32_t K);
 /* The shape the automatic choice takes for a product of `rows` x `cols` outputs, depth `nz` (batch or
  * K slices), `k` per output, on `num_cu` compute units; variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, -1 = unknown.
  * Pure host arithmetic (no device needed); returns the forced shape while one is forced, -1 on bad

@@ -103,6 +103,20 @@ def test_argument_validation_rejects_before_touching_the_device(dh):
     assert t2(s, 1, ok_ptr, ok_ptr, ok_ptr, 2, 4, 4, 4, too_long) == INVALID_VALUE
 
 
+def test_paired_form_is_kept_to_spans_its_32_bit_offsets_reach(dh):
+    fits = dh.lib.dragon_gemm_paired_form_fits
+    NN, T1, T2 = 0, 1, 2
+    assert fits(NN, 1, 4096, 4096, 4096) == 1 and fits(T1, 1, 4096, 4096, 4096) == 1
+    # K-outer operands advance a whole row per k: B[K, M] of 2 GiB and more is out of reach
+    assert fits(NN, 1, 64, 65536, 8188) == 1 and fits(NN, 1, 64, 65536, 8192) == 0
+    assert fits(T1, 1, 65536, 64, 8192) == 0                    # A[K, N] likewise
+    assert fits(T2, 1, 65536, 65536, 8192) == 1                 # both K-inner: 4 bytes per k
+    assert fits(T2, 1, 4, 4, 1 << 29) == 0
+    # split-K: the longest slice counts (the last one takes the remainder)
+    assert fits(NN, 4, 64, 65536, 8192 * 4 - 32) == 1 and fits(NN, 4, 64, 65536, 8192 * 4) == 0
+    assert fits(NN, 0, 4, 4, 4) == -1 and fits(3, 1, 4, 4, 4) == -1
+
+
 def test_python_wrapper_raises_the_exception_type(dh):
     with pytest.raises(dh.CudaException) as e:
         dh.Cuda_matMul.matMul([0], 1, 0, 0, 0, 4, 4, 4)
