@@ -280,6 +280,12 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M) {
 }
 
 void dragon_gemm_force_tile(int32_t tile) { gemm_force_tile(tile); }
+void dragon_gemm_tile_divisor(uint32_t d, uint32_t* mul, uint32_t* shift) {
+    unsigned m = 0, s = 0;
+    gemm_magic_divisor(d, m, s);
+    if (mul) *mul = m;
+    if (shift) *shift = s;
+}
 int32_t dragon_gemm_paired_form_fits(int32_t variant, int32_t GridZ, int32_t N, int32_t M, int32_t K) {
     if (variant < GEMM_NN || variant > GEMM_T2 || GridZ < 1 || N <= 0 || M <= 0 || K <= 0) return -1;
     GemmParams p = {};

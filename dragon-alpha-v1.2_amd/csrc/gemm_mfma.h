@@ -64,7 +64,14 @@ struct GemmParams {
     const float* bias;      // optional row vector added to C[i][j] for i < bias_rows, j < bias_width
     int bias_rows, bias_width;
     int tiles_m, tiles_n;   // filled by the launcher
+    // filled by the launcher (gemm_fill_tile_divisors): the divisors of the tile-index decode as
+    // multiply-and-shift pairs, n / d == mulhi(2 * n, mul) >> shift for 0 <= n < 2^31
+    unsigned div_tiles_mul, div_tiles_shift;   // d = tiles_m * tiles_n
+    unsigned div_band_mul, div_band_shift;     // d = 8 * tiles_n (a band of 8 tile rows)
+    unsigned div_last_mul, div_last_shift;     // d = tile rows of the last, shorter band (tiles_m % 8, or 8)
 };
+void gemm_fill_tile_divisors(GemmParams& p);
+void gemm_magic_divisor(unsigned d, unsigned& mul, unsigned& shift);
 
 // Compute units of the current device (256 when no device answers), cached per device.
 int gemm_device_num_cu();

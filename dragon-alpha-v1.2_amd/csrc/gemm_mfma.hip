@@ -18,6 +18,24 @@ int gemm_device_num_cu() {
     return n;
 }
 
+// n / d == mulhi(2n, mul) >> shift for every 0 <= n < 2^31: mul = ceil(2^(31 + shift) / d) with
+// shift = ceil(log2 d) lies in [2^31, 2^32), and the error n * (mul * d - 2^(31+shift)) stays below 2^(31+shift).
+void gemm_magic_divisor(unsigned d, unsigned& mul, unsigned& shift) {
+    if (d == 0) d = 1;
+    unsigned l = 0;
+    while ((1ull << l) < d) l++;
+    const unsigned long long two = 1ull << (31 + l);
+    mul = (unsigned)((two + d - 1) / d);
+    shift = l;
+}
+
+void gemm_fill_tile_divisors(GemmParams& p) {
+    gemm_magic_divisor((unsigned)(p.tiles_m * p.tiles_n), p.div_tiles_mul, p.div_tiles_shift);
+    gemm_magic_divisor((unsigned)(8 * p.tiles_n), p.div_band_mul, p.div_band_shift);
+    const int last = p.tiles_m % 8;
+    gemm_magic_divisor((unsigned)(last ? last : 8), p.div_last_mul, p.div_last_shift);
+}
+
 bool gemm_pitches_addressable(const GemmParams& p) {
     constexpr long long MAX_PITCH = (OOB_OFFSET / 4 - 256) / 256;   // floats
     return p.lda <= MAX_PITCH && p.ldb <= MAX_PITCH && p.ldc <= MAX_PITCH;

@@ -474,20 +474,28 @@ struct TileCtx {
     int nstage;           // LDS stages to run (>= 1; an empty slice runs one all-zero stage)
 };
 
+// n / d for 0 <= n < 2^31 with the pair gemm_fill_tile_divisors made for d
+__device__ __forceinline__ int div_by(int n, unsigned mul, unsigned shift) {
+    return (int)(__umulhi((unsigned)n << 1, mul) >> shift);
+}
+
 template <bool A_KIN, bool B_KIN, int BM, int BN, int KT, typename LoadA, typename LoadB>
 __device__ __forceinline__ TileCtx decode_tile(const GemmParams& p, int lid) {
     TileCtx c;
+    // the three divisions are multiply-and-shift with host-made constants: a division by a run-time
+    // value costs some 25 instructions, and this runs between the matrix work of two tiles
     const int tiles = p.tiles_m * p.tiles_n;
-    const int z = lid / tiles;
+    const int z = div_by(lid, p.div_tiles_mul, p.div_tiles_shift);
     int tt = lid - z * tiles;
     // bands of 8 tile rows, walked row-fastest, keep one XCD's concurrent tiles compact
     constexpr int BAND = 8;
     const int band_sz = BAND * p.tiles_n;
-    const int band = tt / band_sz;
+    const int band = div_by(tt, p.div_band_mul, p.div_band_shift);
     const int first_m = band * BAND;
-    const int band_rows = (p.tiles_m - first_m < BAND) ? (p.tiles_m - first_m) : BAND;
+    const bool short_band = p.tiles_m - first_m < BAND;
+    const int band_rows = short_band ? (p.tiles_m - first_m) : BAND;
     tt -= band * band_sz;
-    const int tile_n = tt / band_rows;
+    const int tile_n = short_band ? div_by(tt, p.div_last_mul, p.div_last_shift) : (tt >> 3);
     const int tile_m = first_m + (tt - tile_n * band_rows);
     c.row0 = tile_m * BM;
     c.col0 = tile_n * BN;
@@ -875,6 +883,7 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
     if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidValue;
+    gemm_fill_tile_divisors(p);
     // workgroups the device keeps resident: one persistent workgroup per slot
     static std::atomic<int> resident_cache{0};   // per instantiation
     const int resident_per_cu = resident_workgroups(resident_cache, kernel);
@@ -932,6 +941,7 @@ static hipError_t launch_cfg_dma(GemmParams p, hipStream_t stream) {
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
     if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidValue;
+    gemm_fill_tile_divisors(p);
     static std::atomic<int> resident_cache{0};   // per instantiation
     const int resident_per_cu = resident_workgroups(resident_cache, kernel);
     const long long slots = (long long)gemm_device_num_cu() * resident_per_cu;

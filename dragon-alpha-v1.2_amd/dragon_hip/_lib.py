@@ -77,6 +77,7 @@ SIGNATURES = {
     "dragon_gemm_force_tile": (None, [i32]),
     "dragon_gemm_choose_tile": (i32, [i32, i32, i32, i32, i32, i32]),
     "dragon_gemm_paired_form_fits": (i32, [i32, i32, i32, i32, i32]),
+    "dragon_gemm_tile_divisor": (None, [ctypes.c_uint32, POINTER(ctypes.c_uint32), POINTER(ctypes.c_uint32)]),
     # include/dragon_hip_runtime.h
     "dragon_Cuda_malloc": (i64, [i64]),
     "dragon_Cuda_free": (i32, [i64]),

@@ -269,6 +269,10 @@ void dragon_gemm_force_tile(int32_t tile);
  * operand's advance per k (4 bytes, or a row of a K-outer operand) must stay below 2^31; 0 if not (the
  * launch then runs the plain form), -1 on bad arguments.  Host arithmetic only; for tests. */
 int32_t dragon_gemm_paired_form_fits(int32_t variant, int32_t GridZ, int32_t N, int32_t M, int32_t K);
+/* The multiply-and-shift pair the kernels divide a tile index by d with: n / d == (((2n) * mul) >> 32) >> shift
+ * for every 0 <= n < 2^31 (the launcher makes the pairs, the kernels only multiply).  Host arithmetic; for
+ * tests. */
+void dragon_gemm_tile_divisor(uint32_t d, uint32_t* mul, uint32_t* shift);
 /* The shape the automatic choice takes for a product of `rows` x `cols` outputs, depth `nz` (batch or
  * K slices), `k` per output, on `num_cu` compute units; variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, -1 = unknown.
  * Pure host arithmetic (no device needed); returns the forced shape while one is forced, -1 on bad

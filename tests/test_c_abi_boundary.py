@@ -117,6 +117,26 @@ def test_paired_form_is_kept_to_spans_its_32_bit_offsets_reach(dh):
     assert fits(NN, 0, 4, 4, 4) == -1 and fits(3, 1, 4, 4, 4) == -1
 
 
+def test_tile_index_divisors_divide_exactly(dh):
+    """The kernels turn a tile index into (slice or batch, band, column) with multiply-and-shift pairs made
+    on the host: checked against integer division at the edges of every quotient step and at random."""
+    rng = np.random.default_rng(77)
+    ds = list(range(1, 600)) + [2 ** k for k in range(31)] + [2 ** k + 1 for k in range(30)] + \
+        [2 ** k - 1 for k in range(2, 32)] + [int(v) for v in rng.integers(1, 2 ** 31, 300)]
+    mul, shift = ctypes.c_uint32(), ctypes.c_uint32()
+    for d in ds:
+        dh.lib.dragon_gemm_tile_divisor(d, ctypes.byref(mul), ctypes.byref(shift))
+        m, s = mul.value, shift.value
+        assert 2 ** 31 <= m < 2 ** 32
+        ns = [0, 1, d - 1, d, d + 1, 2 ** 31 - 1, 2 ** 31 - 2] + [k * d - 1 for k in range(1, 12)] + \
+            [k * d for k in range(1, 12)] + [int(v) for v in rng.integers(0, 2 ** 31, 40)]
+        top = (2 ** 31 - 1) // d
+        ns += [top * d, top * d - 1, top * d + d - 1]
+        for n in ns:
+            if 0 <= n < 2 ** 31:
+                assert ((((2 * n) & 0xffffffff) * m) >> 32) >> s == n // d, (n, d)
+
+
 def test_python_wrapper_raises_the_exception_type(dh):
     with pytest.raises(dh.CudaException) as e:
         dh.Cuda_matMul.matMul([0], 1, 0, 0, 0, 4, 4, 4)
