@@ -98,13 +98,27 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
     // ---- staging of the K / V tiles ----
     const int s_chunk = t % CPR, s_row = t / CPR;
     v4f kreg[PASSES], vreg[PASSES];
+    // A lane's byte offsets inside a key tile never change (a chunk beyond the head dimension is out of
+    // range for good).  The tile's first key goes into the buffer descriptor's base and the bytes up
+    // to the end of the last key into its size, so the hardware returns zeros for rows beyond the key
+    // count: a step's fetch costs scalar instructions only, no per-lane address or test.
+    int koff[PASSES], voff[PASSES];
+#pragma unroll
+    for (int s = 0; s < PASSES; s++) {
+        const int row = s_row + s * RPP;
+        koff[s] = (s_chunk * 4 < p.dk4) ? (row * p.k_l + s_chunk * 4) * 4 : OOB_OFFSET;
+        voff[s] = (s_chunk * 4 < p.dv4) ? (row * p.v_l + s_chunk * 4) * 4 : OOB_OFFSET;
+    }
     auto fetch = [&](int key0) {
+        const int left = p.nk - key0;   // > 0
+        const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(Kb + (size_t)key0 * p.k_l), 0, left * p.k_l * 4, RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(Vb + (size_t)key0 * p.v_l), 0, left * p.v_l * 4, RSRC_FLAGS);
 #pragma unroll
         for (int s = 0; s < PASSES; s++) {
-            const int key = key0 + s_row + s * RPP;
-            const bool in = key < p.nk;
-            kreg[s] = buffer_load_f4(Kb, (in && s_chunk * 4 < p.dk4) ? (key * p.k_l + s_chunk * 4) * 4 : OOB_OFFSET);
-            vreg[s] = buffer_load_f4(Vb, (in && s_chunk * 4 < p.dv4) ? (key * p.v_l + s_chunk * 4) * 4 : OOB_OFFSET);
+            kreg[s] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rk, koff[s], 0, 0));
+            vreg[s] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rv, voff[s], 0, 0));
         }
     };
     auto stage = [&](int buf) {
