@@ -138,6 +138,21 @@ def test_conv3D_every_tile_shape_with_whole_channel_stages(dh, gpu, tile):
     assert np.array_equal(Y, oracle.conv3D(X, W, 1, 2, 1, 1))
 
 
+@pytest.mark.parametrize("tile", [257, 260, 1])
+def test_conv3D_paired_stages_across_tile_boundaries(dh, gpu, tile):
+    # more tiles than resident workgroups and nine 16-k stages: a workgroup's second tile starts on the odd
+    # LDS buffer, with the filter-tap walk restarted (tile 1: the plain form on the same shape)
+    rng = np.random.default_rng(500 + tile)
+    X = rng.integers(-3, 4, (48, 64, 64, 16)).astype(np.float32)
+    W = rng.integers(-3, 4, (64, 3, 3, 16)).astype(np.float32)
+    dh.force_tile(tile)
+    try:
+        Y, _ = run_conv(dh, X, W, 1, 1, 1, 1)
+    finally:
+        dh.force_tile(-1)
+    assert np.array_equal(Y, oracle.conv3D(X, W, 1, 1, 1, 1))
+
+
 @pytest.mark.parametrize("entry", ["texture", "V2", "np", "W1", "GemmR", "GemmR_W1", "winograd"])
 def test_every_native_family_computes_the_same_convolution(dh, gpu, entry):
     rng = np.random.default_rng(len(entry))
