@@ -83,10 +83,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias,attention,conv,transpose,transfer",
+    ap.add_argument("--configs", default="3,4,5,bias,attention,conv,transpose,transfer,engine",
                     help="which of the other workloads to time (default all): BASELINE configs 3, 4, 5, "
                          "the biased fully-connected layer, the attention chain, the forward convolution, "
-                         "dimension swaps, tensor upload / download")
+                         "dimension swaps, tensor upload / download, the host mirror's own overhead")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
                          "(the known-size copy that FETCH_SIZE / WRITE_SIZE are scaled by)")
@@ -487,6 +487,35 @@ def main():
                                                      "GBps": round(logical / dn / 1e9, 2)}
         Cuda.free(dT)
         Cuda.freeHost(pinned)
+
+    if "engine" in extra:
+        # the config-3 product through the host-side engine (Engine.matMulT1 -> split-K policy -> two-stage
+        # launch -> SplitKSyncer): host-clock time per call including the wait for the result, with the
+        # reference's recycling memory pool behind C and the partial buffer, and with a device allocation
+        # and release per block
+        log("engine mirror ...")
+        from dragon_hip import engine as eng
+        g = synthetic.stream_for(3)
+        K3, N3 = 131072, 256
+        A3 = g.normal((K3, N3), 0.0, 0.05)
+        B3 = g.normal((K3, N3), 0.0, 0.05)
+        for name, pool_bytes in (("memory pool (memp1)", 2 << 30), ("device allocation per block", 0)):
+            eg = eng.cuda_float32(0, 32, max_mem_size=pool_bytes)
+            tA, tB = eg.tensor(A3, K3, N3), eg.tensor(B3, K3, N3)
+
+            def call():
+                tC = eg.matMulT1(tA, tB)     # sync(true): returns when C is there, partial buffer released
+                eg.delete(tC)
+            for _ in range(3):
+                call()
+            reps, t0 = 30, time.perf_counter()
+            for _ in range(reps):
+                call()
+            ms = (time.perf_counter() - t0) / reps * 1e3
+            per_config["engine.matMulT1 256x256 K=131072 (GridZ %d), %s" % (eg.get_param("last_gridZ"), name)] = {
+                "ms": round(ms, 4), "tflops": round(2.0 * N3 * N3 * K3 / ms / 1e9, 2),
+                "pct_peak": round(100 * 2.0 * N3 * N3 * K3 / ms / 1e9 / PEAK_TFLOPS, 1)}
+            eg.close()
 
     Cuda.deleteStream(stream)
     out = {

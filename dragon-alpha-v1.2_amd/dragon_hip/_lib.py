@@ -129,8 +129,10 @@ SIGNATURES = {
     # include/dragon_hip_engine.h
     "dragon_engine_last_error": (c_char_p, []),
     "dragon_engine_last_cuda_code": (i32, []),
+    "dragon_engine_last_status": (i32, []),
     "dragon_engine_cuda_float32": (c_void_p, [i32, i32]),
     "dragon_engine_cuda_float32_buffered": (c_void_p, [i32, i32, i64]),
+    "dragon_engine_cuda_float32_pooled": (c_void_p, [i32, i32, i64, i64]),
     "dragon_engine_delete": (None, [c_void_p]),
     "dragon_engine_check": (i32, [c_void_p, i32]),
     "dragon_engine_sync": (i32, [c_void_p, i32]),

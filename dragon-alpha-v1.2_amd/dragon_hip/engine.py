@@ -70,16 +70,19 @@ MATMUL, MATMUL_T1, MATMUL_T2, BMM, BMM_T1, BMM_T2 = range(6)
 class Engine:
     """alpha.engine.cuda_float32(deviceId, ...)"""
 
-    def __init__(self, device_id=0, stream_pool_size=32, max_trans_buf_size=0):
-        if max_trans_buf_size > 0:
+    def __init__(self, device_id=0, stream_pool_size=32, max_trans_buf_size=0, max_mem_size=0):
+        """max_trans_buf_size > 0: pinned staging pool for uploads / downloads; max_mem_size > 0: device
+        memory pool (alpha.engine.memp1) behind tensors and split-K partial buffers."""
+        if max_mem_size > 0:
+            self._h = lib.dragon_engine_cuda_float32_pooled(device_id, stream_pool_size, max_mem_size,
+                                                            max_trans_buf_size)
+        elif max_trans_buf_size > 0:
             self._h = lib.dragon_engine_cuda_float32_buffered(device_id, stream_pool_size,
                                                               max_trans_buf_size)
         else:
             self._h = lib.dragon_engine_cuda_float32(device_id, stream_pool_size)
         if not self._h:
-            msg = _last_code()
-            code = lib.dragon_engine_last_cuda_code()
-            raise CudaException(code) if code else RuntimeError(msg)
+            _raise(lib.dragon_engine_last_status() or 4)
 
     def close(self):
         if self._h:
@@ -109,13 +112,7 @@ class Engine:
     # ---- tensors ----
     def _wrap(self, h):
         if not h:
-            msg = _last_code()
-            if "null" in msg.lower():
-                raise NullPointerException(msg)
-            code = lib.dragon_engine_last_cuda_code()
-            if msg.startswith("hip") and code:
-                raise CudaException(code)
-            raise IllegalArgumentException(msg)
+            _raise(lib.dragon_engine_last_status() or 4)
         return Tensor(self, h)
 
     def empty(self, *dim):
@@ -260,5 +257,5 @@ class Engine:
         return self.linear2_row(inplace, X1, X2, 1.0, 1.0, 0.0)
 
 
-def cuda_float32(device_id=0, stream_pool_size=32, max_trans_buf_size=0):
-    return Engine(device_id, stream_pool_size, max_trans_buf_size)
+def cuda_float32(device_id=0, stream_pool_size=32, max_trans_buf_size=0, max_mem_size=0):
+    return Engine(device_id, stream_pool_size, max_trans_buf_size, max_mem_size)

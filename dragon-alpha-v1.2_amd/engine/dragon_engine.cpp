@@ -413,32 +413,36 @@ void CudaFloat32EngineBase::set2D(int64_t address, const float* value, int heigh
     streamPool_->returnStream(stream);
 }
 
-// ---- PinnedMempool (PinnedMempool.java:96-200) ---------------------------------------------------
-PinnedMempool::Block PinnedMempool::malloc(int64_t mem_size) {
+// ---- RecyclingPool: Mempool.java:150-225 + Memp1.java:27-80; PinnedMempool.java:96-200 -------------
+RecyclingPool::Block RecyclingPool::malloc(int64_t mem_size) {
     std::lock_guard<std::mutex> g(mu_);
     if (mem_size <= 0) throw IllegalArgumentException("mem_size must be positive");
     mem_size = (mem_size + 3) >> 2 << 2;
+    if (mem_size > max_mem_size_)
+        throw IllegalArgumentException(fmt("mem_size { got %lld } > mempool.max_mem_size { got %lld }",
+                                           (long long)mem_size, (long long)max_mem_size_));
     int64_t size = 0, address = 0;
     auto it = pool_.lower_bound(mem_size);                       // remove_section(size, 1.5 * size)
     if (it != pool_.end() && it->first <= (int64_t)((double)mem_size * 1.5)) {
         size = it->first; address = it->second;
         pool_.erase(it);
     } else {
-        // the Java pool waits up to 10 s for another thread to free memory; this one fails at once
+        // the Java pools wait up to 10 s for the collector or another thread to free memory; this one
+        // fails at once
         if (mem_size > max_mem_size_ - used_mem_size_)
             throw std::runtime_error("[Error] Maximum Memory { " + std::to_string(max_mem_size_ >> 20) +
-                                     " } is insufficient. Try to alloc more");
+                                     " MB } is insufficient. Try to alloc more");
         while (mem_size > max_mem_size_ - total_mem_size_ && !pool_.empty()) {   // alloc_free: largest first
             auto big = std::prev(pool_.end());
-            cu(dragon_Cuda_freeHost(big->second));
+            raw_free(big->second);
             total_mem_size_ -= big->first;
             blocks_.erase(big->second);
             grave_.erase(big->second);
             pool_.erase(big);
         }
-        address = dragon_Cuda_mallocHost(mem_size);
+        address = raw_malloc(mem_size);
         if (address == 0)
-            throw std::runtime_error("Cuda_malloc_host: failed to alloc pinned-memory for [mem_size = " +
+            throw std::runtime_error(std::string("failed to alloc ") + what() + " for [mem_size = " +
                                      std::to_string(mem_size) + " ]");
         size = mem_size;
         total_mem_size_ += size;
@@ -448,20 +452,27 @@ PinnedMempool::Block PinnedMempool::malloc(int64_t mem_size) {
     grave_.erase(address);
     return Block{size >> 2, address};
 }
-bool PinnedMempool::free(int64_t size, int64_t address) {
+bool RecyclingPool::free(int64_t size, int64_t address) {
     std::lock_guard<std::mutex> g(mu_);
     if (address == 0 || grave_.count(address) || !blocks_.count(address)) return false;
-    const int64_t bytes = size << 2;
+    const int64_t bytes = blocks_[address];   // what the block really holds (the caller reports the same)
+    (void)size;
     pool_.emplace(bytes, address);
     grave_.insert(address);
     used_mem_size_ -= bytes;
     return true;
 }
-void PinnedMempool::clear() {
+void RecyclingPool::clear() {
     std::lock_guard<std::mutex> g(mu_);
-    for (auto& kv : blocks_) (void)dragon_Cuda_freeHost(kv.first);
+    for (auto& kv : blocks_) raw_free(kv.first);
     blocks_.clear(); pool_.clear(); grave_.clear();
     total_mem_size_ = used_mem_size_ = 0;
+}
+int64_t PinnedMempool::raw_malloc(int64_t bytes) { return dragon_Cuda_mallocHost(bytes); }
+void PinnedMempool::raw_free(int64_t address) { (void)dragon_Cuda_freeHost(address); }
+int64_t Memp1::raw_malloc(int64_t bytes) { return base_->malloc(bytes); }
+void Memp1::raw_free(int64_t address) {
+    try { base_->free(address); } catch (const std::exception&) {}   // also runs from destructors
 }
 
 // Shared body of matMul / matMulT1 / matMulT2 (:1534-1589, :1751-1806, :1870-1925) and, with a
@@ -774,15 +785,23 @@ EngineCore::Block EngineCore::malloc(int mem_length) {
     if (check && mem_length <= 0)
         throw IllegalArgumentException(fmt("mem_length { got %lld } must be positive", mem_length));
     Block b;
-    b.size = (int64_t)mem_length * 4;
-    b.address = base_->malloc(b.size);
+    if (mempool_) {            // EngineCore.malloc -> Mempool.malloc (EngineCore.java:154-165)
+        const RecyclingPool::Block pb = mempool_->malloc((int64_t)pad4(mem_length) * 4);
+        b.size = pb.size * 4;
+        b.address = pb.address;
+    } else {
+        b.size = (int64_t)mem_length * 4;
+        b.address = base_->malloc(b.size);
+    }
     std::lock_guard<std::mutex> g(mu_);
     live_blocks_++;
     return b;
 }
-void EngineCore::free(int64_t, int64_t address) {
+void EngineCore::free(int64_t size, int64_t address) {
     if (address == 0) return;
-    base_->free(address);
+    if (mempool_) {
+        if (!mempool_->free(size >> 2, address)) return;   // not this pool's, or freed already
+    } else base_->free(address);
     std::lock_guard<std::mutex> g(mu_);
     live_blocks_--;
 }
@@ -1046,13 +1065,17 @@ Tensor& Tensor::c() {
 }
 
 // ---- Engine ------------------------------------------------------------------------------------------------
-Engine::Engine(int deviceId, int streamPool_maxsize, int64_t max_trans_buf_size) {
+Engine::Engine(int deviceId, int streamPool_maxsize, int64_t max_trans_buf_size, int64_t max_mem_size) {
     base_.reset(new CudaFloat32EngineBase(deviceId, streamPool_maxsize));
     if (max_trans_buf_size > 0)
         base_->buf_mempool(std::unique_ptr<PinnedMempool>(new PinnedMempool(max_trans_buf_size)));
     core_.reset(new EngineCore(base_.get(), true));
+    if (max_mem_size > 0) core_->mempool(std::unique_ptr<Memp1>(new Memp1(max_mem_size, base_.get())));
 }
-Engine::~Engine() {}
+Engine::~Engine() {
+    core_.reset();   // the pool hands its blocks back through the engine base, which must still be there
+    base_.reset();
+}
 
 static void equals(int a, const char* an, int b, const char* bn) {
     if (a != b)

@@ -66,28 +66,62 @@ private:
     std::mutex mu_;
 };
 
-// ---- pinned host staging buffers for tensor transfer (z/dragon/engine/cuda/impl/PinnedMempool.java)
-// Blocks are recycled by size: a request takes the smallest free block of [size, 1.5*size], else
-// allocates; when the budget is exhausted free blocks are released largest-first to make room.
-class PinnedMempool {
+// ---- memory pools ------------------------------------------------------------------------------
+// The recycling policy of the reference's pools (z/dragon/engine/memp/Mempool.java:150-225 with
+// Memp1.java:27-80, and cuda/impl/PinnedMempool.java:96-200, which repeats it for pinned memory):
+// blocks are recycled by size -- a request takes the smallest free block of [size, 1.5*size] (equal
+// sizes first in, first out), else allocates; when the budget is exhausted free blocks are released
+// largest-first to make room; an address can be freed once until it is handed out again.
+class RecyclingPool {
 public:
-    explicit PinnedMempool(int64_t maxMemorySize) : max_mem_size_(maxMemorySize) {}
-    ~PinnedMempool() { clear(); }
-    struct Block { int64_t size, address; };   // size in floats (bytes / 4), as the Java pool reports it
+    explicit RecyclingPool(int64_t maxMemorySize) : max_mem_size_(maxMemorySize) {}
+    virtual ~RecyclingPool() {}
+    struct Block { int64_t size, address; };   // size in floats (bytes / 4), as the Java pools report it
     Block malloc(int64_t mem_size);            // mem_size in bytes
     bool free(int64_t size, int64_t address);  // size as returned by malloc
-    void clear();
+    void clear();                              // releases every block, handed out or not
     int64_t max_mem_size() const { return max_mem_size_; }
     int64_t total_mem_size() const { return total_mem_size_; }
     int64_t used_mem_size() const { return used_mem_size_; }
     int physical_block_num() const { return (int)blocks_.size(); }
     int buffered_block_num() const { return (int)pool_.size(); }
+protected:
+    virtual int64_t raw_malloc(int64_t bytes) = 0;   // 0 on failure
+    virtual void raw_free(int64_t address) = 0;
+    virtual const char* what() const = 0;
 private:
     int64_t max_mem_size_, total_mem_size_ = 0, used_mem_size_ = 0;
     std::multimap<int64_t, int64_t> pool_;     // free blocks: size in bytes -> address
     std::map<int64_t, int64_t> blocks_;        // every block this pool owns: address -> size in bytes
     std::set<int64_t> grave_;                  // addresses currently free (guards a double free)
     std::mutex mu_;
+};
+
+// pinned host staging buffers for tensor transfer (z/dragon/engine/cuda/impl/PinnedMempool.java)
+class PinnedMempool : public RecyclingPool {
+public:
+    explicit PinnedMempool(int64_t maxMemorySize) : RecyclingPool(maxMemorySize) {}
+    ~PinnedMempool() override { clear(); }
+protected:
+    int64_t raw_malloc(int64_t bytes) override;
+    void raw_free(int64_t address) override;
+    const char* what() const override { return "pinned-memory"; }
+};
+
+class CudaFloat32EngineBase;
+// device memory for tensors and split-K partials (z/dragon/engine/memp/Memp1.java, the pool the
+// reference's tests build their engines with: alpha.engine.memp1(size)).  Without one, EngineCore
+// allocates and frees every block on the device itself.
+class Memp1 : public RecyclingPool {
+public:
+    Memp1(int64_t maxMemorySize, CudaFloat32EngineBase* base) : RecyclingPool(maxMemorySize), base_(base) {}
+    ~Memp1() override { clear(); }
+protected:
+    int64_t raw_malloc(int64_t bytes) override;
+    void raw_free(int64_t address) override;
+    const char* what() const override { return "device memory"; }
+private:
+    CudaFloat32EngineBase* base_;
 };
 
 // ---- completion handles ----------------------------------------------------------------------
@@ -227,12 +261,14 @@ public:
     CudaFloat32EngineBase* engineBase() { return base_; }
     bool check;
 
-    // a block is {size in bytes, address}; the pool behind it is the caller's business in
-    // the reference, here every block is its own device allocation
+    // a block is {size in bytes, address}.  With a pool (EngineCore(mempool, check) of the reference)
+    // blocks are recycled through it; without one every block is its own device allocation.
     struct Block { int64_t size, address; };
     Block malloc(int mem_length);
     void free(int64_t size, int64_t address);
     int64_t live_blocks() const { return live_blocks_; }
+    void mempool(std::unique_ptr<Memp1> pool) { mempool_ = std::move(pool); }
+    Memp1* mempool() { return mempool_.get(); }
     SyncerPtr memset(int64_t address, int value, int length);
     void get1D(int64_t address, float* value, int length);
     void get2D(int64_t address, float* value, int height, int width);
@@ -269,6 +305,7 @@ private:
                             int sw, int ph, int pw) const;
     CudaFloat32EngineBase* base_;
     int64_t live_blocks_ = 0;
+    std::unique_ptr<Memp1> mempool_;
     std::mutex mu_;
 };
 
@@ -293,8 +330,9 @@ private:
 // ---- Engine: the tensor-level API ------------------------------------------------------------------------
 class Engine {
 public:
-    // max_trans_buf_size > 0 gives the engine a PinnedMempool of that many bytes (Alpha.java:770-790)
-    Engine(int deviceId, int streamPool_maxsize, int64_t max_trans_buf_size = 0);
+    // max_trans_buf_size > 0 gives the engine a PinnedMempool of that many bytes, max_mem_size > 0 a
+    // Memp1 device pool of that many (Alpha.java:770-790)
+    Engine(int deviceId, int streamPool_maxsize, int64_t max_trans_buf_size = 0, int64_t max_mem_size = 0);
     ~Engine();
     EngineCore& engineCore() { return *core_; }
     CudaFloat32EngineBase& engineBase() { return *base_; }

@@ -8,26 +8,27 @@
 
 using namespace dragon;
 
-struct dragon_engine { Engine eg; dragon_engine(int d, int p, int64_t b = 0) : eg(d, p, b) {} };
+struct dragon_engine { Engine eg; dragon_engine(int d, int p, int64_t b = 0, int64_t m = 0) : eg(d, p, b, m) {} };
 struct dragon_tensor { Tensor* ts; };
 
 namespace {
 thread_local std::string g_err;
 thread_local int g_cuda_code = 0;
+thread_local int g_status = DRAGON_OK;
 
 template <typename F>
 int guard(F f) {
     try {
         f();
-        return DRAGON_OK;
+        return g_status = DRAGON_OK;
     } catch (const NullPointerException& e) {
-        g_err = e.what(); return DRAGON_E_NULL_POINTER;
+        g_err = e.what(); return g_status = DRAGON_E_NULL_POINTER;
     } catch (const IllegalArgumentException& e) {
-        g_err = e.what(); return DRAGON_E_ILLEGAL_ARGUMENT;
+        g_err = e.what(); return g_status = DRAGON_E_ILLEGAL_ARGUMENT;
     } catch (const CudaException& e) {
-        g_err = e.what(); g_cuda_code = e.code; return DRAGON_E_CUDA;
+        g_err = e.what(); g_cuda_code = e.code; return g_status = DRAGON_E_CUDA;
     } catch (const std::exception& e) {
-        g_err = e.what(); return DRAGON_E_OTHER;
+        g_err = e.what(); return g_status = DRAGON_E_OTHER;
     }
 }
 std::vector<int> dims(const int32_t* dim, int32_t ndim) {
@@ -48,6 +49,7 @@ extern "C" {
 
 const char* dragon_engine_last_error(void) { return g_err.c_str(); }
 int32_t dragon_engine_last_cuda_code(void) { return g_cuda_code; }
+int32_t dragon_engine_last_status(void) { return g_status; }
 
 dragon_engine* dragon_engine_cuda_float32(int32_t device_id, int32_t stream_pool_size) {
     dragon_engine* e = nullptr;
@@ -58,6 +60,15 @@ dragon_engine* dragon_engine_cuda_float32_buffered(int32_t device_id, int32_t st
                                                    int64_t max_trans_buf_size) {
     dragon_engine* e = nullptr;
     guard([&] { e = new dragon_engine(device_id, stream_pool_size, max_trans_buf_size); });
+    return e;
+}
+dragon_engine* dragon_engine_cuda_float32_pooled(int32_t device_id, int32_t stream_pool_size,
+                                                 int64_t max_mem_size, int64_t max_trans_buf_size) {
+    dragon_engine* e = nullptr;
+    guard([&] {
+        if (max_mem_size <= 0) throw IllegalArgumentException("Mempool.max_mem_size must be positive");
+        e = new dragon_engine(device_id, stream_pool_size, max_trans_buf_size, max_mem_size);
+    });
     return e;
 }
 void dragon_engine_delete(dragon_engine* eg) { delete eg; }
@@ -117,6 +128,14 @@ int32_t dragon_engine_get_param(dragon_engine* eg, const char* name) {
         else if (n == "buf_buffered_blocks") out = b.buf_mempool() ? b.buf_mempool()->buffered_block_num() : -1;
         else if (n == "buf_used_mem_size") out = b.buf_mempool() ? (int32_t)b.buf_mempool()->used_mem_size() : -1;
         else if (n == "buf_total_mem_size_MB") out = b.buf_mempool() ? (int32_t)(b.buf_mempool()->total_mem_size() >> 20) : -1;
+        else if (n == "memp_physical_blocks" || n == "memp_buffered_blocks" || n == "memp_used_mem_size_KB" ||
+                 n == "memp_total_mem_size_KB") {
+            Memp1* mp = eg->eg.engineCore().mempool();
+            out = !mp ? -1 : n == "memp_physical_blocks" ? mp->physical_block_num()
+                : n == "memp_buffered_blocks" ? mp->buffered_block_num()
+                : n == "memp_used_mem_size_KB" ? (int32_t)(mp->used_mem_size() >> 10)
+                : (int32_t)(mp->total_mem_size() >> 10);
+        }
         else throw IllegalArgumentException("unknown parameter: " + n);
     });
     return out;

@@ -34,6 +34,9 @@ enum {
 };
 const char* dragon_engine_last_error(void);
 int32_t dragon_engine_last_cuda_code(void);
+/* status (DRAGON_OK or DRAGON_E_*) of the calling thread's last engine call: tells the kind of failure of
+ * the functions that return a handle (NULL on failure) */
+int32_t dragon_engine_last_status(void);
 
 /* alpha.engine.cuda_float32(deviceId, ...) with a stream pool of the given size (32 in the
  * reference's default constructor). */
@@ -43,6 +46,12 @@ dragon_engine* dragon_engine_cuda_float32(int32_t device_id, int32_t stream_pool
  * Alpha.java:770-790; PinnedMempool.java) */
 dragon_engine* dragon_engine_cuda_float32_buffered(int32_t device_id, int32_t stream_pool_size,
                                                    int64_t max_trans_buf_size);
+/* the same with a device memory pool of max_mem_size bytes behind every tensor and every split-K
+ * partial buffer (alpha.engine.cuda_float32(deviceId, alpha.engine.memp1(max_mem_size), max_trans_buf_size),
+ * Alpha.java:792-805; engine/memp/Mempool.java, Memp1.java): blocks are recycled by size instead of
+ * being allocated and freed on the device per operation.  max_trans_buf_size may be 0. */
+dragon_engine* dragon_engine_cuda_float32_pooled(int32_t device_id, int32_t stream_pool_size,
+                                                 int64_t max_mem_size, int64_t max_trans_buf_size);
 void dragon_engine_delete(dragon_engine* eg);
 int dragon_engine_check(dragon_engine* eg, int32_t flag);   /* Engine.check(boolean) */
 int dragon_engine_sync(dragon_engine* eg, int32_t flag);    /* Engine.sync(boolean)  */
@@ -56,7 +65,8 @@ int dragon_engine_set_param(dragon_engine* eg, const char* name, int32_t value);
 int32_t dragon_engine_get_param(dragon_engine* eg, const char* name);   /* also "last_gridZ",
     "last_stream_count", "live_blocks", "stream_pool_size", and of the staging pool
     "buf_physical_blocks", "buf_buffered_blocks", "buf_used_mem_size", "buf_total_mem_size_MB"
-    (-1 without a pool) */
+    (-1 without a pool), and of the device pool "memp_physical_blocks", "memp_buffered_blocks",
+    "memp_used_mem_size_KB", "memp_total_mem_size_KB" (-1 without a pool) */
 
 /* split-K decision for padded dims; kind 0 matMul, 1 matMulT1, 2 matMulT2, 3 matMul_biased;
  * 1 = no split */

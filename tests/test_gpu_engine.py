@@ -10,10 +10,12 @@ from oracle import oracle
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def eg(gpu):
+@pytest.fixture(scope="module", params=["direct", "pooled"])
+def eg(gpu, request):
+    """Every test runs on an engine that allocates each block on the device itself and on one with the
+    reference's recycling pool (alpha.engine.memp1) behind its tensors and partial buffers."""
     from dragon_hip import engine
-    e = engine.cuda_float32(0, 32)
+    e = engine.cuda_float32(0, 32, max_mem_size=(2 << 30) if request.param == "pooled" else 0)
     yield e
     e.close()
 
