@@ -403,12 +403,16 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
     const int rows_left = p.rows - row0, cols_left = p.cols - col0;
     const int lcol = wn * TN * 32 + TN * r;
     const int lane_off = (lcol < cols_left) ? lane_row * ldc4 + lcol * 4 : OOB_OFFSET;
+    // a wavefront whose 32*TM rows all lie inside C (the same answer for all its lanes) skips the test
+    // per store: two vector instructions less for each of the 16*TM stores of an interior tile
+    auto emit = [&](auto check_rows_tag) __attribute__((always_inline)) {
+    constexpr bool CHECK_ROWS = decltype(check_rows_tag)::value;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
         for (int e = 0; e < 16; e++) {
             const int crow = A_KIN ? (i * 32 + 8 * (e / 4) + (e % 4)) : (TM * (8 * (e / 4) + (e % 4)) + i);
-            const bool row_ok = lane_row < rows_left - crow;
+            const bool row_ok = !CHECK_ROWS || lane_row < rows_left - crow;
             const int row_soff = crow * ldc4;
             float out[TN];
 #pragma unroll
@@ -431,6 +435,9 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
             }
         }
     }
+    };
+    if (rows_left >= (wm + 1) * TM * 32) emit(std::false_type());
+    else emit(std::true_type());
 }
 
 // One group of 8 k: fragments from LDS, then 4 MFMA steps over the wave's TM x TN blocks.
