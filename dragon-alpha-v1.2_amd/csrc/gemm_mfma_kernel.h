@@ -103,6 +103,17 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
     return xcd * per + (xcd < rem ? xcd : rem) + local;
 }
 
+// The tile a persistent workgroup takes after `lid`, or -1.  full_end = (total / G) * G.  The rounds in
+// which every workgroup has a tile are walked in the XCD-contiguous numbering; the tiles of the last,
+// partial round are dealt by the hardware's own workgroup id instead, which spreads them evenly over
+// the XCDs and their compute units (in the contiguous numbering they would all land on the first XCDs).
+__device__ __forceinline__ int next_tile(int lid, int G, int full_end, int total) {
+    if (lid + G < full_end) return lid + G;
+    if (lid >= full_end) return -1;                       // that was the extra tile
+    const int extra = full_end + (int)blockIdx.x;
+    return extra < total ? extra : -1;
+}
+
 // ---------------------------------------------------------------------------
 // Tile staging: global -> registers -> LDS
 // ---------------------------------------------------------------------------
@@ -381,9 +392,9 @@ __device__ __forceinline__ void read_frag_kouter(float (&frag)[T][4], const floa
 // The stores go through a buffer descriptor whose base is the tile's origin: a lane outside C gets
 // an out-of-range offset and the hardware drops its store, so the whole epilogue is straight-line
 // code -- no branch per store and 32-bit offset arithmetic only.
-template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS>
-__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
-                                           int col0, float* c_ptr, int wm, int wn, int r, int h) {
+template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS, bool CHECK_ROWS>
+__device__ __forceinline__ void store_tile_rows(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
+                                                int col0, float* c_ptr, int wm, int wn, int r, int h) {
     constexpr int NT_STORE = 2;   // cache policy bit "nt": C is written once and not read back here
     float bias_v[TN];
     if constexpr (BIAS) {
@@ -403,10 +414,6 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
     const int rows_left = p.rows - row0, cols_left = p.cols - col0;
     const int lcol = wn * TN * 32 + TN * r;
     const int lane_off = (lcol < cols_left) ? lane_row * ldc4 + lcol * 4 : OOB_OFFSET;
-    // a wavefront whose 32*TM rows all lie inside C (the same answer for all its lanes) skips the test
-    // per store: two vector instructions less for each of the 16*TM stores of an interior tile
-    auto emit = [&](auto check_rows_tag) __attribute__((always_inline)) {
-    constexpr bool CHECK_ROWS = decltype(check_rows_tag)::value;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -435,9 +442,24 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const Gemm
             }
         }
     }
-    };
-    if (rows_left >= (wm + 1) * TM * 32) emit(std::false_type());
-    else emit(std::true_type());
+
+}
+
+// A wavefront whose 32*TM rows all lie inside C (the same answer for all its lanes) skips the row test
+// per store: two vector instructions less for each of the 16*TM stores of an interior tile.  Only
+// where the second copy of the epilogue costs no resident wavefront: the four-block wavefronts, whose
+// accumulators pin the register count anyway, and not with the bias row (those kernels spilled).
+template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
+                                           int col0, float* c_ptr, int wm, int wn, int r, int h) {
+    constexpr bool FAST_PATH = !BIAS && TM * TN == 4;
+    if constexpr (FAST_PATH) {
+        if (p.rows - row0 >= (wm + 1) * TM * 32) {
+            store_tile_rows<A_KIN, B_KIN, TM, TN, BIAS, false>(acc, p, row0, col0, c_ptr, wm, wn, r, h);
+            return;
+        }
+    }
+    store_tile_rows<A_KIN, B_KIN, TM, TN, BIAS, true>(acc, p, row0, col0, c_ptr, wm, wn, r, h);
 }
 
 // One group of 8 k: fragments from LDS, then 4 MFMA steps over the wave's TM x TN blocks.
@@ -565,6 +587,7 @@ void gemm_f32_mfma(const GemmParams p) {
     const int total = p.tiles_m * p.tiles_n * p.nz;
     const int G = gridDim.x;
     int lid = xcd_contiguous_id(blockIdx.x, G);   // G <= total, so lid is a valid tile
+    const int full_end = (total / G) * G;
 
     TileCtx cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid);
     LoadA la;
@@ -604,7 +627,8 @@ void gemm_f32_mfma(const GemmParams p) {
     int buf = 0;
 
     for (;;) {
-        const bool has_next = lid + G < total;
+        const int next_lid = next_tile(lid, G, full_end, total);
+        const bool has_next = next_lid >= 0;
         TileCtx nxt = cur;
         const float* a_ptr = cur.a_ptr;
         const float* b_ptr = cur.b_ptr;
@@ -658,7 +682,7 @@ void gemm_f32_mfma(const GemmParams p) {
                 lb.template load<!INNER>(rb, b_ptr, cur.kb_lim - knext);
                 fetched = true;
             } else if (has_next) {       // first stage of the next tile -> registers
-                nxt = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid + G);
+                nxt = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, next_lid);
                 if constexpr (CONV) la.init_conv(t, nxt.row0, p.a_outer, p);
                 else la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
                 lb.init(t, nxt.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
@@ -725,7 +749,7 @@ void gemm_f32_mfma(const GemmParams p) {
         for (int i = 0; i < TM; i++)
             for (int j = 0; j < TN; j++) acc[i][j] = (v16f)(0.0f);
         cur = nxt;
-        lid += G;
+        lid = next_lid;
     }
 }
 
@@ -894,14 +918,11 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     // workgroups the device keeps resident: one persistent workgroup per slot
     static std::atomic<int> resident_cache{0};   // per instantiation
     const int resident_per_cu = resident_workgroups(resident_cache, kernel);
-    // One persistent workgroup per resident slot, trimmed so that every workgroup gets the
-    // same number of tiles (+-1): a static schedule has no tail to balance a ragged last round.
+    // One persistent workgroup per resident slot: every compute unit holds the same number of
+    // workgroups, and the tiles of the last, partial round go one each to workgroups spread over the
+    // units (next_tile), so that no unit has more than one tile above the average.
     const long long slots = (long long)gemm_device_num_cu() * resident_per_cu;
-    long long grid = total;
-    if (total > slots) {
-        const long long rounds = (total + slots - 1) / slots;
-        grid = (total + rounds - 1) / rounds;
-    }
+    const long long grid = total < slots ? total : slots;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
 }
