@@ -171,7 +171,7 @@ def test_tile_choice_on_the_documented_shapes(dh):
     for v in (NN, T1, T2):
         assert ct(v, 4096, 4096, 1, 4096) == 0 + P                # four tiles per compute unit: 16-k stages
         assert ct(v, 2816, 2816, 1, 4096) == 6 + P                # two per unit: 32-k stages cost no co-residency
-        assert ct(v, 2048, 2048, 1, 2048) == 8 + P                # 128x64, two per unit: 32-k stages
+        assert ct(v, 2048, 2048, 1, 2048) == 7 + P                # 64x64, four per unit: 32-k stages
         assert ct(v, 1536, 1536, 1, 1536) == 7 + P                # 64x64, three per unit: 32-k stages
     assert ct(T1, 256, 256, 128, 1024) == 6 + P                   # the split-K weight gradient (GridZ 128 slices of 1024)
     assert ct(NN, 1024, 64, 64, 1024) == 8 + P                    # scores x V of the attention-shaped batch
@@ -182,6 +182,7 @@ def test_tile_choice_on_the_documented_shapes(dh):
     shape = (64 * 20, 128 * 19, 1, 2048)
     if ct(NN, *shape) in (5 + P, 9 + P):
         assert ct(NN, *shape) == 9 + P and ct(T2, *shape) == 9 + P and ct(T1, *shape) == 5 + P
+    assert ct(NN, 3072, 3072, 1, 3072) == 7 + P                 # nine 64x64 tiles per unit: still 32-k stages
     assert ct(NN, 4096, 4096, 1, 256) == 0 and ct(NN, 4096, 4096, 1, 512) == P    # a short K keeps the plain form
     dh.force_tile(7)
     assert ct(NN, 4096, 4096, 1, 4096) == 7                     # a forced shape is reported as it is
