@@ -85,6 +85,22 @@ def test_batched_random_within_tolerance(gpu, variant):
         assert oracle.samePercent_relative(C, R) >= 0.999
 
 
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_more_tiles_than_resident_workgroups_with_a_partial_last_round(gpu, variant):
+    """37 (padded to 40) batches of 1024 x 1024 x 64 are 2560 tiles of 128 x 128 for 1024 resident
+    workgroups: two full rounds and a last round of 512 tiles, dealt over the compute units by the
+    hardware's workgroup id.  Integer inputs: every tile must come out bit for bit, exactly once."""
+    rng = np.random.default_rng(700 + variant)
+    Batch, N, M, K = 37, 1024, 1024, 64
+    if variant == NN:
+        N, M, K = 1024, 1024, 64
+    A, B, dims, cshape, B4 = make_case(variant, rng, Batch, N, M, K, "int")
+    C = run(gpu, variant, A, B, B4, dims, cshape)
+    R = oracle.bmm(variant, A, B, B4, *dims)
+    assert np.array_equal(C, R)
+    assert np.count_nonzero(C[Batch:]) == 0
+
+
 def test_reference_batched_sweep(gpu):
     """The reference's batched sweep (N in 1..82, M in 1..96, K in 7..9, batch 5x3,
     Cuda_batchMatMul_test.java:120-123), thinned; the reference demands sp == 1.0 here."""
