@@ -33,7 +33,7 @@ PEAK_TFLOPS = 157.3      # FP32 MFMA, dense
 HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per 4096^3 launch read off the hardware counters (FETCH_SIZE scaled x2.000 by a
 # known copy, plus WRITE_SIZE); source: profiles/gemm_f32_mfma_4096cubed.md
-MEASURED_TRAFFIC_BYTES = {"A*B": 867.8 * 2 ** 20, "A*B^T": 866.2 * 2 ** 20, "A^T*B": 828.7 * 2 ** 20}
+MEASURED_TRAFFIC_BYTES = {"A*B": 857.3 * 2 ** 20, "A*B^T": 866.4 * 2 ** 20, "A^T*B": 828.8 * 2 ** 20}
 
 
 def log(*a):
