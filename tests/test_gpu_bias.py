@@ -185,10 +185,11 @@ def test_fused_bias_argument_errors(dh, gpu):
 
 # ---- engine level -----------------------------------------------------------------------------------
 
-@pytest.fixture(scope="module")
-def eg(gpu):
+@pytest.fixture(scope="module", params=["direct", "pooled"])
+def eg(gpu, request):
+    """With and without the recycling device memory pool behind the tensors (recycled blocks are dirty)."""
     from dragon_hip import engine
-    e = engine.cuda_float32(0, 32)
+    e = engine.cuda_float32(0, 32, max_mem_size=(2 << 30) if request.param == "pooled" else 0)
     yield e
     e.close()
 
