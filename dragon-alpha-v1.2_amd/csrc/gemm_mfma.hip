@@ -136,6 +136,10 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant)
         const long long per_cu = (total + num_cu - 1) / num_cu;
         if (per_cu >= 2) best = (k >= 256 && per_cu <= 3) ? TILE_128x64_K32 : TILE_128x64;
     }
+    // One tile per compute unit or fewer: the direct-to-LDS kernel was the best a lone workgroup did until
+    // the paired form, which beats it by 2-9 % wherever an operand is K-inner (A*B, A*B^T; measured on
+    // 1000x777x1531, 768^3, 1024^3, 1024x1024x4096, 512x512x8192) and loses 0-5 % on A^T*B.
+    if (best == TILE_DMA_64x64_K32_S4 && variant != GEMM_T1 && k >= 512) best = TILE_64x64_K32;
     // The paired-stage form of the kernel, measured over 2048..4096 x 2048..4096 x K in all layouts: equal
     // at K = 256, 2-5 % faster at 512..1024, 3.5-8 % at 4096; slower on a short K (8 % at K = 64).  The two
     // 256-row shapes spill in it and gain only from K = 2048 on.

@@ -176,7 +176,8 @@ def test_tile_choice_on_the_documented_shapes(dh):
     assert ct(T1, 256, 256, 128, 1024) == 6 + P                   # the split-K weight gradient (GridZ 128 slices of 1024)
     assert ct(NN, 1024, 64, 64, 1024) == 8 + P                    # scores x V of the attention-shaped batch
     assert ct(T2, 1024, 1024, 64, 64) == 0 and ct(T1, 1024, 1024, 64, 64) == 0
-    assert ct(NN, 1000, 780, 1, 1532) in (16, 17)               # fewer tiles than units: direct-to-LDS 64x64
+    assert ct(T1, 1000, 780, 1, 1532) == 17                     # fewer tiles than units: direct-to-LDS 64x64 ...
+    assert ct(NN, 1000, 780, 1, 1532) == 7 + P == ct(T2, 1000, 780, 1, 1532)   # ... or, with a K-inner operand, paired
     assert ct(NN, 257, 388, 36, 129) == 1                       # batch of small ragged products: 64x64
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
