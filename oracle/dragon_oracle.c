@@ -30,8 +30,8 @@
  *   blockNum / nstream / streamSize: pinned -- hand-derived table, brute-force
  *       tile-class decomposition, and the reference's own blockNum where
  *       micro.cuh builds.
- *   gridZ policies (Java float arithmetic): pinned by the hand-derived table of
- *       the survey only; beyond that table "parity unpinned" (no JVM here).
+ *   gridZ policies (Java float arithmetic): pinned by a hand-derived table of
+ *       cases only; beyond that table "parity unpinned" (no JVM here).
  */
 #include <stdint.h>
 #include <stdlib.h>
