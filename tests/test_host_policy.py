@@ -19,6 +19,14 @@ def test_known_answers(dh):
     # biased product splits; fGridZ = (4096 + 2048)/(2*512) = 6, capped by 256*4*0.8/512 = 1 -> raised to 2
     assert hp.gridZ(hp.MATMUL, 2048, 4096, 16384, 256) == 1
     assert hp.gridZ(hp.MATMUL_BIASED, 2048, 4096, 16384, 256) == 2
+    # matMulT2's quirks (CudaFloat32EngineBase.java:1859-1867, 1894): blockNum(N, K) tested against
+    # matMul's 1.2 and used as the divisor of the GridZ3 clamp.  Derivations: see
+    # test_oracle_pins.test_matMulT2_policy_known_answers_that_need_its_quirks.
+    assert hp.gridZ(hp.MATMUL_T2, 64, 64, 8192, 256) == 12         # 32 with blockNum(N, M) in the clamp
+    assert hp.gridZ(hp.MATMUL_T1, 64, 64, 8192, 256) == 32
+    assert hp.gridZ(hp.MATMUL_T2, 64, 64, 65536, 256) == 2         # 128 with blockNum(N, M) in the clamp
+    assert hp.gridZ(hp.MATMUL_T1, 64, 64, 65536, 256) == 128
+    assert hp.gridZ(hp.MATMUL_T2, 6784, 4, 1024, 256) == 2         # 1 with matMulT2's own 1.14
 
 
 def test_policy_matches_oracle_over_a_grid(dh):

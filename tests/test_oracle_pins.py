@@ -290,6 +290,34 @@ def test_heuristics_known_answers():
     assert oracle.gridZ(oracle.MATMUL, 128, 128, 508, 256) == 1
 
 
+def test_matMulT2_policy_known_answers_that_need_its_quirks():
+    """matMulT2 (CudaFloat32EngineBase.java:1859-1867, 1894) tests b2 = blockNum(N, K) -- not the
+    blockNum(N, M) of its own output -- against matMul's constant 1.2 (matMul_sk_minBlock_perSM, not
+    matMulT2_sk_minBlock_perSM = 1.14) and divides by that same b2 in the GridZ3 clamp.  Each answer below
+    is derived by hand from the Java text and comes out differently when one of those is "corrected"."""
+    SM = 256
+    # N = M = 64, K = 8192: b2 = blockNum(64, 8192) = 1 * 64 = 64 < 256 * (1.2 + 8192/9216) = 534.8
+    #   b0 = blockNum(64, 64) = 1, b1 = blockNum(8192, 64) = 64, fGridZ = (64 + 64) / 2 = 64
+    #   GridZ2 = 8192 >> 8 = 32 -> 32;  GridZ3 = int(256 * 4 * (8192/12288) / 64) = int(10.67) = 10 -> 10
+    #   padded to a multiple of 4: 12.   (With b0 in the clamp: GridZ3 = 682 -> 32, which is what
+    #   matMulT1 answers for this shape.)
+    assert oracle.blockNum(64, 8192) == 64 and oracle.blockNum(8192, 64) == 64 and oracle.blockNum(64, 64) == 1
+    assert oracle.gridZ(oracle.MATMUL_T2, 64, 64, 8192, SM) == 12
+    assert oracle.gridZ(oracle.MATMUL_T1, 64, 64, 8192, SM) == 32
+    # K = 65536: b2 = 512 < 256 * (1.2 + 65536/66560) = 559.3; fGridZ = (512 + 512) / 2 = 512
+    #   GridZ2 = 256 -> 256;  GridZ3 = int(1024 * (65536/69632) / 512) = int(1.88) = 1 -> 1 -> raised to 2.
+    #   (With b0 in the clamp: 963 -> 256 -> maxPart 128, matMulT1's answer.)
+    assert oracle.blockNum(64, 65536) == 512
+    assert oracle.gridZ(oracle.MATMUL_T2, 64, 64, 65536, SM) == 2
+    assert oracle.gridZ(oracle.MATMUL_T1, 64, 64, 65536, SM) == 128
+    # The constant alone: N = 6784 (53 tiles of 128), M = 4, K = 1024: b2 = blockNum(6784, 1024) = 53 * 8 = 424
+    #   lies between 256 * (1.14 + 0.5) = 419.8 and 256 * (1.2 + 0.5) = 435.2, so the product is split only
+    #   because matMul's 1.2 is used: b0 = 53, b1 = blockNum(1024, 4) = 8, fGridZ = (8 + 424) / 106 = 4.08
+    #   GridZ2 = 4;  GridZ3 = int(1024 * 0.2 / 424) = 0 -> raised to 2.   (With 1.14: no split, 1.)
+    assert oracle.blockNum(6784, 1024) == 424 and oracle.blockNum(6784, 4) == 53 and oracle.blockNum(1024, 4) == 8
+    assert oracle.gridZ(oracle.MATMUL_T2, 6784, 4, 1024, SM) == 2
+
+
 def test_biased_policy_known_answer():
     # hand-derived (see the arithmetic in test_host_policy.test_known_answers)
     assert oracle.blockNum(2048, 4096) == 512
