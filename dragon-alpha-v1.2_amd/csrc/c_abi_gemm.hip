@@ -4,6 +4,8 @@
 // guarded kernel, and launches on streams[0].
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
+#include <atomic>
 #include "gemm_mfma.h"
 #include "../../include/dragon_hip_gemm.h"
 
@@ -113,6 +115,67 @@ int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC, 
     if (part == 0) return hipSuccess;
     return skbuf_summary_launch((hipStream_t)(intptr_t)stream, (const float*)(intptr_t)dCbuf,
                                 (float*)(intptr_t)dC, part, sizeC);
+}
+
+// ---- the whole split-K product with the partials in memory the library already holds ------------
+
+}  // extern "C"
+
+namespace {
+
+// Partial products of dragon_Cuda_matMul_matMulSK_static: slice z >= 1 at (z-1)*N*M, exactly the
+// layout of the caller's Cbuf in the two-stage entry points.  One copy per GPU, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress: the kernels get
+// the device address that call returns.
+constexpr long long SK_STATIC_FLOATS = 8ll << 20;   // 32 MiB
+static __device__ __align__(256) __attribute__((used)) float scratch[SK_STATIC_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<float*> g_scratch_ptr[MAX_DEVICES];
+
+// The device address of `scratch` on the current device, looked up once per device.
+int static_scratch(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    float* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (ptr == nullptr) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // concurrent first calls store the same value
+    }
+    *out = ptr;
+    return hipSuccess;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dragon_Cuda_matMul_matMulSK_static(const int64_t* streams, int32_t length, int32_t variant, int32_t GridZ,
+                                       int64_t dA, int64_t dB, int64_t dC, int32_t N, int32_t M, int32_t K) {
+    if (variant < GEMM_NN || variant > GEMM_T2) return hipErrorInvalidValue;
+    int e = check_common(streams, length, dA, dB, dC);
+    if (e) return e;
+    if (N <= 0 || M <= 0 || K <= 0 || GridZ < 1 || !x4(N) || !x4(M) || !x4(K)) return hipErrorInvalidValue;
+    if ((long long)N * M > 0x7fffffffLL) return hipErrorInvalidValue;
+    const long long need = (long long)(GridZ - 1) * N * M;
+    if (need > SK_STATIC_FLOATS) {
+        fprintf(stderr,
+                "dragon_Cuda_matMul_matMulSK_static: (GridZ-1)*N*M = %lld floats of partial products do not fit "
+                "the static workspace of %lld floats\n", need, SK_STATIC_FLOATS);
+        return hipErrorOutOfMemory;
+    }
+    if (GridZ == 1) return matmul_2d(variant, streams, length, 1, dA, dB, dC, 0, N, M, K);
+    float* ptr = nullptr;
+    e = static_scratch(&ptr);
+    if (e) return e;
+    // stage 1 writes every float of the GridZ-1 partials it later reads, so nothing has to be cleared
+    e = matmul_2d(variant, streams, length, GridZ, dA, dB, dC, (int64_t)(intptr_t)ptr, N, M, K);
+    if (e) return e;
+    return skbuf_summary_launch((hipStream_t)(intptr_t)streams[0], ptr, (float*)(intptr_t)dC, GridZ - 1, N * M);
 }
 
 int dragon_Cuda_matMul_matMul_biased(const int64_t* streams, int32_t length, int64_t dA, int64_t dB,

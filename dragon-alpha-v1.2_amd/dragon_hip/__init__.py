@@ -227,6 +227,12 @@ class Cuda_matMul:
         _check(lib.dragon_Cuda_matMul_SKbuf_summary(stream, dCbuf, dC, part, sizeC))
 
     @staticmethod
+    def matMulSK_static(streams, length, variant, GridZ, dA, dB, dC, N, M, K):
+        """Both split-K stages with the partials in the library's own static workspace (no allocation)."""
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_matMul_matMulSK_static(arr, length, variant, GridZ, dA, dB, dC, N, M, K))
+
+    @staticmethod
     def matMul(streams, length, dA, dB, dC, N, M, K):
         arr, _ = _stream_array(streams)
         _check(lib.dragon_Cuda_matMul_matMul(arr, length, dA, dB, dC, N, M, K))

@@ -33,6 +33,7 @@ SIGNATURES = {
     "dragon_Cuda_matMul_matMulT1SK": (i32, _MMSK),
     "dragon_Cuda_matMul_matMulT2SK": (i32, _MMSK),
     "dragon_Cuda_matMul_SKbuf_summary": (i32, [i64, i64, i64, i32, i32]),
+    "dragon_Cuda_matMul_matMulSK_static": (i32, [p_i64, i32, i32, i32, i64, i64, i64, i32, i32, i32]),
     "dragon_Cuda_function_linear_dual2D_row": (i32, [i64, i64, i64, i32, f32, f32, f32, i64, i32, i32, i32]),
     "dragon_Cuda_matMul_matMul_biased": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_function_linear2D": (i32, [i64, f32, i64, f32, i64, i32, i32, i32]),

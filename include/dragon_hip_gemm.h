@@ -88,6 +88,24 @@ int dragon_Cuda_matMul_matMulT2SK(const int64_t* streams, int32_t length, int32_
 int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC,
                                      int32_t part, int32_t sizeC);
 
+/* ---- the complete split-K product without any allocation: stage 1 as above (variant 0 = A*B,
+ * 1 = A^T*B, 2 = A*B^T), the GridZ-1 partial products in a workspace that is part of the library's
+ * device image instead of a caller's Cbuf, then the Kahan fold of stage 2 into C, all on streams[0].
+ * Every bit of C equals what matMulSK / matMulT1SK / matMulT2SK + SKbuf_summary leave.
+ * No counterpart in the reference (whose Java side allocates Cbuf per call,
+ * CudaFloat32EngineBase.java:1565-1583); it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid device allocation.  Neither this call nor anything
+ * it runs allocates or frees memory, and it enqueues kernels only (no memset).
+ * Limit: (GridZ-1)*N*M <= 8 388 608 floats (32 MiB, held once per GPU until the process ends); beyond
+ * it the call returns hipErrorOutOfMemory (2) and says so on stderr, without launching anything.
+ * All calls on one GPU share that workspace, which keeps the last call's partials: two calls that
+ * overlap in time on one GPU (different streams or threads) race and must be ordered by the caller.
+ * The first call on a device looks up the workspace's address (which may load the library's device
+ * code); make that call outside a graph capture. */
+int dragon_Cuda_matMul_matMulSK_static(const int64_t* streams, int32_t length, int32_t variant,
+                                       int32_t GridZ, int64_t dA, int64_t dB, int64_t dC,
+                                       int32_t N, int32_t M, int32_t K);
+
 /* ---- bias row -------------------------------------------------------------------- */
 
 /* Y[i] = alpha*X1[i] + beta*X2[i % row_lengthv] + gamma for i < lengthv, then elements whose
