@@ -111,7 +111,7 @@ def main():
         nfl = 64 * 1024 * 1024                      # 256 MiB read + 256 MiB written per launch
         src, dst = dh.DeviceArray(size=nfl), dh.DeviceArray(size=nfl)
         for _ in range(10):
-            rc = dh.lib.dragon_Cuda_copy1D_kernel(stream, dst.address, src.address, nfl)
+            rc = dh.lib.dragon_test_copy1D_kernel(stream, dst.address, src.address, nfl)
             assert rc == 0
         Cuda.streamSynchronize(stream)
         print(json.dumps({"calibrate_copy": {"bytes_read_per_launch": nfl * 4,

@@ -48,7 +48,8 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
         p.bias_width = width;
     }
     const int num_cu = gemm_device_num_cu();
-    int tile = gemm_choose_tile(p.rows, p.cols, 1, p.k_total, num_cu);
+    if (num_cu <= 0) return hipErrorNoDevice;
+    int tile = gemm_forced_tile() != TILE_AUTO ? gemm_forced_tile() : gemm_choose_tile_per_workgroup(p.rows, p.cols, 1, p.k_total, num_cu);
     const bool free_choice = gemm_forced_tile() == TILE_AUTO;   // a forced shape (tests, sweeps) is taken as it is
     if (free_choice) tile &= ~TILE_PAIRED;   // decided below, on the convolution's own measurements
     if (gemm_tile_is_dma(tile)) {   // the direct-to-LDS shapes have no gathering loader: nearest classic shape

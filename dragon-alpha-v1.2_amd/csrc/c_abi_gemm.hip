@@ -8,6 +8,7 @@
 #include <atomic>
 #include "gemm_mfma.h"
 #include "../../include/dragon_hip_gemm.h"
+#include "../../include/dragon_hip_testing.h"
 
 using namespace dragon;
 
@@ -70,7 +71,12 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
         p.split = 1;  // a zero K_slice leaves every slice but the last empty: they write zeros
     }
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total, gemm_device_num_cu(), variant);
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    // K slices go to the caller's buffers one by one: always a tile-per-workgroup kernel
+    const int tile = p.split ? (gemm_forced_tile() != TILE_AUTO ? gemm_forced_tile()
+                                : gemm_choose_tile_per_workgroup(p.rows, p.cols, p.nz, p.k_slice > 0 ? p.k_slice : p.k_total, num_cu, variant))
+                             : gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, num_cu, variant);
     return gemm_launch(variant, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -221,7 +227,9 @@ int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length, 
     p.sA = (long long)N * AK; p.sB = (long long)BK * M; p.sC = (long long)N * M;
     p.nz = Batch;
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, gemm_device_num_cu(), GEMM_NN);
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, num_cu, GEMM_NN);
     return gemm_launch(GEMM_NN, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -249,7 +257,9 @@ int dragon_Cuda_batchMatMul_batchMatMulT1(const int64_t* streams, int32_t length
     p.sA = (long long)K * AN; p.sB = (long long)K * M; p.sC = (long long)CN * M;
     p.nz = Batch;
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, gemm_device_num_cu(), GEMM_T1);
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, num_cu, GEMM_T1);
     return gemm_launch(GEMM_T1, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -271,7 +281,9 @@ int dragon_Cuda_batchMatMul_batchMatMulT2(const int64_t* streams, int32_t length
     p.sA = (long long)N * K; p.sB = (long long)BM * K; p.sC = (long long)N * CM;
     p.nz = Batch;
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
-    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, gemm_device_num_cu(), GEMM_T2);
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, num_cu, GEMM_T2);
     return gemm_launch(GEMM_T2, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 

@@ -29,11 +29,21 @@ enum GemmTile {
     TILE_DMA_64x64_S4 = 16,
     TILE_DMA_64x64_K32_S4 = 17,
     TILE_ALL_COUNT = 18,
+    // Few tiles, long K: persistent workgroups that share the work in equal runs of LDS stages rather than in
+    // whole tiles (gemm_mfma_streamk.hip); 32 k per stage, direct global->LDS staging
+    TILE_SK_64x64 = 18,        // one workgroup per compute unit, 4 stage buffers
+    TILE_SK_128x64 = 19,
+    TILE_SK_64x128 = 20,
+    TILE_SK_128x128 = 21,
+    TILE_SK_64x64_O2 = 22,     // two workgroups per compute unit, 4 stage buffers
+    TILE_SK_128x64_O2 = 23,    // two workgroups per compute unit, 3 stage buffers
+    TILE_SK_END = 24,
     // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
     // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
     // short K; gemm_choose_tile sets it.
     TILE_PAIRED = 0x100
 };
+inline bool gemm_tile_is_streamk(int tile) { return tile >= TILE_SK_64x64 && tile < TILE_SK_END; }
 inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
@@ -69,11 +79,19 @@ struct GemmParams {
     unsigned div_tiles_mul, div_tiles_shift;   // d = tiles_m * tiles_n
     unsigned div_band_mul, div_band_shift;     // d = 8 * tiles_n (a band of 8 tile rows)
     unsigned div_last_mul, div_last_shift;     // d = tile rows of the last, shorter band (tiles_m % 8, or 8)
+    // filled by the launcher of the balanced kernel (gemm_launch_streamk): a tile has sk_S stages, workgroup w
+    // takes sk_q stages (one more for w < sk_rem) of the tiles' stages numbered tile by tile; pieces of shared
+    // tiles go to sk_ws
+    float* sk_ws;
+    int* sk_count;
+    int sk_S, sk_q, sk_rem;
+    unsigned sk_div_S_mul, sk_div_S_shift;
 };
 void gemm_fill_tile_divisors(GemmParams& p);
 void gemm_magic_divisor(unsigned d, unsigned& mul, unsigned& shift);
 
-// Compute units of the current device (256 when no device answers), cached per device.
+// Compute units of the current device, cached per device; 0 when no device answers (the launchers then
+// return hipErrorNoDevice).
 int gemm_device_num_cu();
 // The kernels address an operand tile with 32-bit byte offsets from the tile's origin: up to 256 rows
 // (or k) of pitch.  False when a leading stride is too long for that; the entry points reject such calls.
@@ -83,11 +101,25 @@ bool gemm_pitches_addressable(const GemmParams& p);
 // does not fit 31 bits; the launcher then runs the plain form (advancing 64-bit pointers) instead.
 bool gemm_paired_form_fits(bool a_k_inner, bool b_k_inner, const GemmParams& p);
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant = -1);   // variant: GEMM_* or -1
+// the same without the balanced kernel's shapes
+int gemm_choose_tile_per_workgroup(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
 void gemm_force_tile(int tile);
 int gemm_forced_tile();   // TILE_AUTO when the choice is left to gemm_choose_tile
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
 hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);
+// the three products (batched too) through the balanced kernel (tile ids TILE_SK_*).  It needs the stream's
+// workspace; hipErrorOutOfMemory says that the product cannot go this way (no workspace and none may be made
+// now, or sizes beyond its counters) and the caller takes a tile-per-workgroup kernel instead.
+hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream);
+// The balanced kernel's tile for this product, or -1 where the tile-per-workgroup kernels do as well or
+// better (an estimate fitted to measurements: at most two 64 x 64 tiles per compute unit, and K long enough
+// to carry the balanced kernel's larger fixed time).
+int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
+// The workspace of `stream` on the current device: arrival counters and the slots for pieces of shared tiles.
+// Made at the first balanced launch on that stream (never while the stream is capturing: then nullptr) and kept
+// for later launches on the same handle until the process ends.
+float* gemm_streamk_workspace(hipStream_t stream, size_t* floats);
 // Y = conv(X, W) [+ bias row over OC] as an implicit GEMM (the A * B^T kernel with a gathered A);
 // classic tile ids only
 hipError_t gemm_launch_conv(const GemmParams& p, int tile, hipStream_t stream);

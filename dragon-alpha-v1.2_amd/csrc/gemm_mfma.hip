@@ -8,11 +8,11 @@ namespace dragon {
 int gemm_device_num_cu() {
     static std::atomic<int> cached[64];
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
     int n = cached[dev].load(std::memory_order_relaxed);
     if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
+            return 0;   // no answer: the callers fail the launch rather than guess a grid
         cached[dev].store(n, std::memory_order_relaxed);
     }
     return n;
@@ -51,10 +51,10 @@ bool gemm_paired_form_fits(bool a_k_inner, bool b_k_inner, const GemmParams& p) 
     return a_span < 0x7fffffffLL && b_span < 0x7fffffffLL;
 }
 
-// a test and tuning hook: one setting for the whole process
-static std::atomic<int> g_forced_tile{TILE_AUTO};
-void gemm_force_tile(int tile) { g_forced_tile.store(tile, std::memory_order_relaxed); }
-int gemm_forced_tile() { return g_forced_tile.load(std::memory_order_relaxed); }
+// a test and tuning hook: a setting of the calling thread only
+static thread_local int t_forced_tile = TILE_AUTO;
+void gemm_force_tile(int tile) { t_forced_tile = tile; }
+int gemm_forced_tile() { return t_forced_tile; }
 
 // What the tile shapes are worth, measured on MI355X (fractions of a compute unit's
 // FP32 matrix peak): `alone` is what one resident workgroup sustains by itself (its
@@ -92,6 +92,11 @@ static const TileTraits kTiles[TILE_ALL_COUNT] = {
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant) {
     const int forced = gemm_forced_tile();
     if (forced != TILE_AUTO) return forced;
+    const int balanced = gemm_choose_streamk(rows, cols, nz, k, num_cu, variant);
+    return balanced >= 0 ? balanced : gemm_choose_tile_per_workgroup(rows, cols, nz, k, num_cu, variant);
+}
+
+int gemm_choose_tile_per_workgroup(int rows, int cols, int nz, int k, int num_cu, int variant) {
     int best = TILE_128x128;
     double best_cost = 1e300;
     for (int tile = 0; tile < TILE_ALL_COUNT; tile++) {
@@ -150,6 +155,17 @@ int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant)
 
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream) {
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
+    if (gemm_tile_is_streamk(tile)) {
+        // where the product cannot take the balanced kernel (split-K slices go to the caller's buffers; a
+        // capturing stream that has no workspace yet) a tile-per-workgroup kernel takes over
+        const hipError_t e = gemm_launch_streamk(variant, p, tile, stream);
+        if (e != hipErrorOutOfMemory) return e;
+        (void)hipGetLastError();
+        const int k = p.split ? (p.k_slice > 0 ? p.k_slice : p.k_total) : p.k_total;
+        const int num_cu = gemm_device_num_cu();
+        if (num_cu <= 0) return hipErrorNoDevice;
+        tile = gemm_choose_tile_per_workgroup(p.rows, p.cols, p.nz, k, num_cu, variant);
+    }
     if (p.bias != nullptr)   // the bias row exists for the forward product only
         return variant == GEMM_NN ? gemm_launch_nn_biased(p, tile, stream) : hipErrorInvalidValue;
     if (gemm_tile_is_dma(tile)) return gemm_launch_dma(variant, p, tile, stream);

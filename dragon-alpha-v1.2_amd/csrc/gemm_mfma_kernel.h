@@ -89,6 +89,28 @@ __device__ __forceinline__ void dma_f4(const float* base, float* lds_wave_base, 
                  : "s"(lds_addr), "v"(byte_offset), "s"(rsrc)
                  : "memory", "m0");
 }
+// The same transfer for callers that keep the descriptor in registers and the LDS address as an
+// integer (a wave-uniform base plus a compile-time distance): three instructions per transfer.
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_f4_lean(v4u rsrc, unsigned lds_wave_base, int byte_offset) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_wave_base), "v"(byte_offset), "s"(rsrc), "n"(LDS_IMM)
+                 : "memory", "m0", "scc");
+}
+__device__ __forceinline__ v4u dma_descriptor(const float* base) {
+    const unsigned long long b = (unsigned long long)base;
+    const v4u rsrc = {(unsigned)b, (unsigned)(b >> 32) & 0xffffu, (unsigned)RSRC_RECORDS, (unsigned)RSRC_FLAGS};
+    return rsrc;
+}
+// advance a descriptor's base by `bytes` (addresses stay below 2^48, so the carry never reaches the
+// stride field above the base)
+__device__ __forceinline__ void dma_descriptor_advance(v4u& rsrc, unsigned long long bytes) {
+    unsigned long long b = ((unsigned long long)rsrc.y << 32) | rsrc.x;
+    b += bytes;
+    rsrc.x = (unsigned)b;
+    rsrc.y = (unsigned)(b >> 32);
+}
 #pragma clang diagnostic pop
 
 // s_waitcnt for the vector-memory counter alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
@@ -205,6 +227,12 @@ struct KInner {
         for (int s = 0; s < PASSES; s++)
             dma_f4(base, lds + (s * NTHREADS + wave * 64) * 4, dma_kcol[s] < k_left ? off[s] : OOB_OFFSET);
     }
+    // one of the PASSES transfers of a stage, for callers that place them between other instructions
+    __device__ __forceinline__ void issue_pass(int s, float* lds, const float* base, int k_left, int wave) const {
+        dma_f4(base, lds + (s * NTHREADS + wave * 64) * 4, dma_kcol[s] < k_left ? off[s] : OOB_OFFSET);
+    }
+    // the lane's byte offset for transfer s of a stage with k_left k still inside the operand
+    __device__ __forceinline__ int dma_offset(int s, int k_left) const { return dma_kcol[s] < k_left ? off[s] : OOB_OFFSET; }
     __device__ __forceinline__ static const float* tile_base(const float* X, int row0, int k, int ld) {
         return X + (size_t)row0 * ld + k;
     }
@@ -253,6 +281,10 @@ struct KOuter {
         for (int s = 0; s < PASSES; s++)
             dma_f4(base, lds + (s * NTHREADS + wave * 64) * 4, (krow + s * RPP < k_left) ? off[s] : OOB_OFFSET);
     }
+    __device__ __forceinline__ void issue_pass(int s, float* lds, const float* base, int k_left, int wave) const {
+        dma_f4(base, lds + (s * NTHREADS + wave * 64) * 4, (krow + s * RPP < k_left) ? off[s] : OOB_OFFSET);
+    }
+    __device__ __forceinline__ int dma_offset(int s, int k_left) const { return (krow + s * RPP < k_left) ? off[s] : OOB_OFFSET; }
     __device__ __forceinline__ static const float* tile_base(const float* X, int col0, int k, int ld) {
         return X + (size_t)k * ld + col0;
     }
@@ -928,7 +960,9 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     // One persistent workgroup per resident slot: every compute unit holds the same number of
     // workgroups, and the tiles of the last, partial round go one each to workgroups spread over the
     // units (next_tile), so that no unit has more than one tile above the average.
-    const long long slots = (long long)gemm_device_num_cu() * resident_per_cu;
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const long long slots = (long long)num_cu * resident_per_cu;
     const long long grid = total < slots ? total : slots;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
@@ -979,7 +1013,9 @@ static hipError_t launch_cfg_dma(GemmParams p, hipStream_t stream) {
     gemm_fill_tile_divisors(p);
     static std::atomic<int> resident_cache{0};   // per instantiation
     const int resident_per_cu = resident_workgroups(resident_cache, kernel);
-    const long long slots = (long long)gemm_device_num_cu() * resident_per_cu;
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const long long slots = (long long)num_cu * resident_per_cu;
     long long grid = total;
     if (total > slots) {
         const long long rounds = (total + slots - 1) / slots;

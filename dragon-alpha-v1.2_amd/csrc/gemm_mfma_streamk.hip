@@ -1,0 +1,524 @@
+// The products for shapes with FEWER TILES THAN THE CHIP HAS COMPUTE UNITS (or barely more): one
+// workgroup per compute unit, and the work dealt out in equal runs of LDS stages instead of in
+// whole tiles.
+//
+// Unit of work = one LDS stage (KT k) of one tile; the tiles' stages are numbered tile by tile
+// (tile order of decode_tile) and workgroup w takes the contiguous run [u0(w), u0(w+1)), every run
+// within one unit of the others.  A run may start and end in the middle of a tile's K range: a
+// tile whose stages all fall to one workgroup is stored to C as usual, a tile shared by several
+// workgroups has each of them write its partial sum to a workspace slot (two slots per workgroup:
+// one for a piece of the tile its run starts in, one for a piece of a later tile) and count itself
+// on the tile's arrival counter; the workgroup that arrives last adds the tile's pieces in run
+// order and stores it.  No workgroup ever waits for another.  The split is a pure function of the
+// shape and the unit count and the pieces are added in run order whoever does it, so every bit of
+// the result is the same from run to run.  The reference's answer to the same problem is the host-side split-K policy
+// (CudaFloat32EngineBase.java:1523-1562), which on 256 units still leaves most of them idle or
+// unevenly loaded on such shapes.
+//
+// A workgroup that has a compute unit to itself has nobody to hide its waits behind, so the stage
+// loop is built for that case:
+//   * operands go global -> LDS directly (buffer_load ... lds) through NS stage buffers, NS-2
+//     stages in flight beyond the one that has just landed; no staging registers;
+//   * ONE barrier per stage, placed before the matrix work of the stage's LAST k group: by then
+//     the fragments of that group are in registers, so after the barrier the wavefront first
+//     issues the transfers of a later stage and the fragment reads of the NEXT stage's first
+//     group, and only then multiplies -- the LDS latency that otherwise sits between a barrier and
+//     the first MFMA is covered by the last group's MFMAs.  Within a stage the fragments of group
+//     g+1 are read while group g is multiplied (two fragment sets).
+#include "gemm_mfma_kernel.h"
+#include <utility>
+#include <mutex>
+#include <map>
+
+namespace dragon {
+namespace {
+
+constexpr int SK_MAX_TILES = 4096;   // arrival counters at the head of the workspace
+constexpr size_t SK_MAX_WORKSPACES = 64;
+
+// first unit of workgroup w: the first `rem` workgroups take q+1 units, the others q
+__device__ __forceinline__ int sk_first_unit(int w, int q, int rem) { return w * q + (w < rem ? w : rem); }
+// the workgroup that owns unit u
+__device__ __forceinline__ int sk_owner(int u, int q, int rem) {
+    const int big = rem * (q + 1);
+    return u < big ? u / (q + 1) : rem + (u - big) / q;
+}
+
+// Partial tile in the accumulators' own layout: block (i, j) of wavefront `wave`, element e, lane at
+// float (((wave*TM + i)*TN + j)*16 + e)*64 + lane: a wavefront writes 256 contiguous bytes per store.
+// The pieces travel between workgroups on different XCDs, each with an L2 of its own, inside one
+// launch.  Every access to them is a relaxed atomic of device scope -- a store that writes through
+// to memory, a load that does not take a stale line from the reader's L2 -- so that no cache has to be
+// written back or invalidated as a whole (a device-scope fence does both to the XCD's L2, and with
+// them went the operand reuse: 33 -> 110 us on 1000 x 777 x 1531).
+template <int TM, int TN>
+__device__ __forceinline__ void store_partial(const v16f (&acc)[TM][TN], float* slot, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            float* at = slot + (size_t)(((wave * TM + i) * TN + j) * 16) * 64 + lane;
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                __hip_atomic_store(at + e * 64, acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void add_partial(v16f (&acc)[TM][TN], const float* slot, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const float* at = slot + (size_t)(((wave * TM + i) * TN + j) * 16) * 64 + lane;
+            float v[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) v[e] = __hip_atomic_load(at + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] += v[e];
+        }
+}
+
+template <bool A_KIN, bool B_KIN, int TM, int TN, int BM, int BN, int KT>
+__device__ __forceinline__ void read_group(float (&fa)[TM][4], float (&fb)[TN][4], const float* as, const float* bs,
+                                           int wm, int wn, int g, int r, int h) {
+    if constexpr (A_KIN) read_frag_kinner<TM, KT>(fa, as, wm * TM * 32, g, r, h);
+    else                 read_frag_kouter<TM, BM>(fa, as, wm * TM * 32, g, r, h);
+    if constexpr (B_KIN) read_frag_kinner<TN, KT>(fb, bs, wn * TN * 32, g, r, h);
+    else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
+}
+
+// compile-time loop: f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N-1>)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// The MFMAs of one group of 8 k, with `between(m)` placed after MFMA number m.  A wavefront issues one
+// instruction every four cycles at best and an MFMA keeps the matrix pipe busy for 64: whatever else
+// the wavefront has to do costs nothing while it sits BETWEEN two MFMAs (15 issue slots each) and
+// costs its full issue time anywhere else -- and a workgroup alone on its compute unit has no other
+// wavefront to fill the gap.  The order is pinned with scheduling barriers.
+template <int NACC, int TM, int TN, typename Between>
+__device__ __forceinline__ void mfma_group_with(v16f (&acc)[NACC][TM][TN], const float (&fa)[TM][4], const float (&fb)[TN][4],
+                                                Between&& between) {
+    static_for<4 * TM * TN>([&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        constexpr int q = m / (TM * TN), i = (m / TN) % TM, j = m % TN;
+        // a single-block wavefront alternates between two accumulators: an MFMA that adds to the result
+        // of the one just before it waits for that result
+        constexpr int a = q % NACC;
+        acc[a][i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[a][i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        between(mc);
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC>
+__global__ __launch_bounds__(NTHREADS, OCC)
+void gemm_f32_mfma_streamk(const GemmParams p) {
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    static_assert(NS == 3 || NS == 4, "stage buffers: 3 or 4");
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
+    using LoadB = typename std::conditional<B_KIN, KInner<BN, KT, TN>, KOuter<BN, KT>>::type;
+    constexpr int STAGE_FLOATS = LoadA::LDS_FLOATS + LoadB::LDS_FLOATS;
+    constexpr unsigned STAGE_BYTES = STAGE_FLOATS * 4;
+    constexpr int PA = LoadA::PASSES, PB = LoadB::PASSES;
+    constexpr int XFERS = PA + PB;                             // transfers per wave per stage
+    constexpr int GR = KT / 8;                                 // k groups per stage
+    constexpr int NM = 4 * TM * TN;                            // MFMAs per group
+    static_assert(GR >= 2 && GR % 2 == 0, "an even number of k groups per stage (two fragment sets)");
+    static_assert((NS - 2) * XFERS <= 63, "vmcnt holds 6 bits");
+    static_assert(OCC * NS * STAGE_FLOATS * 4 <= 160 * 1024, "stage buffers exceed the LDS");
+
+    __shared__ __attribute__((aligned(16))) float smem[NS * STAGE_FLOATS];
+    __shared__ int sk_last[2];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+    const unsigned long long a_step8 = (unsigned long long)LoadA::k_advance(p.lda) * 4;
+    const unsigned long long b_step8 = (unsigned long long)LoadB::k_advance(p.ldb) * 4;
+
+    const int S = p.sk_S;
+    // neighbouring runs share a tile's operands: keep them on one XCD (one L2)
+    const int w = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int u0 = sk_first_unit(w, p.sk_q, p.sk_rem);
+    const int n = p.sk_q + (w < p.sk_rem ? 1 : 0);             // >= 1: the grid never exceeds the unit count
+
+    // ---- producer: the stage to fetch next ------------------------------------------------------
+    // Kept as cheap as the hardware allows, because nothing a wavefront does beside its MFMAs is free
+    // (see mfma_group_with): the descriptors point at the stage and move on by a scalar 64-bit add, the
+    // LDS addresses are integers known at compile time up to the wave's base, and the lanes' offsets sit
+    // ready in registers -- their K test is redone only for a stage that is not wholly inside K, and
+    // what has to be looked at per stage is one countdown (f_until).
+    const int first_tile = div_by(u0, p.sk_div_S_mul, p.sk_div_S_shift);
+    int f_tile = first_tile;
+    int f_it = u0 - first_tile * S;   // stage of its tile the producer fetches next, as of the last look
+    int f_left = n;                   // stages of the run not yet fetched, as of the last look
+    int f_span = 0, f_until = 0;      // stages until the next look, at the last look and now
+    int f_interior = 0;               // stages of the tile that lie wholly inside K for both operands
+    TileCtx ft = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, f_tile);
+    LoadA la;
+    LoadB lb;
+    la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+    lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+    v4u rsrc_a = dma_descriptor(ft.a_ptr + (size_t)f_it * LoadA::k_advance(p.lda));
+    v4u rsrc_b = dma_descriptor(ft.b_ptr + (size_t)f_it * LoadB::k_advance(p.ldb));
+    int offa[PA], offb[PB];           // the lanes' offsets for the stage to fetch
+    const unsigned lds_wave = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float*)smem + wave * 1024;
+
+    // decide how the following stages are fetched and for how many of them that holds
+    auto look = [&]() __attribute__((always_inline)) {
+        if (f_left <= 0) {            // past the end of the run: all-zero transfers, so that the count of
+#pragma unroll                        // transfers in flight stays a constant
+            for (int i = 0; i < PA; i++) offa[i] = OOB_OFFSET;
+#pragma unroll
+            for (int i = 0; i < PB; i++) offb[i] = OOB_OFFSET;
+            f_span = 0x40000000;
+        } else {
+            if (f_it == S) {          // next tile
+                f_tile++;
+                ft = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, f_tile);
+                la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+                lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+                rsrc_a = dma_descriptor(ft.a_ptr);
+                rsrc_b = dma_descriptor(ft.b_ptr);
+                f_it = 0;
+            }
+            f_interior = min(ft.ka_lim, ft.kb_lim) / KT;
+            if (f_it < f_interior) {  // stages wholly inside K: no K test
+#pragma unroll
+                for (int i = 0; i < PA; i++) offa[i] = la.off[i];
+#pragma unroll
+                for (int i = 0; i < PB; i++) offb[i] = lb.off[i];
+                f_span = min(f_interior - f_it, f_left);
+            } else {                  // a stage that reaches beyond K: tested lane by lane, one stage at a time
+#pragma unroll
+                for (int i = 0; i < PA; i++) offa[i] = la.dma_offset(i, ft.ka_lim - f_it * KT);
+#pragma unroll
+                for (int i = 0; i < PB; i++) offb[i] = lb.dma_offset(i, ft.kb_lim - f_it * KT);
+                f_span = 1;
+            }
+        }
+        f_until = f_span;
+    };
+    // transfer number i of the stage to fetch, into the stage buffer at LDS byte address stage_lds (+ the wave's part)
+    auto xfer = [&](auto ic, unsigned stage_lds) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i < PA) dma_f4_lean<i * NTHREADS * 16>(rsrc_a, stage_lds, offa[i]);
+        else dma_f4_lean<LoadA::LDS_FLOATS * 4 + (i - PA) * NTHREADS * 16>(rsrc_b, stage_lds, offb[i - PA]);
+    };
+    // after a stage's transfers
+    auto advance = [&]() __attribute__((always_inline)) {
+        dma_descriptor_advance(rsrc_a, a_step8);
+        dma_descriptor_advance(rsrc_b, b_step8);
+        if (--f_until == 0) {
+            f_it += f_span;
+            f_left -= f_span;
+            look();
+        }
+    };
+    look();
+
+    // ---- consumer: the tile being multiplied -------------------------------------------------------
+    TileCtx cur = ft;
+    int c_tile = first_tile, c_it = f_it;
+    int left = n;                     // stages of the run not yet multiplied
+    int rec_tile0 = 0, rec_tile1 = 0; // shared tiles this run has left a piece of
+    int n_rec = 0;
+
+    constexpr int NACC = (TM * TN == 1) ? 2 : 1;
+    v16f acc[NACC][TM][TN];
+#pragma unroll
+    for (int a = 0; a < NACC; a++)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[a][i][j] = (v16f)(0.0f);
+
+    float fa[2][TM][4], fb[2][TN][4];
+
+    // prologue: NS-1 stages on their way, the first one landed and visible, its first fragments read
+#pragma unroll
+    for (int s = 0; s < NS - 1; s++) {
+        static_for<XFERS>([&](auto ic) { xfer(ic, lds_wave + s * STAGE_BYTES); });
+        advance();
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * XFERS));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(fa[0], fb[0], smem, smem + LoadA::LDS_FLOATS, wm, wn, 0, r, h);
+
+    // One stage, multiplied from stage buffer SLOT (a compile-time constant: every LDS address of the
+    // stage is a lane's base register plus an immediate).
+    auto stage = [&](auto slot_c) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        const float* as = smem + SLOT * STAGE_FLOATS;
+        const float* bs = as + LoadA::LDS_FLOATS;
+        const float* nas = smem + ((SLOT + 1) % NS) * STAGE_FLOATS;
+        const unsigned fetch_stage = lds_wave + ((SLOT + NS - 1) % NS) * STAGE_BYTES;   // the buffer of the stage before
+        static_for<GR>([&](auto gc) {
+            constexpr int g = decltype(gc)::value;
+            if constexpr (g + 1 < GR) {
+                // the fragments of the next group are read behind this group's first MFMA
+                mfma_group_with<NACC, TM, TN>(acc, fa[g & 1], fb[g & 1], [&](auto mc) {
+                    if constexpr (decltype(mc)::value == 0)
+                        read_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(fa[(g + 1) & 1], fb[(g + 1) & 1], as, bs, wm, wn, g + 1, r, h);
+                });
+            } else {
+                // Last group: every fragment of this stage is in registers.  Spread between its MFMAs:
+                //   piece 0          own transfers of the next stage landed (vmcnt retires in order: at most
+                //                    the younger stages may be outstanding; stores issued in between only
+                //                    make this wait longer), then the barrier: everybody's part of that
+                //                    stage is visible and nobody reads the buffer of the stage before any more
+                //   pieces 1..XFERS  the transfers of the stage NS-1 ahead into that buffer
+                //   then             the producer's bookkeeping; the next stage's first fragments
+                constexpr int NP = XFERS + 3;
+                mfma_group_with<NACC, TM, TN>(acc, fa[g & 1], fb[g & 1], [&](auto mc) {
+                    constexpr int m = decltype(mc)::value;
+                    constexpr int lo = m * NP / NM, hi = (m + 1) * NP / NM;
+                    static_for<hi - lo>([&](auto pc) {
+                        constexpr int piece = lo + decltype(pc)::value;
+                        if constexpr (piece == 0) {
+                            __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 3) * XFERS));
+                            __builtin_amdgcn_s_barrier();
+                            asm volatile("" ::: "memory");
+                        } else if constexpr (piece <= XFERS) {
+                            xfer(std::integral_constant<int, piece - 1>{}, fetch_stage);
+                        } else if constexpr (piece == XFERS + 1) {
+                            advance();
+                        } else {
+                            read_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(fa[0], fb[0], nas, nas + LoadA::LDS_FLOATS, wm, wn, 0, r, h);
+                        }
+                    });
+                });
+            }
+        });
+    };
+
+    int phase = 0;                    // stage buffer of the next stage to multiply
+    for (;;) {
+        // ---- one piece: the stages of this run that belong to tile c_tile ----
+        const int piece_len = min(S - c_it, left);
+        const bool whole = c_it == 0 && piece_len == S;
+        int todo = piece_len;
+        // the stage buffers take turns; the loop is unrolled over them and entered where the last piece left off
+        bool more = true;
+        while (more) {
+            switch (phase) {
+                case 0:
+                    stage(std::integral_constant<int, 0>{});
+                    if (--todo == 0) { phase = 1; more = false; break; }
+                    [[fallthrough]];
+                case 1:
+                    stage(std::integral_constant<int, 1>{});
+                    if (--todo == 0) { phase = 2; more = false; break; }
+                    [[fallthrough]];
+                case 2:
+                    stage(std::integral_constant<int, 2>{});
+                    if (--todo == 0) { phase = (NS == 3) ? 0 : 3; more = false; break; }
+                    if constexpr (NS == 3) { phase = 0; break; }
+                    [[fallthrough]];
+                default:
+                    if constexpr (NS == 4) {
+                        stage(std::integral_constant<int, 3>{});
+                        phase = 0;
+                        if (--todo == 0) more = false;
+                    }
+                    break;
+            }
+        }
+        left -= piece_len;
+
+        if constexpr (NACC == 2) acc[0][0][0] += acc[1][0][0];
+        if (whole) {
+            store_tile<A_KIN, B_KIN, TM, TN, false>(acc[0], p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
+        } else {
+            // A piece of a shared tile goes to the workspace: slot 2w for a piece of the tile the run starts
+            // in, 2w+1 for a piece of a later tile.  It is counted at the end of the run.
+            store_partial<TM, TN>(acc[0], p.sk_ws + (size_t)(2 * w + (c_tile != first_tile ? 1 : 0)) * (BM * BN), wave, lane);
+            if (n_rec == 0) rec_tile0 = c_tile; else rec_tile1 = c_tile;
+            n_rec++;
+        }
+        if (left == 0) break;
+        c_tile++;
+        c_it = 0;
+        cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, c_tile);
+#pragma unroll
+        for (int a = 0; a < NACC; a++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int jj = 0; jj < TN; jj++) acc[a][i][jj] = (v16f)(0.0f);
+    }
+    // nothing of this wave may still be on its way into LDS when the wave ends, and every piece it stored
+    // has arrived in memory before the workgroup is counted
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    if (n_rec == 0) return;
+
+    // ---- the shared tiles this run has left a piece of (at most two) ----
+    // The pieces are counted per tile; whoever counts last adds up all the tile's pieces -- its own
+    // included, read back like the others, in run order whatever the order of arrival -- and stores the
+    // tile.  Nobody waits for anybody.  The last one also puts the counter back to zero for the next launch.
+    __syncthreads();
+    if (t < n_rec) {
+        const int tile = t == 0 ? rec_tile0 : rec_tile1;
+        const int wa = sk_owner(tile * S, p.sk_q, p.sk_rem), wb = sk_owner(tile * S + S - 1, p.sk_q, p.sk_rem);
+        const int arrived = atomicAdd(p.sk_count + tile, 1);
+        const int last = arrived == wb - wa;
+        if (last) atomicExch(p.sk_count + tile, 0);
+        sk_last[t] = last;
+    }
+    __syncthreads();
+    for (int i = 0; i < n_rec; i++) {
+        if (!sk_last[i]) continue;
+        const int tile = i == 0 ? rec_tile0 : rec_tile1;
+        const int wa = sk_owner(tile * S, p.sk_q, p.sk_rem), wb = sk_owner(tile * S + S - 1, p.sk_q, p.sk_rem);
+#pragma unroll
+        for (int ii = 0; ii < TM; ii++)
+#pragma unroll
+            for (int jj = 0; jj < TN; jj++) acc[0][ii][jj] = (v16f)(0.0f);
+        for (int w2 = wa; w2 <= wb; w2++) {
+            const int w2_first_tile = div_by(sk_first_unit(w2, p.sk_q, p.sk_rem), p.sk_div_S_mul, p.sk_div_S_shift);
+            add_partial<TM, TN>(acc[0], p.sk_ws + (size_t)(2 * w2 + (w2_first_tile == tile ? 0 : 1)) * (BM * BN), wave, lane);
+        }
+        const TileCtx c = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, tile);
+        store_tile<A_KIN, B_KIN, TM, TN, false>(acc[0], p, c.row0, c.col0, c.c_ptr, wm, wn, r, h);
+    }
+}
+
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC = 1>
+static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws, size_t ws_floats) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    if (p.split || p.bias != nullptr) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
+    p.tiles_m = (p.rows + BM - 1) / BM;
+    p.tiles_n = (p.cols + BN - 1) / BN;
+    const long long tiles = (long long)p.tiles_m * p.tiles_n * p.nz;
+    const long long S = ((long long)p.k_total + KT - 1) / KT;
+    const long long units = tiles * S;
+    if (tiles <= 0 || S <= 0) return hipErrorInvalidValue;
+    if (units > 0x3fffffffLL) return hipErrorOutOfMemory;
+    gemm_fill_tile_divisors(p);
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const long long slots = (long long)num_cu * OCC;
+    const long long grid = units < slots ? units : slots;
+    if (ws == nullptr || tiles > SK_MAX_TILES || SK_MAX_TILES + (size_t)(2 * grid) * BM * BN > ws_floats)
+        return hipErrorOutOfMemory;
+    p.sk_count = (int*)ws;            // one arrival counter per tile, zero between launches
+    p.sk_ws = ws + SK_MAX_TILES;
+    p.sk_S = (int)S;
+    gemm_magic_divisor((unsigned)S, p.sk_div_S_mul, p.sk_div_S_shift);
+    p.sk_q = (int)(units / grid);
+    p.sk_rem = (int)(units % grid);
+    hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC>), dim3((unsigned)grid),
+                       dim3(NTHREADS), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <bool A_KIN, bool B_KIN>
+static hipError_t launch_streamk_variant(const GemmParams& p, int tile, hipStream_t stream, float* ws, size_t ws_floats) {
+    switch (tile) {
+        case TILE_SK_64x64:     return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 32, 4, 1>(p, stream, ws, ws_floats);
+        case TILE_SK_128x64:    return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 32, 4, 1>(p, stream, ws, ws_floats);
+        case TILE_SK_64x128:    return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 1, 2, 32, 4, 1>(p, stream, ws, ws_floats);
+        case TILE_SK_128x128:   return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 2, 2, 32, 4, 1>(p, stream, ws, ws_floats);
+        case TILE_SK_64x64_O2:  return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 32, 4, 2>(p, stream, ws, ws_floats);
+        case TILE_SK_128x64_O2: return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 32, 3, 2>(p, stream, ws, ws_floats);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// ---- the workspace: one per (device, stream), made at the first balanced launch on that stream ----
+struct Workspace { float* ptr; size_t floats; };
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
+
+}  // namespace
+
+size_t gemm_streamk_workspace_floats(int num_cu) { return SK_MAX_TILES + (size_t)2 * num_cu * 128 * 128; }
+
+float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_ws.find({dev, stream});
+    if (it != g_ws.end()) {
+        *floats = it->second.floats;
+        return it->second.ptr;
+    }
+    // never allocate under a stream capture: the caller takes the tile-per-workgroup kernel instead
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return nullptr;
+    // a host that keeps making streams with new handles does not make the library hold ever more memory
+    if (g_ws.size() >= SK_MAX_WORKSPACES) return nullptr;
+    Workspace w = {nullptr, gemm_streamk_workspace_floats(num_cu)};
+    if (hipMalloc((void**)&w.ptr, w.floats * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    // the arrival counters start at zero and every launch leaves them there
+    if (hipMemset(w.ptr, 0, SK_MAX_TILES * sizeof(int)) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(w.ptr);
+        return nullptr;
+    }
+    g_ws[{dev, stream}] = w;
+    *floats = w.floats;
+    return w.ptr;
+}
+
+// Fitted to times measured on MI355X (1000 x 780 x K for K = 128 ... 6128, 512 ... 2048-wide squares and panels
+// with K up to 131072, all three layouts), in microseconds:
+//   tile-per-workgroup kernels, at most two 64 x 64 tiles per compute unit: 4.5 + 0.575 per 32-k stage of a tile
+//                                                                           (0.615 for A^T*B), times the tiles per unit
+//   balanced kernel, two workgroups per unit, runs of 64 x 64 tiles: 9.5 + 1.05 per stage of a run;
+//   runs of 128 x 64 tiles (two MFMA blocks per wavefront, fewer other instructions per MFMA, but pieces twice
+//   the size): 14 + 1.75 per stage, ahead from runs of 24 stages on.
+// The balanced kernel's extra fixed time is its pieces crossing the chip through memory; its stages run at 77-79 % of
+// the matrix peak with every unit busy.  Runs shorter than 12 stages consist of pieces only and do not pay unless the
+// tiles leave more than half the chip idle.  Measured gains where it is taken: 4-9 % at 1000 x 777 x 1531, 13 % at
+// 1024 x 1024 x 4096, 3.6 x at 512 x 512 x 8192, 17 x at 256 x 256 x 131072.
+int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant) {
+    if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
+    const long long t64 = (long long)((rows + 63) / 64) * ((cols + 63) / 64) * nz;
+    if (t64 > 2LL * num_cu || t64 > SK_MAX_TILES) return -1;
+    const long long stages = ((long long)k + 31) / 32;
+    const long long slots = 2LL * num_cu;
+    const long long t128 = (long long)((rows + 127) / 128) * ((cols + 63) / 64) * nz;
+    const long long runs64 = (t64 * stages + slots - 1) / slots, runs128 = (t128 * stages + slots - 1) / slots;
+    if (runs64 < 12 && 2 * t64 >= num_cu) return -1;
+    const bool wide = runs128 >= 24;
+    const double t_balanced = wide ? 14.0 + 1.75 * (double)runs128 : 9.5 + 1.05 * (double)runs64;
+    const double per_unit = (double)((t64 + num_cu - 1) / num_cu);
+    const double t_tiles = 4.5 + (variant == GEMM_T1 ? 0.615 : 0.575) * (double)stages * per_unit;
+    if (t_balanced > 0.97 * t_tiles) return -1;
+    return wide ? TILE_SK_128x64_O2 : TILE_SK_64x64_O2;
+}
+
+hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream) {
+    size_t floats = 0;
+    float* ws = gemm_streamk_workspace(stream, &floats);
+    if (ws == nullptr) return hipErrorOutOfMemory;
+    switch (variant) {
+        case GEMM_NN: return launch_streamk_variant<true, false>(p, tile, stream, ws, floats);
+        case GEMM_T1: return launch_streamk_variant<false, false>(p, tile, stream, ws, floats);
+        case GEMM_T2: return launch_streamk_variant<true, true>(p, tile, stream, ws, floats);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace dragon

@@ -9,14 +9,17 @@
 #include <atomic>
 #include <vector>
 #include "../../include/dragon_hip_runtime.h"
+#include "../../include/dragon_hip_testing.h"
 #include "runtime_internal.h"
 
 namespace {
-std::atomic<int> g_last_error{0};
+// per host thread, like the runtime's own last error (cudaGetLastError in the reference,
+// Cuda/Cuda/Cuda_Exception.cuh:21-27): one thread never takes another thread's error code
+thread_local int t_last_error = 0;
 }
 namespace dragon_rt {
 int note(hipError_t e) {
-    if (e != hipSuccess) g_last_error.store((int)e, std::memory_order_relaxed);
+    if (e != hipSuccess) t_last_error = (int)e;
     return (int)e;
 }
 }  // namespace dragon_rt
@@ -225,7 +228,8 @@ int dragon_Cuda_streamsWaitEvent_default(const int64_t* streams, int32_t length,
 const char* dragon_Cuda_getExceptionName(int32_t type) { return hipGetErrorName((hipError_t)type); }
 const char* dragon_Cuda_getExceptionInfo(int32_t type) { return hipGetErrorString((hipError_t)type); }
 int32_t dragon_Cuda_getLastExceptionType(void) {
-    int e = g_last_error.exchange(0, std::memory_order_relaxed);
+    const int e = t_last_error;
+    t_last_error = 0;
     hipError_t h = hipGetLastError();
     return e ? e : (int)h;
 }
@@ -246,7 +250,7 @@ int dragon_Cuda_set2D_value(int64_t stream, int64_t address, float value, int32_
     return note(hipGetLastError());
 }
 
-int dragon_Cuda_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t length) {
+int dragon_test_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t length) {
     if (dst == 0 || src == 0 || length <= 0 || (length & 3) || ((dst | src) & 15))
         return note(hipErrorInvalidValue);
     const long long n4 = length >> 2;

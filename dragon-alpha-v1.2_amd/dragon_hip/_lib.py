@@ -1,5 +1,6 @@
 """ctypes binding of libdragon_hip.so: the C ABI declared in include/dragon_hip_gemm.h
-and include/dragon_hip_runtime.h, and the host-side engine of include/dragon_hip_engine.h.
+and include/dragon_hip_runtime.h, the host-side engine of include/dragon_hip_engine.h and the
+test hooks of include/dragon_hip_testing.h.
 
 The library is loaded from the package directory.  There is no fallback: if the shared
 object is missing or a symbol cannot be resolved the import fails, and every compute
@@ -126,7 +127,7 @@ SIGNATURES = {
     "dragon_Cuda_get2D_v2": (i32, [i64, i64, c_void_p, i64, i32, i32, i32]),
     "dragon_Cuda_set1D_v2": (i32, [i64, i64, c_void_p, i64, i32]),
     "dragon_Cuda_set2D_v2": (i32, [i64, i64, c_void_p, i64, i32, i32, i32]),
-    "dragon_Cuda_copy1D_kernel": (i32, [i64, i64, i64, i64]),
+    "dragon_test_copy1D_kernel": (i32, [i64, i64, i64, i64]),
     # include/dragon_hip_engine.h
     "dragon_engine_last_error": (c_char_p, []),
     "dragon_engine_last_cuda_code": (i32, []),

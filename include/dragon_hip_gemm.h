@@ -18,12 +18,19 @@
  * Conventions shared by all entry points (same as the reference):
  *   - Letters follow the reference: N = rows of C, M = columns of C, K = contraction.
  *   - Row-major FP32.  Addresses are device pointers owned by the caller, 16-byte
- *     aligned; nothing is allocated, freed or retained here.
+ *     aligned; no caller memory is freed or retained here.  The one thing the library allocates:
+ *     for products with few tiles and a long K (at most two 64 x 64 tiles of C per compute
+ *     unit) the first call on a stream makes a 32 MiB workspace that later calls on the same
+ *     stream handle reuse (partial tiles of workgroups that share the K range of a tile pass
+ *     through it); it is kept until the process ends, at most 64 of them exist, and none is
+ *     ever made while the stream is being captured into a graph -- such a call runs the
+ *     ordinary kernel instead, as does every call when the allocation fails.
  *   - C is overwritten (no alpha/beta).  Padded rows/columns of C receive exact zeros.
  *   - streams[0..length) are valid stream handles, 1 <= length <= 10.  Work is issued
  *     asynchronously on streams[0]; the other handles are left idle (the caller joins
  *     all of them into streams[0] anyway).  The call returns without waiting.
- *   - Callable from any host thread; no host-side global state is modified.
+ *   - Callable from any host thread; the only host-side state is the table of those
+ *     workspaces (behind a mutex) and per-kernel occupancy figures cached on first use.
  *   - Errors: hipErrorInvalidValue (1) for a null address, a non-positive dimension, a
  *     stream count outside 1..10, a dimension that violates the x4 padding contract, or
  *     a misaligned address, or a size beyond the limits below; otherwise the launch
@@ -270,32 +277,6 @@ int dragon_Cuda_batchMatMul_batchMatMulT2_mma(int32_t useTexture,
 int32_t dragon_Cuda_matMul_blockNum(int32_t N, int32_t M);
 int32_t dragon_Cuda_matMul_nstream(int32_t N, int32_t M);
 int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M);
-
-/* ---- tuning hook (no counterpart in the reference): force one tile shape for every
- * following launch of this process, -1 restores the automatic choice.  For benchmarks
- * and tests that sweep the kernel variants; not thread-safe against concurrent calls.
- * Shapes: 0 = 128x128, 1 = 64x64, 2 = 256x64, 3 = 64x256, 4 = 128x64, 5 = 64x128 (16 k per
- * LDS stage); 6 = 128x128, 7 = 64x64, 8 = 128x64, 9 = 64x128 with 32 k per stage; 10 = 64x64
- * with 64 k, 11 = 64x64 with 128 k, 12 = 128x128, 13 = 128x64, 14 = 64x128 with 64 k per stage;
- * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
- * directly through four stage buffers.  Adding 256 to a shape 0..9 selects its paired-stage form
- * (stages run two by two with compile-time LDS buffers; what the automatic choice takes from
- * K = 512 on). */
-void dragon_gemm_force_tile(int32_t tile);
-/* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
- * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the
- * operand's advance per k (4 bytes, or a row of a K-outer operand) must stay below 2^31; 0 if not (the
- * launch then runs the plain form), -1 on bad arguments.  Host arithmetic only; for tests. */
-int32_t dragon_gemm_paired_form_fits(int32_t variant, int32_t GridZ, int32_t N, int32_t M, int32_t K);
-/* The multiply-and-shift pair the kernels divide a tile index by d with: n / d == (((2n) * mul) >> 32) >> shift
- * for every 0 <= n < 2^31 (the launcher makes the pairs, the kernels only multiply).  Host arithmetic; for
- * tests. */
-void dragon_gemm_tile_divisor(uint32_t d, uint32_t* mul, uint32_t* shift);
-/* The shape the automatic choice takes for a product of `rows` x `cols` outputs, depth `nz` (batch or
- * K slices), `k` per output, on `num_cu` compute units; variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, -1 = unknown.
- * Pure host arithmetic (no device needed); returns the forced shape while one is forced, -1 on bad
- * arguments.  For inspection and tests; no counterpart in the reference. */
-int32_t dragon_gemm_choose_tile(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu);
 
 #ifdef __cplusplus
 }

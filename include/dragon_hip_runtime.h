@@ -88,10 +88,6 @@ int dragon_Cuda_get2D(int64_t stream, int64_t address, float* value,
 int dragon_Cuda_set1D(int64_t stream, int64_t address, const float* value, int32_t length);  /* :214 */
 int dragon_Cuda_set2D(int64_t stream, int64_t address, const float* value,
                       int32_t height, int32_t width, int32_t stride);                        /* :311 */
-/* Device-to-device copy of `length` floats (a multiple of 4, 16-byte aligned) done by an
- * ordinary kernel rather than the copy engine.  No counterpart in the reference: it is the
- * known-size copy that hardware byte counters are calibrated against when profiling. */
-int dragon_Cuda_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t length);
 /* _v2: the caller provides a pinned staging buffer of height*stride (or length) floats. */
 int dragon_Cuda_get1D_v2(int64_t stream, int64_t address, float* value, int64_t buf, int32_t length);
 int dragon_Cuda_get2D_v2(int64_t stream, int64_t address, float* value, int64_t buf,

@@ -1,0 +1,50 @@
+/*
+ * dragon_hip_testing.h -- inspection and test hooks of libdragon_hip.so.
+ *
+ * NOT part of the drop-in boundary: nothing here has a counterpart in the reference and no host
+ * needs it to run the engine.  The hooks exist so that tests and benchmarks can sweep the kernel
+ * variants, check host arithmetic without a device, and calibrate profiler byte counters.
+ */
+#ifndef DRAGON_HIP_TESTING_H
+#define DRAGON_HIP_TESTING_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Force one tile shape for the following launches OF THE CALLING THREAD (the setting is
+ * thread-local: no other thread's kernel choice changes); -1 restores the automatic choice.
+ * Shapes: 0 = 128x128, 1 = 64x64, 2 = 256x64, 3 = 64x256, 4 = 128x64, 5 = 64x128 (16 k per
+ * LDS stage); 6 = 128x128, 7 = 64x64, 8 = 128x64, 9 = 64x128 with 32 k per stage; 10 = 64x64
+ * with 64 k, 11 = 64x64 with 128 k, 12 = 128x128, 13 = 128x64, 14 = 64x128 with 64 k per stage;
+ * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
+ * directly through four stage buffers.  Adding 256 to a shape 0..9 selects its paired-stage form
+ * (stages run two by two with compile-time LDS buffers; what the automatic choice takes from
+ * K = 512 on).  18..23: the balanced kernel for few tiles and a long K (workgroups share the work
+ * in equal runs of LDS stages): 18 = 64x64, 19 = 128x64, 20 = 64x128, 21 = 128x128 with one
+ * workgroup per compute unit, 22 = 64x64 and 23 = 128x64 with two. */
+void dragon_gemm_force_tile(int32_t tile);
+/* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
+ * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the
+ * operand's advance per k (4 bytes, or a row of a K-outer operand) must stay below 2^31; 0 if not (the
+ * launch then runs the plain form), -1 on bad arguments.  Host arithmetic only. */
+int32_t dragon_gemm_paired_form_fits(int32_t variant, int32_t GridZ, int32_t N, int32_t M, int32_t K);
+/* The multiply-and-shift pair the kernels divide a tile index by d with: n / d == (((2n) * mul) >> 32) >> shift
+ * for every 0 <= n < 2^31 (the launcher makes the pairs, the kernels only multiply).  Host arithmetic. */
+void dragon_gemm_tile_divisor(uint32_t d, uint32_t* mul, uint32_t* shift);
+/* The shape the automatic choice takes for a product of `rows` x `cols` outputs, depth `nz` (batch or
+ * K slices), `k` per output, on `num_cu` compute units; variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, -1 = unknown.
+ * Pure host arithmetic (no device needed); returns the forced shape while the calling thread forces one,
+ * -1 on bad arguments. */
+int32_t dragon_gemm_choose_tile(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu);
+/* Device-to-device copy of `length` floats (a multiple of 4, 16-byte aligned) done by an ordinary
+ * kernel rather than the copy engine: the known-size copy that hardware byte counters are
+ * calibrated against when profiling. */
+int dragon_test_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t length);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRAGON_HIP_TESTING_H */

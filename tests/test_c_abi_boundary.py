@@ -11,7 +11,8 @@ import pytest
 from oracle import oracle
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("dragon_hip_gemm.h", "dragon_hip_conv.h", "dragon_hip_runtime.h", "dragon_hip_engine.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("dragon_hip_gemm.h", "dragon_hip_conv.h", "dragon_hip_runtime.h", "dragon_hip_engine.h",
+                                                    "dragon_hip_testing.h")]
 INVALID_VALUE = 1   # hipErrorInvalidValue
 
 
@@ -176,8 +177,17 @@ def test_tile_choice_on_the_documented_shapes(dh):
     assert ct(T1, 256, 256, 128, 1024) == 6 + P                   # the split-K weight gradient (GridZ 128 slices of 1024)
     assert ct(NN, 1024, 64, 64, 1024) == 8 + P                    # scores x V of the attention-shaped batch
     assert ct(T2, 1024, 1024, 64, 64) == 0 and ct(T1, 1024, 1024, 64, 64) == 0
-    assert ct(T1, 1000, 780, 1, 1532) == 17                     # fewer tiles than units: direct-to-LDS 64x64 ...
-    assert ct(NN, 1000, 780, 1, 1532) == 7 + P == ct(T2, 1000, 780, 1, 1532)   # ... or, with a K-inner operand, paired
+    # Few tiles and a long K: the balanced kernel (22 = 64x64, 23 = 128x64, two workgroups per unit) where its
+    # estimated time is ahead; 128x64 once its runs are 24 stages long
+    for v in (NN, T1, T2):
+        assert ct(v, 1000, 780, 1, 1532) == 22                  # 208 tiles x 48 stages over 512 workgroups: runs of 19.5
+        assert ct(v, 256, 256, 1, 131072) == 23                 # the tall-K weight gradient through the unsplit entry
+        assert ct(v, 1024, 1024, 1, 4096) == 23 and ct(v, 512, 512, 1, 8192) == 22
+        assert ct(v, 1000, 780, 1, 6128) == 23 and ct(v, 1000, 780, 1, 3064) == 22
+    assert ct(NN, 1000, 780, 1, 1024) == 7 + P == ct(T2, 1000, 780, 1, 1024)   # a shorter K: one paired 64x64 tile per workgroup
+    assert ct(NN, 1024, 1024, 1, 1024) == 7 + P and ct(T1, 1024, 1024, 1, 1024) == 17   # ... or direct-to-LDS for A^T*B
+    assert ct(NN, 768, 768, 1, 768) == 7 + P                    # runs of 7 stages would be pieces only
+    assert ct(NN, 1000, 780, 2, 760) == 22                      # a batch of two ragged products is balanced as one
     assert ct(NN, 257, 388, 36, 129) == 1                       # batch of small ragged products: 64x64
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
