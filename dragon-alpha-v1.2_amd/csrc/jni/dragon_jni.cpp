@@ -8,8 +8,9 @@
 // non-zero status into z.dragon.engine.cuda.impl.CudaException(int), as the reference's
 // handleError / throwCudaException do (Cuda_matMul/Cuda_matMul/JNITool.cuh:9-25).
 //
-// Built only where a JDK provides <jni.h> (build_jni.sh next to this file); the rest of the
-// library does not depend on it.
+// Built where a JDK provides <jni.h> (build_jni.sh next to this file); the rest of the library does not
+// depend on it.  Without a JDK the CPU tests still compile it, against a minimal stand-in header, and
+// compare its exports with the reference's names.
 #if __has_include(<jni.h>)
 #include <jni.h>
 #include <stddef.h>
@@ -118,6 +119,18 @@ DEF_MM2D(matMulT2_1mma, dragon_Cuda_matMul_matMulT2_mma)
 DEF_MMSK(matMulSK, dragon_Cuda_matMul_matMulSK)
 DEF_MMSK(matMulT1SK, dragon_Cuda_matMul_matMulT1SK)
 DEF_MMSK(matMulT2SK, dragon_Cuda_matMul_matMulT2SK)
+
+// Both split-K stages without any allocation (the partials stay in the library's static device workspace).
+// The reference has no such native: a maintainer who wants it declares `public static native void
+// matMulSK_static(long[] streamArray, int length, int variant, int GridZ, long dA_address, long dB_address,
+// long dC_address, int N, int M, int K)` in Cuda_matMul.java.
+JNIEXPORT void JNICALL MM(matMulSK_1static)(JNIEnv* env, jclass, jlongArray streamArray, jint length,
+                                            jint variant, jint GridZ, jlong dA, jlong dB, jlong dC, jint N,
+                                            jint M, jint K) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_matMul_matMulSK_static(st.s, st.n, variant, GridZ, dA, dB, dC, N, M, K));
+}
 
 // One launch for matMul + bias row.  The reference has no such native: a maintainer who wants it
 // declares `public static native void matMul_biased(long[] streamArray, int length, long dA_address,
