@@ -31,9 +31,74 @@ for _p in (ROOT, os.path.join(ROOT, "dragon-alpha-v1.2_amd")):
 
 PEAK_TFLOPS = 157.3      # FP32 MFMA, dense
 HBM_PEAK_GBS = 8000.0
-# HBM-side bytes per 4096^3 launch read off the hardware counters (FETCH_SIZE scaled x2.000 by a
-# known copy, plus WRITE_SIZE); source: profiles/gemm_f32_mfma_4096cubed.md
-MEASURED_TRAFFIC_BYTES = {"A*B": 857.3 * 2 ** 20, "A*B^T": 866.4 * 2 ** 20, "A^T*B": 828.8 * 2 ** 20}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_f32_mfma_4096cubed.md")
+# the sources the headline kernels are compiled from: a counter reading belongs to one state of them
+KERNEL_SOURCES = [os.path.join(ROOT, "dragon-alpha-v1.2_amd", "csrc", f)
+                  for f in ("gemm_mfma_kernel.h", "gemm_mfma.hip", "gemm_mfma.h", "build.sh")]
+
+
+def kernel_sources_sha16():
+    import hashlib
+    h = hashlib.sha256()
+    for f in KERNEL_SOURCES:
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic():
+    """HBM-side bytes per 4096^3 launch as the hardware counters read them (FETCH_SIZE and WRITE_SIZE, each
+    scaled by what the same counter reads on a copy kernel of known size): the machine-readable block
+    that `bench.py --summarize-traffic` printed into profiles/gemm_f32_mfma_4096cubed.md.  Counters cannot
+    be read inside a timed run, so this is a recorded figure; it is marked stale when the kernel sources
+    have changed since."""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+        block = re.search(r"```json traffic\n(.*?)\n```", text, flags=re.S)
+        rec = json.loads(block.group(1))
+        rec["stale"] = rec.get("kernel_sources_sha16") != kernel_sources_sha16()
+        return rec
+    except Exception as e:      # no block, unreadable: no traffic figure rather than a made-up one
+        return {"error": "%s: %s" % (type(e).__name__, e)}
+
+
+def summarize_traffic(root):
+    """Reads the four rocprofv3 --pmc result databases under `root` (fetch/, write/: the headline run;
+    cfetch/, cwrite/: `bench.py --calibrate-copy`) and prints the traffic block for the profile summary."""
+    import glob
+    import sqlite3
+
+    def per_kernel(sub, counter):
+        db = sqlite3.connect(glob.glob(os.path.join(root, sub, "**", "*.db"), recursive=True)[0])
+        cols = [r[1] for r in db.execute("pragma table_info(counters_collection)")]
+        out = {}
+        for row in db.execute("select * from counters_collection"):
+            d = dict(zip(cols, row))
+            if d["counter_name"] == counter:
+                out.setdefault(d["kernel_name"], []).append(float(d["value"]))
+        return {k: sum(v) / len(v) for k, v in out.items()}        # KiB per dispatch
+
+    copy_bytes = 64 * 1024 * 1024 * 4.0
+    cf = [v for k, v in per_kernel("cfetch", "FETCH_SIZE").items() if "copy4_kernel" in k][0]
+    cw = [v for k, v in per_kernel("cwrite", "WRITE_SIZE").items() if "copy4_kernel" in k][0]
+    scale_f, scale_w = copy_bytes / (cf * 1024), copy_bytes / (cw * 1024)
+    fetch, write = per_kernel("fetch", "FETCH_SIZE"), per_kernel("write", "WRITE_SIZE")
+    names = {"<true, false,": "A*B", "<true, true,": "A*B^T", "<false, false,": "A^T*B"}
+    per = {}
+    for k in fetch:
+        if "gemm_f32_mfma" not in k:
+            continue
+        label = [v for pat, v in names.items() if pat in k]
+        if not label:
+            continue
+        rd, wr = fetch[k] * 1024 * scale_f, write.get(k, 0.0) * 1024 * scale_w
+        per[label[0]] = {"kernel": k.split("(dragon::GemmParams")[0].replace("void dragon::(anonymous namespace)::", ""), "read_bytes": round(rd), "written_bytes": round(wr),
+                         "traffic_bytes": round(rd + wr)}
+    print("```json traffic")
+    print(json.dumps({"kernel_sources_sha16": kernel_sources_sha16(),
+                      "fetch_scale": round(scale_f, 4), "write_scale": round(scale_w, 4),
+                      "algorithmic_bytes": 3 * 4096 * 4096 * 4, "per_launch": per}, indent=1))
+    print("```")
 
 
 def log(*a):
@@ -83,14 +148,21 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias,attention,conv,transpose,transfer,engine",
+    ap.add_argument("--configs", default="3,4,5,bias,attention,conv,hbm,transpose,transfer,engine",
                     help="which of the other workloads to time (default all): BASELINE configs 3, 4, 5, "
                          "the biased fully-connected layer, the attention chain, the forward convolution, "
                          "dimension swaps, tensor upload / download, the host mirror's own overhead")
+    ap.add_argument("--summarize-traffic", metavar="DIR", default=None,
+                    help="no GPU needed: read the rocprofv3 --pmc databases under DIR/fetch, DIR/write (the "
+                         "headline run) and DIR/cfetch, DIR/cwrite (--calibrate-copy) and print the traffic "
+                         "block that profiles/gemm_f32_mfma_4096cubed.md carries")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: run a 256 MiB device copy kernel 10 times and exit "
                          "(the known-size copy that FETCH_SIZE / WRITE_SIZE are scaled by)")
     args = ap.parse_args()
+    if args.summarize_traffic:
+        summarize_traffic(args.summarize_traffic)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this engine runs on ONE GPU (one process, no collectives); "
                  "run it with --gpus 1")
@@ -154,12 +226,16 @@ def main():
                                                "pct_peak": round(100 * tf / PEAK_TFLOPS, 1)}
     slowest = max(kernel_ms, key=kernel_ms.get)
     achieved = flop / (kernel_ms[slowest] * 1e-3) / 1e12
+    rec = recorded_traffic()
+    rec_kernel = rec.get("per_launch", {}).get(slowest)
     roofline = {"bound": "mfma", "kernel": "gemm_f32_mfma %s 4096^3" % slowest,
                 "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_TFLOPS, 4),
-                "traffic": round(MEASURED_TRAFFIC_BYTES[slowest]),
-                "traffic_note": "bytes per launch at the L2-fabric boundary from rocprofv3 counters "
-                                "(includes Infinity-Cache hits); algorithmic = 201326592"}
+                "traffic": rec_kernel["traffic_bytes"] if rec_kernel else None,
+                "traffic_stale": bool(rec.get("stale", True)),
+                "traffic_note": "bytes per launch at the L2-fabric boundary (Infinity-Cache hits included), recorded "
+                                "from rocprofv3 FETCH_SIZE / WRITE_SIZE in profiles/gemm_f32_mfma_4096cubed.md, not "
+                                "measured by this run; stale = the kernel sources changed since; algorithmic = 201326592"}
 
     # ---------------- CPU baseline: the oracle on the same three products ---------------------
     cpu_baseline = None
@@ -229,6 +305,18 @@ def main():
         ms = timer.per_launch_ms(cfg3, iters=50)
         record("cfg3 A^T*B 256x256 K=131072 split-K GZ=%d + reduction" % GZ, 2.0 * N3 * N3 * K3, ms,
                4.0 * (2 * K3 * N3 + N3 * N3))
+        if cpu_baseline is not None:
+            # the stated gate of this config, measured: relative Frobenius error against the CPU matmul
+            from oracle import oracle
+            g3 = synthetic.stream_for(3)
+            A3, B3 = g3.normal((K3, N3), 0.0, 0.05), g3.normal((K3, N3), 0.0, 0.05)
+            R3 = oracle.matmul(1, A3, B3)
+            Cuda.streamSynchronize(stream)
+            C3 = dC.get((N3, N3))
+            cpu_baseline["rel_frobenius_gpu_vs_cpu_cfg3_A^T*B_splitK"] = float(
+                np.linalg.norm(C3.astype(np.float64) - R3) / np.linalg.norm(R3.astype(np.float64)))
+            cpu_baseline["rel_frobenius_gate"] = 1e-5
+            del A3, B3, R3, C3
         ms = timer.per_launch_ms(
             lambda: MM.matMulT1(S, 1, dA.address, dB.address, dC.address, N3, N3, K3), iters=20)
         record("cfg3 same shape through the unsplit entry", 2.0 * N3 * N3 * K3, ms)
@@ -327,9 +415,9 @@ def main():
         record("fullconnect_biased 8192x4096x4096 product + linear_dual2D_row", flb, ms)
         ms = timer.per_launch_ms(lambda: FN.linear_dual2D_row(
             stream, dY.address, db.address, Mb, 1.0, 1.0, 0.0, dY.address, Nb * Mb, Mb, Mb), iters=50)
-        per_config["linear_dual2D_row 8192x4096 (HBM-bound)"] = {
-            "ms": round(ms, 4), "alg_GBps": round(8.0 * Nb * Mb / (ms * 1e-3) / 1e9, 1),
-            "pct_hbm_peak": round(100 * 8.0 * Nb * Mb / (ms * 1e-3) / 8e12, 1)}
+        # 128 MiB in place: the tensor sits in the 256 MB Infinity Cache, so this is not an HBM figure
+        per_config["linear_dual2D_row 8192x4096 in place (128 MiB: served by the Infinity Cache)"] = {
+            "ms": round(ms, 4), "alg_GBps": round(8.0 * Nb * Mb / (ms * 1e-3) / 1e9, 1), "bound": "mall"}
         for x in (dX, dW, db, dY):
             x.free()
 
@@ -365,14 +453,13 @@ def main():
             pv()
         ms = timer.per_launch_ms(lambda: RD.softmax2D(stream, dP.address, dP.address, Bt * Sq, Sq, Sq, Sq,
                                                       0.125), iters=30)
-        per_config["softmax2D 65536 rows of 1024, in place (HBM-bound, 512 MiB)"] = {
-            "ms": round(ms, 4), "alg_GBps": round(8.0 * nP / (ms * 1e-3) / 1e9, 1),
-            "pct_hbm_peak": round(100 * 8.0 * nP / (ms * 1e-3) / 8e12, 1)}
+        # 256 MiB in place: as large as the Infinity Cache, largely served by it
+        per_config["softmax2D 65536 rows of 1024 in place (256 MiB: Infinity-Cache assisted)"] = {
+            "ms": round(ms, 4), "alg_GBps": round(8.0 * nP / (ms * 1e-3) / 1e9, 1), "bound": "mall"}
         ms = timer.per_launch_ms(lambda: FN.linear2D(stream, 0.125, dP.address, 0.0, dP.address, nP, Sq, Sq),
                                  iters=30)
-        per_config["linear2D (sdiv) 64 Mi floats in place (HBM-bound, 512 MiB)"] = {
-            "ms": round(ms, 4), "alg_GBps": round(8.0 * nP / (ms * 1e-3) / 1e9, 1),
-            "pct_hbm_peak": round(100 * 8.0 * nP / (ms * 1e-3) / 8e12, 1)}
+        per_config["linear2D (sdiv) 64 Mi floats in place (256 MiB: Infinity-Cache assisted)"] = {
+            "ms": round(ms, 4), "alg_GBps": round(8.0 * nP / (ms * 1e-3) / 1e9, 1), "bound": "mall"}
         fl_chain = 2 * 2.0 * Bt * Sq * Sq * D
         ms = timer.per_launch_ms(chain_fused_scale, iters=20)
         record("attention chain Q.K^T -> softmax(x/8) -> P.V, batch 64 x 1024 x 64 (3 launches)", fl_chain, ms)
@@ -433,6 +520,28 @@ def main():
             for x in (dXc, dWc, dbc, dYc):
                 x.free()
 
+    if "hbm" in extra:
+        # the HBM-bound kernels of the widenings on tensors of 1 GiB (four times the 256 MB Infinity Cache), in
+        # place: 1 GiB read + 1 GiB written per launch
+        log("HBM-bound kernels on 1 GiB tensors ...")
+        RD, FN = dh.Cuda_reduce, dh.Cuda_function
+        rows_h, width_h = 32768, 8192
+        nH = rows_h * width_h
+        dH = dh.DeviceArray(size=nH)
+        dbH = dh.DeviceArray(size=width_h)
+        for name, fn in (
+            ("linear_dual2D_row 32768x8192 in place", lambda: FN.linear_dual2D_row(
+                stream, dH.address, dbH.address, width_h, 1.0, 1.0, 0.0, dH.address, nH, width_h, width_h)),
+            ("linear2D 32768x8192 in place", lambda: FN.linear2D(stream, 0.5, dH.address, 0.0, dH.address, nH,
+                                                                 width_h, width_h)),
+            ("softmax2D 262144 rows of 1024 in place", lambda: RD.softmax2D(
+                stream, dH.address, dH.address, nH // 1024, 1024, 1024, 1024, 1.0))):
+            ms = timer.per_launch_ms(fn, iters=20)
+            per_config[name + " (HBM-bound, 1 GiB tensor)"] = {
+                "ms": round(ms, 4), "alg_GBps": round(8.0 * nH / (ms * 1e-3) / 1e9, 1), "bound": "hbm",
+                "pct_hbm_peak": round(100 * 8.0 * nH / (ms * 1e-3) / 8e12, 1)}
+        dH.free(), dbH.free()
+
     if "transpose" in extra:
         # the layout step of attention blocks: [B, S, H, D] <-> [B, H, S, D] (whole rows move) and the
         # last-two-dimension swap K -> K^T per head (LDS-tiled); HBM-bound, read + write once
@@ -449,8 +558,8 @@ def main():
             ("transpose2D [8192,8192]", lambda: E2.transpose2D(
                 stream, dX2.address, dY2.address, 8192, 8192, 8192, 8192, nq))):
             ms = timer.per_launch_ms(fn, iters=50)
-            per_config[name + " (HBM-bound)"] = {
-                "ms": round(ms, 4), "alg_GBps": round(8.0 * nq / (ms * 1e-3) / 1e9, 1),
+            per_config[name + " (HBM-bound, 256 MiB in + 256 MiB out)"] = {
+                "ms": round(ms, 4), "alg_GBps": round(8.0 * nq / (ms * 1e-3) / 1e9, 1), "bound": "hbm",
                 "pct_hbm_peak": round(100 * 8.0 * nq / (ms * 1e-3) / 8e12, 1)}
         dX2.free(), dY2.free()
 
