@@ -38,12 +38,17 @@ enum GemmTile {
     TILE_SK_64x64_O2 = 22,     // two workgroups per compute unit, 4 stage buffers
     TILE_SK_128x64_O2 = 23,    // two workgroups per compute unit, 3 stage buffers
     TILE_SK_END = 24,
+    // Short K (at most 64), large C: a workgroup keeps a band of 128 rows of A in LDS, walks along its
+    // column tiles with the whole K in one stage and stores a tile while it multiplies the next
+    // (gemm_mfma_band.hip)
+    TILE_BAND_128x128 = 24,
     // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
     // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
     // short K; gemm_choose_tile sets it.
     TILE_PAIRED = 0x100
 };
 inline bool gemm_tile_is_streamk(int tile) { return tile >= TILE_SK_64x64 && tile < TILE_SK_END; }
+inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128; }
 inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
@@ -86,6 +91,9 @@ struct GemmParams {
     int* sk_count;
     int sk_S, sk_q, sk_rem;
     unsigned sk_div_S_mul, sk_div_S_shift;
+    // filled by the launcher of the band kernel (gemm_launch_band): a band's tiles_n column tiles are dealt
+    // out in bd_chunks runs of bd_chunk_tiles
+    int bd_chunks, bd_chunk_tiles;
 };
 void gemm_fill_tile_divisors(GemmParams& p);
 void gemm_magic_divisor(unsigned d, unsigned& mul, unsigned& shift);
@@ -120,6 +128,14 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
 // Made at the first balanced launch on that stream (never while the stream is capturing: then nullptr) and kept
 // for later launches on the same handle until the process ends.
 float* gemm_streamk_workspace(hipStream_t stream, size_t* floats);
+// The band kernel (tile id TILE_BAND_128x128) for the three products, batched too, with K <= 64.
+// hipErrorOutOfMemory says that the product cannot go this way (a longer K, K slices, a bias row) and the
+// caller takes a tile-per-workgroup kernel instead.
+hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream);
+// TILE_BAND_128x128 where the band kernel is the better choice, else -1
+int gemm_choose_band(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
+// how the band kernel deals a band's column tiles to workgroups
+void gemm_band_split(long long bands, int tiles_n, int num_cu, int& chunks, int& chunk_tiles);
 // Y = conv(X, W) [+ bias row over OC] as an implicit GEMM (the A * B^T kernel with a gathered A);
 // classic tile ids only
 hipError_t gemm_launch_conv(const GemmParams& p, int tile, hipStream_t stream);

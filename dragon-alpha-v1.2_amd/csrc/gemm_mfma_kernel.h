@@ -42,6 +42,7 @@
 #include <hip/hip_runtime.h>
 #include <atomic>
 #include <type_traits>
+#include <utility>
 #include <stdint.h>
 #include "gemm_mfma.h"
 
@@ -112,6 +113,16 @@ __device__ __forceinline__ void dma_descriptor_advance(v4u& rsrc, unsigned long 
     rsrc.y = (unsigned)(b >> 32);
 }
 #pragma clang diagnostic pop
+
+// compile-time loop: f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N-1>)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // s_waitcnt for the vector-memory counter alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
 // expcnt 6:4 and lgkmcnt 11:8 left at "no wait")

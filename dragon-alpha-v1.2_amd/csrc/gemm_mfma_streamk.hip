@@ -88,16 +88,6 @@ __device__ __forceinline__ void read_group(float (&fa)[TM][4], float (&fb)[TN][4
     else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
 }
 
-// compile-time loop: f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N-1>)
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 // The MFMAs of one group of 8 k, with `between(m)` placed after MFMA number m.  A wavefront issues one
 // instruction every four cycles at best and an MFMA keeps the matrix pipe busy for 64: whatever else
 // the wavefront has to do costs nothing while it sits BETWEEN two MFMAs (15 issue slots each) and

@@ -176,7 +176,12 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 1536, 1536, 1, 1536) == 7 + P                # 64x64, three per unit: 32-k stages
     assert ct(T1, 256, 256, 128, 1024) == 6 + P                   # the split-K weight gradient (GridZ 128 slices of 1024)
     assert ct(NN, 1024, 64, 64, 1024) == 8 + P                    # scores x V of the attention-shaped batch
-    assert ct(T2, 1024, 1024, 64, 64) == 0 and ct(T1, 1024, 1024, 64, 64) == 0
+    # A K that fits one LDS stage of 64 under a large C: the band kernel (24), from two tiles per compute unit on;
+    # not for a K of 56 or less, rows of C off the 128-byte lines, or a C that leaves its tiles mostly empty
+    for v in (NN, T1, T2):
+        assert ct(v, 1024, 1024, 64, 64) == 24 and ct(v, 4096, 4096, 1, 60) == 24 and ct(v, 2048, 256, 64, 64) == 24
+        assert ct(v, 1024, 1024, 64, 56) != 24 and ct(v, 1024, 1000, 64, 64) != 24 and ct(v, 1024, 1024, 1, 64) != 24
+        assert ct(v, 130, 1024, 64, 64) != 24 and ct(v, 1024, 1024, 64, 68) != 24
     # Few tiles and a long K: the balanced kernel (22 = 64x64, 23 = 128x64, two workgroups per unit) where its
     # estimated time is ahead; 128x64 once its runs are 24 stages long
     for v in (NN, T1, T2):
