@@ -113,7 +113,7 @@ template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS
 __global__ __launch_bounds__(NTHREADS, OCC)
 void gemm_f32_mfma_streamk(const GemmParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
-    static_assert(NS == 3 || NS == 4, "stage buffers: 3 or 4");
+    static_assert(NS == 3 || NS == 4, "stage buffers: 3 or 4 (deeper ones measured slower)");
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
     using LoadB = typename std::conditional<B_KIN, KInner<BN, KT, TN>, KOuter<BN, KT>>::type;
@@ -225,7 +225,7 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     int rec_tile0 = 0, rec_tile1 = 0; // shared tiles this run has left a piece of
     int n_rec = 0;
 
-    constexpr int NACC = (TM * TN == 1) ? 2 : 1;
+    constexpr int NACC = 1;   // MFMAs that add to the same block issue back to back at the full rate (measured)
     v16f acc[NACC][TM][TN];
 #pragma unroll
     for (int a = 0; a < NACC; a++)
@@ -294,41 +294,17 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
         });
     };
 
-    int phase = 0;                    // stage buffer of the next stage to multiply
-    for (;;) {
-        // ---- one piece: the stages of this run that belong to tile c_tile ----
-        const int piece_len = min(S - c_it, left);
-        const bool whole = c_it == 0 && piece_len == S;
-        int todo = piece_len;
-        // the stage buffers take turns; the loop is unrolled over them and entered where the last piece left off
-        bool more = true;
-        while (more) {
-            switch (phase) {
-                case 0:
-                    stage(std::integral_constant<int, 0>{});
-                    if (--todo == 0) { phase = 1; more = false; break; }
-                    [[fallthrough]];
-                case 1:
-                    stage(std::integral_constant<int, 1>{});
-                    if (--todo == 0) { phase = 2; more = false; break; }
-                    [[fallthrough]];
-                case 2:
-                    stage(std::integral_constant<int, 2>{});
-                    if (--todo == 0) { phase = (NS == 3) ? 0 : 3; more = false; break; }
-                    if constexpr (NS == 3) { phase = 0; break; }
-                    [[fallthrough]];
-                default:
-                    if constexpr (NS == 4) {
-                        stage(std::integral_constant<int, 3>{});
-                        phase = 0;
-                        if (--todo == 0) more = false;
-                    }
-                    break;
-            }
-        }
+    // ---- the run, piece by piece: a piece = the stages of this run that belong to one tile ----
+    // The stage buffers take turns in a fixed order, so the loop below is unrolled over them and always
+    // entered at buffer 0; a piece may end behind any stage, and what then has to be done (store the tile
+    // or the piece, move on to the next tile) stands behind each of the NS stages.  One loop, no way into
+    // its middle: the accumulators stay in the registers they are in.
+    int piece_len = min(S - c_it, left);
+    bool whole = c_it == 0 && piece_len == S;
+    int todo = piece_len;
+    // the piece of c_tile that this run holds has been multiplied; true when that was the run's last
+    auto piece_end = [&]() __attribute__((always_inline)) -> bool {
         left -= piece_len;
-
-        if constexpr (NACC == 2) acc[0][0][0] += acc[1][0][0];
         if (whole) {
             store_tile<A_KIN, B_KIN, TM, TN, false>(acc[0], p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
         } else {
@@ -338,16 +314,32 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
             if (n_rec == 0) rec_tile0 = c_tile; else rec_tile1 = c_tile;
             n_rec++;
         }
-        if (left == 0) break;
+        if (left == 0) return true;
         c_tile++;
-        c_it = 0;
         cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, c_tile);
 #pragma unroll
-        for (int a = 0; a < NACC; a++)
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int jj = 0; jj < TN; jj++) acc[a][i][jj] = (v16f)(0.0f);
+            for (int jj = 0; jj < TN; jj++) acc[0][i][jj] = (v16f)(0.0f);
+        piece_len = min(S, left);
+        whole = piece_len == S;
+        todo = piece_len;
+        return false;
+    };
+    // one stage from buffer SLOT, then whatever the end of a piece asks for; true when the run is over
+    auto step = [&](auto slot_c) __attribute__((always_inline)) -> bool {
+        stage(slot_c);
+        return --todo == 0 && piece_end();
+    };
+    // turn after turn through the buffers, until a step ends the run (written out: with the turn folded into
+    // one expression the compiler's code was 8 % slower)
+    for (;;) {
+        if (step(std::integral_constant<int, 0>{})) break;
+        if (step(std::integral_constant<int, 1>{})) break;
+        if (step(std::integral_constant<int, 2>{})) break;
+        if constexpr (NS == 4) {
+            if (step(std::integral_constant<int, 3>{})) break;
+        }
     }
     // nothing of this wave may still be on its way into LDS when the wave ends, and every piece it stored
     // has arrived in memory before the workgroup is counted
@@ -471,32 +463,37 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
     return w.ptr;
 }
 
-// Fitted to times measured on MI355X (1000 x 780 x K for K = 128 ... 6128, 512 ... 2048-wide squares and panels
-// with K up to 131072, all three layouts), in microseconds:
-//   tile-per-workgroup kernels, at most two 64 x 64 tiles per compute unit: 4.5 + 0.575 per 32-k stage of a tile
-//                                                                           (0.615 for A^T*B), times the tiles per unit
-//   balanced kernel, two workgroups per unit, runs of 64 x 64 tiles: 9.5 + 1.05 per stage of a run;
-//   runs of 128 x 64 tiles (two MFMA blocks per wavefront, fewer other instructions per MFMA, but pieces twice
-//   the size): 14 + 1.75 per stage, ahead from runs of 24 stages on.
-// The balanced kernel's extra fixed time is its pieces crossing the chip through memory; its stages run at 77-79 % of
-// the matrix peak with every unit busy.  Runs shorter than 12 stages consist of pieces only and do not pay unless the
-// tiles leave more than half the chip idle.  Measured gains where it is taken: 4-9 % at 1000 x 777 x 1531, 13 % at
-// 1024 x 1024 x 4096, 3.6 x at 512 x 512 x 8192, 17 x at 256 x 256 x 131072.
+// Fitted to times measured on MI355X (256 ... 2048-wide squares and panels, 1000 x 780 x 1532, K from 64 to
+// 131072, all three layouts), in microseconds, with S = 32-k stages per tile and `run` = stages per workgroup:
+//   tile-per-workgroup kernels, at most two 64 x 64 tiles per compute unit: 4.5 + 0.575 S (0.615 for A^T*B) per
+//                                                                           tile of the busiest unit;
+//   balanced, one workgroup per unit: 0.5 per stage of a run (85 % of the matrix peak with every unit busy)
+//     + 3 where every run is whole tiles, else 7.5 (the pieces cross the chip through memory, and the last
+//     arriver adds them one after the other: 0.4 more for every piece of a tile beyond the second);
+//   balanced, two workgroups per unit: behind the former except where its runs are whole tiles and the
+//     former's are not (512 tiles on 256 units: 18.2 against 19.6).
+// Products with fewer stages than two per unit stay with the tile-per-workgroup kernels (256^3: 7.9 against
+// 9.7).  Measured gains where it is taken: 15 % at 1000 x 777 x 1531, 17 % at 1024^3 and 1536 x 1024 x 1024,
+// 25 % at 512^3, 18 % at 2048 x 512 x 2048, 2.2 x at 128 x 128 x 4096, 17 x at 256 x 256 x 131072 (where it
+// equals the host's split into 128 slices plus the fold: 138 us).
 int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant) {
     if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
     const long long t64 = (long long)((rows + 63) / 64) * ((cols + 63) / 64) * nz;
     if (t64 > 2LL * num_cu || t64 > SK_MAX_TILES) return -1;
-    const long long stages = ((long long)k + 31) / 32;
-    const long long slots = 2LL * num_cu;
-    const long long t128 = (long long)((rows + 127) / 128) * ((cols + 63) / 64) * nz;
-    const long long runs64 = (t64 * stages + slots - 1) / slots, runs128 = (t128 * stages + slots - 1) / slots;
-    if (runs64 < 12 && 2 * t64 >= num_cu) return -1;
-    const bool wide = runs128 >= 24;
-    const double t_balanced = wide ? 14.0 + 1.75 * (double)runs128 : 9.5 + 1.05 * (double)runs64;
+    const long long S = ((long long)k + 31) / 32;
+    const long long units = t64 * S;
+    if (units < 2LL * num_cu) return -1;
+    const long long run1 = (units + num_cu - 1) / num_cu;
+    const bool whole1 = t64 % num_cu == 0;
+    const double pieces = run1 < S ? (double)S / (double)run1 : 0.0;
+    const double t_one = (whole1 ? 3.0 : 7.5 + 0.4 * (pieces > 2.0 ? pieces - 2.0 : 0.0)) + 0.5 * (double)run1;
+    const bool whole2 = t64 % (2LL * num_cu) == 0;
+    const double t_two = whole2 ? 3.5 + 0.92 * (double)(units / (2LL * num_cu)) : 1e300;
     const double per_unit = (double)((t64 + num_cu - 1) / num_cu);
-    const double t_tiles = 4.5 + (variant == GEMM_T1 ? 0.615 : 0.575) * (double)stages * per_unit;
+    const double t_tiles = 4.5 + (variant == GEMM_T1 ? 0.615 : 0.575) * (double)S * per_unit;
+    const double t_balanced = t_two < t_one ? t_two : t_one;
     if (t_balanced > 0.97 * t_tiles) return -1;
-    return wide ? TILE_SK_128x64_O2 : TILE_SK_64x64_O2;
+    return t_two < t_one ? TILE_SK_64x64_O2 : TILE_SK_64x64;
 }
 
 hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream) {

@@ -182,17 +182,16 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 1024, 1024, 64, 64) == 24 and ct(v, 4096, 4096, 1, 60) == 24 and ct(v, 2048, 256, 64, 64) == 24
         assert ct(v, 1024, 1024, 64, 56) != 24 and ct(v, 1024, 1000, 64, 64) != 24 and ct(v, 1024, 1024, 1, 64) != 24
         assert ct(v, 130, 1024, 64, 64) != 24 and ct(v, 1024, 1024, 64, 68) != 24
-    # Few tiles and a long K: the balanced kernel (22 = 64x64, 23 = 128x64, two workgroups per unit) where its
-    # estimated time is ahead; 128x64 once its runs are 24 stages long
+    # At most two 64x64 tiles per compute unit and at least two 32-k stages per unit: the balanced kernel where its
+    # estimated time is ahead (18 = one workgroup per unit; 22 = two, where only that makes the runs whole tiles)
     for v in (NN, T1, T2):
-        assert ct(v, 1000, 780, 1, 1532) == 22                  # 208 tiles x 48 stages over 512 workgroups: runs of 19.5
-        assert ct(v, 256, 256, 1, 131072) == 23                 # the tall-K weight gradient through the unsplit entry
-        assert ct(v, 1024, 1024, 1, 4096) == 23 and ct(v, 512, 512, 1, 8192) == 22
-        assert ct(v, 1000, 780, 1, 6128) == 23 and ct(v, 1000, 780, 1, 3064) == 22
-    assert ct(NN, 1000, 780, 1, 1024) == 7 + P == ct(T2, 1000, 780, 1, 1024)   # a shorter K: one paired 64x64 tile per workgroup
-    assert ct(NN, 1024, 1024, 1, 1024) == 7 + P and ct(T1, 1024, 1024, 1, 1024) == 17   # ... or direct-to-LDS for A^T*B
-    assert ct(NN, 768, 768, 1, 768) == 7 + P                    # runs of 7 stages would be pieces only
-    assert ct(NN, 1000, 780, 2, 760) == 22                      # a batch of two ragged products is balanced as one
+        assert ct(v, 1000, 780, 1, 1532) == 18                  # 208 tiles x 48 stages over 256 workgroups: runs of 39
+        assert ct(v, 256, 256, 1, 131072) == 18                 # the tall-K weight gradient through the unsplit entry
+        assert ct(v, 1024, 1024, 1, 4096) == 18 and ct(v, 512, 512, 1, 8192) == 18
+        assert ct(v, 1024, 1024, 1, 1024) == 18 and ct(v, 768, 768, 1, 768) == 18 and ct(v, 512, 512, 1, 512) == 18
+        assert ct(v, 2048, 1024, 1, 512) == 22                  # 512 tiles: one whole tile for each of 512 workgroups
+        assert ct(v, 256, 256, 1, 256) == 17 and ct(v, 512, 512, 1, 64) == 17   # too few stages to share out
+    assert ct(NN, 1000, 780, 2, 760) == 18                      # a batch of two ragged products is balanced as one
     assert ct(NN, 257, 388, 36, 129) == 1                       # batch of small ragged products: 64x64
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)

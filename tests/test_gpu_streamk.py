@@ -68,8 +68,8 @@ def test_runs_that_start_and_end_inside_tiles_bitwise(gpu, variant, tile):
 @pytest.mark.parametrize("variant", [NN, T1, T2])
 def test_the_automatic_choice_takes_it_and_stays_within_tolerance(gpu, variant):
     # the chooser sends these through the balanced kernel (pinned on the CPU in test_c_abi_boundary)
-    assert gpu.choose_tile(variant, 1000, 780, 1, 1532) == 22 and gpu.choose_tile(variant, 256, 256, 1, 8192) == 22
-    assert gpu.choose_tile(variant, 512, 500, 1, 12000) == 23
+    assert gpu.choose_tile(variant, 1000, 780, 1, 1532) == 18 and gpu.choose_tile(variant, 256, 256, 1, 8192) == 18
+    assert gpu.choose_tile(variant, 512, 500, 1, 12000) == 18
     rng = np.random.default_rng(60 + variant)
     for (N, M, K), dist in (((1000, 777, 1531), "uniform"), ((256, 256, 8192), "normal"), ((512, 500, 11999), "normal")):
         A, B = logical_operands(variant, rng, N, M, K, dist=dist)
