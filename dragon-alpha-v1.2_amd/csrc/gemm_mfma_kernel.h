@@ -523,6 +523,27 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[TM][TN], const float* as, 
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
 }
 
+// The same for a tile's last stage, of which only `k_here` k exist from this group on (>= 1): the steps
+// whose k lie beyond for both lane halves are left out (their operands would be zeros).
+template <bool A_KIN, bool B_KIN, int TM, int TN, int BM, int BN, int KT>
+__device__ __forceinline__ void mma_group_upto(v16f (&acc)[TM][TN], const float* as, const float* bs, int wm,
+                                               int wn, int g, int r, int h, int k_here) {
+    float fa[TM][4], fb[TN][4];
+    if constexpr (A_KIN) read_frag_kinner<TM, KT>(fa, as, wm * TM * 32, g, r, h);
+    else                 read_frag_kouter<TM, BM>(fa, as, wm * TM * 32, g, r, h);
+    if constexpr (B_KIN) read_frag_kinner<TN, KT>(fb, bs, wn * TN * 32, g, r, h);
+    else                 read_frag_kouter<TN, BN>(fb, bs, wn * TN * 32, g, r, h);
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        if (q < k_here) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
+        }
+}
+
 // ---------------------------------------------------------------------------
 // The kernel
 //   A_KIN / B_KIN : operand is K-inner
@@ -748,9 +769,20 @@ void gemm_f32_mfma(const GemmParams p) {
             __builtin_amdgcn_sched_barrier(0);
             const float* as = LDS_BY_POINTER ? As_ptr[b] : As[b];
             const float* bs = LDS_BY_POINTER ? Bs_ptr[b] : Bs[b];
+            // A tile's last stage: only the k that exist (K = 129 ends one k into its ninth stage of 16).  For the
+            // single-block wavefronts only: in the larger tiles the second form of the matrix work costs registers
+            // (the 128 x 128 paired kernels spilled some 200 with it), and a short K is not their business.
+            if (TM * TN == 1 && !CONV && last) {
+                const int k_stage = min(cur.ka_lim, cur.kb_lim) - (cur.k0 + it * KT);
 #pragma unroll
-            for (int g = 0; g < KT / 8; g++)
-                mma_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(acc, as, bs, wm, wn, g, r, h);
+                for (int g = 0; g < KT / 8; g++)
+                    if (g * 8 < k_stage)
+                        mma_group_upto<A_KIN, B_KIN, TM, TN, BM, BN, KT>(acc, as, bs, wm, wn, g, r, h, k_stage - g * 8);
+            } else {
+#pragma unroll
+                for (int g = 0; g < KT / 8; g++)
+                    mma_group<A_KIN, B_KIN, TM, TN, BM, BN, KT>(acc, as, bs, wm, wn, g, r, h);
+            }
             if (fetched) {
                 // one wait for all of the stage's loads (issued a whole stage of matrix work ago) instead
                 // of one per staging register: vmcnt(0), the other counters left alone
