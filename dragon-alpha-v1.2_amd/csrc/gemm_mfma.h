@@ -94,6 +94,10 @@ struct GemmParams {
     // filled by the launcher of the band kernel (gemm_launch_band): a band's tiles_n column tiles are dealt
     // out in bd_chunks runs of bd_chunk_tiles
     int bd_chunks, bd_chunk_tiles;
+    // filled by gemm_rim_applies for the 64 x 64 kernels with a rim (see rim_job in gemm_mfma_kernel.h): the last
+    // rim_rows rows and rim_cols columns of C (0..4 each) are computed by the launch's first rim_wgs workgroups,
+    // the tiles cover the rest
+    int rim_rows, rim_cols, rim_wgs;
 };
 void gemm_fill_tile_divisors(GemmParams& p);
 void gemm_magic_divisor(unsigned d, unsigned& mul, unsigned& shift);
@@ -101,6 +105,10 @@ void gemm_magic_divisor(unsigned d, unsigned& mul, unsigned& shift);
 // Compute units of the current device, cached per device; 0 when no device answers (the launchers then
 // return hipErrorNoDevice).
 int gemm_device_num_cu();
+// True where C's extent is 1..4 rows and / or columns past a multiple of 64 and leaving those to the rim's
+// workgroups saves at least an eighth of the 64 x 64 tiles (and K is short enough for the rim's serial
+// walk along it); fills p.rim_rows / p.rim_cols.
+bool gemm_rim_applies(GemmParams& p);
 // The kernels address an operand tile with 32-bit byte offsets from the tile's origin: up to 256 rows
 // (or k) of pitch.  False when a leading stride is too long for that; the entry points reject such calls.
 bool gemm_pitches_addressable(const GemmParams& p);

@@ -51,6 +51,20 @@ bool gemm_paired_form_fits(bool a_k_inner, bool b_k_inner, const GemmParams& p) 
     return a_span < 0x7fffffffLL && b_span < 0x7fffffffLL;
 }
 
+bool gemm_rim_applies(GemmParams& p) {
+    p.rim_rows = p.rim_cols = p.rim_wgs = 0;
+    if (p.split || p.k_total > 256) return false;
+    const int rr = p.rows % 64, rc = p.cols % 64;
+    const bool use_r = rr >= 1 && rr <= 4 && p.rows > 64, use_c = rc >= 1 && rc <= 4 && p.cols > 64;
+    if (!use_r && !use_c) return false;
+    const long long before = (long long)((p.rows + 63) / 64) * ((p.cols + 63) / 64);
+    const long long after = (long long)((p.rows - (use_r ? rr : 0) + 63) / 64) * ((p.cols - (use_c ? rc : 0) + 63) / 64);
+    if (after * 8 > before * 7) return false;
+    p.rim_rows = use_r ? rr : 0;
+    p.rim_cols = use_c ? rc : 0;
+    return true;
+}
+
 // a test and tuning hook: a setting of the calling thread only
 static thread_local int t_forced_tile = TILE_AUTO;
 void gemm_force_tile(int tile) { t_forced_tile = tile; }

@@ -140,10 +140,10 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
 // which every workgroup has a tile are walked in the XCD-contiguous numbering; the tiles of the last,
 // partial round are dealt by the hardware's own workgroup id instead, which spreads them evenly over
 // the XCDs and their compute units (in the contiguous numbering they would all land on the first XCDs).
-__device__ __forceinline__ int next_tile(int lid, int G, int full_end, int total) {
+__device__ __forceinline__ int next_tile(int lid, int G, int full_end, int total, int block) {
     if (lid + G < full_end) return lid + G;
     if (lid >= full_end) return -1;                       // that was the extra tile
-    const int extra = full_end + (int)blockIdx.x;
+    const int extra = full_end + block;
     return extra < total ? extra : -1;
 }
 
@@ -545,6 +545,118 @@ __device__ __forceinline__ void mma_group_upto(v16f (&acc)[TM][TN], const float*
 }
 
 // ---------------------------------------------------------------------------
+// The rim: the last 1..4 rows and / or columns of a C whose extent is that much past a multiple of
+// the tile.  A whole row or column of tiles for them would be all but empty (257 x 385 in 64 x 64
+// tiles: 35 tiles where 24 hold all but one row and one column); the reference carves such edges
+// down to tiles of 4 (MM/matMul.cuh:24-43) and has kernels for a C of 4 columns
+// (MM/matMul_sernel.cuh:17-30).  Here the tiles cover the part of C that fills them, and the first
+// rim_wgs workgroups of the same launch compute the rim with plain FMAs, straight from memory: the
+// rim's matrix work is tiny (a few rows), what it needs is every byte of one operand once more, and
+// that comes out of the L2 while the tiles run.
+// One job = 64 outputs along the rim x up to 4 across it: the workgroup's four wavefronts each take a
+// quarter of K (contiguous, so a lane that walks along a row of its own stays on a cache line), the
+// quarters meet in LDS and are added in k order.  Row jobs: rows R0 .. R0+rr-1, 64 columns; column
+// jobs: 64 rows below R0, columns C0 .. C0+rc-1.
+// Four consecutive k of one operand line: a K-inner line (k contiguous, padded to a multiple of 4 in memory)
+// in one 16-byte load, a K-outer one (k is the row) in four loads that stop where the operand ends.
+template <bool KIN>
+__device__ __forceinline__ v4f rim_load4(const float* line, size_t sk, int k, int k_end) {
+    if constexpr (KIN) {
+        return *(const v4f*)(line + k);
+    } else {
+        // every load is made (of the operand's last k where its own lies beyond) and the value dropped
+        // afterwards: no branch around a load, so that they all are on their way together
+        const int last = k_end - 1;
+        v4f v;
+        v.x = line[(size_t)min(k + 0, last) * sk];
+        v.y = line[(size_t)min(k + 1, last) * sk];
+        v.z = line[(size_t)min(k + 2, last) * sk];
+        v.w = line[(size_t)min(k + 3, last) * sk];
+        v.y = k + 1 < k_end ? v.y : 0.0f;
+        v.z = k + 2 < k_end ? v.z : 0.0f;
+        v.w = k + 3 < k_end ? v.w : 0.0f;
+        return v;
+    }
+}
+
+// acc[x] += sum over k in [k0, k1) of walk(k) * fixed[x](k): `walk` is the lane's own operand line (64 lanes,
+// 64 lines), the `fixed` ones are the same for every lane.  16 k per turn, the loads ahead of the FMAs.
+template <bool WALK_KIN, bool FIXED_KIN>
+__device__ __forceinline__ void rim_dot(float (&acc)[4], const float* walk, size_t w_sk, const float* const (&fixed)[4],
+                                        size_t f_sk, int k0, int k1, int k_end) {
+#pragma unroll 4
+    for (int k = k0; k < k1; k += 4) {
+        const v4f w = rim_load4<WALK_KIN>(walk, w_sk, k, k_end);
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+            const v4f f = rim_load4<FIXED_KIN>(fixed[x], f_sk, k, k_end);
+            acc[x] = fmaf(w.x, f.x, acc[x]);
+            acc[x] = fmaf(w.y, f.y, acc[x]);
+            acc[x] = fmaf(w.z, f.z, acc[x]);
+            acc[x] = fmaf(w.w, f.w, acc[x]);
+        }
+    }
+}
+
+template <bool A_KIN, bool B_KIN, bool BIAS>
+__device__ __forceinline__ void rim_job(const GemmParams& p, float* lds, int job) {
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int R0 = p.rows, C0 = p.cols;                    // the tiles' part of C
+    const int rr = p.rim_rows, rc = p.rim_cols;
+    const int row_jobs = rr > 0 ? (C0 + rc + 63) / 64 : 0, col_jobs = rc > 0 ? (R0 + 63) / 64 : 0;
+    const int per_z = row_jobs + col_jobs;
+    const int z = job / per_z;
+    if (z >= p.nz) return;                                 // the job count is rounded up to whole groups of 8
+    int seg = job - z * per_z;
+    const bool row_job = seg < row_jobs;
+    if (!row_job) seg -= row_jobs;
+    const float* A = p.A + (size_t)z * p.sA;
+    const float* B = p.B + (size_t)z * p.sB;
+    float* C = p.C + (size_t)z * p.sC;
+    const size_t a_si = A_KIN ? p.lda : 1, a_sk = A_KIN ? 1 : p.lda;     // A(i, k) = A[i * a_si + k * a_sk]
+    const size_t b_sk = B_KIN ? 1 : p.ldb, b_sj = B_KIN ? p.ldb : 1;     // B(k, j) = B[k * b_sk + j * b_sj]
+    const int a_rows = A_KIN ? p.a_outer : p.a_inner, b_cols = B_KIN ? p.b_outer : p.b_inner;   // that exist in memory
+    // the k both operands have; a K-inner operand's lines are padded with zeros to a multiple of 4
+    const int K = min(p.k_total, min(A_KIN ? p.a_inner : p.a_outer, B_KIN ? p.b_inner : p.b_outer));
+    const int kq = (K + 15) / 16 * 4;                      // a quarter of K, in whole groups of 4
+    const int k0 = wave * kq, k1 = min(K, k0 + kq);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    bool ok;
+    if (row_job) {      // rows R0 .. R0+rr-1 of A against the lane's column of B
+        const int j = seg * 64 + lane;
+        ok = j < b_cols;
+        const float* const fixed[4] = {A + (size_t)min(R0, a_rows - 1) * a_si, A + (size_t)min(R0 + (1 < rr ? 1 : 0), a_rows - 1) * a_si,
+                                       A + (size_t)min(R0 + (2 < rr ? 2 : 0), a_rows - 1) * a_si,
+                                       A + (size_t)min(R0 + (3 < rr ? 3 : 0), a_rows - 1) * a_si};
+        rim_dot<B_KIN, A_KIN>(acc, B + (ok ? (size_t)j * b_sj : 0), b_sk, fixed, a_sk, k0, k1, K);
+    } else {            // the lane's row of A against columns C0 .. C0+rc-1 of B
+        const int i = seg * 64 + lane;
+        ok = i < R0 && i < a_rows;
+        const float* const fixed[4] = {B + (size_t)min(C0, b_cols - 1) * b_sj, B + (size_t)min(C0 + (1 < rc ? 1 : 0), b_cols - 1) * b_sj,
+                                       B + (size_t)min(C0 + (2 < rc ? 2 : 0), b_cols - 1) * b_sj,
+                                       B + (size_t)min(C0 + (3 < rc ? 3 : 0), b_cols - 1) * b_sj};
+        rim_dot<A_KIN, B_KIN>(acc, A + (ok ? (size_t)i * a_si : 0), a_sk, fixed, b_sk, k0, k1, K);
+    }
+#pragma unroll
+    for (int x = 0; x < 4; x++) lds[(wave * 4 + x) * 64 + lane] = acc[x];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+        const float sum = ((lds[(0 * 4 + x) * 64 + lane] + lds[(1 * 4 + x) * 64 + lane]) + lds[(2 * 4 + x) * 64 + lane]) +
+                          lds[(3 * 4 + x) * 64 + lane];
+        // a row of A or a column of B that does not exist in memory (the operand's own padding) gives zeros
+        const int i = row_job ? R0 + x : seg * 64 + lane, j = row_job ? seg * 64 + lane : C0 + x;
+        const bool inside = row_job ? (x < rr && j < C0 + rc) : (x < rc && i < R0);
+        float value = (ok && (row_job ? i < a_rows : j < b_cols)) ? sum : 0.0f;
+        if constexpr (BIAS) {   // as the tiles' epilogue adds it (see store_tile_rows)
+            if (inside && i < p.bias_rows) value = (value + (j < p.bias_width ? p.bias[j] : 0.0f)) + 0.0f;
+        }
+        if (inside) C[(size_t)i * p.ldc + j] = value;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // The kernel
 //   A_KIN / B_KIN : operand is K-inner
 //   WM x WN       : wavefront grid in the workgroup (WM*WN == 4)
@@ -626,7 +738,7 @@ constexpr int target_occupancy() {
 }
 
 template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, bool BIAS, bool CONV = false,
-          bool PAIRED = false>
+          bool PAIRED = false, bool RIM = false>
 __global__ __launch_bounds__(NTHREADS, (target_occupancy<A_KIN, B_KIN, WM * TM * 32, WN * TN * 32, KT>()))
 void gemm_f32_mfma(const GemmParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -656,8 +768,18 @@ void gemm_f32_mfma(const GemmParams p) {
     const int a_step4 = (int)(a_step * 4), b_step4 = (int)(b_step * 4);
 
     const int total = p.tiles_m * p.tiles_n * p.nz;
-    const int G = gridDim.x;
-    int lid = xcd_contiguous_id(blockIdx.x, G);   // G <= total, so lid is a valid tile
+    int block = blockIdx.x, G = gridDim.x;
+    if constexpr (RIM) {
+        // the launch's first workgroups compute the rim of C (see rim_job); the others are the tiles'
+        static_assert(LoadA::LDS_FLOATS >= 1024, "the rim's partial sums take 1024 floats of LDS");
+        if (block < p.rim_wgs) {
+            rim_job<A_KIN, B_KIN, BIAS>(p, &As[0][0], block);
+            return;
+        }
+        block -= p.rim_wgs;
+        G -= p.rim_wgs;
+    }
+    int lid = xcd_contiguous_id(block, G);   // G <= total, so lid is a valid tile
     const int full_end = (total / G) * G;
 
     TileCtx cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, lid);
@@ -698,7 +820,7 @@ void gemm_f32_mfma(const GemmParams p) {
     int buf = 0;
 
     for (;;) {
-        const int next_lid = next_tile(lid, G, full_end, total);
+        const int next_lid = next_tile(lid, G, full_end, total, block);
         const bool has_next = next_lid >= 0;
         TileCtx nxt = cur;
         const float* a_ptr = cur.a_ptr;
@@ -988,10 +1110,19 @@ static int resident_workgroups(std::atomic<int>& cache, Kernel kernel) {
 }
 
 template <bool A_KIN, bool B_KIN, bool BIAS, int WM, int WN, int TM, int TN, int KT, bool CONV = false,
-          bool PAIRED = false>
+          bool PAIRED = false, bool RIM = false>
 static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    auto kernel = gemm_f32_mfma<A_KIN, B_KIN, WM, WN, TM, TN, KT, BIAS, CONV, PAIRED>;
+    auto kernel = gemm_f32_mfma<A_KIN, B_KIN, WM, WN, TM, TN, KT, BIAS, CONV, PAIRED, RIM>;
+    if constexpr (RIM) {
+        // the tiles take the part of C that fills them; the rim's jobs (64 outputs along it each) go first
+        // in the grid, in whole groups of 8 so that the tiles' workgroups keep their places on the XCDs
+        static_assert(BM == 64 && BN == 64, "the rim's jobs are 64 outputs long");
+        const int row_jobs = p.rim_rows > 0 ? (p.cols + 63) / 64 : 0, col_jobs = p.rim_cols > 0 ? (p.rows - p.rim_rows + 63) / 64 : 0;
+        p.rows -= p.rim_rows;
+        p.cols -= p.rim_cols;
+        p.rim_wgs = (int)((((long long)(row_jobs + col_jobs) * p.nz) + 7) / 8 * 8);
+    }
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long total = (long long)p.tiles_m * p.tiles_n * p.nz;
@@ -1006,7 +1137,7 @@ static hipError_t launch_cfg(GemmParams p, hipStream_t stream) {
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return hipErrorNoDevice;
     const long long slots = (long long)num_cu * resident_per_cu;
-    const long long grid = total < slots ? total : slots;
+    const long long grid = (total < slots ? total : slots) + (RIM ? p.rim_wgs : 0);
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
 }
@@ -1017,8 +1148,13 @@ static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stre
     switch (tile & ~TILE_PAIRED) {
         case TILE_128x128: return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV, true>(p, stream)
                                          : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 16, CONV>(p, stream);
-        case TILE_64x64:   return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, CONV, true>(p, stream)
-                                         : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, CONV>(p, stream);
+        case TILE_64x64:
+            if constexpr (!CONV) {
+                GemmParams q = p;
+                if (!paired && gemm_rim_applies(q)) return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, CONV, false, true>(q, stream);
+            }
+            return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, CONV, true>(p, stream)
+                          : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 16, CONV>(p, stream);
         case TILE_256x64:  return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 4, 1, 2, 2, 16, CONV, true>(p, stream)
                                          : launch_cfg<A_KIN, B_KIN, BIAS, 4, 1, 2, 2, 16, CONV>(p, stream);
         case TILE_64x256:  return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 1, 4, 2, 2, 16, CONV, true>(p, stream)
@@ -1029,8 +1165,13 @@ static hipError_t launch_variant(const GemmParams& p, int tile, hipStream_t stre
                                          : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 16, CONV>(p, stream);
         case TILE_128x128_K32: return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 32, CONV, true>(p, stream)
                                              : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 2, 32, CONV>(p, stream);
-        case TILE_64x64_K32:   return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, CONV, true>(p, stream)
-                                             : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, CONV>(p, stream);
+        case TILE_64x64_K32:
+            if constexpr (!CONV) {
+                GemmParams q = p;
+                if (!paired && gemm_rim_applies(q)) return launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, CONV, false, true>(q, stream);
+            }
+            return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, CONV, true>(p, stream)
+                          : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 1, 32, CONV>(p, stream);
         case TILE_128x64_K32:  return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 32, CONV, true>(p, stream)
                                              : launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 2, 1, 32, CONV>(p, stream);
         case TILE_64x128_K32:  return paired ? launch_cfg<A_KIN, B_KIN, BIAS, 2, 2, 1, 2, 32, CONV, true>(p, stream)
