@@ -128,6 +128,14 @@ __device__ __forceinline__ void static_for(F&& f) {
 // expcnt 6:4 and lgkmcnt 11:8 left at "no wait")
 constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
+// The value as if it had just been read: the compiler works out what depends on it HERE instead of once
+// at the top of the kernel and keeping the results in registers all the way (the lanes' row offsets of a
+// tile's loads, needed once per tile: kept live, they were what the 128 x 128 kernels spilled).
+__device__ __forceinline__ int fresh(int v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with a private L2.
 // Re-number them so that one XCD owns a contiguous range of logical ids.
 __device__ __forceinline__ int xcd_contiguous_id(int pid, int nwg) {
@@ -435,9 +443,9 @@ __device__ __forceinline__ void read_frag_kouter(float (&frag)[T][4], const floa
 // The stores go through a buffer descriptor whose base is the tile's origin: a lane outside C gets
 // an out-of-range offset and the hardware drops its store, so the whole epilogue is straight-line
 // code -- no branch per store and 32-bit offset arithmetic only.
-template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS, bool CHECK_ROWS>
-__device__ __forceinline__ void store_tile_rows(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
-                                                int col0, float* c_ptr, int wm, int wn, int r, int h) {
+template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
+                                           int col0, float* c_ptr, int wm, int wn, int r, int h) {
     constexpr int NT_STORE = 2;   // cache policy bit "nt": C is written once and not read back here
     float bias_v[TN];
     if constexpr (BIAS) {
@@ -447,14 +455,16 @@ __device__ __forceinline__ void store_tile_rows(const v16f (&acc)[TM][TN], const
             bias_v[j] = col < p.bias_width ? p.bias[col] : 0.0f;
         }
     }
-    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(c_ptr + (size_t)row0 * p.ldc + col0), 0, RSRC_RECORDS, RSRC_FLAGS);
-    const int ldc4 = p.ldc * 4;
     // A store's address = tile origin (descriptor) + lane part (vector offset: the lane's first row
-    // and its column) + row part (scalar offset: a compile-time row count times the row pitch).
-    // Only the lane part is range-checked by the hardware, so "outside C" is expressed there.
-    const int lane_row = wm * TM * 32 + (A_KIN ? 4 * h : TM * 4 * h);
+    // and its column) + row part (scalar offset: a compile-time row count times the row pitch).  The
+    // hardware checks vector + scalar offset against the descriptor's size, which ends behind C's last
+    // row: the rows of the tile beyond C are dropped there, with no instruction spent on them; a lane
+    // whose columns lie beyond C carries an offset that is out of range from the start.
+    const int ldc4 = p.ldc * 4;
     const int rows_left = p.rows - row0, cols_left = p.cols - col0;
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(c_ptr + (size_t)row0 * p.ldc + col0), 0, rows_left > 0 ? (rows_left > 256 ? 256 : rows_left) * ldc4 : 0, RSRC_FLAGS);   // a tile has at most 256 rows
+    const int lane_row = wm * TM * 32 + (A_KIN ? 4 * h : TM * 4 * h);
     const int lcol = wn * TN * 32 + TN * r;
     const int lane_off = (lcol < cols_left) ? lane_row * ldc4 + lcol * 4 : OOB_OFFSET;
 #pragma unroll
@@ -462,7 +472,6 @@ __device__ __forceinline__ void store_tile_rows(const v16f (&acc)[TM][TN], const
 #pragma unroll
         for (int e = 0; e < 16; e++) {
             const int crow = A_KIN ? (i * 32 + 8 * (e / 4) + (e % 4)) : (TM * (8 * (e / 4) + (e % 4)) + i);
-            const bool row_ok = !CHECK_ROWS || lane_row < rows_left - crow;
             const int row_soff = crow * ldc4;
             float out[TN];
 #pragma unroll
@@ -471,38 +480,19 @@ __device__ __forceinline__ void store_tile_rows(const v16f (&acc)[TM][TN], const
                 if constexpr (BIAS)
                     if (row0 + lane_row + crow < p.bias_rows) out[j] = (out[j] + bias_v[j]) + 0.0f;
             }
-            const int off = row_ok ? lane_off : OOB_OFFSET;
             if constexpr (TN == 1) {
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[0]), rsrc, off, row_soff,
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out[0]), rsrc, lane_off, row_soff,
                                                       NT_STORE);
             } else if constexpr (TN == 2) {
                 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
                 const v2f v = {out[0], out[1]};
-                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rsrc, off, row_soff, NT_STORE);
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rsrc, lane_off, row_soff, NT_STORE);
             } else {
                 const v4f v = {out[0], out[1], out[2], out[3]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc, off, row_soff, NT_STORE);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc, lane_off, row_soff, NT_STORE);
             }
         }
     }
-
-}
-
-// A wavefront whose 32*TM rows all lie inside C (the same answer for all its lanes) skips the row test
-// per store: two vector instructions less for each of the 16*TM stores of an interior tile.  Only
-// where the second copy of the epilogue costs no resident wavefront: the four-block wavefronts, whose
-// accumulators pin the register count anyway, and not with the bias row (those kernels spilled).
-template <bool A_KIN, bool B_KIN, int TM, int TN, bool BIAS>
-__device__ __forceinline__ void store_tile(const v16f (&acc)[TM][TN], const GemmParams& p, int row0,
-                                           int col0, float* c_ptr, int wm, int wn, int r, int h) {
-    constexpr bool FAST_PATH = !BIAS && TM * TN == 4;
-    if constexpr (FAST_PATH) {
-        if (p.rows - row0 >= (wm + 1) * TM * 32) {
-            store_tile_rows<A_KIN, B_KIN, TM, TN, BIAS, false>(acc, p, row0, col0, c_ptr, wm, wn, r, h);
-            return;
-        }
-    }
-    store_tile_rows<A_KIN, B_KIN, TM, TN, BIAS, true>(acc, p, row0, col0, c_ptr, wm, wn, r, h);
 }
 
 // One group of 8 k: fragments from LDS, then 4 MFMA steps over the wave's TM x TN blocks.
@@ -877,8 +867,8 @@ void gemm_f32_mfma(const GemmParams p) {
             } else if (has_next) {       // first stage of the next tile -> registers
                 nxt = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, next_lid);
                 if constexpr (CONV) la.init_conv(t, nxt.row0, p.a_outer, p);
-                else la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
-                lb.init(t, nxt.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+                else la.init(t, nxt.row0, A_KIN ? p.a_outer : p.a_inner, fresh(p.lda));
+                lb.init(t, nxt.col0, B_KIN ? p.b_outer : p.b_inner, fresh(p.ldb));
                 if constexpr (CONV) {
                     if (cv_walk) la.load_conv_tap(ra, nxt.a_ptr, 0, 0, 0, p);
                     else la.load_conv(ra, nxt.a_ptr, nxt.ka_lim - nxt.k0, nxt.k0, p);
