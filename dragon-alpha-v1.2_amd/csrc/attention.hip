@@ -54,13 +54,18 @@ struct AttnParams {
     long long v_n, v_h; int v_l;
     long long y_n, y_h; int y_l;
     float c;                     // scale * log2(e): the exponentials are base 2
+    const float* M;              // optional factor on the probabilities, M[.., query, key]
+    long long m_b; int m_l;      // its element strides: (image, head) slice (0: one mask for all), row
 };
 
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
 // DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32), 2 (d <= 64) or 4 (d <= 128);
-// KB = 32-key blocks per step
-template <int DB, int KB>
+// KB = 32-key blocks per step;
+// MASK: the probabilities are multiplied by M[query, key] AFTER the softmax, as the block's mask unit does
+// (ChannelMHA.java:75-76: P = softmax(...); P = mask.forward(P)): the sum that normalises them runs over the
+// unmasked terms, the second product takes the masked ones.
+template <int DB, int KB, bool MASK>
 __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnParams p) {
     constexpr int AK = KB * 32;            // keys per step
     constexpr int DW = DB * 32;            // tile width in floats
@@ -130,6 +135,22 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
         }
     };
 
+    // ---- this lane's row of the mask: keys 32kb + 8g + 4h .. +3 of a step in one 16-byte load; zeros beyond
+    // the row's end (the descriptor ends there) and for a query that does not exist ----
+    const float* Mrow = MASK ? p.M + (size_t)bh * p.m_b + (size_t)(q < p.nq ? q : 0) * p.m_l : nullptr;
+    v4f mreg[MASK ? KB * 4 : 1];
+    auto fetch_mask = [&](int key0) {
+        if constexpr (MASK) {
+            const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(
+                (void*)(Mrow + key0), 0, q < p.nq ? (p.m_l - key0) * 4 : 0, RSRC_FLAGS);   // to the end of the row
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    mreg[kb * 4 + g] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rm, (32 * kb + 8 * g + 4 * h) * 4, 0, 0));
+        }
+    };
+
     v16f o[DB];
 #pragma unroll
     for (int b = 0; b < DB; b++) o[b] = (v16f)(0.0f);
@@ -143,6 +164,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
     for (int it = 0; it < steps; it++) {
         const bool more = it + 1 < steps;
         if (more) fetch((it + 1) * AK);
+        fetch_mask(it * AK);      // used behind the first product and the exponentials
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- S^T[key][query] for this step's keys, one 32-key block after the other ----
@@ -195,6 +217,25 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
                 sum += s[kb][v];
             }
         l += sum;
+        if constexpr (MASK) {
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    s[kb][4 * g + 0] *= mreg[kb * 4 + g].x;
+                    s[kb][4 * g + 1] *= mreg[kb * 4 + g].y;
+                    s[kb][4 * g + 2] *= mreg[kb * 4 + g].z;
+                    s[kb][4 * g + 3] *= mreg[kb * 4 + g].w;
+                }
+            if (!more && (p.nk & (AK - 1))) {       // whatever the mask's row holds beyond the last key does not count
+                const int left = p.nk - it * AK;
+#pragma unroll
+                for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        if (32 * kb + 8 * (v / 4) + 4 * h + (v % 4) >= left) s[kb][v] = 0.0f;
+            }
+        }
 
         // ---- Y^T[d][query] += V^T[d][key] * P^T[key][query] ----
         const float* vs = Vs[buf];
@@ -240,15 +281,17 @@ using namespace dragon;
 
 extern "C" {
 
-int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
-                                  int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL, int32_t dK4,
-                                  int32_t dV4, int32_t head_inner, float scale) {
+static int attention_launch(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV, int64_t dMask,
+                            int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL, int32_t dK4, int32_t dV4,
+                            int32_t head_inner, float scale, int32_t mask_pitch, int32_t mask_per_head) {
     if (streams == nullptr || length < 1 || length > 10) return hipErrorInvalidValue;
     if (dQ == 0 || dK == 0 || dV == 0 || dY == 0 || !aligned16(dQ) || !aligned16(dK) || !aligned16(dV) ||
         !aligned16(dY))
         return hipErrorInvalidValue;
     if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 128 ||
         dV4 > 128 || !(scale - scale == 0.0f))   // NaN and the infinities fail the last test
+        return hipErrorInvalidValue;
+    if (dMask != 0 && (!aligned16(dMask) || mask_pitch < VL || (mask_pitch & 3) || (long long)mask_pitch * 4 >= 0x7ffffff0LL))
         return hipErrorInvalidValue;
     // offsets inside one (image, head) slice travel as 32-bit byte offsets
     const long long rowK = head_inner ? (long long)head * dK4 : dK4, rowV = head_inner ? (long long)head * dV4 : dV4;
@@ -258,6 +301,9 @@ int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_
     AttnParams p;
     p.Q = (const float*)(intptr_t)dQ; p.K = (const float*)(intptr_t)dK; p.V = (const float*)(intptr_t)dV;
     p.Y = (float*)(intptr_t)dY;
+    p.M = (const float*)(intptr_t)dMask;
+    p.m_l = mask_pitch;
+    p.m_b = mask_per_head ? (long long)QL * mask_pitch : 0;
     p.head = head; p.nq = QL; p.nk = VL; p.dk4 = dK4; p.dv4 = dV4;
     p.qtiles = (QL + AQ - 1) / AQ;
     if (head_inner) {   // [N, L, head, d]: a row of a head lies head*d apart from the next
@@ -274,10 +320,32 @@ int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_
     p.c = scale * 1.44269504088896340736f;
     hipStream_t s = (hipStream_t)(intptr_t)streams[0];
     const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);
-    if (dK4 <= 32 && dV4 <= 32) hipLaunchKernelGGL((attention_f32_mfma<1, 2>), grid, block, 0, s, p);
-    else if (dK4 <= 64 && dV4 <= 64) hipLaunchKernelGGL((attention_f32_mfma<2, 2>), grid, block, 0, s, p);
-    else hipLaunchKernelGGL((attention_f32_mfma<4, 1>), grid, block, 0, s, p);
+    const int db = (dK4 <= 32 && dV4 <= 32) ? 1 : (dK4 <= 64 && dV4 <= 64) ? 2 : 4;
+    if (dMask == 0) {
+        if (db == 1) hipLaunchKernelGGL((attention_f32_mfma<1, 2, false>), grid, block, 0, s, p);
+        else if (db == 2) hipLaunchKernelGGL((attention_f32_mfma<2, 2, false>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((attention_f32_mfma<4, 1, false>), grid, block, 0, s, p);
+    } else {
+        if (db == 1) hipLaunchKernelGGL((attention_f32_mfma<1, 2, true>), grid, block, 0, s, p);
+        else if (db == 2) hipLaunchKernelGGL((attention_f32_mfma<2, 2, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((attention_f32_mfma<4, 1, true>), grid, block, 0, s, p);
+    }
     return hipGetLastError();
+}
+
+int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
+                                  int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL, int32_t dK4,
+                                  int32_t dV4, int32_t head_inner, float scale) {
+    return attention_launch(streams, length, dQ, dK, dV, 0, dY, N, head, QL, VL, dK4, dV4, head_inner, scale, 0, 0);
+}
+
+int dragon_Cuda_attention_forward_masked(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
+                                         int64_t dMask, int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL,
+                                         int32_t dK4, int32_t dV4, int32_t head_inner, float scale,
+                                         int32_t mask_pitch, int32_t mask_per_head) {
+    if (dMask == 0) return hipErrorInvalidValue;
+    return attention_launch(streams, length, dQ, dK, dV, dMask, dY, N, head, QL, VL, dK4, dV4, head_inner, scale,
+                            mask_pitch, mask_per_head);
 }
 
 }  // extern "C"

@@ -59,8 +59,8 @@ static constexpr int OOB_OFFSET = 0x7ffffff0; // >= num_records: the load return
 static constexpr int RSRC_RECORDS = 0x7ffffff0;
 static constexpr int RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format
 
-// byte_offset is the lane's part (range-checked by the hardware), scalar_offset a wave-uniform part
-// added to it unchecked
+// byte_offset is the lane's part, scalar_offset a wave-uniform part on top of it; the hardware checks
+// their sum against the descriptor's size (measured on gfx950)
 __device__ __forceinline__ v4f buffer_load_f4(const float* base, int byte_offset, int scalar_offset = 0) {
     __amdgpu_buffer_rsrc_t r =
         __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, RSRC_RECORDS, RSRC_FLAGS);

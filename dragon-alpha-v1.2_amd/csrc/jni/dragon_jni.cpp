@@ -338,6 +338,19 @@ JNIEXPORT void JNICALL BMM(attention)(JNIEnv* env, jclass, jlongArray streamArra
                                               head_inner ? 1 : 0, scale));
 }
 
+// ... and `attention_masked(long[] streamArray, int length, long dQ_address, long dK_address, long dV_address,
+// long dMask_address, long dY_address, int N, int head, int QL, int VL, int dK4, int dV4, boolean head_inner,
+// float scale, int mask_pitch, boolean mask_per_head)` for a mask unit that multiplies element by element.
+JNIEXPORT void JNICALL BMM(attention_1masked)(JNIEnv* env, jclass, jlongArray streamArray, jint length, jlong dQ,
+                                              jlong dK, jlong dV, jlong dMask, jlong dY, jint N, jint head, jint QL,
+                                              jint VL, jint dK4, jint dV4, jboolean head_inner, jfloat scale,
+                                              jint mask_pitch, jboolean mask_per_head) {
+    Streams st(env, streamArray, length);
+    if (!st.ok) return;
+    handle(env, dragon_Cuda_attention_forward_masked(st.s, st.n, dQ, dK, dV, dMask, dY, N, head, QL, VL, dK4, dV4,
+                                                     head_inner ? 1 : 0, scale, mask_pitch, mask_per_head ? 1 : 0));
+}
+
 #define DEF_BMM_MMA(jname, cname)                                                                \
     JNIEXPORT void JNICALL BMM(jname)(JNIEnv* env, jclass, jboolean useTexture,                  \
                                       jlongArray streamArray, jint length, jlong dA, jlong dB,   \

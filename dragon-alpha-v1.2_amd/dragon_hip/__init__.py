@@ -387,6 +387,13 @@ class Cuda_attention:
         _check(lib.dragon_Cuda_attention_forward(arr, length, dQ, dK, dV, dY, N, head, QL, VL, dK4, dV4,
                                                  int(head_inner), scale))
 
+    @staticmethod
+    def forward_masked(streams, length, dQ, dK, dV, dMask, dY, N, head, QL, VL, dK4, dV4, head_inner, scale,
+                       mask_pitch, mask_per_head):
+        arr, _ = _stream_array(streams)
+        _check(lib.dragon_Cuda_attention_forward_masked(arr, length, dQ, dK, dV, dMask, dY, N, head, QL, VL, dK4, dV4,
+                                                        int(head_inner), scale, mask_pitch, int(mask_per_head)))
+
 
 class Cuda_expk2:
     """The dimension-swap natives of Cuda_expk2.java."""

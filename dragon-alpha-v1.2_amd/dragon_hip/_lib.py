@@ -40,6 +40,8 @@ SIGNATURES = {
     "dragon_Cuda_function_linear2D": (i32, [i64, f32, i64, f32, i64, i32, i32, i32]),
     "dragon_Cuda_reduce_softmax2D": (i32, [i64, i64, i64, i32, i32, i32, i32, f32]),
     "dragon_Cuda_attention_forward": (i32, [p_i64, i32, i64, i64, i64, i64, i32, i32, i32, i32, i32, i32, i32, f32]),
+    "dragon_Cuda_attention_forward_masked": (i32, [p_i64, i32, i64, i64, i64, i64, i64, i32, i32, i32, i32, i32, i32, i32,
+                                                   f32, i32, i32]),
     "dragon_Cuda_expk2_transpose2D": (i32, [i64, i64, i64, i32, i32, i32, i32, i32]),
     "dragon_Cuda_expk2_transpose3D": (i32, [i64, i64, i64] + [i32] * 9),
     "dragon_Cuda_expk2_transpose4D": (i32, [i64, i64, i64] + [i32] * 11),
@@ -164,6 +166,7 @@ SIGNATURES = {
     "dragon_engine_conv3D_into": (i32, [c_void_p, c_void_p, c_void_p, c_void_p, i32, i32, i32, i32, c_void_p]),
     "dragon_policy_conv3D_GEMM_nstream": (i32, [i32, i32]),
     "dragon_engine_attention": (c_void_p, [c_void_p, c_void_p, c_void_p, c_void_p, i32, f32]),
+    "dragon_engine_attention_masked": (c_void_p, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, i32, f32]),
     "dragon_engine_linear": (c_void_p, [c_void_p, i32, f32, c_void_p, f32]),
     "dragon_engine_softmax": (c_void_p, [c_void_p, i32, c_void_p, i32, f32]),
     "dragon_engine_transpose": (c_void_p, [c_void_p, i32, c_void_p, i32, i32]),

@@ -242,9 +242,12 @@ class Engine:
         h = lib.dragon_engine_softmax(self._h, int(inplace), X._h if X else None, features, scale)
         return X if (inplace and h) else self._wrap(h)
 
-    def attention(self, Q, K, V, head, scale=0.0):
-        """softmax(scale * Q.K^T).V per head in one launch; scale = 0: 1/sqrt(Q.lastDim)."""
+    def attention(self, Q, K, V, head, scale=0.0, mask=None):
+        """softmax(scale * Q.K^T).V per head in one launch; scale = 0: 1/sqrt(Q.lastDim).  mask: a tensor
+        [QL, VL] or [N, head, QL, VL] that multiplies the probabilities after the softmax."""
         hs = [x._h if x is not None else None for x in (Q, K, V)]
+        if mask is not None:
+            return self._wrap(lib.dragon_engine_attention_masked(self._h, hs[0], hs[1], hs[2], mask._h, head, scale))
         return self._wrap(lib.dragon_engine_attention(self._h, hs[0], hs[1], hs[2], head, scale))
 
     def transpose(self, inplace, X, dimIdx1, dimIdx2):

@@ -703,10 +703,15 @@ SyncerPtr CudaFloat32EngineBase::softmax2D(int64_t Y, int64_t X, int field_lengt
     return SyncerPtr(new StreamSyncer(streamPool_.get(), stream));
 }
 SyncerPtr CudaFloat32EngineBase::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL,
-                                           int VL, int dK4, int dV4, bool head_inner, float scale) {
+                                           int VL, int dK4, int dV4, bool head_inner, float scale, int64_t Mask,
+                                           int mask_pitch, bool mask_per_head) {
     std::vector<int64_t> s = streamPool_->getStreamArray(1);
     last_gridZ = 1; last_stream_count = (int)s.size();
     try {
+        if (Mask != 0)
+            cu(dragon_Cuda_attention_forward_masked(s.data(), (int)s.size(), Q, K, V, Mask, Y, N, head, QL, VL, dK4,
+                                                    dV4, head_inner ? 1 : 0, scale, mask_pitch, mask_per_head ? 1 : 0));
+        else
         cu(dragon_Cuda_attention_forward(s.data(), (int)s.size(), Q, K, V, Y, N, head, QL, VL, dK4, dV4,
                                          head_inner ? 1 : 0, scale));
     } catch (...) { streamPool_->returnStreamArray(s); throw; }
@@ -966,7 +971,8 @@ SyncerPtr EngineCore::conv3D_biased(int64_t Y, int OH, int OW, int64_t X, int IH
                                 Bias, lengthv, OC);
 }
 SyncerPtr EngineCore::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL, int VL,
-                                int dK, int dV, bool head_inner, float scale) {
+                                int dK, int dV, bool head_inner, float scale, int64_t Mask, int mask_width,
+                                bool mask_per_head) {
     if (check) {
         if (Y == 0) throw NullPointerException("Tensor Y is null");
         if (Q == 0) throw NullPointerException("Tensor Q is null");
@@ -984,7 +990,11 @@ SyncerPtr EngineCore::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int 
         if (pad4(dK) > 128 || pad4(dV) > 128)
             throw IllegalArgumentException("head dimensions { got " + s(dK) + ", " + s(dV) + " } must <= 128");
     }
-    return base_->attention(Y, Q, K, V, N, head, QL, VL, pad4(dK), pad4(dV), head_inner, scale);
+    if (check && Mask != 0 && mask_width != VL)
+        throw IllegalArgumentException("mask.width { got " + std::to_string(mask_width) + " } != V.seq_len { got " +
+                                       std::to_string(VL) + " }");
+    return base_->attention(Y, Q, K, V, N, head, QL, VL, pad4(dK), pad4(dV), head_inner, scale, Mask, pad4(mask_width),
+                            mask_per_head);
 }
 SyncerPtr EngineCore::linear2_2D_row(int64_t Y, int64_t X1, int64_t X2, int row_lengthv, float alpha,
                                      float beta, float gamma, int lengthv, int width) {   // :1965-1983
@@ -1556,7 +1566,7 @@ Tensor* Engine::transpose(bool inplace, Tensor* X, int dimIdx1, int dimIdx2) {
     return X;
 }
 
-Tensor* Engine::attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale) {
+Tensor* Engine::attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale, Tensor* mask) {
     require(Q, "Q"); require(K, "K"); require(V, "V");
     if (check_) {    // ChannelMHA.java:45-63
         must_greater_equal(Q->ndim(), "Q.ndim", 2); must_greater_equal(K->ndim(), "K.ndim", 2);
@@ -1576,12 +1586,21 @@ Tensor* Engine::attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale
         throw IllegalArgumentException("K.seq_len { got " + std::to_string(KL) + " } != V.seq_len { got " +
                                        std::to_string(VL) + " }");
     if (scale == 0.0f) scale = 1.0f / sqrtf((float)KC);
+    bool mask_per_head = false;
+    if (mask != nullptr) {   // [QL, VL] for every image and head, or [N, head, QL, VL]
+        const std::vector<int>& md = mask->dim;
+        const bool one = md.size() == 2 && md[0] == QL && md[1] == VL;
+        mask_per_head = md.size() == 4 && md[0] == N && md[1] == head && md[2] == QL && md[3] == VL;
+        if (!one && !mask_per_head)
+            throw IllegalArgumentException("mask.dim must be [Q.seq_len, V.seq_len] or [batch, head, Q.seq_len, V.seq_len]");
+    }
     std::vector<int> Ydim = Q->dim;
     Ydim.back() = VC;
     Tensor* Y = &empty(Ydim)->c();
     try {
         finish(Y, core_->attention(Y->address, Q->address, K->address, V->address, N, head, QL, VL, KC / head,
-                                   VC / head, true, scale));
+                                   VC / head, true, scale, mask ? mask->address : 0, mask ? mask->lastDim() : 0,
+                                   mask_per_head));
     } catch (...) { deleteTensor(Y); throw; }
     return Y;
 }

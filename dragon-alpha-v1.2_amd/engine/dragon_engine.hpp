@@ -233,8 +233,11 @@ public:
     SyncerPtr memcpy(int64_t dst, int64_t src, int64_t memsize);
     // softmax(scale * Q.K^T).V per (image, head) in one launch; not a Java method (the reference's block
     // issues transposes, batchMatMulT2, sdiv, softmax, batchMatMul: nn/unit/complex/block/ChannelMHA.java:66-83)
+    // Mask != 0: the probabilities are multiplied by it after the softmax (the block's mask unit); rows of
+    // mask_pitch floats, one [QL, mask_pitch] slice for all or one per (image, head)
     SyncerPtr attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL, int VL, int dK4,
-                        int dV4, bool head_inner, float scale);
+                        int dV4, bool head_inner, float scale, int64_t Mask = 0, int mask_pitch = 0,
+                        bool mask_per_head = false);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int BK, int AK);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int CN, int AN, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int CM, int BM, int K);
@@ -293,7 +296,8 @@ public:
     SyncerPtr memcpy(int64_t dst, int64_t src, int length);
     // head dimensions arrive unpadded; with more than one head they must be multiples of 4 already
     SyncerPtr attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int N, int head, int QL, int VL, int dK,
-                        int dV, bool head_inner, float scale);
+                        int dV, bool head_inner, float scale, int64_t Mask = 0, int mask_width = 0,
+                        bool mask_per_head = false);
     SyncerPtr batchMatMul(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT1(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
     SyncerPtr batchMatMulT2(int64_t C, int64_t A, int64_t B, int Batch, int N, int M, int K);
@@ -396,7 +400,10 @@ public:
     // Y[N, QL, VC] = per head softmax(scale * Q.K^T).V.  scale = 0 means the block's own 1/sqrt(KC).
     // Needs KC/head and VC/head <= 128 (and multiples of 4 when head > 1); other shapes take the operator
     // chain (transpose, batchMatMulT2, softmax_scaled, batchMatMul, transpose).  Not a Java method.
-    Tensor* attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale = 0.0f);
+    // mask (optional): a tensor [QL, VL] (one for every image and head) or [N, head, QL, VL] that multiplies the
+    // probabilities after the softmax, which is what the block does with a mask unit that multiplies element by
+    // element (ChannelMHA.java:75-76).
+    Tensor* attention(Tensor* Q, Tensor* K, Tensor* V, int head, float scale = 0.0f, Tensor* mask = nullptr);
 
     // Y = alpha*X1 + beta*X2 + gamma with the row vector X2 broadcast over the rows of X1
     Tensor* add_row(bool inplace, Tensor* X1, Tensor* X2) { return linear2_row(inplace, X1, X2, 1.0f, 1.0f, 0.0f); }

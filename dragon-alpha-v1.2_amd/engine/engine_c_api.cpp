@@ -327,6 +327,16 @@ dragon_tensor* dragon_engine_attention(dragon_engine* eg, dragon_tensor* Q, drag
     });
     return t ? wrap(t) : nullptr;
 }
+dragon_tensor* dragon_engine_attention_masked(dragon_engine* eg, dragon_tensor* Q, dragon_tensor* K, dragon_tensor* V,
+                                              dragon_tensor* Mask, int32_t head, float scale) {
+    Tensor* t = nullptr;
+    guard([&] {
+        if (!eg) throw NullPointerException("engine");
+        if (!Mask) throw NullPointerException("Tensor mask is null");
+        t = eg->eg.attention(T(Q), T(K), T(V), head, scale, T(Mask));
+    });
+    return t ? wrap(t) : nullptr;
+}
 dragon_tensor* dragon_engine_transpose(dragon_engine* eg, int32_t inplace, dragon_tensor* X,
                                        int32_t dimIdx1, int32_t dimIdx2) {
     Tensor* t = nullptr;

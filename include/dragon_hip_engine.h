@@ -134,6 +134,11 @@ int32_t dragon_policy_conv3D_GEMM_nstream(int32_t GM, int32_t OC);
  * otherwise: such shapes take the operator chain).  Not a Java method. */
 dragon_tensor* dragon_engine_attention(dragon_engine* eg, dragon_tensor* Q, dragon_tensor* K, dragon_tensor* V,
                                        int32_t head, float scale);
+/* The same with the block's mask (ChannelMHA.java:75-76, `P = mask.forward(P)` between the softmax and the second
+ * product) for a mask unit that multiplies element by element: Mask[QL, VL] for every image and head, or
+ * Mask[N, head, QL, VL]. */
+dragon_tensor* dragon_engine_attention_masked(dragon_engine* eg, dragon_tensor* Q, dragon_tensor* K, dragon_tensor* V,
+                                              dragon_tensor* Mask, int32_t head, float scale);
 
 /* Engine.linear(inplace, alpha, X, beta): Y = alpha*X + beta (Engine.java:4005-4013); Engine.sdiv(X, C)
  * is linear(1/C, X, 0).  inplace != 0 writes into X and returns X itself. */

@@ -196,10 +196,22 @@ int dragon_Cuda_reduce_softmax2D(int64_t stream, int64_t dX, int64_t dY, int32_t
  * The score matrix is never stored.  No native of this shape in the reference, which runs
  * batchMatMulT2, linear2D (sdiv), row_max, row_softmax, div2D_field, batchMatMul and four transposes
  * (alpha-Dragon-v1.2/src/z/dragon/nn/unit/complex/block/ChannelMHA.java:66-83); a host that owns that
- * block calls this instead when no mask is set and the head dimensions fit.  Work goes to streams[0]. */
+ * block calls this instead when the head dimensions fit (and the next entry when a mask is set).  Work goes
+ * to streams[0]. */
 int dragon_Cuda_attention_forward(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
                                   int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL, int32_t dK4,
                                   int32_t dV4, int32_t head_inner, float scale);
+
+/* The same with the block's mask: the probabilities are multiplied by a tensor AFTER the softmax,
+ *     Y[n, h, i, :] = sum_j softmax_j(...)[j] * M[.., i, j] * V[n, h, j, :]
+ * which is what `if (mask != null) P = mask.forward(P)` does for a mask unit that multiplies element by
+ * element (a dropout pattern, a causal 0/1 pattern; ChannelMHA.java:75-76).  dMask: rows of mask_pitch floats
+ * (a multiple of 4, >= VL), QL rows per slice; mask_per_head = 0: one [QL, mask_pitch] mask for every
+ * (image, head), 1: [N, head, QL, mask_pitch].  Every other argument as above. */
+int dragon_Cuda_attention_forward_masked(const int64_t* streams, int32_t length, int64_t dQ, int64_t dK, int64_t dV,
+                                         int64_t dMask, int64_t dY, int32_t N, int32_t head, int32_t QL, int32_t VL,
+                                         int32_t dK4, int32_t dV4, int32_t head_inner, float scale,
+                                         int32_t mask_pitch, int32_t mask_per_head);
 
 /* ---- batched products (grid depth = Batch) --------------------------------------- */
 

@@ -222,10 +222,12 @@ def softmax2D(Xp, width, features=None, scale=1.0):
     return Y
 
 
-def attention(Q, K, V, alpha):
+def attention(Q, K, V, alpha, mask=None):
     """Y = softmax(alpha * Q.K^T).V per batch entry, as the reference chains its operators
-    (nn/unit/complex/block/ChannelMHA.java:74-78: batchMatMulT2, sdiv, softmax, batchMatMul).
-    Logical float32 arrays Q[B, QL, dk], K[B, VL, dk], V[B, VL, dv] -> Y[B, QL, dv]."""
+    (nn/unit/complex/block/ChannelMHA.java:74-78: batchMatMulT2, sdiv, softmax, [mask], batchMatMul).
+    Logical float32 arrays Q[B, QL, dk], K[B, VL, dk], V[B, VL, dv] -> Y[B, QL, dv].  mask: a float32
+    array [QL, VL] or [B, QL, VL] that multiplies the probabilities element by element after the softmax
+    (one float32 product each, what an element-wise mask unit computes)."""
     def pad_last(x):
         s = (x.shape[-1] + 3) // 4 * 4
         out = np.zeros(x.shape[:-1] + (s,), np.float32)
@@ -238,6 +240,10 @@ def attention(Q, K, V, alpha):
     P = bmm(T2, Qp, Kp, B, QL, VL4, VL, dk4)                       # [B, QL, VL4], columns >= VL zero
     P = linear2D(alpha, P.reshape(B * QL, VL4), 0.0, VL)           # sdiv(C, P) = linear(1/C, P, 0)
     P = softmax2D(P, VL)
+    if mask is not None:
+        Mp = np.zeros((B, QL, VL4), np.float32)
+        Mp[:, :, :VL] = np.broadcast_to(np.asarray(mask, np.float32), (B, QL, VL))
+        P = (P.reshape(B, QL, VL4) * Mp).astype(np.float32)
     Y = bmm(NN, P.reshape(B, QL, VL4), Vp, B, QL, dv4, VL, VL4)    # [B, QL, dv4]
     return Y[:, :, :dv]
 

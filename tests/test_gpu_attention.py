@@ -263,3 +263,134 @@ def test_engine_attention_error_behaviour(eg):
     with pytest.raises(NullPointerException):
         eg.attention(None, tK, tV, 1)
     assert eg.attention(tQ, tK, tV, 2).dim == [2, 8, 24]
+
+
+# ---- the block's mask: a tensor that multiplies the probabilities after the softmax (ChannelMHA.java:75-76) ----
+
+def attention_masked_f64(Q, K, V, scale, M):
+    S = np.einsum("nhqd,nhkd->nhqk", Q.astype(np.float64), K.astype(np.float64)) * np.float64(np.float32(scale))
+    P = np.exp(S - S.max(-1, keepdims=True))
+    P /= P.sum(-1, keepdims=True)
+    return np.einsum("nhqk,nhkd->nhqd", P * M.astype(np.float64), V.astype(np.float64))
+
+
+def run_attention_masked(dh, Q, K, V, M, scale, head_inner, garbage_pad=False):
+    """M[QL, VL] (one mask for every image and head) or M[N, head, QL, VL]."""
+    N, H, QL, dk = Q.shape
+    VL, dv = V.shape[2], V.shape[3]
+    Qp, Kp, Vp, Mp = pad_last(Q), pad_last(K), pad_last(V), pad_last(M)
+    if garbage_pad:                                      # nothing beyond the last key may count
+        Mp[..., VL:] = np.float32("inf")
+    dk4, dv4 = Qp.shape[-1], Vp.shape[-1]
+    if head_inner:
+        Qp, Kp, Vp = (np.ascontiguousarray(x.transpose(0, 2, 1, 3)) for x in (Qp, Kp, Vp))
+    dQ, dK, dV, dM = dh.DeviceArray(Qp), dh.DeviceArray(Kp), dh.DeviceArray(Vp), dh.DeviceArray(Mp)
+    ny = N * H * QL * dv4
+    dY = dh.DeviceArray(size=ny + 16)
+    dY.fill(3.0)
+    dh.Cuda_attention.forward_masked([0], 1, dQ.address, dK.address, dV.address, dM.address, dY.address, N, H, QL, VL,
+                                     dk4, dv4, head_inner, scale, Mp.shape[-1], M.ndim == 4)
+    dh.Cuda.streamSynchronize(0)
+    raw = dY.get()
+    for d in (dQ, dK, dV, dM, dY):
+        d.free()
+    assert np.all(raw[ny:] == 3.0)
+    Yp = raw[:ny].reshape((N, QL, H, dv4) if head_inner else (N, H, QL, dv4))
+    if head_inner:
+        Yp = Yp.transpose(0, 2, 1, 3)
+    assert not Yp[..., dv:].any()
+    return Yp[..., :dv]
+
+
+MASKED_SHAPES = [(1, 1, 1, 1, 4, 4), (2, 3, 37, 29, 20, 20), (1, 2, 128, 128, 64, 64), (2, 2, 130, 257, 64, 64),
+                 (1, 2, 200, 333, 128, 96), (3, 1, 65, 64, 32, 8), (1, 4, 300, 70, 12, 100)]
+
+
+@pytest.mark.parametrize("head_inner", [False, True])
+@pytest.mark.parametrize("kind", ["causal", "dropout", "signed", "per head"])
+def test_masked_block_against_the_chain_and_fp64(dh, gpu, head_inner, kind):
+    rng = np.random.default_rng(515 + len(kind) + 7 * head_inner)
+    for (N, H, QL, VL, dk, dv) in MASKED_SHAPES:
+        Q = rng.uniform(-1, 1, (N, H, QL, dk)).astype(np.float32)
+        K = rng.uniform(-1, 1, (N, H, VL, dk)).astype(np.float32)
+        V = rng.uniform(-1, 1, (N, H, VL, dv)).astype(np.float32)
+        if kind == "causal":
+            M = (np.arange(VL)[None, :] <= np.arange(QL)[:, None] * VL // QL).astype(np.float32)
+        elif kind == "dropout":
+            M = (rng.uniform(0, 1, (QL, VL)) >= 0.3).astype(np.float32) / np.float32(0.7)
+        elif kind == "signed":
+            M = rng.uniform(-2, 2, (QL, VL)).astype(np.float32)
+        else:
+            M = rng.uniform(0, 1.5, (N, H, QL, VL)).astype(np.float32)
+        scale = 1.0 / np.sqrt(dk)
+        Y = run_attention_masked(dh, Q, K, V, M, scale, head_inner, garbage_pad=(kind == "signed"))
+        M4 = np.broadcast_to(M, (N, H, QL, VL))
+        R64 = attention_masked_f64(Q, K, V, scale, M4)
+        R32 = oracle.attention(Q.reshape(N * H, QL, dk), K.reshape(N * H, VL, dk), V.reshape(N * H, VL, dv), scale,
+                               mask=M4.reshape(N * H, QL, VL)).reshape(N, H, QL, dv)
+        assert np.isfinite(Y).all()
+        e_dev, e_ref = np.abs(Y - R64).max(), np.abs(R32 - R64).max()
+        bound = 1e-4 * np.sqrt(dk) * np.abs(V).max() * np.abs(M).max() * (1 + abs(scale) * np.abs(Q).max() * np.abs(K).max())
+        assert np.linalg.norm(Y - R64) <= 1e-5 * max(np.linalg.norm(R64), 1e-30) + 1e-7, (kind, N, H, QL, VL, dk, dv)
+        assert e_dev <= bound and e_dev <= 2 * e_ref + 1e-6, (kind, e_dev, e_ref, bound)
+
+
+def test_masked_block_exact_cases(dh, gpu):
+    rng = np.random.default_rng(77)
+    N, H, QL, VL, d = 1, 2, 70, 90, 16
+    Q = rng.uniform(-1, 1, (N, H, QL, d)).astype(np.float32)
+    K = rng.uniform(-1, 1, (N, H, VL, d)).astype(np.float32)
+    V = rng.uniform(-1, 1, (N, H, VL, d)).astype(np.float32)
+    # a mask of ones is no mask: the same bits as the unmasked entry point
+    Y1 = run_attention_masked(dh, Q, K, V, np.ones((QL, VL), np.float32), 0.25, False)
+    Y0 = run_attention(dh, Q, K, V, 0.25, False)
+    assert np.array_equal(Y1, Y0)
+    # a mask of zeros gives zeros; a mask that keeps one key gives that key's row of V times its probability
+    assert not run_attention_masked(dh, Q, K, V, np.zeros((QL, VL), np.float32), 0.25, False).any()
+    M = np.zeros((QL, VL), np.float32)
+    M[:, 5] = 1.0
+    Y = run_attention_masked(dh, Q * 0, K, V, M, 0.25, False)          # equal scores: probability 1 / VL
+    assert np.allclose(Y, V[:, :, 5:6, :] / VL, rtol=1e-6, atol=1e-7)
+
+
+def test_masked_block_argument_errors(dh, gpu):
+    d = dh.DeviceArray(size=4096)
+    a = d.address
+    f = dh.Cuda_attention.forward_masked
+    with pytest.raises(dh.CudaException):
+        f([0], 1, a, a, a, 0, a, 1, 1, 8, 8, 4, 4, False, 1.0, 8, False)        # no mask
+    with pytest.raises(dh.CudaException):
+        f([0], 1, a, a, a, a, a, 1, 1, 8, 8, 4, 4, False, 1.0, 4, False)        # pitch below the key count
+    with pytest.raises(dh.CudaException):
+        f([0], 1, a, a, a, a, a, 1, 1, 8, 6, 4, 4, False, 1.0, 6, False)        # pitch not a multiple of 4
+    with pytest.raises(dh.CudaException):
+        f([0], 1, a, a, a, a + 4, a, 1, 1, 8, 8, 4, 4, False, 1.0, 8, False)    # mask not 16-byte aligned
+    d.free()
+
+
+@pytest.mark.parametrize("per_head", [False, True])
+def test_engine_attention_with_a_mask(eg, per_head):
+    # ChannelMHA with a mask unit that multiplies element by element, through the engine mirror
+    from dragon_hip.engine import IllegalArgumentException
+    N, QL, VL, head, dk, dv = 2, 70, 45, 3, 16, 12
+    rng = np.random.default_rng(1234 + per_head)
+    KC, VC = head * dk, head * dv
+    Q = rng.uniform(-1, 1, (N, QL, KC)).astype(np.float32)
+    K = rng.uniform(-1, 1, (N, VL, KC)).astype(np.float32)
+    V = rng.uniform(-1, 1, (N, VL, VC)).astype(np.float32)
+    M = (rng.uniform(0, 1, (N, head, QL, VL) if per_head else (QL, VL)) >= 0.25).astype(np.float32) / np.float32(0.75)
+    base = eg.get_param("live_blocks")
+    tQ, tK, tV, tM = (eg.tensor(x, *x.shape) for x in (Q, K, V, M))
+    tY = eg.attention(tQ, tK, tV, head, mask=tM)
+    assert tY.dim == [N, QL, VC]
+    Y = eg.valueOf(tY).reshape(N, QL, head, dv).transpose(0, 2, 1, 3)
+    R = attention_masked_f64(Q.reshape(N, QL, head, dk).transpose(0, 2, 1, 3), K.reshape(N, VL, head, dk).transpose(0, 2, 1, 3),
+                             V.reshape(N, VL, head, dv).transpose(0, 2, 1, 3), 1 / np.sqrt(KC),
+                             np.broadcast_to(M, (N, head, QL, VL)))
+    assert np.linalg.norm(Y - R) <= 1e-5 * np.linalg.norm(R)
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(tQ, tK, tV, head, mask=eg.zeros(QL, VL + 1))          # not [QL, VL]
+    with pytest.raises(IllegalArgumentException):
+        eg.attention(tQ, tK, tV, head, mask=eg.zeros(N, head + 1, QL, VL))
+    eg.delete(tQ, tK, tV, tM, tY)
+    assert eg.get_param("live_blocks") <= base + 2          # the two rejected masks stay with the caller

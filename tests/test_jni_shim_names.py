@@ -60,7 +60,7 @@ def test_every_exported_name_is_one_the_java_side_binds(shim_names):
     *_mma natives (declared in Java, native source unpublished) or one of the documented additions."""
     g = golden()
     additions = {PREFIX["MM"] + "matMul_1biased", PREFIX["MM"] + "matMulSK_1static",
-                 PREFIX["CV"] + "conv3D_1biased", PREFIX["BMM"] + "attention",
+                 PREFIX["CV"] + "conv3D_1biased", PREFIX["BMM"] + "attention", PREFIX["BMM"] + "attention_1masked",
                  "Java_z_dragon_engine_cuda_impl_math_Cuda_1reduce_softmax2D"}
     mma = {PREFIX["MM"] + n for n in ("matMul_1mma", "matMulT1_1mma", "matMulT2_1mma")} | \
           {PREFIX["BMM"] + n for n in ("batchMatMul_1mma", "batchMatMulT1_1mma", "batchMatMulT2_1mma")}
