@@ -220,8 +220,11 @@ int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length, 
     p.A = (const float*)(intptr_t)dA;   // A[Batch, N, AK]
     p.B = (const float*)(intptr_t)dB;   // B[Batch, BK, M]
     p.C = (float*)(intptr_t)dC;         // C[Batch, N, M]
-    p.rows = N; p.cols = M; p.k_total = AK;
-    p.lda = AK; p.a_outer = N;  p.a_inner = AK;
+    // A is read up to the last 16-byte chunk that holds a k below BK: its columns beyond are never touched
+    // (the reference's loop stops at BK, BMM/batchMatMul.cuh:15)
+    const int k_read = (BK + 3) / 4 * 4 < AK ? (BK + 3) / 4 * 4 : AK;
+    p.rows = N; p.cols = M; p.k_total = k_read;
+    p.lda = AK; p.a_outer = N;  p.a_inner = k_read;
     p.ldb = M;  p.b_outer = BK; p.b_inner = M;
     p.ldc = M;
     p.sA = (long long)N * AK; p.sB = (long long)BK * M; p.sC = (long long)N * M;

@@ -216,7 +216,10 @@ int dragon_Cuda_attention_forward_masked(const int64_t* streams, int32_t length,
 /* ---- batched products (grid depth = Batch) --------------------------------------- */
 
 /* C[b][N,M] = A[b][N,AK] * B[b][BK,M], k < BK.  M and AK are multiples of 4, N and BK
- * are arbitrary; batch strides N*AK, BK*M, N*M.
+ * are arbitrary; batch strides N*AK, BK*M, N*M.  Rows of B from BK on are never read and columns
+ * of A from the multiple of 4 at or above BK on neither; the up to three columns of A between BK and
+ * that multiple are read and multiplied by zeros, so they must hold finite values (they are zeros in
+ * the engine's layout).
  * Replaces ..._Cuda_1batchMatMul_batchMatMul and batchMatMul_texture (BMM/A.cu:20-62,
  * JM/Cuda_batchMatMul.java:90,137, dispatcher BMM/batchMatMul.cuh:48-254).  The texture
  * entry is the same computation (textures only served the reference's edge tiles). */

@@ -127,3 +127,20 @@ def test_neighbouring_batch_does_not_leak_into_the_k_tail(gpu):
     R = oracle.bmm(NN, A, B, B4, *dims)
     C = run(gpu, NN, A, B, B4, dims, cshape)
     assert np.isfinite(C[0]).all() and np.array_equal(C[0], R[0])
+
+
+def test_columns_of_a_beyond_the_k_that_exist_are_not_read(gpu):
+    # AK may be wider than BK rounded up to 4 (a view into a wider tensor): whatever lies there, NaN included,
+    # stays out of the product, as in the reference, whose loop over k stops at BK (BMM/batchMatMul.cuh:15)
+    rng = np.random.default_rng(14)
+    Batch, N, M, K, AK = 4, 70, 36, 129, 144
+    A = np.full((Batch, N, AK), np.nan, np.float32)
+    A[:, :, :K] = rng.integers(-3, 4, (Batch, N, K))
+    A[:, :, K:132] = 0.0                                  # the rest of the last 16-byte chunk: finite
+    B = rng.integers(-3, 4, (Batch, K, M)).astype(np.float32)
+    for tile in (-1, 1, 7, 0):
+        gpu.force_tile(tile)
+        C = run(gpu, NN, A, B, Batch, (N, M, K, AK), (Batch, N, M))
+        gpu.force_tile(-1)
+        R = np.einsum("bnk,bkm->bnm", A[:, :, :K].astype(np.float64), B.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(C, R), tile

@@ -167,3 +167,19 @@ def test_reference_correctness_sweep(gpu, variant):
     assert worst <= 1e-5
     for x in (dA, dB, dC):
         x.free()
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_every_row_and_column_count_up_to_255(gpu, variant):
+    """The sweep above samples the reference's 1..255 x 1..255 grid; this one walks EVERY row count against four
+    column counts and every column count against four row counts (K = 129), so that no residue of the tile,
+    block and rim arithmetic goes unvisited."""
+    rng = np.random.default_rng(4242 + variant)
+    K = 129
+    cases = [(n, m) for n in range(1, 256) for m in (1, 64, 130, 255)] + \
+            [(n, m) for m in range(1, 256) for n in (3, 65, 128, 254)]
+    for (n, m) in cases:
+        A, B = logical_operands(variant, rng, n, m, K, dist="int")
+        C, Cp = gpu_matmul_2d(gpu, variant, A, B, fill=5.0)
+        assert np.array_equal(C, oracle.matmul(variant, A, B)), (n, m)
+        assert np.count_nonzero(Cp[n:, :]) == 0 and np.count_nonzero(Cp[:, m:]) == 0, (n, m)
