@@ -476,9 +476,35 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
 // 9.7).  Measured gains where it is taken: 15 % at 1000 x 777 x 1531, 17 % at 1024^3 and 1536 x 1024 x 1024,
 // 25 % at 512^3, 18 % at 2048 x 512 x 2048, 2.2 x at 128 x 128 x 4096, 17 x at 256 x 256 x 131072 (where it
 // equals the host's split into 128 slices plus the fold: 138 us).
+//
+// LARGE products take the balanced kernel too, with 128 x 128 tiles: its stages carry no vector-ALU instruction
+// (which would exclude MFMAs on the SIMD), so one workgroup per unit keeps the matrix pipes as busy as four of the
+// tile-per-workgroup kernel do, and the equal runs leave no unit idle in a last, partial round of tiles.  Measured
+// against the best tile-per-workgroup shape: 4096^3 918 against 934 us (95 % of the peak), 8192 x 4096 x 4096 1835 /
+// 1882, 3584^3 636 / 721, 3072^3 404 / 425, 2560^3 241 / 283-299, 2048^3 119 / 128, 1024 x 8192 x 1024 121 / 128;
+// level at K = 512 ... 1024 and behind below, where the plain tile kernels' shorter set-up counts.  Between the two
+// regimes (more than two 64 x 64 tiles per unit, fewer than one of 128 x 128) the tile is 128 x 64 or 64 x 128:
+// 1536^3 61 against 74 us, 1792^3 92 / 111.
 int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant) {
     if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
     const long long t64 = (long long)((rows + 63) / 64) * ((cols + 63) / 64) * nz;
+    if (k >= 768 && t64 > 2LL * num_cu) {
+        const long long rm = (rows + 127) / 128, cn = (cols + 127) / 128, rm64 = (rows + 63) / 64, cn64 = (cols + 63) / 64;
+        const double area = (double)rows * (double)cols;
+        const long long t128 = rm * cn * nz;
+        if (t128 >= num_cu && t128 <= SK_MAX_TILES && area >= 0.85 * (double)(rm * 128) * (double)(cn * 128))
+            return TILE_SK_128x128;
+        // the half-size tile that wastes less of C
+        const bool tall = (double)(rm * 128) * (double)(cn64 * 64) <= (double)(rm64 * 64) * (double)(cn * 128);
+        const long long th = (tall ? rm * cn64 : rm64 * cn) * nz;
+        const double padded = tall ? (double)(rm * 128) * (double)(cn64 * 64) : (double)(rm64 * 64) * (double)(cn * 128);
+        if (th >= num_cu && th <= SK_MAX_TILES && area >= 0.85 * padded) {
+            // two workgroups per compute unit where that deals whole tiles
+            if (tall && th % (2LL * num_cu) == 0) return TILE_SK_128x64_O2;
+            return tall ? TILE_SK_128x64 : TILE_SK_64x128;
+        }
+        return -1;
+    }
     if (t64 > 2LL * num_cu || t64 > SK_MAX_TILES) return -1;
     const long long S = ((long long)k + 31) / 32;
     const long long units = t64 * S;

@@ -169,13 +169,19 @@ def test_tile_choice_on_the_documented_shapes(dh):
     P = 256
     ct = dh.choose_tile
     dh.force_tile(-1)
+    # More than two 64x64 tiles per compute unit and K from 768 on: the balanced kernel with 128x128 tiles (21),
+    # or with the half-size tile (19 = 128x64, 20 = 64x128; 23 = 128x64 with two workgroups per unit, where that
+    # deals whole tiles) where 128x128 tiles are fewer than the units or would stand mostly empty
     for v in (NN, T1, T2):
-        assert ct(v, 4096, 4096, 1, 4096) == 0 + P                # four tiles per compute unit: 16-k stages
-        assert ct(v, 2816, 2816, 1, 4096) == 6 + P                # two per unit: 32-k stages cost no co-residency
-        assert ct(v, 2048, 2048, 1, 2048) == 7 + P                # 64x64, four per unit: 32-k stages
-        assert ct(v, 1536, 1536, 1, 1536) == 7 + P                # 64x64, three per unit: 32-k stages
-    assert ct(T1, 256, 256, 128, 1024) == 6 + P                   # the split-K weight gradient (GridZ 128 slices of 1024)
-    assert ct(NN, 1024, 64, 64, 1024) == 8 + P                    # scores x V of the attention-shaped batch
+        assert ct(v, 4096, 4096, 1, 4096) == 21 and ct(v, 8192, 4096, 1, 4096) == 21
+        assert ct(v, 2816, 2816, 1, 4096) == 21 and ct(v, 2048, 2048, 1, 2048) == 21
+        assert ct(v, 4096, 4096, 1, 768) == 21 and ct(v, 3000, 3000, 1, 3000) == 21
+        assert ct(v, 1536, 1536, 1, 1536) == 19                   # 144 tiles of 128x128 for 256 units: 128x64
+        assert ct(v, 4096, 4096, 1, 512) == P                     # a shorter K: a tile per workgroup, paired stages
+        assert ct(v, 16384, 16384, 1, 1024) == P                  # more tiles than the balanced kernel counts
+    assert ct(T1, 256, 256, 128, 1024) == 21                      # a batch of 128 such products (the split-K entry
+    #                                                               chooses among the tile-per-workgroup kernels)
+    assert ct(NN, 1024, 64, 64, 1024) == 23                       # scores x V of the attention-shaped batch
     # A K that fits one LDS stage of 64 under a large C: the band kernel (24), from two tiles per compute unit on;
     # not for a K of 56 or less, rows of C off the 128-byte lines, or a C that leaves its tiles mostly empty
     for v in (NN, T1, T2):
@@ -197,7 +203,7 @@ def test_tile_choice_on_the_documented_shapes(dh):
     shape = (64 * 20, 128 * 19, 1, 2048)
     if ct(NN, *shape) in (5 + P, 9 + P):
         assert ct(NN, *shape) == 9 + P and ct(T2, *shape) == 9 + P and ct(T1, *shape) == 5 + P
-    assert ct(NN, 3072, 3072, 1, 3072) == 7 + P                 # nine 64x64 tiles per unit: still 32-k stages
+    assert ct(NN, 3072, 3072, 1, 512) == 7 + P                  # nine 64x64 tiles per unit: still 32-k stages
     assert ct(NN, 4096, 4096, 1, 256) == 0 and ct(NN, 4096, 4096, 1, 512) == P    # a short K keeps the plain form
     dh.force_tile(7)
     assert ct(NN, 4096, 4096, 1, 4096) == 7                     # a forced shape is reported as it is

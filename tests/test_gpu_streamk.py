@@ -135,7 +135,7 @@ def test_host_threads_force_tiles_independently(gpu):
     th = threading.Thread(target=other)
     th.start()
     th.join()
-    assert seen == {"before": 256, "after": 3}
+    assert seen == {"before": 21, "after": 3}
     assert gpu.choose_tile(NN, 4096, 4096, 1, 4096) == 22
 
 
