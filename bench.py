@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_f32_mfma_4096cubed.md")
 # the sources the headline kernels are compiled from: a counter reading belongs to one state of them
 KERNEL_SOURCES = [os.path.join(ROOT, "dragon-alpha-v1.2_amd", "csrc", f)
-                  for f in ("gemm_mfma_kernel.h", "gemm_mfma.hip", "gemm_mfma.h", "build.sh")]
+                  for f in ("gemm_mfma_kernel.h", "gemm_mfma_streamk.hip", "gemm_mfma.hip", "gemm_mfma.h", "build.sh")]
 
 
 def kernel_sources_sha16():

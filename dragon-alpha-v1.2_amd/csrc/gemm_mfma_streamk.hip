@@ -109,7 +109,7 @@ __device__ __forceinline__ void mfma_group_with(v16f (&acc)[NACC][TM][TN], const
     });
 }
 
-template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC>
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC, bool BIAS>
 __global__ __launch_bounds__(NTHREADS, OCC)
 void gemm_f32_mfma_streamk(const GemmParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -306,7 +306,7 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     auto piece_end = [&]() __attribute__((always_inline)) -> bool {
         left -= piece_len;
         if (whole) {
-            store_tile<A_KIN, B_KIN, TM, TN, false>(acc[0], p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
+            store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc[0], p, cur.row0, cur.col0, cur.c_ptr, wm, wn, r, h);
         } else {
             // A piece of a shared tile goes to the workspace: slot 2w for a piece of the tile the run starts
             // in, 2w+1 for a piece of a later tile.  It is counted at the end of the run.
@@ -373,14 +373,17 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
             add_partial<TM, TN>(acc[0], p.sk_ws + (size_t)(2 * w2 + (w2_first_tile == tile ? 0 : 1)) * (BM * BN), wave, lane);
         }
         const TileCtx c = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, tile);
-        store_tile<A_KIN, B_KIN, TM, TN, false>(acc[0], p, c.row0, c.col0, c.c_ptr, wm, wn, r, h);
+        store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc[0], p, c.row0, c.col0, c.c_ptr, wm, wn, r, h);
     }
 }
 
 template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC = 1>
 static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws, size_t ws_floats) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    if (p.split || p.bias != nullptr) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
+    // the bias row exists for the forward product only (added where a tile is stored: once, by whoever holds
+    // the whole sum)
+    constexpr bool CAN_BIAS = A_KIN && !B_KIN;
+    if (p.split || (p.bias != nullptr && !CAN_BIAS)) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long tiles = (long long)p.tiles_m * p.tiles_n * p.nz;
@@ -401,7 +404,14 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     gemm_magic_divisor((unsigned)S, p.sk_div_S_mul, p.sk_div_S_shift);
     p.sk_q = (int)(units / grid);
     p.sk_rem = (int)(units % grid);
-    hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC>), dim3((unsigned)grid),
+    if constexpr (CAN_BIAS) {
+        if (p.bias != nullptr) {
+            hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, true>), dim3((unsigned)grid),
+                               dim3(NTHREADS), 0, stream, p);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false>), dim3((unsigned)grid),
                        dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
 }
