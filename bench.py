@@ -228,7 +228,11 @@ def main():
     achieved = flop / (kernel_ms[slowest] * 1e-3) / 1e12
     rec = recorded_traffic()
     rec_kernel = rec.get("per_launch", {}).get(slowest)
-    roofline = {"bound": "mfma", "kernel": "gemm_f32_mfma %s 4096^3" % slowest,
+    variant_id = {"A*B": 0, "A^T*B": 1, "A*B^T": 2}[slowest]
+    tile_id = dh.choose_tile(variant_id, n, n, 1, n, SM)
+    kernel_name = ("gemm_f32_mfma_streamk" if 18 <= tile_id < 24 else "gemm_f32_mfma_band" if tile_id == 24
+                   else "gemm_f32_mfma_dma" if 15 <= tile_id < 18 else "gemm_f32_mfma")
+    roofline = {"bound": "mfma", "kernel": "%s (tile id %d) %s 4096^3" % (kernel_name, tile_id, slowest),
                 "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_TFLOPS, 4),
                 "traffic": rec_kernel["traffic_bytes"] if rec_kernel else None,
