@@ -26,10 +26,12 @@ int check_common(const int64_t* streams, int length, int64_t dA, int64_t dB, int
     return hipSuccess;
 }
 
-// 2-D products, optionally cut into gz K slices.
+// 2-D products, optionally cut into gz K slices.  sk_ws: a workspace of GEMM_SK_WS_FLOATS_256CU floats for the
+// balanced kernel, from a caller that may not allocate (the kernel otherwise makes one per stream at its first
+// launch there).
 int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t dA, int64_t dB,
               int64_t dC, int64_t dCbuf, int N, int M, int K, int64_t dBias = 0, int bias_rows = 0,
-              int bias_width = 0) {
+              int bias_width = 0, float* sk_ws = nullptr) {
     int e = check_common(streams, length, dA, dB, dC);
     if (e) return e;
     if (N <= 0 || M <= 0 || K <= 0 || gz < 1) return hipErrorInvalidValue;
@@ -73,10 +75,11 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return hipErrorNoDevice;
-    // K slices go to the caller's buffers one by one: always a tile-per-workgroup kernel
-    const int tile = p.split ? (gemm_forced_tile() != TILE_AUTO ? gemm_forced_tile()
-                                : gemm_choose_tile_per_workgroup(p.rows, p.cols, p.nz, p.k_slice > 0 ? p.k_slice : p.k_total, num_cu, variant))
-                             : gemm_choose_tile(p.rows, p.cols, p.nz, p.k_total, num_cu, variant);
+    // K slices are tiles like batches are: (slice, tile of C) pairs, each slice k_slice long
+    const int k_tile = p.split && p.k_slice > 0 ? p.k_slice : p.k_total;
+    const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, k_tile, num_cu, variant);
+    p.sk_ws_given = sk_ws;
+    p.sk_ws_given_floats = sk_ws != nullptr ? GEMM_SK_WS_FLOATS_256CU : 0;
     return gemm_launch(variant, p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 
@@ -129,12 +132,18 @@ int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC, 
 
 namespace {
 
-// Partial products of dragon_Cuda_matMul_matMulSK_static: slice z >= 1 at (z-1)*N*M, exactly the
-// layout of the caller's Cbuf in the two-stage entry points.  One copy per GPU, held until the
-// process ends.  In host code this name is only a handle for hipGetSymbolAddress: the kernels get
-// the device address that call returns.
+// Scratch memory of dragon_Cuda_matMul_matMulSK_static, one copy per GPU, held until the process ends:
+//   [0, SK_STATIC_FLOATS)          the partial products, slice z >= 1 at (z-1)*N*M, exactly the layout of the
+//                                  caller's Cbuf in the two-stage entry points;
+//   [SK_STATIC_FLOATS, + GEMM_SK_WS_FLOATS_256CU)
+//                                  the balanced kernel's workspace (arrival counters, pieces of shared tiles),
+//                                  which the other entry points keep per stream in allocated memory.  The
+//                                  counters start at zero with the array (a device variable without an
+//                                  initialiser is zero) and every launch leaves them there.
+// In host code the array's name is only a handle for hipGetSymbolAddress: the kernels get the device address
+// that call returns.
 constexpr long long SK_STATIC_FLOATS = 8ll << 20;   // 32 MiB
-static __device__ __align__(256) __attribute__((used)) float scratch[SK_STATIC_FLOATS];
+static __device__ __align__(256) __attribute__((used)) float scratch[SK_STATIC_FLOATS + GEMM_SK_WS_FLOATS_256CU];
 
 constexpr int MAX_DEVICES = 64;
 std::atomic<float*> g_scratch_ptr[MAX_DEVICES];
@@ -174,12 +183,13 @@ int dragon_Cuda_matMul_matMulSK_static(const int64_t* streams, int32_t length, i
                 "the static workspace of %lld floats\n", need, SK_STATIC_FLOATS);
         return hipErrorOutOfMemory;
     }
-    if (GridZ == 1) return matmul_2d(variant, streams, length, 1, dA, dB, dC, 0, N, M, K);
     float* ptr = nullptr;
     e = static_scratch(&ptr);
     if (e) return e;
+    float* sk_ws = ptr + SK_STATIC_FLOATS;
+    if (GridZ == 1) return matmul_2d(variant, streams, length, 1, dA, dB, dC, 0, N, M, K, 0, 0, 0, sk_ws);
     // stage 1 writes every float of the GridZ-1 partials it later reads, so nothing has to be cleared
-    e = matmul_2d(variant, streams, length, GridZ, dA, dB, dC, (int64_t)(intptr_t)ptr, N, M, K);
+    e = matmul_2d(variant, streams, length, GridZ, dA, dB, dC, (int64_t)(intptr_t)ptr, N, M, K, 0, 0, 0, sk_ws);
     if (e) return e;
     return skbuf_summary_launch((hipStream_t)(intptr_t)streams[0], ptr, (float*)(intptr_t)dC, GridZ - 1, N * M);
 }

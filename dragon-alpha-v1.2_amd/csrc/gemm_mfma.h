@@ -91,6 +91,13 @@ struct GemmParams {
     int* sk_count;
     int sk_S, sk_q, sk_rem;
     unsigned sk_div_S_mul, sk_div_S_shift;
+    // set by a caller that may not allocate: a workspace of its own for the balanced kernel (arrival counters
+    // zero) instead of the stream's
+    float* sk_ws_given;
+    size_t sk_ws_given_floats;
+    // K slices: the tiles from number sk_T1 on (the last slice's) have sk_S_last stages
+    int sk_S_last, sk_T1;
+    unsigned sk_div_Sl_mul, sk_div_Sl_shift;
     // filled by the launcher of the band kernel (gemm_launch_band): a band's tiles_n column tiles are dealt
     // out in bd_chunks runs of bd_chunk_tiles
     int bd_chunks, bd_chunk_tiles;
@@ -125,13 +132,18 @@ hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t s
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
 hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // the three products (batched too) through the balanced kernel (tile ids TILE_SK_*).  It needs the stream's
-// workspace; hipErrorOutOfMemory says that the product cannot go this way (no workspace and none may be made
-// now, or sizes beyond its counters) and the caller takes a tile-per-workgroup kernel instead.
+// workspace (or the one in p.sk_ws_given); hipErrorOutOfMemory says that the product cannot go this way (no
+// workspace and none may be made now, sizes beyond its counters, K slices shorter than a stage) and the caller
+// takes a tile-per-workgroup kernel instead.
 hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // The balanced kernel's tile for this product, or -1 where the tile-per-workgroup kernels do as well or
 // better (an estimate fitted to measurements: at most two 64 x 64 tiles per compute unit, and K long enough
 // to carry the balanced kernel's larger fixed time).
 int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
+// Floats of a balanced-kernel workspace for a device of num_cu compute units (GEMM_SK_WS_FLOATS_256CU: the
+// same for 256 units, as a constant for static storage)
+size_t gemm_streamk_workspace_floats(int num_cu);
+constexpr size_t GEMM_SK_WS_FLOATS_256CU = 4096 + (size_t)2 * 256 * 128 * 128;
 // The workspace of `stream` on the current device: arrival counters and the slots for pieces of shared tiles.
 // Made at the first balanced launch on that stream (never while the stream is capturing: then nullptr) and kept
 // for later launches on the same handle until the process ends.

@@ -172,8 +172,8 @@ int gemm_choose_tile_per_workgroup(int rows, int cols, int nz, int k, int num_cu
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream) {
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     if (gemm_tile_is_streamk(tile) || gemm_tile_is_band(tile)) {
-        // where the product cannot take the balanced kernel (split-K slices go to the caller's buffers; a
-        // capturing stream that has no workspace yet; a bias row on a transposed product) or the band kernel (a K beyond one stage, K slices, a
+        // where the product cannot take the balanced kernel (K slices shorter than a stage; a capturing
+        // stream that has no workspace yet; a bias row on a transposed product) or the band kernel (a K beyond one stage, K slices, a
         // bias row) a tile-per-workgroup kernel takes over
         const hipError_t e = gemm_tile_is_band(tile) ? gemm_launch_band(variant, p, stream)
                                                      : gemm_launch_streamk(variant, p, tile, stream);

@@ -109,7 +109,10 @@ __device__ __forceinline__ void mfma_group_with(v16f (&acc)[NACC][TM][TN], const
     });
 }
 
-template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC, bool BIAS>
+// SPLIT: the tiles are (K slice, tile of C) pairs of a split-K launch; the tiles of the last slice, which takes
+// the remainder of K, have their own stage count (they come last in the tile order), and a tile's K limits
+// count from the slice's first k.
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC, bool BIAS, bool SPLIT>
 __global__ __launch_bounds__(NTHREADS, OCC)
 void gemm_f32_mfma_streamk(const GemmParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -138,6 +141,31 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     const unsigned long long b_step8 = (unsigned long long)LoadB::k_advance(p.ldb) * 4;
 
     const int S = p.sk_S;
+    // tile -> its stage count and first unit, unit -> tile (two regimes under SPLIT: the slices before the last
+    // with S stages per tile, the sk_T1-th tile onwards with sk_S_last)
+    auto stages_of = [&](int tile) __attribute__((always_inline)) -> int {
+        if constexpr (SPLIT) return tile >= p.sk_T1 ? p.sk_S_last : S;
+        else return S;
+    };
+    auto first_unit_of = [&](int tile) __attribute__((always_inline)) -> int {
+        if constexpr (SPLIT) return tile >= p.sk_T1 ? p.sk_T1 * S + (tile - p.sk_T1) * p.sk_S_last : tile * S;
+        else return tile * S;
+    };
+    auto tile_of = [&](int u) __attribute__((always_inline)) -> int {
+        if constexpr (SPLIT) {
+            const int u1 = p.sk_T1 * S;
+            if (u >= u1) return p.sk_T1 + div_by(u - u1, p.sk_div_Sl_mul, p.sk_div_Sl_shift);
+        }
+        return div_by(u, p.sk_div_S_mul, p.sk_div_S_shift);
+    };
+    auto decode = [&](int tile) __attribute__((always_inline)) -> TileCtx {
+        TileCtx c = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, tile);
+        if constexpr (SPLIT) {   // K limits relative to the slice's first k, like the stage index
+            c.ka_lim -= c.k0;
+            c.kb_lim -= c.k0;
+        }
+        return c;
+    };
     // neighbouring runs share a tile's operands: keep them on one XCD (one L2)
     const int w = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int u0 = sk_first_unit(w, p.sk_q, p.sk_rem);
@@ -149,13 +177,14 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     // LDS addresses are integers known at compile time up to the wave's base, and the lanes' offsets sit
     // ready in registers -- their K test is redone only for a stage that is not wholly inside K, and
     // what has to be looked at per stage is one countdown (f_until).
-    const int first_tile = div_by(u0, p.sk_div_S_mul, p.sk_div_S_shift);
+    const int first_tile = tile_of(u0);
     int f_tile = first_tile;
-    int f_it = u0 - first_tile * S;   // stage of its tile the producer fetches next, as of the last look
+    int f_it = u0 - first_unit_of(first_tile);   // stage of its tile the producer fetches next, as of the last look
+    int f_S = stages_of(first_tile);  // stages of the tile the producer is in
     int f_left = n;                   // stages of the run not yet fetched, as of the last look
     int f_span = 0, f_until = 0;      // stages until the next look, at the last look and now
     int f_interior = 0;               // stages of the tile that lie wholly inside K for both operands
-    TileCtx ft = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, f_tile);
+    TileCtx ft = decode(f_tile);
     LoadA la;
     LoadB lb;
     la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
@@ -174,9 +203,10 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
             for (int i = 0; i < PB; i++) offb[i] = OOB_OFFSET;
             f_span = 0x40000000;
         } else {
-            if (f_it == S) {          // next tile
+            if (f_it == f_S) {        // next tile
                 f_tile++;
-                ft = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, f_tile);
+                if constexpr (SPLIT) f_S = stages_of(f_tile);
+                ft = decode(f_tile);
                 la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
                 lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
                 rsrc_a = dma_descriptor(ft.a_ptr);
@@ -299,8 +329,9 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     // entered at buffer 0; a piece may end behind any stage, and what then has to be done (store the tile
     // or the piece, move on to the next tile) stands behind each of the NS stages.  One loop, no way into
     // its middle: the accumulators stay in the registers they are in.
-    int piece_len = min(S - c_it, left);
-    bool whole = c_it == 0 && piece_len == S;
+    int c_S = stages_of(first_tile);  // stages of the tile being multiplied (the producer may be a tile ahead)
+    int piece_len = min(c_S - c_it, left);
+    bool whole = c_it == 0 && piece_len == c_S;
     int todo = piece_len;
     // the piece of c_tile that this run holds has been multiplied; true when that was the run's last
     auto piece_end = [&]() __attribute__((always_inline)) -> bool {
@@ -316,13 +347,14 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
         }
         if (left == 0) return true;
         c_tile++;
-        cur = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, c_tile);
+        if constexpr (SPLIT) c_S = stages_of(c_tile);
+        cur = decode(c_tile);
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int jj = 0; jj < TN; jj++) acc[0][i][jj] = (v16f)(0.0f);
-        piece_len = min(S, left);
-        whole = piece_len == S;
+        piece_len = min(c_S, left);
+        whole = piece_len == c_S;
         todo = piece_len;
         return false;
     };
@@ -353,7 +385,8 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     __syncthreads();
     if (t < n_rec) {
         const int tile = t == 0 ? rec_tile0 : rec_tile1;
-        const int wa = sk_owner(tile * S, p.sk_q, p.sk_rem), wb = sk_owner(tile * S + S - 1, p.sk_q, p.sk_rem);
+        const int wa = sk_owner(first_unit_of(tile), p.sk_q, p.sk_rem);
+        const int wb = sk_owner(first_unit_of(tile) + stages_of(tile) - 1, p.sk_q, p.sk_rem);
         const int arrived = atomicAdd(p.sk_count + tile, 1);
         const int last = arrived == wb - wa;
         if (last) atomicExch(p.sk_count + tile, 0);
@@ -363,16 +396,17 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     for (int i = 0; i < n_rec; i++) {
         if (!sk_last[i]) continue;
         const int tile = i == 0 ? rec_tile0 : rec_tile1;
-        const int wa = sk_owner(tile * S, p.sk_q, p.sk_rem), wb = sk_owner(tile * S + S - 1, p.sk_q, p.sk_rem);
+        const int wa = sk_owner(first_unit_of(tile), p.sk_q, p.sk_rem);
+        const int wb = sk_owner(first_unit_of(tile) + stages_of(tile) - 1, p.sk_q, p.sk_rem);
 #pragma unroll
         for (int ii = 0; ii < TM; ii++)
 #pragma unroll
             for (int jj = 0; jj < TN; jj++) acc[0][ii][jj] = (v16f)(0.0f);
         for (int w2 = wa; w2 <= wb; w2++) {
-            const int w2_first_tile = div_by(sk_first_unit(w2, p.sk_q, p.sk_rem), p.sk_div_S_mul, p.sk_div_S_shift);
+            const int w2_first_tile = tile_of(sk_first_unit(w2, p.sk_q, p.sk_rem));
             add_partial<TM, TN>(acc[0], p.sk_ws + (size_t)(2 * w2 + (w2_first_tile == tile ? 0 : 1)) * (BM * BN), wave, lane);
         }
-        const TileCtx c = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, tile);
+        const TileCtx c = decode(tile);
         store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc[0], p, c.row0, c.col0, c.c_ptr, wm, wn, r, h);
     }
 }
@@ -383,12 +417,17 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     // the bias row exists for the forward product only (added where a tile is stored: once, by whoever holds
     // the whole sum)
     constexpr bool CAN_BIAS = A_KIN && !B_KIN;
-    if (p.split || (p.bias != nullptr && !CAN_BIAS)) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
+    if (p.bias != nullptr && (!CAN_BIAS || p.split)) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
     const long long tiles = (long long)p.tiles_m * p.tiles_n * p.nz;
-    const long long S = ((long long)p.k_total + KT - 1) / KT;
-    const long long units = tiles * S;
+    // K slices: every slice but the last is k_slice long, the last takes the rest of K
+    const long long k_first = p.split ? p.k_slice : p.k_total;
+    const long long k_last = p.split ? (long long)p.k_total - (long long)(p.nz - 1) * p.k_slice : p.k_total;
+    if (p.split && (p.k_slice < KT || k_last < KT)) return hipErrorOutOfMemory;   // slices shorter than a stage
+    const long long S = (k_first + KT - 1) / KT, S_last = (k_last + KT - 1) / KT;
+    const long long tiles_before = p.split ? (long long)p.tiles_m * p.tiles_n * (p.nz - 1) : tiles;
+    const long long units = tiles_before * S + (tiles - tiles_before) * S_last;
     if (tiles <= 0 || S <= 0) return hipErrorInvalidValue;
     if (units > 0x3fffffffLL) return hipErrorOutOfMemory;
     gemm_fill_tile_divisors(p);
@@ -402,17 +441,25 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     p.sk_ws = ws + SK_MAX_TILES;
     p.sk_S = (int)S;
     gemm_magic_divisor((unsigned)S, p.sk_div_S_mul, p.sk_div_S_shift);
+    p.sk_S_last = (int)S_last;
+    p.sk_T1 = (int)tiles_before;
+    gemm_magic_divisor((unsigned)S_last, p.sk_div_Sl_mul, p.sk_div_Sl_shift);
     p.sk_q = (int)(units / grid);
     p.sk_rem = (int)(units % grid);
     if constexpr (CAN_BIAS) {
         if (p.bias != nullptr) {
-            hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, true>), dim3((unsigned)grid),
-                               dim3(NTHREADS), 0, stream, p);
+            hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, true, false>),
+                               dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
             return hipGetLastError();
         }
     }
-    hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false>), dim3((unsigned)grid),
-                       dim3(NTHREADS), 0, stream, p);
+    if (p.split) {
+        hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false, true>),
+                           dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false, false>),
+                       dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -437,6 +484,7 @@ std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
 }  // namespace
 
 size_t gemm_streamk_workspace_floats(int num_cu) { return SK_MAX_TILES + (size_t)2 * num_cu * 128 * 128; }
+static_assert(GEMM_SK_WS_FLOATS_256CU == SK_MAX_TILES + (size_t)2 * 256 * 128 * 128, "the constant in the header");
 
 float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
     int dev = 0;
@@ -533,8 +581,8 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
 }
 
 hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream) {
-    size_t floats = 0;
-    float* ws = gemm_streamk_workspace(stream, &floats);
+    size_t floats = p.sk_ws_given_floats;
+    float* ws = p.sk_ws_given != nullptr ? p.sk_ws_given : gemm_streamk_workspace(stream, &floats);
     if (ws == nullptr) return hipErrorOutOfMemory;
     switch (variant) {
         case GEMM_NN: return launch_streamk_variant<true, false>(p, tile, stream, ws, floats);

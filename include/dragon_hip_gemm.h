@@ -19,10 +19,10 @@
  *   - Letters follow the reference: N = rows of C, M = columns of C, K = contraction.
  *   - Row-major FP32.  Addresses are device pointers owned by the caller, 16-byte
  *     aligned; no caller memory is freed or retained here.  The one thing the library allocates:
- *     for products with few tiles and a long K (at most two 64 x 64 tiles of C per compute
- *     unit) the first call on a stream makes a 32 MiB workspace that later calls on the same
- *     stream handle reuse (partial tiles of workgroups that share the K range of a tile pass
- *     through it); it is kept until the process ends, at most 64 of them exist, and none is
+ *     for large products (K from 768 on), for products with few tiles and a long K (at most two
+ *     64 x 64 tiles of C per compute unit) and for their split-K forms the first call on a stream
+ *     makes a 32 MiB workspace that later calls on the same stream handle reuse (partial tiles of
+ *     workgroups that share the K range of a tile pass through it); it is kept until the process ends, at most 64 of them exist, and none is
  *     ever made while the stream is being captured into a graph -- such a call runs the
  *     ordinary kernel instead, as does every call when the allocation fails.
  *   - C is overwritten (no alpha/beta).  Padded rows/columns of C receive exact zeros.
@@ -103,8 +103,11 @@ int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC,
  * CudaFloat32EngineBase.java:1565-1583); it is for callers that cannot allocate: code under HIP graph
  * capture, tight serving loops, harnesses that forbid device allocation.  Neither this call nor anything
  * it runs allocates or frees memory, and it enqueues kernels only (no memset).
- * Limit: (GridZ-1)*N*M <= 8 388 608 floats (32 MiB, held once per GPU until the process ends); beyond
- * it the call returns hipErrorOutOfMemory (2) and says so on stderr, without launching anything.
+ * Limit: (GridZ-1)*N*M <= 8 388 608 floats (32 MiB); beyond it the call returns hipErrorOutOfMemory (2)
+ * and says so on stderr, without launching anything.  The same array holds, behind the partials, the
+ * 32 MiB of arrival counters and pieces of shared tiles that the balanced kernel needs (the other entry
+ * points keep those per stream in allocated memory), so that this call runs the very kernels they run:
+ * 64 MiB in all, held once per GPU until the process ends.
  * All calls on one GPU share that workspace, which keeps the last call's partials: two calls that
  * overlap in time on one GPU (different streams or threads) race and must be ordered by the caller.
  * The first call on a device looks up the workspace's address (which may load the library's device

@@ -179,8 +179,8 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 1536, 1536, 1, 1536) == 19                   # 144 tiles of 128x128 for 256 units: 128x64
         assert ct(v, 4096, 4096, 1, 512) == P                     # a shorter K: a tile per workgroup, paired stages
         assert ct(v, 16384, 16384, 1, 1024) == P                  # more tiles than the balanced kernel counts
-    assert ct(T1, 256, 256, 128, 1024) == 21                      # a batch of 128 such products (the split-K entry
-    #                                                               chooses among the tile-per-workgroup kernels)
+    assert ct(T1, 256, 256, 128, 1024) == 21                      # the split-K weight gradient: 128 slices of 1024
+    #                                                               are tiles like 128 batches would be
     assert ct(NN, 1024, 64, 64, 1024) == 23                       # scores x V of the attention-shaped batch
     # A K that fits one LDS stage of 64 under a large C: the band kernel (24), from two tiles per compute unit on;
     # not for a K of 56 or less, rows of C off the 128-byte lines, or a C that leaves its tiles mostly empty

@@ -83,7 +83,7 @@ def test_split_k_equals_unsplit_within_tolerance(gpu, variant):
         assert rel_fro(C, oracle.SKbuf_summary(Cb0, C0, GZ - 1)) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [1, 6, 7, 9, 10, 11, 12, 14, 15, 16, 17, 256, 257, 262, 263, 265])
+@pytest.mark.parametrize("tile", [1, 6, 7, 9, 10, 11, 12, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 256, 257, 262, 263, 265])
 def test_split_k_with_every_stage_depth(gpu, tile):
     # K slices that are not multiples of the k stage (16 or 32), on forced tile shapes
     rng = np.random.default_rng(50 + tile)
@@ -94,6 +94,26 @@ def test_split_k_with_every_stage_depth(gpu, tile):
             C, Cbuf = run_sk(gpu, variant, A, B, 6, summary=False)
             C0, Cb0 = oracle.matMulSK(variant, 6, A, B)
             assert np.array_equal(C, C0) and np.array_equal(Cbuf, Cb0)
+    finally:
+        gpu.force_tile(-1)
+
+
+@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22, 23])
+@pytest.mark.parametrize("shape_gz", [((300, 260, 5000), 5), ((256, 256, 4100), 3), ((64, 200, 40000), 37),
+                                      ((520, 136, 2056), 2)])
+def test_k_slices_through_the_balanced_kernel(gpu, tile, shape_gz):
+    """The balanced kernel takes (K slice, tile) pairs as its tiles: the last slice is longer than the others
+    ((256, 256, 4100) in 3: 1360, 1360, 1380), runs cross from one slice into the next, and tiles shared by
+    several workgroups are put together from pieces.  Integer inputs: every partial is exact."""
+    (N, M, K), GZ = shape_gz
+    rng = np.random.default_rng(K + GZ + tile)
+    gpu.force_tile(tile)
+    try:
+        for variant in (NN, T1, T2):
+            A, B = logical_operands(variant, rng, N, M, K, dist="int")
+            C, Cbuf = run_sk(gpu, variant, A, B, GZ, summary=False)
+            C0, Cb0 = oracle.matMulSK(variant, GZ, A, B)
+            assert np.array_equal(C, C0) and np.array_equal(Cbuf, Cb0), (variant, shape_gz, tile)
     finally:
         gpu.force_tile(-1)
 
