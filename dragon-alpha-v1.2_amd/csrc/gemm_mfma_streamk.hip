@@ -540,16 +540,28 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
 // tile-per-workgroup kernel do, and the equal runs leave no unit idle in a last, partial round of tiles.  Measured
 // against the best tile-per-workgroup shape: 4096^3 918 against 934 us (95 % of the peak), 8192 x 4096 x 4096 1835 /
 // 1882, 3584^3 636 / 721, 3072^3 404 / 425, 2560^3 241 / 283-299, 2048^3 119 / 128, 1024 x 8192 x 1024 121 / 128;
-// level at K = 512 ... 1024 and behind below, where the plain tile kernels' shorter set-up counts.  Between the two
+// level at K = 512 ... 768 (within +-5 % either way over ten shapes), so the rule starts at 768.  From K = 256 on
+// one case is taken besides: 128 x 64 tiles that can be dealt whole, one to three each, to two workgroups per
+// unit (2048^2 x 512: 33.2 / 35.9; 8192 x 1024 x 512: 63.5 / 67.4; 2048^2 x 256: 19.2 / 20.4; 6144 x 2048 x 256:
+// 50.0 / 51.7).  Between the two
 // regimes (more than two 64 x 64 tiles per unit, fewer than one of 128 x 128) the tile is 128 x 64 or 64 x 128:
 // 1536^3 61 against 74 us, 1792^3 92 / 111.
 int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant) {
     if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
     const long long t64 = (long long)((rows + 63) / 64) * ((cols + 63) / 64) * nz;
-    if (k >= 768 && t64 > 2LL * num_cu) {
+    if (k >= 256 && t64 > 2LL * num_cu) {
         const long long rm = (rows + 127) / 128, cn = (cols + 127) / 128, rm64 = (rows + 63) / 64, cn64 = (cols + 63) / 64;
         const double area = (double)rows * (double)cols;
         const long long t128 = rm * cn * nz;
+        if (k < 768) {
+            // a shorter K: 128 x 64 tiles, two workgroups per unit, where that deals whole tiles, up to three each
+            // (with four, 4096^2 x 512, the 128 x 128 tile-per-workgroup kernel is 1-2 % ahead again); other
+            // shapes measured within +-5 % of the best tile-per-workgroup shape either way and stay there
+            const long long th = rm * cn64 * nz;
+            if (th % (2LL * num_cu) == 0 && th <= 6LL * num_cu && area >= 0.85 * (double)(rm * 128) * (double)(cn64 * 64))
+                return TILE_SK_128x64_O2;
+            return -1;
+        }
         if (t128 >= num_cu && t128 <= SK_MAX_TILES && area >= 0.85 * (double)(rm * 128) * (double)(cn * 128))
             return TILE_SK_128x128;
         // the half-size tile that wastes less of C
