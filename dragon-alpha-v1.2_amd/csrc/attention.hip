@@ -60,19 +60,24 @@ struct AttnParams {
 
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
-// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32), 2 (d <= 64) or 4 (d <= 128);
+// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32), 2 (d <= 64), 4 (d <= 128) or 8
+// (d <= 256: one workgroup per compute unit, its query and output registers fill the register file);
 // KB = 32-key blocks per step;
 // MASK: the probabilities are multiplied by M[query, key] AFTER the softmax, as the block's mask unit does
 // (ChannelMHA.java:75-76: P = softmax(...); P = mask.forward(P)): the sum that normalises them runs over the
 // unmasked terms, the second product takes the masked ones.
 template <int DB, int KB, bool MASK>
-__global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnParams p) {
+__global__ __launch_bounds__(NTHREADS, DB > 4 ? 1 : 2) void attention_f32_mfma(const AttnParams p) {
     constexpr int AK = KB * 32;            // keys per step
     constexpr int DW = DB * 32;            // tile width in floats
     constexpr int CPR = DW / 4;            // 16-byte chunks per tile row
     constexpr int RPP = NTHREADS / CPR;    // tile rows staged per pass
     constexpr int PASSES = AK / RPP;       // = DB * KB
     constexpr int NG = DW / 8;             // groups of 8 d (4 MFMA steps each)
+    // DB = 8: the query and output registers leave no room for staging registers, so the K / V tiles go from
+    // global memory straight into the other LDS buffer (a lane's 16 bytes land at the wave's base + 16 * lane:
+    // the chunk swizzle of the K tile moves to the global side)
+    constexpr bool DMA = DB > 4;
     static_assert(PASSES * RPP == AK, "the key tile divides over the workgroup");
 
     __shared__ __attribute__((aligned(16))) float Ks[2][AK * DW];
@@ -102,7 +107,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
 
     // ---- staging of the K / V tiles ----
     const int s_chunk = t % CPR, s_row = t / CPR;
-    v4f kreg[PASSES], vreg[PASSES];
+    v4f kreg[DMA ? 1 : PASSES], vreg[DMA ? 1 : PASSES];
     // A lane's byte offsets inside a key tile never change (a chunk beyond the head dimension is out of
     // range for good).  The tile's first key goes into the buffer descriptor's base and the bytes up
     // to the end of the last key into its size, so the hardware returns zeros for rows beyond the key
@@ -111,9 +116,27 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
 #pragma unroll
     for (int s = 0; s < PASSES; s++) {
         const int row = s_row + s * RPP;
-        koff[s] = (s_chunk * 4 < p.dk4) ? (row * p.k_l + s_chunk * 4) * 4 : OOB_OFFSET;
+        const int kchunk = DMA ? (s_chunk ^ kin_swizzle<DW>(row)) : s_chunk;   // the chunk that belongs at this LDS slot
+        koff[s] = (kchunk * 4 < p.dk4) ? (row * p.k_l + kchunk * 4) * 4 : OOB_OFFSET;
         voff[s] = (s_chunk * 4 < p.dv4) ? (row * p.v_l + s_chunk * 4) * 4 : OOB_OFFSET;
     }
+    const unsigned lds_k = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float*)&Ks[0][0];
+    const unsigned lds_v = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float*)&Vs[0][0];
+    const unsigned lds_wave = __builtin_amdgcn_readfirstlane(wave) * 1024;
+    // DMA: the tiles of the step that starts at key0, into LDS buffer `into`
+    auto fetch_direct = [&](int key0, int into) {
+        const int left = p.nk - key0;   // > 0
+        const unsigned long long bk = (unsigned long long)(Kb + (size_t)key0 * p.k_l);
+        const unsigned long long bv = (unsigned long long)(Vb + (size_t)key0 * p.v_l);
+        const v4u rk = {(unsigned)bk, (unsigned)(bk >> 32) & 0xffffu, (unsigned)(left * p.k_l * 4), (unsigned)RSRC_FLAGS};
+        const v4u rv = {(unsigned)bv, (unsigned)(bv >> 32) & 0xffffu, (unsigned)(left * p.v_l * 4), (unsigned)RSRC_FLAGS};
+        const unsigned tile_bytes = into * (AK * DW * 4);
+        static_for<PASSES>([&](auto sc) {
+            constexpr int s = decltype(sc)::value;
+            dma_f4_lean<s * NTHREADS * 16>(rk, lds_k + tile_bytes + lds_wave, koff[s]);
+            dma_f4_lean<s * NTHREADS * 16>(rv, lds_v + tile_bytes + lds_wave, voff[s]);
+        });
+    };
     auto fetch = [&](int key0) {
         const int left = p.nk - key0;   // > 0
         const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
@@ -157,13 +180,21 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
     float m = -__builtin_inff(), l = 0.0f;      // reference maximum (shared by the halves), this half's sum
 
     const int steps = (p.nk + AK - 1) / AK;
-    fetch(0);
-    stage(0);
+    if constexpr (DMA) {
+        fetch_direct(0, 0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    } else {
+        fetch(0);
+        stage(0);
+    }
     __syncthreads();
     int buf = 0;
     for (int it = 0; it < steps; it++) {
         const bool more = it + 1 < steps;
-        if (more) fetch((it + 1) * AK);
+        if (more) {
+            if constexpr (DMA) fetch_direct((it + 1) * AK, buf ^ 1);   // nobody reads that buffer during this step
+            else fetch((it + 1) * AK);
+        }
         fetch_mask(it * AK);      // used behind the first product and the exponentials
         __builtin_amdgcn_sched_barrier(0);
 
@@ -249,7 +280,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attention_f32_mfma(const AttnPara
                     o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * DW + b * 32 + r], s[kb][v], o[b], 0, 0, 0);
             }
 
-        if (more) stage(buf ^ 1);
+        if constexpr (DMA) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // this wave's part of the next tiles has landed
+        else if (more) stage(buf ^ 1);
         __syncthreads();
         buf ^= 1;
     }
@@ -288,8 +320,8 @@ static int attention_launch(const int64_t* streams, int32_t length, int64_t dQ, 
     if (dQ == 0 || dK == 0 || dV == 0 || dY == 0 || !aligned16(dQ) || !aligned16(dK) || !aligned16(dV) ||
         !aligned16(dY))
         return hipErrorInvalidValue;
-    if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 128 ||
-        dV4 > 128 || !(scale - scale == 0.0f))   // NaN and the infinities fail the last test
+    if (N <= 0 || head <= 0 || QL <= 0 || VL <= 0 || dK4 <= 0 || dV4 <= 0 || (dK4 & 3) || (dV4 & 3) || dK4 > 256 ||
+        dV4 > 256 || !(scale - scale == 0.0f))   // NaN and the infinities fail the last test
         return hipErrorInvalidValue;
     if (dMask != 0 && (!aligned16(dMask) || mask_pitch < VL || (mask_pitch & 3) || (long long)mask_pitch * 4 >= 0x7ffffff0LL))
         return hipErrorInvalidValue;
@@ -320,15 +352,18 @@ static int attention_launch(const int64_t* streams, int32_t length, int64_t dQ, 
     p.c = scale * 1.44269504088896340736f;
     hipStream_t s = (hipStream_t)(intptr_t)streams[0];
     const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);
-    const int db = (dK4 <= 32 && dV4 <= 32) ? 1 : (dK4 <= 64 && dV4 <= 64) ? 2 : 4;
+    const int dmax = dK4 > dV4 ? dK4 : dV4;
+    const int db = dmax <= 32 ? 1 : dmax <= 64 ? 2 : dmax <= 128 ? 4 : 8;
     if (dMask == 0) {
         if (db == 1) hipLaunchKernelGGL((attention_f32_mfma<1, 2, false>), grid, block, 0, s, p);
         else if (db == 2) hipLaunchKernelGGL((attention_f32_mfma<2, 2, false>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((attention_f32_mfma<4, 1, false>), grid, block, 0, s, p);
+        else if (db == 4) hipLaunchKernelGGL((attention_f32_mfma<4, 1, false>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((attention_f32_mfma<8, 1, false>), grid, block, 0, s, p);
     } else {
         if (db == 1) hipLaunchKernelGGL((attention_f32_mfma<1, 2, true>), grid, block, 0, s, p);
         else if (db == 2) hipLaunchKernelGGL((attention_f32_mfma<2, 2, true>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((attention_f32_mfma<4, 1, true>), grid, block, 0, s, p);
+        else if (db == 4) hipLaunchKernelGGL((attention_f32_mfma<4, 1, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((attention_f32_mfma<8, 1, true>), grid, block, 0, s, p);
     }
     return hipGetLastError();
 }

@@ -168,7 +168,7 @@ __device__ __forceinline__ int next_tile(int lid, int G, int full_end, int total
 // contiguous run.
 template <int KT>
 __device__ __forceinline__ int kin_swizzle(int row) {
-    static_assert(KT == 16 || KT == 32 || KT == 64 || KT == 128, "k per stage: 16, 32, 64 or 128");
+    static_assert(KT == 16 || KT == 32 || KT == 64 || KT == 128 || KT == 256, "k per row: 16, 32, 64, 128 or 256");
     return (KT == 16) ? ((row >> 2) & 3) : (KT == 32) ? ((row >> 1) & 7) : (row & 15);
 }
 

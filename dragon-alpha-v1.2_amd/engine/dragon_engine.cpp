@@ -987,8 +987,8 @@ SyncerPtr EngineCore::attention(int64_t Y, int64_t Q, int64_t K, int64_t V, int 
         if (head > 1 && ((dK & 3) || (dV & 3)))
             throw IllegalArgumentException("with several heads the head dimensions { got " + s(dK) + ", " + s(dV) +
                                            " } must be multiples of 4");
-        if (pad4(dK) > 128 || pad4(dV) > 128)
-            throw IllegalArgumentException("head dimensions { got " + s(dK) + ", " + s(dV) + " } must <= 128");
+        if (pad4(dK) > 256 || pad4(dV) > 256)
+            throw IllegalArgumentException("head dimensions { got " + s(dK) + ", " + s(dV) + " } must <= 256");
     }
     if (check && Mask != 0 && mask_width != VL)
         throw IllegalArgumentException("mask.width { got " + std::to_string(mask_width) + " } != V.seq_len { got " +

@@ -398,7 +398,7 @@ public:
     // The attention block of ChannelMHA (nn/unit/complex/block/ChannelMHA.java:66-83) in one launch:
     // Q[N, QL, KC], K[N, VL, KC], V[N, VL, VC] hold `head` heads side by side in their last dimension;
     // Y[N, QL, VC] = per head softmax(scale * Q.K^T).V.  scale = 0 means the block's own 1/sqrt(KC).
-    // Needs KC/head and VC/head <= 128 (and multiples of 4 when head > 1); other shapes take the operator
+    // Needs KC/head and VC/head <= 256 (and multiples of 4 when head > 1); other shapes take the operator
     // chain (transpose, batchMatMulT2, softmax_scaled, batchMatMul, transpose).  Not a Java method.
     // mask (optional): a tensor [QL, VL] (one for every image and head) or [N, head, QL, VL] that multiplies the
     // probabilities after the softmax, which is what the block does with a mask unit that multiplies element by

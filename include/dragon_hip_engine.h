@@ -130,7 +130,7 @@ int32_t dragon_policy_conv3D_GEMM_nstream(int32_t GM, int32_t OC);
 /* The attention block of nn/unit/complex/block/ChannelMHA.java:66-83 in one launch: Q[N, QL, KC],
  * K[N, VL, KC], V[N, VL, VC] with `head` heads side by side in the last dimension ->
  * Y[N, QL, VC] = per head softmax(scale * Q.K^T).V; scale = 0 selects the block's 1/sqrt(KC).
- * KC/head and VC/head must be <= 128 and, with several heads, multiples of 4 (IllegalArgumentException
+ * KC/head and VC/head must be <= 256 and, with several heads, multiples of 4 (IllegalArgumentException
  * otherwise: such shapes take the operator chain).  Not a Java method. */
 dragon_tensor* dragon_engine_attention(dragon_engine* eg, dragon_tensor* Q, dragon_tensor* K, dragon_tensor* V,
                                        int32_t head, float scale);

@@ -80,7 +80,9 @@ SHAPES = [  # N, head, QL, VL, dk, dv
     (1, 1, 1, 1, 4, 4), (2, 3, 37, 29, 20, 20), (1, 2, 128, 128, 64, 64), (2, 2, 130, 257, 64, 64),
     (1, 4, 300, 31, 32, 32), (1, 1, 64, 1000, 61, 64), (3, 1, 5, 33, 7, 40), (1, 2, 129, 64, 40, 12),
     (1, 1, 255, 96, 64, 8), (1, 2, 100, 150, 128, 128), (1, 1, 70, 90, 96, 72), (2, 1, 33, 65, 100, 128),
-    (1, 1, 129, 40, 16, 125)]
+    (1, 1, 129, 40, 16, 125),
+    # head dimensions above 128: eight 32-wide blocks per query, one workgroup per compute unit
+    (1, 2, 130, 70, 132, 132), (2, 1, 100, 257, 256, 256), (1, 1, 64, 64, 192, 40), (1, 3, 37, 90, 20, 200)]
 
 
 @pytest.mark.parametrize("head_inner", [0, 1])
@@ -198,7 +200,7 @@ def test_attention_argument_errors(dh, gpu):
                                   g["QL"], g["VL"], g["dK4"], g["dV4"], g["hi"], g["scale"])
     call()
     for bad in (dict(dQ=0), dict(dK=0), dict(dV=0), dict(dY=0), dict(dQ=a + 4), dict(N=0), dict(head=0), dict(QL=0),
-                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=132), dict(dV4=256), dict(scale=float("nan")), dict(scale=float("inf")),
+                dict(VL=0), dict(dK4=6), dict(dV4=0), dict(dK4=260), dict(dV4=512), dict(scale=float("nan")), dict(scale=float("inf")),
                 dict(length=0), dict(length=11)):
         with pytest.raises(dh.CudaException) as e:
             call(**bad)
@@ -259,7 +261,7 @@ def test_engine_attention_error_behaviour(eg):
     with pytest.raises(IllegalArgumentException):
         eg.attention(tQ, tK, eg.zeros(2, 10, 24), 1)           # K.seq_len != V.seq_len
     with pytest.raises(IllegalArgumentException):
-        eg.attention(eg.zeros(2, 8, 136), eg.zeros(2, 9, 136), tV, 1)   # head dimension above 128
+        eg.attention(eg.zeros(2, 8, 260), eg.zeros(2, 9, 260), tV, 1)   # head dimension above 256
     with pytest.raises(NullPointerException):
         eg.attention(None, tK, tV, 1)
     assert eg.attention(tQ, tK, tV, 2).dim == [2, 8, 24]
@@ -303,7 +305,7 @@ def run_attention_masked(dh, Q, K, V, M, scale, head_inner, garbage_pad=False):
 
 
 MASKED_SHAPES = [(1, 1, 1, 1, 4, 4), (2, 3, 37, 29, 20, 20), (1, 2, 128, 128, 64, 64), (2, 2, 130, 257, 64, 64),
-                 (1, 2, 200, 333, 128, 96), (3, 1, 65, 64, 32, 8), (1, 4, 300, 70, 12, 100)]
+                 (1, 2, 200, 333, 128, 96), (3, 1, 65, 64, 32, 8), (1, 4, 300, 70, 12, 100), (1, 2, 70, 100, 160, 256)]
 
 
 @pytest.mark.parametrize("head_inner", [False, True])
