@@ -145,8 +145,8 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
 size_t gemm_streamk_workspace_floats(int num_cu);
 constexpr size_t GEMM_SK_WS_FLOATS_256CU = 4096 + (size_t)2 * 256 * 128 * 128;
 // The workspace of `stream` on the current device: arrival counters and the slots for pieces of shared tiles.
-// Made at the first balanced launch on that stream (never while the stream is capturing: then nullptr) and kept
-// for later launches on the same handle until the process ends.
+// Made at the first balanced launch on that stream and kept for later launches on the same handle until the
+// process ends; nullptr while the stream is capturing (a graph's launches may run next to the stream's own).
 float* gemm_streamk_workspace(hipStream_t stream, size_t* floats);
 // The band kernel (tile id TILE_BAND_128x128) for the three products, batched too, with K <= 64.
 // hipErrorOutOfMemory says that the product cannot go this way (a longer K, K slices, a bias row) and the

@@ -489,17 +489,19 @@ static_assert(GEMM_SK_WS_FLOATS_256CU == SK_MAX_TILES + (size_t)2 * 256 * 128 * 
 float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    // Not under a stream capture: nothing may be allocated there, and a graph may later be launched on ANOTHER
+    // stream, next to eager launches that use this stream's workspace -- two launches on one workspace at a
+    // time would mix their pieces.  The caller takes the tile-per-workgroup kernel instead.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     auto it = g_ws.find({dev, stream});
     if (it != g_ws.end()) {
         *floats = it->second.floats;
         return it->second.ptr;
-    }
-    // never allocate under a stream capture: the caller takes the tile-per-workgroup kernel instead
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-        (void)hipGetLastError();
-        return nullptr;
     }
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return nullptr;

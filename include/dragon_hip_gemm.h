@@ -22,9 +22,10 @@
  *     for large products (K from 768 on), for products with few tiles and a long K (at most two
  *     64 x 64 tiles of C per compute unit) and for their split-K forms the first call on a stream
  *     makes a 32 MiB workspace that later calls on the same stream handle reuse (partial tiles of
- *     workgroups that share the K range of a tile pass through it); it is kept until the process ends, at most 64 of them exist, and none is
- *     ever made while the stream is being captured into a graph -- such a call runs the
- *     ordinary kernel instead, as does every call when the allocation fails.
+ *     workgroups that share the K range of a tile pass through it); it is kept until the process
+ *     ends, at most 64 of them exist, and none is made or used while the stream is being
+ *     captured into a graph -- such a call runs the ordinary kernel instead, as does every call
+ *     when the allocation fails.
  *   - C is overwritten (no alpha/beta).  Padded rows/columns of C receive exact zeros.
  *   - streams[0..length) are valid stream handles, 1 <= length <= 10.  Work is issued
  *     asynchronously on streams[0]; the other handles are left idle (the caller joins
