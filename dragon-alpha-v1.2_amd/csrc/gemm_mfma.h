@@ -143,7 +143,7 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
 // Floats of a balanced-kernel workspace for a device of num_cu compute units (GEMM_SK_WS_FLOATS_256CU: the
 // same for 256 units, as a constant for static storage)
 size_t gemm_streamk_workspace_floats(int num_cu);
-constexpr size_t GEMM_SK_WS_FLOATS_256CU = 4096 + (size_t)2 * 256 * 128 * 128;
+constexpr size_t GEMM_SK_WS_FLOATS_256CU = 65536 + (size_t)2 * 256 * 128 * 128;
 // The workspace of `stream` on the current device: arrival counters and the slots for pieces of shared tiles.
 // Made at the first balanced launch on that stream and kept for later launches on the same handle until the
 // process ends; nullptr while the stream is capturing (a graph's launches may run next to the stream's own).

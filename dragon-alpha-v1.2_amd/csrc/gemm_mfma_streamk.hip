@@ -33,7 +33,7 @@
 namespace dragon {
 namespace {
 
-constexpr int SK_MAX_TILES = 4096;   // arrival counters at the head of the workspace
+constexpr int SK_MAX_TILES = 65536;   // arrival counters at the head of the workspace
 constexpr size_t SK_MAX_WORKSPACES = 64;
 
 // first unit of workgroup w: the first `rem` workgroups take q+1 units, the others q
