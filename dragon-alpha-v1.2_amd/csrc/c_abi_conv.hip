@@ -79,6 +79,14 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     // the paired-stage form pays later here than in the plain products (the gathering loader needs the
     // registers): 3-5 % faster on 7x7x64 and 3x3x512 filters, 4-8 % slower on 3x3x64 and 1x1x256
     if (free_choice && GK >= 3072 && tile != TILE_256x64 && tile != TILE_64x256) tile |= TILE_PAIRED;
+    // Large layers whose output channels fill 128-wide tiles take the balanced kernel (the gather staged straight
+    // into LDS, a filter tap at a time; channels in multiples of 32): 3x3 layers with 128 ... 512 channels 5 - 13 %
+    // faster (290 -> 276, 298 -> 267, 302 -> 263 us), level for a K below 768, and behind with 64 output
+    // channels, where its 128 x 64 tiles lose to the paired tile-per-workgroup kernel (823 against 782 us on the
+    // 7x7 layer).  gemm_launch_conv falls back where the stream has no workspace and may not make one.
+    if (free_choice && (IC & 31) == 0 && FH <= 32 && FW <= 32 &&
+        gemm_choose_streamk(p.rows, p.cols, 1, p.k_total, num_cu, GEMM_T2) == TILE_SK_128x128)
+        tile = TILE_SK_128x128;
     return gemm_launch_conv(p, tile, (hipStream_t)(intptr_t)streams[0]);
 }
 

@@ -76,6 +76,12 @@ struct GemmParams {
     int cv_IH, cv_IW, cv_IC, cv_FW, cv_OH, cv_OW, cv_sh, cv_sw, cv_ph, cv_pw;
     float cv_rcp_IC, cv_rcp_FW;
     int cv_walk;          // 1: visit the K chunks filter-column fastest (see the kernel), 0: in storage order
+    // filled by the launcher of the balanced kernel's convolution form (gemm_launch_streamk_conv): filter rows,
+    // LDS stages per filter tap (IC / 32), the bytes the lanes' offsets are raised by so that a pixel above or left
+    // of the image still has a non-negative one, and multiply-and-shift pairs for OW, OH, cv_spt and FW
+    int cv_FH, cv_spt, cv_bias;
+    unsigned cv_div_OW_mul, cv_div_OW_shift, cv_div_OH_mul, cv_div_OH_shift;
+    unsigned cv_div_spt_mul, cv_div_spt_shift, cv_div_FW_mul, cv_div_FW_shift;
     const float* bias;      // optional row vector added to C[i][j] for i < bias_rows, j < bias_width
     int bias_rows, bias_width;
     int tiles_m, tiles_n;   // filled by the launcher
@@ -144,6 +150,10 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
 // same for 256 units, as a constant for static storage)
 size_t gemm_streamk_workspace_floats(int num_cu);
 constexpr size_t GEMM_SK_WS_FLOATS_256CU = 65536 + (size_t)2 * 256 * 128 * 128;
+// The forward convolution (A gathered from the image, see ConvDirect) through the balanced kernel, for channel
+// counts that are multiples of 32 and filters of at most 32 x 32; hipErrorOutOfMemory as above (then
+// gemm_launch_conv takes over).
+hipError_t gemm_launch_streamk_conv(const GemmParams& p, int tile, hipStream_t stream);
 // The workspace of `stream` on the current device: arrival counters and the slots for pieces of shared tiles.
 // Made at the first balanced launch on that stream and kept for later launches on the same handle until the
 // process ends; nullptr while the stream is capturing (a graph's launches may run next to the stream's own).

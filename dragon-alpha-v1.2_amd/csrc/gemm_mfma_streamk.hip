@@ -109,16 +109,69 @@ __device__ __forceinline__ void mfma_group_with(v16f (&acc)[NACC][TM][TN], const
     });
 }
 
+// The A operand of the forward convolution, gathered from the image X[N, IH, IW, IC] straight into LDS, for
+// channel counts that are multiples of KT: a stage then lies inside one filter tap (fh, fw), which is the same
+// for every lane.  off[s] is the lane's byte offset for tap (0, 0), channel 0, measured from cv_bias bytes BELOW
+// X, so that a pixel above or left of the image -- which a later tap moves inside -- still has a non-negative
+// one; bit f of vh[s] / vw[s] says whether filter row / column f reads inside the image for the lane's pixel.
+// Per tap the lanes are left with a shift, an and and a select per transfer; the tap's own offset travels in
+// the descriptor's base.
+template <int R, int KT>
+struct ConvDirect {
+    static constexpr int CPR = KT / 4;
+    static constexpr int RPP = NTHREADS / CPR;
+    static constexpr int PASSES = R / RPP;
+    static constexpr int LDS_FLOATS = R * KT;
+    static_assert(R % RPP == 0 && PASSES >= 1, "tile does not divide over the workgroup");
+    int off[PASSES];
+    unsigned vh[PASSES], vw[PASSES];
+
+    // bits [lo, hi) set, 0 <= lo, hi <= 32
+    __device__ __forceinline__ static unsigned bit_range(int lo, int hi) {
+        if (hi <= lo) return 0u;
+        const unsigned upto_hi = hi >= 32 ? 0xffffffffu : ((1u << hi) - 1u);
+        return upto_hi & ~((1u << lo) - 1u);
+    }
+    __device__ __forceinline__ void init_conv(int t, int row0, int gm, const GemmParams& p) {
+        const int slot = t % CPR, r0 = t / CPR;
+#pragma unroll
+        for (int s = 0; s < PASSES; s++) {
+            const int rr = r0 + s * RPP;                       // LDS row = tile row
+            const int c = slot ^ kin_swizzle<KT>(rr);          // the chunk that belongs at this LDS slot
+            const int m = row0 + rr;
+            const int q = div_by(m, p.cv_div_OW_mul, p.cv_div_OW_shift), ow = m - q * p.cv_OW;
+            const int n = div_by(q, p.cv_div_OH_mul, p.cv_div_OH_shift), oh = q - n * p.cv_OH;
+            const int ih0 = oh * p.cv_sh - p.cv_ph, iw0 = ow * p.cv_sw - p.cv_pw;
+            off[s] = (((n * p.cv_IH + ih0) * p.cv_IW + iw0) * p.cv_IC + c * 4) * 4 + p.cv_bias;
+            // filter row f reads image row ih0 + f: inside for max(0, -ih0) <= f < min(FH, IH - ih0)
+            vh[s] = m < gm ? bit_range(max(0, -ih0), min(p.cv_FH, p.cv_IH - ih0)) : 0u;
+            vw[s] = bit_range(max(0, -iw0), min(p.cv_FW, p.cv_IW - iw0));
+        }
+    }
+    __device__ __forceinline__ int tap_offset(int s, int fh, int fw) const {
+        return (((vh[s] >> fh) & (vw[s] >> fw)) & 1u) ? off[s] : OOB_OFFSET;
+    }
+    // the interface of the other loaders where the kernel's common code names it (never reached for a gather)
+    __device__ __forceinline__ void init_dma(int, int, int, int) {}
+    __device__ __forceinline__ int dma_offset(int s, int) const { return off[s]; }
+    __device__ __forceinline__ static const float* tile_base(const float* X, int, int, int) { return X; }
+    __device__ __forceinline__ static size_t k_advance(int) { return KT; }
+};
+
 // SPLIT: the tiles are (K slice, tile of C) pairs of a split-K launch; the tiles of the last slice, which takes
 // the remainder of K, have their own stage count (they come last in the tile order), and a tile's K limits
 // count from the slice's first k.
-template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC, bool BIAS, bool SPLIT>
+// CONV: A is gathered from an image (ConvDirect), B holds the filters K-inner, C is the output image.
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC, bool BIAS, bool SPLIT,
+          bool CONV = false>
 __global__ __launch_bounds__(NTHREADS, OCC)
 void gemm_f32_mfma_streamk(const GemmParams p) {
+    static_assert(!CONV || (A_KIN && B_KIN && !SPLIT), "the convolution is an A * B^T product, unsplit");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     static_assert(NS == 3 || NS == 4, "stage buffers: 3 or 4 (deeper ones measured slower)");
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    using LoadA = typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type;
+    using LoadA = typename std::conditional<CONV, ConvDirect<BM, KT>,
+                  typename std::conditional<A_KIN, KInner<BM, KT>, KOuter<BM, KT>>::type>::type;
     using LoadB = typename std::conditional<B_KIN, KInner<BN, KT, TN>, KOuter<BN, KT>>::type;
     constexpr int STAGE_FLOATS = LoadA::LDS_FLOATS + LoadB::LDS_FLOATS;
     constexpr unsigned STAGE_BYTES = STAGE_FLOATS * 4;
@@ -187,8 +240,17 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     TileCtx ft = decode(f_tile);
     LoadA la;
     LoadB lb;
-    la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+    if constexpr (CONV) la.init_conv(t, ft.row0, p.a_outer, p);
+    else la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
     lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
+    // CONV: the filter tap the producer is in and the stage inside it (cv_spt stages of KT channels per tap)
+    int f_fh = 0, f_fw = 0, f_ic = 0;
+    if constexpr (CONV) {
+        const int tap = div_by(f_it, p.cv_div_spt_mul, p.cv_div_spt_shift);
+        f_ic = f_it - tap * p.cv_spt;
+        f_fh = div_by(tap, p.cv_div_FW_mul, p.cv_div_FW_shift);
+        f_fw = tap - f_fh * p.cv_FW;
+    }
     v4u rsrc_a = dma_descriptor(ft.a_ptr + (size_t)f_it * LoadA::k_advance(p.lda));
     v4u rsrc_b = dma_descriptor(ft.b_ptr + (size_t)f_it * LoadB::k_advance(p.ldb));
     int offa[PA], offb[PB];           // the lanes' offsets for the stage to fetch
@@ -207,19 +269,29 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
                 f_tile++;
                 if constexpr (SPLIT) f_S = stages_of(f_tile);
                 ft = decode(f_tile);
-                la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
+                if constexpr (CONV) la.init_conv(t, ft.row0, p.a_outer, p);
+                else la.init_dma(t, ft.row0, A_KIN ? p.a_outer : p.a_inner, p.lda);
                 lb.init_dma(t, ft.col0, B_KIN ? p.b_outer : p.b_inner, p.ldb);
                 rsrc_a = dma_descriptor(ft.a_ptr);
                 rsrc_b = dma_descriptor(ft.b_ptr);
                 f_it = 0;
+                if constexpr (CONV) f_fh = f_fw = f_ic = 0;
             }
             f_interior = min(ft.ka_lim, ft.kb_lim) / KT;
             if (f_it < f_interior) {  // stages wholly inside K: no K test
+                if constexpr (CONV) {
+                    // the rest of the current tap: which lanes' pixels it reads, and where it starts
 #pragma unroll
-                for (int i = 0; i < PA; i++) offa[i] = la.off[i];
+                    for (int i = 0; i < PA; i++) offa[i] = la.tap_offset(i, f_fh, f_fw);
+                    rsrc_a = dma_descriptor(p.A + ((ptrdiff_t)(f_fh * p.cv_IW + f_fw) * p.cv_IC + f_ic * KT) - p.cv_bias / 4);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < PA; i++) offa[i] = la.off[i];
+                }
 #pragma unroll
                 for (int i = 0; i < PB; i++) offb[i] = lb.off[i];
                 f_span = min(f_interior - f_it, f_left);
+                if constexpr (CONV) f_span = min(f_span, p.cv_spt - f_ic);
             } else {                  // a stage that reaches beyond K: tested lane by lane, one stage at a time
 #pragma unroll
                 for (int i = 0; i < PA; i++) offa[i] = la.dma_offset(i, ft.ka_lim - f_it * KT);
@@ -243,6 +315,13 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
         if (--f_until == 0) {
             f_it += f_span;
             f_left -= f_span;
+            if constexpr (CONV) {
+                f_ic += f_span;
+                if (f_ic == p.cv_spt) {   // next tap
+                    f_ic = 0;
+                    if (++f_fw == p.cv_FW) { f_fw = 0; f_fh++; }
+                }
+            }
             look();
         }
     };
@@ -411,12 +490,13 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     }
 }
 
-template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC = 1>
+template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC = 1, bool CONV = false>
 static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws, size_t ws_floats) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    // the bias row exists for the forward product only (added where a tile is stored: once, by whoever holds
-    // the whole sum)
-    constexpr bool CAN_BIAS = A_KIN && !B_KIN;
+    // the bias row exists for the forward product and the convolution only (added where a tile is stored:
+    // once, by whoever holds the whole sum)
+    constexpr bool CAN_BIAS = (A_KIN && !B_KIN) || CONV;
+    if (CONV && p.split) return hipErrorOutOfMemory;
     if (p.bias != nullptr && (!CAN_BIAS || p.split)) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
@@ -448,10 +528,15 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     p.sk_rem = (int)(units % grid);
     if constexpr (CAN_BIAS) {
         if (p.bias != nullptr) {
-            hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, true, false>),
+            hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, true, false, CONV>),
                                dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
             return hipGetLastError();
         }
+    }
+    if constexpr (CONV) {
+        hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false, false, true>),
+                           dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
+        return hipGetLastError();
     }
     if (p.split) {
         hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false, true>),
@@ -592,6 +677,39 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
     const double t_balanced = t_two < t_one ? t_two : t_one;
     if (t_balanced > 0.97 * t_tiles) return -1;
     return t_two < t_one ? TILE_SK_64x64_O2 : TILE_SK_64x64;
+}
+
+hipError_t gemm_launch_streamk_conv(const GemmParams& p0, int tile, hipStream_t stream) {
+    GemmParams p = p0;
+    // a stage of 32 channels inside one filter tap; the taps' validity bits in one register each; every byte
+    // offset (the image's extent plus the bias that keeps offsets non-negative) below the out-of-range mark
+    if (p.cv_IC <= 0 || (p.cv_IC & 31) != 0 || p.cv_FW <= 0 || p.cv_FW > 32 || p.split) return hipErrorOutOfMemory;
+    const long long taps_k = (long long)p.cv_FW * p.cv_IC;
+    if (p.k_total <= 0 || p.k_total % taps_k != 0) return hipErrorInvalidValue;
+    p.cv_FH = (int)(p.k_total / taps_k);
+    if (p.cv_FH > 32) return hipErrorOutOfMemory;
+    const long long bias = ((long long)p.cv_ph * p.cv_IW + p.cv_pw) * p.cv_IC * 4;
+    // the image as far as the lanes' rows can reach: rows beyond the last output pixel (tile padding) are
+    // switched off by their validity bits, whatever their offset
+    const long long n_images = ((long long)p.rows + (long long)p.cv_OH * p.cv_OW - 1) / ((long long)p.cv_OH * p.cv_OW);
+    const long long extent = n_images * p.cv_IH * p.cv_IW * p.cv_IC * 4;
+    if (extent + 2 * bias + 4096 >= (long long)OOB_OFFSET) return hipErrorOutOfMemory;
+    p.cv_bias = (int)bias;
+    p.cv_spt = p.cv_IC / 32;
+    gemm_magic_divisor((unsigned)p.cv_OW, p.cv_div_OW_mul, p.cv_div_OW_shift);
+    gemm_magic_divisor((unsigned)p.cv_OH, p.cv_div_OH_mul, p.cv_div_OH_shift);
+    gemm_magic_divisor((unsigned)p.cv_spt, p.cv_div_spt_mul, p.cv_div_spt_shift);
+    gemm_magic_divisor((unsigned)p.cv_FW, p.cv_div_FW_mul, p.cv_div_FW_shift);
+    size_t floats = p.sk_ws_given_floats;
+    float* ws = p.sk_ws_given != nullptr ? p.sk_ws_given : gemm_streamk_workspace(stream, &floats);
+    if (ws == nullptr) return hipErrorOutOfMemory;
+    switch (tile) {
+        case TILE_SK_64x64:   return launch_streamk_cfg<true, true, 2, 2, 1, 1, 32, 4, 1, true>(p, stream, ws, floats);
+        case TILE_SK_128x64:  return launch_streamk_cfg<true, true, 2, 2, 2, 1, 32, 4, 1, true>(p, stream, ws, floats);
+        case TILE_SK_64x128:  return launch_streamk_cfg<true, true, 2, 2, 1, 2, 32, 4, 1, true>(p, stream, ws, floats);
+        case TILE_SK_128x128: return launch_streamk_cfg<true, true, 2, 2, 2, 2, 32, 4, 1, true>(p, stream, ws, floats);
+        default: return hipErrorOutOfMemory;   // the shapes with two workgroups per unit are not built for the gather
+    }
 }
 
 hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream) {

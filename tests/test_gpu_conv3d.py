@@ -110,7 +110,7 @@ def test_conv3D_matches_oracle(dh, gpu, geom):
     assert np.array_equal(Yi, oracle.conv3D(Xi, Wi, sh, sw, ph, pw))
 
 
-@pytest.mark.parametrize("tile", list(range(-1, 18)) + list(range(256, 266)))
+@pytest.mark.parametrize("tile", list(range(-1, 24)) + list(range(256, 266)))
 def test_conv3D_every_tile_shape(dh, gpu, tile):
     rng = np.random.default_rng(300 + tile)
     X = rng.integers(-3, 4, (3, 11, 9, 12)).astype(np.float32)
@@ -136,6 +136,34 @@ def test_conv3D_every_tile_shape_with_whole_channel_stages(dh, gpu, tile):
     finally:
         dh.force_tile(-1)
     assert np.array_equal(Y, oracle.conv3D(X, W, 1, 2, 1, 1))
+
+
+# IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw with channel counts that are multiples of 32
+BALANCED_GEOMS = [(9, 8, 3, 3, 2, 128, 40, 1, 2, 1, 1), (14, 14, 3, 3, 5, 64, 70, 1, 1, 1, 1), (7, 7, 1, 1, 9, 96, 130, 1, 1, 0, 0),
+                  (12, 10, 7, 7, 3, 32, 64, 2, 2, 3, 3), (6, 6, 5, 4, 2, 64, 12, 1, 1, 4, 3), (20, 20, 3, 3, 2, 32, 200, 3, 1, 0, 2)]
+
+
+@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22, 23])
+@pytest.mark.parametrize("geom", BALANCED_GEOMS)
+def test_conv3D_through_the_balanced_kernel(dh, gpu, tile, geom):
+    """The gathered operand staged straight into LDS, a filter tap at a time, by workgroups that share the tiles'
+    stages in equal runs (tiles 22 and 23 have no such form and fall back).  Integer inputs: bit for bit; with the
+    bias row: equal to the oracle's convolution plus the row."""
+    IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw = geom
+    rng = np.random.default_rng(sum(geom) + tile)
+    X = rng.integers(-3, 4, (N, IH, IW, IC)).astype(np.float32)
+    W = rng.integers(-3, 4, (OC, FH, FW, IC)).astype(np.float32)
+    bias = rng.integers(-5, 6, OC).astype(np.float32)
+    R = oracle.conv3D(X, W, sh, sw, ph, pw)
+    dh.force_tile(tile)
+    try:
+        Y, Yp = run_conv(dh, X, W, sh, sw, ph, pw)
+        Yb, _ = run_conv(dh, X, W, sh, sw, ph, pw, entry="biased", bias=bias)
+    finally:
+        dh.force_tile(-1)
+    assert np.array_equal(Y, R)
+    assert not Yp[N:].any() and not Yp[..., OC:].any()
+    assert np.array_equal(Yb, R + bias[None, None, None, :])
 
 
 @pytest.mark.parametrize("tile", [257, 260, 1])
