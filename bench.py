@@ -230,7 +230,7 @@ def main():
     rec_kernel = rec.get("per_launch", {}).get(slowest)
     variant_id = {"A*B": 0, "A^T*B": 1, "A*B^T": 2}[slowest]
     tile_id = dh.choose_tile(variant_id, n, n, 1, n, SM)
-    kernel_name = ("gemm_f32_mfma_streamk" if 18 <= tile_id < 24 else "gemm_f32_mfma_band" if tile_id == 24
+    kernel_name = ("gemm_f32_mfma_streamk" if 18 <= tile_id < 24 or tile_id == 25 else "gemm_f32_mfma_band" if tile_id == 24
                    else "gemm_f32_mfma_dma" if 15 <= tile_id < 18 else "gemm_f32_mfma")
     roofline = {"bound": "mfma", "kernel": "%s (tile id %d) %s 4096^3" % (kernel_name, tile_id, slowest),
                 "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",

@@ -42,12 +42,15 @@ enum GemmTile {
     // column tiles with the whole K in one stage and stores a tile while it multiplies the next
     // (gemm_mfma_band.hip)
     TILE_BAND_128x128 = 24,
+    // one more balanced shape: 256 x 64, four wavefronts of 64 x 64 one above the other, 3 stage buffers -- for a
+    // C of 64 columns, where it has the 128 x 128 tile's ratio of matrix work to LDS traffic
+    TILE_SK_256x64 = 25,
     // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
     // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
     // short K; gemm_choose_tile sets it.
     TILE_PAIRED = 0x100
 };
-inline bool gemm_tile_is_streamk(int tile) { return tile >= TILE_SK_64x64 && tile < TILE_SK_END; }
+inline bool gemm_tile_is_streamk(int tile) { return (tile >= TILE_SK_64x64 && tile < TILE_SK_END) || tile == TILE_SK_256x64; }
 inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128; }
 inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
 

@@ -557,6 +557,7 @@ static hipError_t launch_streamk_variant(const GemmParams& p, int tile, hipStrea
         case TILE_SK_128x128:   return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 2, 2, 32, 4, 1>(p, stream, ws, ws_floats);
         case TILE_SK_64x64_O2:  return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 1, 1, 32, 4, 2>(p, stream, ws, ws_floats);
         case TILE_SK_128x64_O2: return launch_streamk_cfg<A_KIN, B_KIN, 2, 2, 2, 1, 32, 3, 2>(p, stream, ws, ws_floats);
+        case TILE_SK_256x64:    return launch_streamk_cfg<A_KIN, B_KIN, 4, 1, 2, 2, 32, 3, 1>(p, stream, ws, ws_floats);
         default: return hipErrorInvalidValue;
     }
 }
@@ -708,6 +709,7 @@ hipError_t gemm_launch_streamk_conv(const GemmParams& p0, int tile, hipStream_t 
         case TILE_SK_128x64:  return launch_streamk_cfg<true, true, 2, 2, 2, 1, 32, 4, 1, true>(p, stream, ws, floats);
         case TILE_SK_64x128:  return launch_streamk_cfg<true, true, 2, 2, 1, 2, 32, 4, 1, true>(p, stream, ws, floats);
         case TILE_SK_128x128: return launch_streamk_cfg<true, true, 2, 2, 2, 2, 32, 4, 1, true>(p, stream, ws, floats);
+        case TILE_SK_256x64:  return launch_streamk_cfg<true, true, 4, 1, 2, 2, 32, 3, 1, true>(p, stream, ws, floats);
         default: return hipErrorOutOfMemory;   // the shapes with two workgroups per unit are not built for the gather
     }
 }

@@ -137,11 +137,11 @@ def _biased_both_ways(dh, A, B, bias, tile):
     return C1, C2
 
 
-@pytest.mark.parametrize("tile", list(range(-1, 24)) + list(range(256, 266)))
+@pytest.mark.parametrize("tile", list(range(-1, 24)) + [25] + list(range(256, 266)))
 def test_fused_bias_equals_two_launches_bitwise(dh, gpu, tile):
     rng = np.random.default_rng(1000 + tile)
     shapes = [(130, 203, 77), (1, 5, 300), (257, 64, 129)]
-    if 18 <= tile < 24:     # the balanced kernel: tiles whose sum is put together from several workgroups' pieces
+    if 18 <= tile < 24 or tile == 25:     # the balanced kernel: tiles whose sum is put together from several workgroups' pieces
         shapes += [(70, 130, 3001), (300, 260, 1030)]
     for (N, M, K) in shapes:
         A = rng.uniform(-1, 1, (N, K)).astype(np.float32)

@@ -143,7 +143,7 @@ BALANCED_GEOMS = [(9, 8, 3, 3, 2, 128, 40, 1, 2, 1, 1), (14, 14, 3, 3, 5, 64, 70
                   (12, 10, 7, 7, 3, 32, 64, 2, 2, 3, 3), (6, 6, 5, 4, 2, 64, 12, 1, 1, 4, 3), (20, 20, 3, 3, 2, 32, 200, 3, 1, 0, 2)]
 
 
-@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22, 23])
+@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22, 23, 25])
 @pytest.mark.parametrize("geom", BALANCED_GEOMS)
 def test_conv3D_through_the_balanced_kernel(dh, gpu, tile, geom):
     """The gathered operand staged straight into LDS, a filter tap at a time, by workgroups that share the tiles'

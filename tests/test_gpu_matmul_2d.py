@@ -20,7 +20,8 @@ TILES = {-1: "auto", 0: "128x128", 1: "64x64", 2: "256x64", 3: "64x256", 4: "128
          18: "balanced 64x64", 19: "balanced 128x64", 20: "balanced 64x128", 21: "balanced 128x128",
          22: "balanced 64x64 x2", 23: "balanced 128x64 x2",
          # a band of 128 rows of A held in LDS, the whole K (at most 64) in one stage; a longer K falls back
-         24: "band 128x128"}
+         24: "band 128x128",
+         25: "balanced 256x64"}
 # + 256: the paired-stage form of the shapes 0..9 (what the automatic choice takes for a long K)
 PAIRED = 256
 TILES.update({PAIRED + t: TILES[t] + " paired" for t in range(10)})

@@ -98,7 +98,7 @@ def test_split_k_with_every_stage_depth(gpu, tile):
         gpu.force_tile(-1)
 
 
-@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22, 23])
+@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22, 23, 25])
 @pytest.mark.parametrize("shape_gz", [((300, 260, 5000), 5), ((256, 256, 4100), 3), ((64, 200, 40000), 37),
                                       ((520, 136, 2056), 2)])
 def test_k_slices_through_the_balanced_kernel(gpu, tile, shape_gz):

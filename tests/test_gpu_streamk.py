@@ -14,7 +14,7 @@ from helpers import (NN, T1, T2, VARIANT_NAMES, assert_within_tolerance, logical
 
 pytestmark = pytest.mark.gpu
 
-BALANCED = {18: "64x64", 19: "128x64", 20: "64x128", 21: "128x128", 22: "64x64 x2", 23: "128x64 x2"}
+BALANCED = {18: "64x64", 19: "128x64", 20: "64x128", 21: "128x128", 22: "64x64 x2", 23: "128x64 x2", 25: "256x64"}
 
 
 @pytest.fixture(autouse=True)
