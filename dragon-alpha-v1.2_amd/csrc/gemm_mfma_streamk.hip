@@ -79,6 +79,28 @@ __device__ __forceinline__ void add_partial(v16f (&acc)[TM][TN], const float* sl
         }
 }
 
+// N pieces at a time: the loads of all of them are on their way before the first is added (the order of the
+// additions stays the order of the pieces).
+template <int N, int TM, int TN>
+__device__ __forceinline__ void add_partials(v16f (&acc)[TM][TN], const float* const (&slot)[N], int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const size_t at = (size_t)(((wave * TM + i) * TN + j) * 16) * 64 + lane;
+            float v[N][16];
+#pragma unroll
+            for (int k = 0; k < N; k++)
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    v[k][e] = __hip_atomic_load(slot[k] + at + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int k = 0; k < N; k++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][j][e] += v[k][e];
+        }
+}
+
 template <bool A_KIN, bool B_KIN, int TM, int TN, int BM, int BN, int KT>
 __device__ __forceinline__ void read_group(float (&fa)[TM][4], float (&fb)[TN][4], const float* as, const float* bs,
                                            int wm, int wn, int g, int r, int h) {
@@ -481,10 +503,17 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
         for (int ii = 0; ii < TM; ii++)
 #pragma unroll
             for (int jj = 0; jj < TN; jj++) acc[0][ii][jj] = (v16f)(0.0f);
-        for (int w2 = wa; w2 <= wb; w2++) {
+        auto piece_of = [&](int w2) __attribute__((always_inline)) -> const float* {
             const int w2_first_tile = tile_of(sk_first_unit(w2, p.sk_q, p.sk_rem));
-            add_partial<TM, TN>(acc[0], p.sk_ws + (size_t)(2 * w2 + (w2_first_tile == tile ? 0 : 1)) * (BM * BN), wave, lane);
+            return p.sk_ws + (size_t)(2 * w2 + (w2_first_tile == tile ? 0 : 1)) * (BM * BN);
+        };
+        // two at a time (four at a time made the compiler's code of the 64 x 64 kernel's main loop 5 % slower)
+        int w2 = wa;
+        for (; w2 + 1 <= wb; w2 += 2) {
+            const float* const two[2] = {piece_of(w2), piece_of(w2 + 1)};
+            add_partials<2, TM, TN>(acc[0], two, wave, lane);
         }
+        if (w2 <= wb) add_partial<TM, TN>(acc[0], piece_of(w2), wave, lane);
         const TileCtx c = decode(tile);
         store_tile<A_KIN, B_KIN, TM, TN, BIAS>(acc[0], p, c.row0, c.col0, c.c_ptr, wm, wn, r, h);
     }
