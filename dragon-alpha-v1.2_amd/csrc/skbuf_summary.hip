@@ -9,7 +9,8 @@
 // HBM-bound: reads part*sizeC floats once.  The sum over the partials is a serial
 // chain per element, so the bytes in flight come from the elements: a C of at least
 // 1M floats uses one float4 per thread, a smaller one a single float per thread (four
-// times the threads), and the loads of 16 partials are issued ahead of the chain.
+// times the threads), and the loads of 16 partials (64 for a small C with 48 partials or more) are issued ahead
+// of the chain.
 #include <hip/hip_runtime.h>
 #include "gemm_mfma.h"
 
@@ -25,12 +26,11 @@ __device__ __forceinline__ void kahan_step(V& v, V& c, V vbuf) {
     v = t;
 }
 
-template <typename V>
+template <typename V, int AHEAD>
 __global__ __launch_bounds__(256) void skbuf_summary_kernel(const float* __restrict__ Cbuf,
                                                             float* __restrict__ C,
                                                             int part, int nvec, size_t sizeC) {
     constexpr int W = sizeof(V) / sizeof(float);
-    constexpr int AHEAD = 16;
     const int stride = gridDim.x * blockDim.x;
     for (int iv = blockIdx.x * blockDim.x + threadIdx.x; iv < nvec; iv += stride) {
         const size_t at = (size_t)iv * W;
@@ -67,12 +67,19 @@ hipError_t skbuf_summary_launch(hipStream_t stream, const float* Cbuf, float* C,
         const int nvec = sizeC >> 2;
         int blocks = (nvec + threads - 1) / threads;
         if (blocks > 65536) blocks = 65536;
-        hipLaunchKernelGGL(skbuf_summary_kernel<v4f>, dim3(blocks), dim3(threads), 0, stream, Cbuf,
+        hipLaunchKernelGGL((skbuf_summary_kernel<v4f, 16>), dim3(blocks), dim3(threads), 0, stream, Cbuf,
                            C, part, nvec, (size_t)sizeC);
     } else {
         const int blocks = (sizeC + threads - 1) / threads;
-        hipLaunchKernelGGL(skbuf_summary_kernel<float>, dim3(blocks), dim3(threads), 0, stream, Cbuf,
-                           C, part, sizeC, (size_t)sizeC);
+        // many partials of a small C (the tall-K weight gradient: 127 x 65536): few elements, so each thread keeps
+        // 64 loads on their way (8.8 -> 6.4 us); the remainder's loads are predicated one by one, which a short
+        // fold does not earn back (part = 1: 4.9 -> 12.8 us), so it keeps 16
+        if (part >= 48)
+            hipLaunchKernelGGL((skbuf_summary_kernel<float, 64>), dim3(blocks), dim3(threads), 0, stream, Cbuf,
+                               C, part, sizeC, (size_t)sizeC);
+        else
+            hipLaunchKernelGGL((skbuf_summary_kernel<float, 16>), dim3(blocks), dim3(threads), 0, stream, Cbuf,
+                               C, part, sizeC, (size_t)sizeC);
     }
     return hipGetLastError();
 }
