@@ -193,8 +193,9 @@ int dragon_Cuda_reduce_softmax2D(int64_t stream, int64_t dX, int64_t dY, int32_t
  * for QL queries and VL keys, head dimensions dK4 (Q, K) and dV4 (V, Y), both multiples of 4 and at
  * most 256 (pad columns of Q, K, V zero, as everywhere; the pad columns of Y get zeros).  Above 128 a
  * query's registers fill the register file and one workgroup runs per compute unit: there the call is
- * about as fast as the three-launch chain (batchMatMulT2, softmax2D with the scale, batchMatMul) and
- * saves that chain's score matrix; up to 128 it is 1.1 - 1.9 times faster than the chain.
+ * level with the three-launch chain (batchMatMulT2, softmax2D with the scale, batchMatMul) at 256 and
+ * behind it in between (the key tile is 256 wide whatever the dimension), and saves that chain's score
+ * matrix; up to 128 it is 1.4 - 1.9 times faster than the chain.
  * head_inner = 0: tensors laid out [N, head, L, d4] -- the operands of the reference's
  *                 batchMatMulT2 / batchMatMul after its transpose(1, 2);
  * head_inner = 1: tensors laid out [N, L, head, d4] (= [N, L, head*d4]) -- as the layer holds them
