@@ -657,16 +657,17 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
 // tile-per-workgroup kernel do, and the equal runs leave no unit idle in a last, partial round of tiles.  Measured
 // against the best tile-per-workgroup shape: 4096^3 918 against 934 us (95 % of the peak), 8192 x 4096 x 4096 1835 /
 // 1882, 3584^3 636 / 721, 3072^3 404 / 425, 2560^3 241 / 283-299, 2048^3 119 / 128, 1024 x 8192 x 1024 121 / 128;
-// level at K = 512 ... 768 (within +-5 % either way over ten shapes), so the rule starts at 768.  From K = 256 on
+// level at K = 512 ... 768 (within +-5 % either way over ten shapes), so the rule starts at 768.  From K = 96 on
 // one case is taken besides: 128 x 64 tiles that can be dealt whole, one to three each, to two workgroups per
 // unit (2048^2 x 512: 33.2 / 35.9; 8192 x 1024 x 512: 63.5 / 67.4; 2048^2 x 256: 19.2 / 20.4; 6144 x 2048 x 256:
-// 50.0 / 51.7).  Between the two
+// 50.0 / 51.7; K = 96 ... 192: batch 64 of 256 x 256 x 128 11.5 / 12.8, batch 16 of 512 x 512 x 192 15.1 / 17.2,
+// 2048^2 x 128 11.9 / 12.8, twelve such shapes 4 - 12 % ahead).  Between the two
 // regimes (more than two 64 x 64 tiles per unit, fewer than one of 128 x 128) the tile is 128 x 64 or 64 x 128:
 // 1536^3 61 against 74 us, 1792^3 92 / 111.
 int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant) {
     if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
     const long long t64 = (long long)((rows + 63) / 64) * ((cols + 63) / 64) * nz;
-    if (k >= 256 && t64 > 2LL * num_cu) {
+    if (k >= 96 && t64 > 2LL * num_cu) {
         const long long rm = (rows + 127) / 128, cn = (cols + 127) / 128, rm64 = (rows + 63) / 64, cn64 = (cols + 63) / 64;
         const double area = (double)rows * (double)cols;
         const long long t128 = rm * cn * nz;

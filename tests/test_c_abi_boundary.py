@@ -178,9 +178,9 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 4096, 4096, 1, 768) == 21 and ct(v, 3000, 3000, 1, 3000) == 21
         assert ct(v, 1536, 1536, 1, 1536) == 19                   # 144 tiles of 128x128 for 256 units: 128x64
         assert ct(v, 4096, 4096, 1, 512) == P                     # a shorter K: a tile per workgroup, paired stages
-        # ... except where 128x64 tiles can be dealt whole, one to three each, to two workgroups per unit (K >= 256)
+        # ... except where 128x64 tiles can be dealt whole, one to three each, to two workgroups per unit (K >= 96)
         assert ct(v, 2048, 2048, 1, 512) == 23 and ct(v, 8192, 1024, 1, 512) == 23 and ct(v, 6144, 2048, 1, 256) == 23
-        assert ct(v, 2048, 2048, 1, 128) != 23
+        assert ct(v, 2048, 2048, 1, 128) == 23 and ct(v, 256, 256, 64, 128) == 23 and ct(v, 2048, 2048, 1, 80) != 23
         assert ct(v, 16384, 16384, 1, 1024) == 21                 # 16384 tiles
         assert not 18 <= ct(v, 32768 + 128, 32768, 1, 1024) < 24  # more tiles than the balanced kernel has counters for
     assert ct(T1, 256, 256, 128, 1024) == 21                      # the split-K weight gradient: 128 slices of 1024
