@@ -1,6 +1,9 @@
-// The products for shapes with FEWER TILES THAN THE CHIP HAS COMPUTE UNITS (or barely more): one
-// workgroup per compute unit, and the work dealt out in equal runs of LDS stages instead of in
-// whole tiles.
+// The balanced kernel: one workgroup per compute unit (two in two of its shapes), and the work dealt out in
+// equal runs of LDS stages instead of in whole tiles.  Written for shapes with FEWER TILES THAN THE CHIP HAS
+// COMPUTE UNITS (or barely more), where whole tiles leave units idle; its stage loop, which carries no
+// vector-ALU instruction, turned out to be the fastest for large products as well (gemm_choose_streamk), and
+// it also runs the K slices of a split-K launch ((slice, tile) pairs as its tiles) and the forward
+// convolution (ConvDirect: the gathered operand staged a filter tap at a time).
 //
 // Unit of work = one LDS stage (KT k) of one tile; the tiles' stages are numbered tile by tile
 // (tile order of decode_tile) and workgroup w takes the contiguous run [u0(w), u0(w+1)), every run
