@@ -22,9 +22,12 @@ extern "C" {
  * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
  * directly through four stage buffers.  Adding 256 to a shape 0..9 selects its paired-stage form
  * (stages run two by two with compile-time LDS buffers; what the automatic choice takes from
- * K = 512 on).  18..23: the balanced kernel for few tiles and a long K (workgroups share the work
- * in equal runs of LDS stages): 18 = 64x64, 19 = 128x64, 20 = 64x128, 21 = 128x128 with one
- * workgroup per compute unit, 22 = 64x64 and 23 = 128x64 with two. */
+ * K = 512 on).  18..23 and 25: the balanced kernel (workgroups share the work in equal runs of LDS
+ * stages; taken for few tiles and a long K, for large products, their K slices and large
+ * convolutions): 18 = 64x64, 19 = 128x64, 20 = 64x128, 21 = 128x128 with one workgroup per
+ * compute unit, 22 = 64x64 and 23 = 128x64 with two, 25 = 256x64 with one.  24: the band kernel
+ * for a K of at most 64 under a large C (a band of 128 rows of A stays in LDS; a longer K falls
+ * back to the automatic choice). */
 void dragon_gemm_force_tile(int32_t tile);
 /* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
  * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the
