@@ -610,6 +610,9 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
     // Not under a stream capture: nothing may be allocated there, and a graph may later be launched on ANOTHER
     // stream, next to eager launches that use this stream's workspace -- two launches on one workspace at a
     // time would mix their pieces.  The caller takes the tile-per-workgroup kernel instead.
+    // Nor on the per-thread default stream: one handle that stands for a different stream in every host thread,
+    // whose launches may run side by side.
+    if (stream == hipStreamPerThread) return nullptr;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
         (void)hipGetLastError();
