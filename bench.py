@@ -148,8 +148,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,bias,attention,conv,hbm,transpose,transfer,engine",
-                    help="which of the other workloads to time (default all): BASELINE configs 3, 4, 5, "
+    ap.add_argument("--configs", default="3,4,5,sizes,bias,attention,conv,hbm,transpose,transfer,engine",
+                    help="which of the other workloads to time (default all): BASELINE configs 3, 4, 5, other sizes, "
                          "the biased fully-connected layer, the attention chain, the forward convolution, "
                          "dimension swaps, tensor upload / download, the host mirror's own overhead")
     ap.add_argument("--summarize-traffic", metavar="DIR", default=None,
@@ -393,6 +393,24 @@ def main():
             S, 1, da.address, db.address, dc.address, p4(Bt5), n5, p4(m5), k5, p4(k5)), iters=100)
         record("cfg5 batchMatMul batch33 257x129 by 129x385", 2.0 * Bt5 * n5 * m5 * k5, ms)
         for x in (da, db, dc):
+            x.free()
+
+    if "sizes" in extra:
+        # the three products at other sizes: smaller and larger squares, panels, a short and a medium K
+        log("other sizes ...")
+        shapes = [(1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (3072, 3072, 3072), (5120, 5120, 5120),
+                  (8192, 4096, 4096), (4096, 11008, 4096), (4096, 4096, 512), (2048, 2048, 256)]
+        na = max(r * k for r, c, k in shapes)
+        nb = max(k * c for r, c, k in shapes)
+        nc = max(r * c for r, c, k in shapes)
+        g = synthetic.stream_for(8)
+        dA, dB, dC = dh.DeviceArray(g.normal((na,), 0.0, 1.0)), dh.DeviceArray(g.normal((nb,), 0.0, 1.0)), dh.DeviceArray(size=nc)
+        for (r, c, k) in shapes:
+            assert r * k <= na and k * c <= nb and r * c <= nc
+            for name, fn in products:
+                ms = timer.per_launch_ms(lambda: fn(S, 1, dA.address, dB.address, dC.address, r, c, k), iters=20)
+                record("%s %dx%dx%d" % (name, r, c, k), 2.0 * r * c * k, ms)
+        for x in (dA, dB, dC):
             x.free()
 
     if "bias" in extra:
