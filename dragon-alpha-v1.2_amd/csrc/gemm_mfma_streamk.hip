@@ -677,6 +677,13 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
         const long long rm = (rows + 127) / 128, cn = (cols + 127) / 128, rm64 = (rows + 63) / 64, cn64 = (cols + 63) / 64;
         const double area = (double)rows * (double)cols;
         const long long t128 = rm * cn * nz;
+        // A batch whose products are up to 64 columns wide and give exactly one 256 x 64 tile per unit: that shape
+        // (the 128 x 128 tile's ratio of matrix work to LDS traffic) measured 0 - 5 % ahead of the 128 x 64 tiles
+        // dealt two per unit on batches of 1024 / 2048 / 4096 x 64 x 1024 (68.4-70.9 against 72.2-73.0 us,
+        // 67.1-67.4 / 67.5-68.0, 65.1-65.4 / 66.8-67.3), level at K = 2048, behind at K = 512 and for one product
+        if (nz > 1 && cols > 32 && cols <= 64 && k >= 768 && k <= 1536 && rows % 256 == 0 &&
+            (long long)(rows / 256) * nz == num_cu)
+            return TILE_SK_256x64;
         if (k < 768) {
             // a shorter K: 128 x 64 tiles, two workgroups per unit, where that deals whole tiles, up to three each
             // (with four, 4096^2 x 512, the 128 x 128 tile-per-workgroup kernel is 1-2 % ahead again); other

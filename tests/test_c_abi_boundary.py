@@ -185,7 +185,9 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert not 18 <= ct(v, 32768 + 128, 32768, 1, 1024) < 24  # more tiles than the balanced kernel has counters for
     assert ct(T1, 256, 256, 128, 1024) == 21                      # the split-K weight gradient: 128 slices of 1024
     #                                                               are tiles like 128 batches would be
-    assert ct(NN, 1024, 64, 64, 1024) == 23                       # scores x V of the attention-shaped batch
+    assert ct(NN, 1024, 64, 64, 1024) == 25                       # scores x V of the attention-shaped batch: one
+    #                                                               256x64 tile per unit
+    assert ct(NN, 1024, 64, 64, 2048) == 23 and ct(NN, 65536, 64, 1, 1024) == 23   # otherwise 128x64, two per unit
     # A K that fits one LDS stage of 64 under a large C: the band kernel (24), from two tiles per compute unit on;
     # not for a K of 56 or less, rows of C off the 128-byte lines, or a C that leaves its tiles mostly empty
     for v in (NN, T1, T2):
