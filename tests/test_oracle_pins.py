@@ -490,6 +490,37 @@ def test_attention_oracle_is_the_chain_and_matches_fp64():
     assert np.abs(oracle.attention(Q, K, V, 1.0) - V[0, 6]).max() <= 1e-6   # one key dominates: its row of V
 
 
+def test_attention_oracle_applies_the_mask_after_the_softmax():
+    # ChannelMHA.java:74-78: P = softmax(...); if (mask != null) P = mask.forward(P) -- the mask multiplies the
+    # probabilities, the rows are NOT normalised again.  Against that mathematics in FP64, and on cases that a
+    # mask applied before the softmax (the other common convention) would get wrong.
+    B, QL, VL, dk, dv, alpha = 2, 7, 13, 8, 5, 0.4
+    Q = RNG.standard_normal((B, QL, dk)).astype(np.float32)
+    K = RNG.standard_normal((B, VL, dk)).astype(np.float32)
+    V = RNG.standard_normal((B, VL, dv)).astype(np.float32)
+    ones = np.ones((QL, VL), np.float32)
+    assert np.array_equal(oracle.attention(Q, K, V, alpha, mask=ones), oracle.attention(Q, K, V, alpha))
+    causal = np.tril(np.ones((QL, VL), np.float32))
+    per_entry = RNG.uniform(0, 2, (B, QL, VL)).astype(np.float32)
+    S = np.einsum("bqd,bkd->bqk", Q.astype(np.float64), K.astype(np.float64)) * np.float64(np.float32(alpha))
+    P = np.exp(S - S.max(-1, keepdims=True))
+    P /= P.sum(-1, keepdims=True)
+    for M in (causal, per_entry):
+        R = np.einsum("bqk,bkd->bqd", P * np.broadcast_to(M, P.shape), V.astype(np.float64))
+        assert np.abs(oracle.attention(Q, K, V, alpha, mask=M) - R).max() <= 1e-5 * max(1.0, np.abs(V).max())
+    # a zero on the one key that holds all the probability: the output is (nearly) zero, where masking the
+    # score before the softmax would have handed the weight to the other keys
+    Q = np.zeros((1, 1, 4), np.float32); Q[..., 0] = 60.0
+    K = np.zeros((1, 9, 4), np.float32); K[0, 6, 0] = 1.0
+    V = np.ones((1, 9, 3), np.float32)
+    M = np.ones((1, 9), np.float32); M[0, 6] = 0.0
+    assert np.abs(oracle.attention(Q, K, V, 1.0, mask=M)).max() <= 1e-6
+    # a zero mask gives exact zeros; a mask of twos doubles the output exactly
+    assert not oracle.attention(Q, K, V, 1.0, mask=np.zeros((1, 9), np.float32)).any()
+    Y1 = oracle.attention(Q, K, V, 1.0)
+    assert np.array_equal(oracle.attention(Q, K, V, 1.0, mask=2 * np.ones((1, 9), np.float32)), 2 * Y1)
+
+
 def test_reference_micro_helpers_when_built():
     ref = oracle.load_ref()
     if ref is None:
