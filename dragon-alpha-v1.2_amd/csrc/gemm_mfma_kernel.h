@@ -569,16 +569,18 @@ __device__ __forceinline__ v4f rim_load4(const float* line, size_t sk, int k, in
     }
 }
 
-// acc[x] += sum over k in [k0, k1) of walk(k) * fixed[x](k): `walk` is the lane's own operand line (64 lanes,
-// 64 lines), the `fixed` ones are the same for every lane.  16 k per turn, the loads ahead of the FMAs.
-template <bool WALK_KIN, bool FIXED_KIN>
+// acc[x] += sum over k in [k0, k1) of walk(k) * fixed[x](k) for x < NX: `walk` is the lane's own operand line
+// (64 lanes, 64 lines), the `fixed` ones are the same for every lane.  16 k per turn, the loads ahead of the
+// FMAs.  NX = 1 for a rim of a single row or column (the commonest: an extent one past a multiple of 64): a
+// quarter of the loads and FMAs of NX = 4, and these vector instructions keep the SIMD's MFMAs waiting.
+template <bool WALK_KIN, bool FIXED_KIN, int NX>
 __device__ __forceinline__ void rim_dot(float (&acc)[4], const float* walk, size_t w_sk, const float* const (&fixed)[4],
                                         size_t f_sk, int k0, int k1, int k_end) {
 #pragma unroll 4
     for (int k = k0; k < k1; k += 4) {
         const v4f w = rim_load4<WALK_KIN>(walk, w_sk, k, k_end);
 #pragma unroll
-        for (int x = 0; x < 4; x++) {
+        for (int x = 0; x < NX; x++) {
             const v4f f = rim_load4<FIXED_KIN>(fixed[x], f_sk, k, k_end);
             acc[x] = fmaf(w.x, f.x, acc[x]);
             acc[x] = fmaf(w.y, f.y, acc[x]);
@@ -618,14 +620,16 @@ __device__ __forceinline__ void rim_job(const GemmParams& p, float* lds, int job
         const float* const fixed[4] = {A + (size_t)min(R0, a_rows - 1) * a_si, A + (size_t)min(R0 + (1 < rr ? 1 : 0), a_rows - 1) * a_si,
                                        A + (size_t)min(R0 + (2 < rr ? 2 : 0), a_rows - 1) * a_si,
                                        A + (size_t)min(R0 + (3 < rr ? 3 : 0), a_rows - 1) * a_si};
-        rim_dot<B_KIN, A_KIN>(acc, B + (ok ? (size_t)j * b_sj : 0), b_sk, fixed, a_sk, k0, k1, K);
+        if (rr == 1) rim_dot<B_KIN, A_KIN, 1>(acc, B + (ok ? (size_t)j * b_sj : 0), b_sk, fixed, a_sk, k0, k1, K);
+        else         rim_dot<B_KIN, A_KIN, 4>(acc, B + (ok ? (size_t)j * b_sj : 0), b_sk, fixed, a_sk, k0, k1, K);
     } else {            // the lane's row of A against columns C0 .. C0+rc-1 of B
         const int i = seg * 64 + lane;
         ok = i < R0 && i < a_rows;
         const float* const fixed[4] = {B + (size_t)min(C0, b_cols - 1) * b_sj, B + (size_t)min(C0 + (1 < rc ? 1 : 0), b_cols - 1) * b_sj,
                                        B + (size_t)min(C0 + (2 < rc ? 2 : 0), b_cols - 1) * b_sj,
                                        B + (size_t)min(C0 + (3 < rc ? 3 : 0), b_cols - 1) * b_sj};
-        rim_dot<A_KIN, B_KIN>(acc, A + (ok ? (size_t)i * a_si : 0), a_sk, fixed, b_sk, k0, k1, K);
+        if (rc == 1) rim_dot<A_KIN, B_KIN, 1>(acc, A + (ok ? (size_t)i * a_si : 0), a_sk, fixed, b_sk, k0, k1, K);
+        else         rim_dot<A_KIN, B_KIN, 4>(acc, A + (ok ? (size_t)i * a_si : 0), a_sk, fixed, b_sk, k0, k1, K);
     }
 #pragma unroll
     for (int x = 0; x < 4; x++) lds[(wave * 4 + x) * 64 + lane] = acc[x];
