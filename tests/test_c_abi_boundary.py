@@ -215,3 +215,29 @@ def test_tile_choice_on_the_documented_shapes(dh):
     assert ct(NN, 4096, 4096, 1, 4096) == 7                     # a forced shape is reported as it is
     dh.force_tile(-1)
     assert ct(NN, 0, 4, 1, 4) == -1
+
+
+def test_tile_choice_stays_inside_what_the_kernels_accept(dh):
+    # host arithmetic only, over random shapes: whatever the choice is, the chosen kernel can run it -- a
+    # balanced shape never has more tiles than the kernel has arrival counters, the band kernel only gets a K
+    # that fits its one stage, and every id is one that exists
+    rng = np.random.default_rng(20240607)
+    dims = {18: (64, 64), 19: (128, 64), 20: (64, 128), 21: (128, 128), 22: (64, 64), 23: (128, 64), 25: (256, 64)}
+    valid = set(range(0, 26)) | set(range(256, 266))
+    dh.force_tile(-1)
+    seen = set()
+    for _ in range(20000):
+        rows = int(rng.choice([4, 64, 256, 1000, 1024, 4096, 16384, 65536])) + int(rng.integers(0, 3)) * 4
+        cols = int(rng.choice([4, 64, 128, 780, 1024, 4096, 11008, 32768])) + int(rng.integers(0, 3)) * 4
+        nz = int(rng.choice([1, 1, 1, 2, 33, 64, 128, 1024]))
+        k = int(rng.choice([4, 60, 64, 96, 128, 132, 256, 512, 768, 1024, 4096, 131072]))
+        for v in (0, 1, 2):
+            t = dh.choose_tile(v, rows, cols, nz, k, 256)
+            assert t in valid, (v, rows, cols, nz, k, t)
+            seen.add(t)
+            if t in dims:
+                bm, bn = dims[t]
+                assert -(-rows // bm) * -(-cols // bn) * nz <= 65536, (v, rows, cols, nz, k, t)
+            if t == 24:
+                assert 56 < k <= 64 and cols % 32 == 0, (v, rows, cols, nz, k)
+    assert {21, 24} <= seen and seen & {18, 22} and seen & {19, 20, 23}      # the sample reaches every family
