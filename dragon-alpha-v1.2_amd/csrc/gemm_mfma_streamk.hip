@@ -712,6 +712,16 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
     if (units < 2LL * num_cu) return -1;
     const long long run1 = (units + num_cu - 1) / num_cu;
     const bool whole1 = t64 % num_cu == 0;
+    // Many tiles with a long K whose runs are not whole tiles: neighbouring workgroups then sit at different k of
+    // the same operand panels, nothing is shared through the L2, and 64 x 64 tiles -- 16 FLOP per byte staged --
+    // become bound by the fabric (1000 x 780 x 8192: 0.7 us per stage instead of 0.5).  The half-size tile stages
+    // a third fewer bytes per FLOP: 148 -> 110 us there, 768^2 x 8192 90 -> 79, 1280^2 x 4096 119 -> 105; with
+    // fewer tiles or a shorter K (640^2 x 4096, 512^2 x 16384, 1000 x 780 x 3072, 1536 x 768 x 2048) level or behind.
+    if (!whole1 && t64 >= num_cu / 2 && S >= 128) {
+        const long long rm = (rows + 127) / 128, cn = (cols + 127) / 128, rm64 = (rows + 63) / 64, cn64 = (cols + 63) / 64;
+        const bool tall = (double)(rm * 128) * (double)(cn64 * 64) <= (double)(rm64 * 64) * (double)(cn * 128);
+        return tall ? TILE_SK_128x64 : TILE_SK_64x128;
+    }
     const double pieces = run1 < S ? (double)S / (double)run1 : 0.0;
     const double t_one = (whole1 ? 3.0 : 7.5 + 0.4 * (pieces > 2.0 ? pieces - 2.0 : 0.0)) + 0.5 * (double)run1;
     const bool whole2 = t64 % (2LL * num_cu) == 0;

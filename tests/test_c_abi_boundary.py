@@ -204,6 +204,9 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 2048, 1024, 1, 512) == 22                  # 512 tiles: one whole tile for each of 512 workgroups
         assert ct(v, 256, 256, 1, 256) == 17 and ct(v, 512, 512, 1, 64) == 17   # too few stages to share out
     assert ct(NN, 1000, 780, 2, 760) == 18                      # a batch of two ragged products is balanced as one
+    # many tiles, a long K, runs that are not whole tiles: the half-size tile (fewer bytes staged per FLOP)
+    assert ct(NN, 1000, 780, 1, 8192) == 19 and ct(NN, 768, 768, 1, 8192) == 19 and ct(NN, 1280, 1280, 1, 4096) in (19, 20)
+    assert ct(NN, 640, 640, 1, 4096) == 18 and ct(NN, 1000, 780, 1, 3072) == 18 and ct(NN, 1024, 1024, 1, 4096) == 18
     assert ct(NN, 257, 388, 36, 129) == 1                       # batch of small ragged products: 64x64
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
