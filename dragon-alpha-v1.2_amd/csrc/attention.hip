@@ -60,20 +60,23 @@ struct AttnParams {
 
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
-// DB = 32-wide blocks of the head dimension held per query: 1 (d <= 32), 2 (d <= 64), 4 (d <= 128) or 8
-// (d <= 256: one workgroup per compute unit, its query and output registers fill the register file);
+// DB = 32-wide blocks of the head dimension in a row of the K / V tiles in LDS: 1 (d <= 32), 2 (d <= 64),
+// 4 (d <= 128) or 8 (d <= 256: one workgroup per compute unit, its query and output registers fill the
+// register file); DC <= DB = the blocks that hold anything for this head dimension -- only those are
+// multiplied and kept in registers (d = 192: 6 of 8, a quarter of the matrix work less);
 // KB = 32-key blocks per step;
 // MASK: the probabilities are multiplied by M[query, key] AFTER the softmax, as the block's mask unit does
 // (ChannelMHA.java:75-76: P = softmax(...); P = mask.forward(P)): the sum that normalises them runs over the
 // unmasked terms, the second product takes the masked ones.
-template <int DB, int KB, bool MASK>
+template <int DB, int DC, int KB, bool MASK>
 __global__ __launch_bounds__(NTHREADS, DB > 4 ? 1 : 2) void attention_f32_mfma(const AttnParams p) {
+    static_assert(DC >= 1 && DC <= DB && 2 * DC > DB, "a narrower tile row would do");
     constexpr int AK = KB * 32;            // keys per step
     constexpr int DW = DB * 32;            // tile width in floats
     constexpr int CPR = DW / 4;            // 16-byte chunks per tile row
     constexpr int RPP = NTHREADS / CPR;    // tile rows staged per pass
     constexpr int PASSES = AK / RPP;       // = DB * KB
-    constexpr int NG = DW / 8;             // groups of 8 d (4 MFMA steps each)
+    constexpr int NG = DC * 4;             // groups of 8 d (4 MFMA steps each) that the head dimension reaches
     // DB = 8: the query and output registers leave no room for staging registers, so the K / V tiles go from
     // global memory straight into the other LDS buffer (a lane's 16 bytes land at the wave's base + 16 * lane:
     // the chunk swizzle of the K tile moves to the global side)
@@ -174,9 +177,9 @@ __global__ __launch_bounds__(NTHREADS, DB > 4 ? 1 : 2) void attention_f32_mfma(c
         }
     };
 
-    v16f o[DB];
+    v16f o[DC];
 #pragma unroll
-    for (int b = 0; b < DB; b++) o[b] = (v16f)(0.0f);
+    for (int b = 0; b < DC; b++) o[b] = (v16f)(0.0f);
     float m = -__builtin_inff(), l = 0.0f;      // reference maximum (shared by the halves), this half's sum
 
     const int steps = (p.nk + AK - 1) / AK;
@@ -235,7 +238,7 @@ __global__ __launch_bounds__(NTHREADS, DB > 4 ? 1 : 2) void attention_f32_mfma(c
             m = m_new;
             l *= alpha;
 #pragma unroll
-            for (int b = 0; b < DB; b++)
+            for (int b = 0; b < DC; b++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) o[b][v] *= alpha;
         }
@@ -276,7 +279,7 @@ __global__ __launch_bounds__(NTHREADS, DB > 4 ? 1 : 2) void attention_f32_mfma(c
             for (int v = 0; v < 16; v++) {
                 const int key = 32 * kb + 8 * (v / 4) + 4 * h + (v % 4);
 #pragma unroll
-                for (int b = 0; b < DB; b++)
+                for (int b = 0; b < DC; b++)
                     o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * DW + b * 32 + r], s[kb][v], o[b], 0, 0, 0);
             }
 
@@ -292,7 +295,7 @@ __global__ __launch_bounds__(NTHREADS, DB > 4 ? 1 : 2) void attention_f32_mfma(c
     if (q < p.nq) {
         float* yrow = Yb + (size_t)q * p.y_l;
 #pragma unroll
-        for (int b = 0; b < DB; b++)
+        for (int b = 0; b < DC; b++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int d = 32 * b + 8 * g + 4 * h;
@@ -353,18 +356,25 @@ static int attention_launch(const int64_t* streams, int32_t length, int64_t dQ, 
     hipStream_t s = (hipStream_t)(intptr_t)streams[0];
     const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);
     const int dmax = dK4 > dV4 ? dK4 : dV4;
-    const int db = dmax <= 32 ? 1 : dmax <= 64 ? 2 : dmax <= 128 ? 4 : 8;
-    if (dMask == 0) {
-        if (db == 1) hipLaunchKernelGGL((attention_f32_mfma<1, 2, false>), grid, block, 0, s, p);
-        else if (db == 2) hipLaunchKernelGGL((attention_f32_mfma<2, 2, false>), grid, block, 0, s, p);
-        else if (db == 4) hipLaunchKernelGGL((attention_f32_mfma<4, 1, false>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((attention_f32_mfma<8, 1, false>), grid, block, 0, s, p);
-    } else {
-        if (db == 1) hipLaunchKernelGGL((attention_f32_mfma<1, 2, true>), grid, block, 0, s, p);
-        else if (db == 2) hipLaunchKernelGGL((attention_f32_mfma<2, 2, true>), grid, block, 0, s, p);
-        else if (db == 4) hipLaunchKernelGGL((attention_f32_mfma<4, 1, true>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((attention_f32_mfma<8, 1, true>), grid, block, 0, s, p);
+    const int dc = (dmax + 31) / 32;   // 32-wide blocks of the head dimension that hold anything
+    const bool masked = dMask != 0;
+#define ATTN_CASE(DB_, DC_, KB_)                                                                          \
+    case DC_:                                                                                             \
+        if (masked) hipLaunchKernelGGL((attention_f32_mfma<DB_, DC_, KB_, true>), grid, block, 0, s, p);  \
+        else hipLaunchKernelGGL((attention_f32_mfma<DB_, DC_, KB_, false>), grid, block, 0, s, p);        \
+        break;
+    switch (dc) {
+        ATTN_CASE(1, 1, 2)
+        ATTN_CASE(2, 2, 2)
+        ATTN_CASE(4, 3, 1)
+        ATTN_CASE(4, 4, 1)
+        ATTN_CASE(8, 5, 1)
+        ATTN_CASE(8, 6, 1)
+        ATTN_CASE(8, 7, 1)
+        ATTN_CASE(8, 8, 1)
+        default: return hipErrorInvalidValue;
     }
+#undef ATTN_CASE
     return hipGetLastError();
 }
 

@@ -82,7 +82,8 @@ SHAPES = [  # N, head, QL, VL, dk, dv
     (1, 1, 255, 96, 64, 8), (1, 2, 100, 150, 128, 128), (1, 1, 70, 90, 96, 72), (2, 1, 33, 65, 100, 128),
     (1, 1, 129, 40, 16, 125),
     # head dimensions above 128: eight 32-wide blocks per query, one workgroup per compute unit
-    (1, 2, 130, 70, 132, 132), (2, 1, 100, 257, 256, 256), (1, 1, 64, 64, 192, 40), (1, 3, 37, 90, 20, 200)]
+    (1, 2, 130, 70, 132, 132), (2, 1, 100, 257, 256, 256), (1, 1, 64, 64, 192, 40), (1, 3, 37, 90, 20, 200),
+    (1, 1, 200, 130, 192, 192), (1, 2, 66, 200, 160, 160), (1, 1, 129, 65, 224, 224), (1, 1, 129, 130, 80, 80)]
 
 
 @pytest.mark.parametrize("head_inner", [0, 1])
@@ -305,7 +306,9 @@ def run_attention_masked(dh, Q, K, V, M, scale, head_inner, garbage_pad=False):
 
 
 MASKED_SHAPES = [(1, 1, 1, 1, 4, 4), (2, 3, 37, 29, 20, 20), (1, 2, 128, 128, 64, 64), (2, 2, 130, 257, 64, 64),
-                 (1, 2, 200, 333, 128, 96), (3, 1, 65, 64, 32, 8), (1, 4, 300, 70, 12, 100), (1, 2, 70, 100, 160, 256)]
+                 (1, 2, 200, 333, 128, 96), (3, 1, 65, 64, 32, 8), (1, 4, 300, 70, 12, 100), (1, 2, 70, 100, 160, 256),
+                 # three, five, six and seven of the tile row's 32-wide blocks in use
+                 (1, 2, 50, 80, 72, 96), (1, 1, 40, 64, 160, 132), (1, 2, 70, 100, 192, 160), (1, 1, 40, 64, 36, 224)]
 
 
 @pytest.mark.parametrize("head_inner", [False, True])
