@@ -40,8 +40,9 @@ hipError_t linear_dual2D_row_launch(hipStream_t stream, const float* X1, const f
                                     int lengthv, int width, int stride) {
     const int length4 = lengthv >> 2;
     if (length4 <= 0) return hipSuccess;
-    int blocks = (length4 + 255) / 256;
-    if (blocks > 8192) blocks = 8192;
+    // one 16-byte element per thread, workgroups in address order: measured on a 1 GiB tensor in place 6.0 TB/s,
+    // against 4.7 for 8192 workgroups that stride over the tensor (neighbours in time then touch addresses far apart)
+    const int blocks = (length4 + 255) / 256;
     hipLaunchKernelGGL(linear_dual2D_row_kernel, dim3(blocks), dim3(256), 0, stream, X1, X2, row_lengthv,
                        alpha, beta, gamma, Y, length4, width, stride);
     return hipGetLastError();

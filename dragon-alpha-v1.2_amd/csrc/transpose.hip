@@ -52,11 +52,11 @@ __global__ __launch_bounds__(256) void transpose_last_kernel(const float* __rest
                                                              int tiles_p, int tiles_q) {
     __shared__ float tile[TP][TP + 1];
     long long b = blockIdx.x;
-    // tiles are walked along diagonals of the (p, q) plane: neighbouring workgroups then differ in
-    // both their X rows and their Y rows, which spreads power-of-two strides over the HBM channels
-    const int tj = (int)(b % tiles_q); b /= tiles_q;
-    const int tp = (int)(b % tiles_p); b /= tiles_p;
-    const int tq = (tj + tp) % tiles_q;
+    // tiles are walked along diagonals of the (p, q) plane: from one workgroup to the next both the tile row
+    // and the tile column move on, so neighbours differ in their X rows, X columns, Y rows and Y columns, which
+    // spreads power-of-two strides over the HBM channels on both sides
+    const int tq = (int)(b % tiles_q); b /= tiles_q;
+    const int tp = (int)((b % tiles_p + tq) % tiles_p); b /= tiles_p;
     // the two dimensions that stay in place, o1 < o2
     const int o1 = (a == 0) ? 1 : 0, o2 = (a == 2) ? 1 : 2;
     int x[4];
@@ -120,8 +120,8 @@ int transpose_launch(int64_t stream, int64_t dX, int64_t dY, Dims4 xd, int i1, i
     if (i2 < 3) {
         if (strideX != strideY) return hipErrorInvalidValue;
         const long long rows = (long long)xd.d[0] * xd.d[1] * xd.d[2];
-        long long blocks = (rows * (strideX >> 2) + 255) / 256;
-        if (blocks > 16384) blocks = 16384;
+        const long long blocks = (rows * (strideX >> 2) + 255) / 256;   // one 16-byte element per thread, in address order
+        if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
         hipLaunchKernelGGL(transpose_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1, i2,
                            strideX, rows);
     } else {

@@ -46,7 +46,9 @@ CASES = [((1, 1), 0, 1), ((5, 7), 0, 1), ((7, 5), 1, 0), ((64, 64), 0, 1), ((257
          ((3, 1), 0, 1), ((1, 300), 0, 1),
          ((2, 3, 5), 0, 1), ((2, 3, 5), 1, 2), ((2, 3, 5), 0, 2), ((33, 257, 129), 1, 2), ((4, 100, 8), 2, 0),
          ((2, 3, 4, 6), 0, 1), ((2, 3, 4, 6), 1, 2), ((2, 3, 4, 6), 0, 2), ((2, 3, 4, 6), 2, 3), ((2, 3, 4, 6), 1, 3),
-         ((2, 3, 4, 6), 0, 3), ((8, 128, 12, 64), 1, 2), ((8, 12, 128, 64), 2, 3), ((3, 70, 2, 65), 3, 1)]
+         ((2, 3, 4, 6), 0, 3), ((8, 128, 12, 64), 1, 2), ((8, 12, 128, 64), 2, 3), ((3, 70, 2, 65), 3, 1),
+         # planes of many tiles, square and not: the diagonal tile order visits each tile once
+         ((1024, 1024), 0, 1), ((2048, 1021), 0, 1), ((2, 1024, 2, 1024), 1, 3), ((1021, 3, 2048), 0, 2)]
 
 
 @pytest.mark.parametrize("dims,i1,i2", CASES)
