@@ -79,6 +79,20 @@ def test_the_automatic_choice_takes_it_and_stays_within_tolerance(gpu, variant):
         assert_within_tolerance(C, oracle.matmul_f64(variant, A, B), K, A, B, what + " vs FP64 oracle")
 
 
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_many_tiles_with_a_long_k_take_the_half_size_tile(gpu, variant):
+    """Many 64 x 64 tiles, K >= 4096 and runs that are not whole tiles: the automatic choice is the 128 x 64 / 64 x 128
+    balanced tile (fewer bytes staged per FLOP).  Integer inputs: every bit against the exact product."""
+    assert gpu.choose_tile(variant, 1000, 780, 1, 4352) in (19, 20) and gpu.choose_tile(variant, 768, 772, 1, 8192) in (19, 20)
+    rng = np.random.default_rng(900 + variant)
+    for (N, M, K) in ((1000, 777, 4351), (768, 770, 8192)):
+        A, B = logical_operands(variant, rng, N, M, K, dist="int")
+        C, Cp = gpu_matmul_2d(gpu, variant, A, B, fill=3.0)
+        R = oracle.matmul_f64(variant, A, B).astype(np.float32)
+        assert np.array_equal(C, R), (VARIANT_NAMES[variant], N, M, K)
+        assert np.count_nonzero(Cp[N:, :]) == 0 and np.count_nonzero(Cp[:, M:]) == 0
+
+
 @pytest.mark.parametrize("tile", [22, 23, 18])
 def test_every_bit_is_the_same_from_run_to_run(gpu, tile):
     """The pieces of a shared tile are added in run order whichever workgroup arrives last, so rounding
