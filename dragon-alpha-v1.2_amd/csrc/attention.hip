@@ -352,6 +352,7 @@ static int attention_launch(const int64_t* streams, int32_t length, int64_t dQ, 
         p.v_h = (long long)VL * dV4; p.y_h = (long long)QL * dV4;
         p.q_n = p.q_h * head; p.k_n = p.k_h * head; p.v_n = p.v_h * head; p.y_n = p.y_h * head;
     }
+    dragon::split_ledger_touch(p.Y, (size_t)N * (size_t)p.y_n * 4);
     p.c = scale * 1.44269504088896340736f;
     hipStream_t s = (hipStream_t)(intptr_t)streams[0];
     const dim3 grid((unsigned)((long long)N * head * p.qtiles)), block(NTHREADS);

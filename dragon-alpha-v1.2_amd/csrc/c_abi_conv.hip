@@ -5,6 +5,7 @@
 #include "../../include/dragon_hip_conv.h"
 #include "../../include/dragon_hip_gemm.h"
 #include "gemm_mfma.h"
+#include "runtime_internal.h"
 
 using namespace dragon;
 
@@ -25,6 +26,7 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     const long long sizeX = (long long)N * IH * IW * IC;
     if (GM > 0x7fffffffLL || GK >= (1LL << 24) || sizeX >= (1LL << 29) || GM * OC > 0x7fffffffLL)
         return hipErrorInvalidValue;
+    split_ledger_touch((const void*)(intptr_t)dY, (size_t)(GM * OC) * 4);
     GemmParams p = {};
     p.A = (const float*)(intptr_t)dX;
     p.B = (const float*)(intptr_t)dW;

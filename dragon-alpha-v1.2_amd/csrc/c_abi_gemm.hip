@@ -6,7 +6,10 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <atomic>
+#include <mutex>
+#include <vector>
 #include "gemm_mfma.h"
+#include "runtime_internal.h"
 #include "../../include/dragon_hip_gemm.h"
 #include "../../include/dragon_hip_testing.h"
 
@@ -17,6 +20,61 @@ namespace {
 constexpr int MAX_STREAMS = 10;  // the reference copies the handles into jlong streams[10]
 
 inline bool aligned16(int64_t a) { return (a & 15) == 0; }
+
+// How the split-K entry points treat the caller's GridZ: -1 the estimate decides (gemm_split_loses), 0 always
+// as asked, 1 declined wherever the unsplit product can take the balanced kernel.  A test hook, per thread.
+thread_local int t_split_policy = -1;
+std::atomic<long long> g_declined{0};   // split-K calls that ran unsplit (read by tests)
+
+// ---- the ledger of declined splits ------------------------------------------------------------------------
+// A declined split leaves the whole product in C and zeros in the partial buffers; the fold the host then asks
+// for (SKbuf_summary with the same stream, Cbuf, C, part and sizeC) would add zeros to C: a launch, three
+// passes over C, and no change.  The entry point remembers the call here, and SKbuf_summary, finding its exact
+// arguments, returns without launching.  An entry dies with its first use, with any write the library sees to
+// its C or its partial buffers (every entry point that writes device memory reports the range), with a free of
+// that memory, and when 64 younger ones exist; the buffers hold their zeros in any case, so a fold that does run
+// (another stream, other arguments, an entry that died) is right as well.
+struct DeclinedSplit { int dev; hipStream_t stream; uintptr_t cbuf, cbuf_end, c, c_end; int part, sizeC; };
+std::mutex g_led_mutex;
+std::vector<DeclinedSplit> g_led;
+std::atomic<int> g_led_n{0};
+std::atomic<int> g_fold_skip{1};          // test hook: 0 = every fold is launched
+std::atomic<long long> g_folds_skipped{0};
+
+void ledger_note(hipStream_t stream, int64_t dCbuf, int64_t dC, int part, int sizeC) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    const uintptr_t cb = (uintptr_t)dCbuf, c = (uintptr_t)dC;
+    std::lock_guard<std::mutex> lock(g_led_mutex);
+    if (g_led.size() >= 64) g_led.erase(g_led.begin());
+    g_led.push_back({dev, stream, cb, cb + (uintptr_t)part * (uintptr_t)sizeC * 4, c, c + (uintptr_t)sizeC * 4, part, sizeC});
+    g_led_n.store((int)g_led.size(), std::memory_order_release);
+}
+
+// true: this fold is the no-op that follows a declined split
+bool ledger_fold_is_noop(hipStream_t stream, int64_t dCbuf, int64_t dC, int part, int sizeC) {
+    if (g_led_n.load(std::memory_order_acquire) == 0) return false;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    std::lock_guard<std::mutex> lock(g_led_mutex);
+    for (size_t i = 0; i < g_led.size(); i++) {
+        const DeclinedSplit& e = g_led[i];
+        if (e.cbuf != (uintptr_t)dCbuf) continue;
+        const bool same = e.dev == dev && e.stream == stream && e.c == (uintptr_t)dC && e.part == part && e.sizeC == sizeC;
+        g_led.erase(g_led.begin() + i);
+        g_led_n.store((int)g_led.size(), std::memory_order_release);
+        return same && g_fold_skip.load(std::memory_order_relaxed) != 0;
+    }
+    return false;
+}
+
+inline void touch(int64_t address, long long floats) { split_ledger_touch((const void*)(intptr_t)address, (size_t)floats * 4); }
+
+bool split_declined(int variant, int N, int M, int gz, int K, int k_slice, int num_cu) {
+    if (gemm_forced_tile() != TILE_AUTO || t_split_policy == 0) return false;
+    if (t_split_policy == 1) return k_slice >= 32 && gemm_choose_streamk(N, M, 1, K, num_cu, variant) >= 0;
+    return gemm_split_loses(variant, N, M, gz, K, k_slice, num_cu);
+}
 inline bool x4(int v) { return (v & 3) == 0; }
 
 int check_common(const int64_t* streams, int length, int64_t dA, int64_t dB, int64_t dC) {
@@ -39,6 +97,8 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
     if (gz > 1 && (dCbuf == 0 || !aligned16(dCbuf))) return hipErrorInvalidValue;
     if ((long long)N * M > 0x7fffffffLL) return hipErrorInvalidValue;
 
+    touch(dC, (long long)N * M);
+    if (gz > 1) touch(dCbuf, (long long)(gz - 1) * N * M);
     GemmParams p = {};
     p.A = (const float*)(intptr_t)dA;
     p.B = (const float*)(intptr_t)dB;
@@ -75,15 +135,51 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return hipErrorNoDevice;
+    p.sk_ws_given = sk_ws;
+    p.sk_ws_given_floats = sk_ws != nullptr ? GEMM_SK_WS_FLOATS_256CU : 0;
+    hipStream_t stream = (hipStream_t)(intptr_t)streams[0];
+    // A split that loses is declined: the balanced kernel deals equal runs of stages to the compute units by
+    // itself, and where the unsplit product through it is estimated to beat the slices plus their fold, the
+    // whole product goes to C and the partial buffers get zeros -- SKbuf_summary then adds zeros and leaves C
+    // as it is (the caller sees the sum it asked for; which slice holds what is the kernel's business).  A
+    // forced tile shape (tests, tuning) always honours the split.
+    if (gz > 1 && dBias == 0 && split_declined(variant, N, M, gz, K, p.k_slice, num_cu)) {
+        GemmParams q = p;
+        q.nz = 1; q.split = 0; q.k_slice = 0; q.sizeC = 0; q.Cbuf = nullptr;
+        q.zero_buf = p.Cbuf;
+        q.zero_floats = (long long)(gz - 1) * N * M;
+        const int tile1 = gemm_choose_streamk(N, M, 1, K, num_cu, variant);
+        const hipError_t e1 = gemm_launch_streamk(variant, q, tile1, stream);
+        if (e1 != hipErrorOutOfMemory) {
+            if (e1 == hipSuccess) {
+                g_declined.fetch_add(1, std::memory_order_relaxed);
+                if (sk_ws == nullptr) ledger_note(stream, dCbuf, dC, gz - 1, N * M);   // (the static entry folds nothing)
+            }
+            return e1;
+        }
+        (void)hipGetLastError();   // no workspace may be made now (a capturing stream): the slices as asked
+    }
     // K slices are tiles like batches are: (slice, tile of C) pairs, each slice k_slice long
     const int k_tile = p.split && p.k_slice > 0 ? p.k_slice : p.k_total;
     const int tile = gemm_choose_tile(p.rows, p.cols, p.nz, k_tile, num_cu, variant);
-    p.sk_ws_given = sk_ws;
-    p.sk_ws_given_floats = sk_ws != nullptr ? GEMM_SK_WS_FLOATS_256CU : 0;
-    return gemm_launch(variant, p, tile, (hipStream_t)(intptr_t)streams[0]);
+    return gemm_launch(variant, p, tile, stream);
 }
 
 }  // namespace
+
+namespace dragon {
+void split_ledger_touch(const void* ptr, size_t bytes) {
+    if (g_led_n.load(std::memory_order_acquire) == 0) return;
+    const uintptr_t lo = (uintptr_t)ptr, hi = bytes == 0 ? ~(uintptr_t)0 : lo + bytes;
+    std::lock_guard<std::mutex> lock(g_led_mutex);
+    for (size_t i = 0; i < g_led.size();) {
+        const DeclinedSplit& e = g_led[i];
+        if ((lo < e.cbuf_end && e.cbuf < hi) || (lo < e.c_end && e.c < hi)) g_led.erase(g_led.begin() + i);
+        else i++;
+    }
+    g_led_n.store((int)g_led.size(), std::memory_order_release);
+}
+}  // namespace dragon
 
 extern "C" {
 
@@ -122,6 +218,12 @@ int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC, 
         return hipErrorInvalidValue;
     if (part > 0 && (dCbuf == 0 || !aligned16(dCbuf))) return hipErrorInvalidValue;
     if (part == 0) return hipSuccess;
+    // the fold that follows a declined split adds zeros: nothing to launch
+    if (ledger_fold_is_noop((hipStream_t)(intptr_t)stream, dCbuf, dC, part, sizeC)) {
+        g_folds_skipped.fetch_add(1, std::memory_order_relaxed);
+        return hipSuccess;
+    }
+    touch(dC, sizeC);
     return skbuf_summary_launch((hipStream_t)(intptr_t)stream, (const float*)(intptr_t)dCbuf,
                                 (float*)(intptr_t)dC, part, sizeC);
 }
@@ -187,6 +289,21 @@ int dragon_Cuda_matMul_matMulSK_static(const int64_t* streams, int32_t length, i
     e = static_scratch(&ptr);
     if (e) return e;
     float* sk_ws = ptr + SK_STATIC_FLOATS;
+    // While the stream is capturing, the balanced kernel stays out of it: replays of a graph may overlap with
+    // each other or with eager calls, and two launches at a time on the one static workspace would mix their
+    // pieces and could leave its arrival counters off zero for every later call.  The tile-per-workgroup
+    // kernels need no workspace; the partials still go to the static array.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)(intptr_t)streams[0], &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusActive;
+    }
+    if (cap != hipStreamCaptureStatusNone) sk_ws = nullptr;
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    // a split that loses is declined as in the two-stage entry points; here nobody folds afterwards, so the
+    // unsplit product is the whole call
+    if (GridZ > 1 && sk_ws != nullptr && split_declined(variant, N, M, GridZ, K, ((K / GridZ) >> 3) << 3, num_cu)) GridZ = 1;
     if (GridZ == 1) return matmul_2d(variant, streams, length, 1, dA, dB, dC, 0, N, M, K, 0, 0, 0, sk_ws);
     // stage 1 writes every float of the GridZ-1 partials it later reads, so nothing has to be cleared
     e = matmul_2d(variant, streams, length, GridZ, dA, dB, dC, (int64_t)(intptr_t)ptr, N, M, K, 0, 0, 0, sk_ws);
@@ -212,6 +329,7 @@ int dragon_Cuda_function_linear_dual2D_row(int64_t stream, int64_t dX1, int64_t 
         !x4(lengthv) || !x4(row_lengthv) || !x4(stride) || lengthv % stride != 0 ||
         lengthv % row_lengthv != 0 || row_lengthv % stride != 0)
         return hipErrorInvalidValue;
+    touch(dY, lengthv);
     return linear_dual2D_row_launch((hipStream_t)(intptr_t)stream, (const float*)(intptr_t)dX1,
                                     (const float*)(intptr_t)dX2, row_lengthv, alpha, beta, gamma,
                                     (float*)(intptr_t)dY, lengthv, width, stride);
@@ -239,6 +357,7 @@ int dragon_Cuda_batchMatMul_batchMatMul(const int64_t* streams, int32_t length, 
     p.ldc = M;
     p.sA = (long long)N * AK; p.sB = (long long)BK * M; p.sC = (long long)N * M;
     p.nz = Batch;
+    touch(dC, p.sC * Batch);
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return hipErrorNoDevice;
@@ -269,6 +388,7 @@ int dragon_Cuda_batchMatMul_batchMatMulT1(const int64_t* streams, int32_t length
     p.ldc = M;
     p.sA = (long long)K * AN; p.sB = (long long)K * M; p.sC = (long long)CN * M;
     p.nz = Batch;
+    touch(dC, p.sC * Batch);
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return hipErrorNoDevice;
@@ -293,6 +413,7 @@ int dragon_Cuda_batchMatMul_batchMatMulT2(const int64_t* streams, int32_t length
     p.ldc = CM;
     p.sA = (long long)N * K; p.sB = (long long)BM * K; p.sC = (long long)N * CM;
     p.nz = Batch;
+    touch(dC, p.sC * Batch);
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return hipErrorNoDevice;
@@ -368,6 +489,20 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M) {
 }
 
 void dragon_gemm_force_tile(int32_t tile) { gemm_force_tile(tile); }
+int32_t dragon_gemm_release_workspaces(void) { return gemm_streamk_release_workspaces(); }
+int32_t dragon_gemm_workspace_count(void) { return gemm_streamk_workspace_count(); }
+int64_t dragon_gemm_workspaces_refused(void) { return gemm_streamk_workspaces_refused(); }
+void dragon_gemm_fold_skip(int32_t on) { g_fold_skip.store(on ? 1 : 0, std::memory_order_relaxed); }
+int64_t dragon_gemm_folds_skipped(void) { return g_folds_skipped.load(std::memory_order_relaxed); }
+void dragon_gemm_split_policy(int32_t mode) { t_split_policy = mode < -1 || mode > 1 ? -1 : mode; }
+int64_t dragon_gemm_declined_splits(void) { return g_declined.load(std::memory_order_relaxed); }
+int32_t dragon_gemm_split_loses(int32_t variant, int32_t N, int32_t M, int32_t GridZ, int32_t K, int32_t num_cu) {
+    if (variant < GEMM_NN || variant > GEMM_T2 || GridZ < 1 || N <= 0 || M <= 0 || K <= 0 || num_cu <= 0) return -1;
+    return gemm_split_loses(variant, N, M, GridZ, K, ((K / GridZ) >> 3) << 3, num_cu) ? 1 : 0;
+}
+double dragon_gemm_estimate_us(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu) {
+    return gemm_estimate_us(rows, cols, nz, k, num_cu, variant);
+}
 void dragon_gemm_tile_divisor(uint32_t d, uint32_t* mul, uint32_t* shift) {
     unsigned m = 0, s = 0;
     gemm_magic_divisor(d, m, s);

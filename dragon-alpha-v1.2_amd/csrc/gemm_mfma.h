@@ -45,6 +45,10 @@ enum GemmTile {
     // one more balanced shape: 256 x 64, four wavefronts of 64 x 64 one above the other, 3 stage buffers -- for a
     // C of 64 columns, where it has the 128 x 128 tile's ratio of matrix work to LDS traffic
     TILE_SK_256x64 = 25,
+    // A K of 89 ... 144 under a ragged C, batch after batch: 64 x 64 tiles with the whole K of a tile resident in
+    // LDS, one persistent workgroup per compute unit, the rim of C (1 ... 4 rows / columns past a multiple of 64)
+    // as strips of 4 x 4 MFMA blocks beside the tiles (gemm_mfma_shortk.hip)
+    TILE_SHORTK_64x64 = 26,
     // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
     // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
     // short K; gemm_choose_tile sets it.
@@ -52,6 +56,7 @@ enum GemmTile {
 };
 inline bool gemm_tile_is_streamk(int tile) { return (tile >= TILE_SK_64x64 && tile < TILE_SK_END) || tile == TILE_SK_256x64; }
 inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128; }
+inline bool gemm_tile_is_shortk(int tile) { return tile == TILE_SHORTK_64x64; }
 inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
 
 // One product C[z] = op(A[z]) * op(B[z]) or one K slice of it.
@@ -107,6 +112,10 @@ struct GemmParams {
     // K slices: the tiles from number sk_T1 on (the last slice's) have sk_S_last stages
     int sk_S_last, sk_T1;
     unsigned sk_div_Sl_mul, sk_div_Sl_shift;
+    // a split-K call whose split was declined (gemm_split_loses): the whole product goes to C and the balanced
+    // kernel's workgroups write zeros over the zero_floats floats (a multiple of 4) of the caller's partial buffers
+    float* zero_buf;
+    long long zero_floats;
     // filled by the launcher of the band kernel (gemm_launch_band): a band's tiles_n column tiles are dealt
     // out in bd_chunks runs of bd_chunk_tiles
     int bd_chunks, bd_chunk_tiles;
@@ -138,6 +147,12 @@ int gemm_choose_tile_per_workgroup(int rows, int cols, int nz, int k, int num_cu
 void gemm_force_tile(int tile);
 int gemm_forced_tile();   // TILE_AUTO when the choice is left to gemm_choose_tile
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream);
+// The resident-K kernel (tile id TILE_SHORTK_64x64) for the three products, batched too, with 88 < K <= 144.
+// hipErrorOutOfMemory says that the product cannot go this way (another K, K slices, a bias row) and the caller
+// takes a tile-per-workgroup kernel instead.
+hipError_t gemm_launch_shortk(int variant, const GemmParams& p, hipStream_t stream);
+// TILE_SHORTK_64x64 where that kernel is the better choice, else -1
+int gemm_choose_shortk(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
 hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);
 // the three products (batched too) through the balanced kernel (tile ids TILE_SK_*).  It needs the stream's
@@ -149,6 +164,14 @@ hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipSt
 // better (an estimate fitted to measurements: at most two 64 x 64 tiles per compute unit, and K long enough
 // to carry the balanced kernel's larger fixed time).
 int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
+// The fitted estimate behind that choice, in microseconds: what the product takes through the kernel
+// gemm_choose_tile names (few 64 x 64 tiles: the measured per-stage and per-launch costs of the balanced and the
+// tile-per-workgroup kernels; more tiles: the padded matrix work at the rate the large kernels sustain).
+double gemm_estimate_us(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
+// True where cutting K into gz slices (k_slice each, partials folded by SKbuf_summary afterwards) is estimated
+// to take longer than the unsplit product through the balanced kernel, which deals equal runs of stages to the
+// compute units by itself: the split-K entry points then run the unsplit product and zero the partial buffers.
+bool gemm_split_loses(int variant, int rows, int cols, int gz, int k, int k_slice, int num_cu);
 // Floats of a balanced-kernel workspace for a device of num_cu compute units (GEMM_SK_WS_FLOATS_256CU: the
 // same for 256 units, as a constant for static storage)
 size_t gemm_streamk_workspace_floats(int num_cu);
@@ -157,10 +180,20 @@ constexpr size_t GEMM_SK_WS_FLOATS_256CU = 65536 + (size_t)2 * 256 * 128 * 128;
 // counts that are multiples of 32 and filters of at most 32 x 32; hipErrorOutOfMemory as above (then
 // gemm_launch_conv takes over).
 hipError_t gemm_launch_streamk_conv(const GemmParams& p, int tile, hipStream_t stream);
-// The workspace of `stream` on the current device: arrival counters and the slots for pieces of shared tiles.
-// Made at the first balanced launch on that stream and kept for later launches on the same handle until the
-// process ends; nullptr while the stream is capturing (a graph's launches may run next to the stream's own).
+// The workspace of `stream` on the stream's device: arrival counters and the slots for pieces of shared tiles.
+// Made at the first balanced launch on that stream (a device allocation, and a small kernel on that stream that
+// clears the counters) and kept for later launches on the same handle until the stream is deleted through the
+// runtime bridge or the workspaces are released; nullptr while the stream is capturing (a graph's launches may
+// run next to the stream's own) and when the library already holds its maximum number of workspaces.
 float* gemm_streamk_workspace(hipStream_t stream, size_t* floats);
+// Gives the stream's workspace back (after the stream's work is done); the runtime bridge calls it before it
+// destroys a stream.  Nothing happens for a stream that has none.
+void gemm_streamk_release_workspace(hipStream_t stream);
+// The same for every workspace the library holds, on every device (each device is synchronised first);
+// returns how many there were.  Streams that launch the balanced kernel again get a new one.
+int gemm_streamk_release_workspaces();
+int gemm_streamk_workspace_count();               // workspaces held now
+long long gemm_streamk_workspaces_refused();      // balanced launches that found the table full and took another kernel
 // The band kernel (tile id TILE_BAND_128x128) for the three products, batched too, with K <= 64.
 // hipErrorOutOfMemory says that the product cannot go this way (a longer K, K slices, a bias row) and the
 // caller takes a tile-per-workgroup kernel instead.

@@ -47,6 +47,11 @@ __device__ __forceinline__ int sk_owner(int u, int q, int rem) {
     return u < big ? u / (q + 1) : rem + (u - big) / q;
 }
 
+// The hand-over of pieces between workgroups below is written for gfx950's memory system and for nothing else.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "the balanced kernel's piece hand-over relies on gfx950's cache behaviour (see store_partial)"
+#endif
+
 // Partial tile in the accumulators' own layout: block (i, j) of wavefront `wave`, element e, lane at
 // float (((wave*TM + i)*TN + j)*16 + e)*64 + lane: a wavefront writes 256 contiguous bytes per store.
 // The pieces travel between workgroups on different XCDs, each with an L2 of its own, inside one
@@ -54,6 +59,18 @@ __device__ __forceinline__ int sk_owner(int u, int q, int rem) {
 // to memory, a load that does not take a stale line from the reader's L2 -- so that no cache has to be
 // written back or invalidated as a whole (a device-scope fence does both to the XCD's L2, and with
 // them went the operand reuse: 33 -> 110 us on 1000 x 777 x 1531).
+// What the ordering rests on, instruction by instruction (gfx950; the formal memory model promises less):
+//   * writer: the piece's stores carry the device-scope bit (sc1), i.e. they write through the XCD's L2
+//     to memory and are acknowledged -- the wave's vmcnt counts them down -- only once they are there;
+//     `s_waitcnt vmcnt(0)` after the run therefore means "every float of my pieces is in memory";
+//   * the workgroup barrier behind it makes that true for all four wavefronts before thread 0 / 1 bumps the
+//     tile's arrival counter with an atomic add that executes at the memory side (device scope as well);
+//   * reader: the workgroup whose add returns the last count reads the pieces with device-scope loads
+//     (sc1), which do not hit in its own L2, so a line of the workspace left there by an earlier launch is
+//     never taken; its loads are issued after the add has returned and the workgroup has met at a barrier.
+//   * the compiler keeps atomics of one address space in program order across the s_waitcnt builtin and the
+//     barrier; the "memory" clobbers on the inline-assembly transfers pin the rest.
+// The run-to-run bitwise test and the two-stream test in tests/test_gpu_streamk.py guard this.
 template <int TM, int TN>
 __device__ __forceinline__ void store_partial(const v16f (&acc)[TM][TN], float* slot, int wave, int lane) {
 #pragma unroll
@@ -187,8 +204,11 @@ struct ConvDirect {
 // the remainder of K, have their own stage count (they come last in the tile order), and a tile's K limits
 // count from the slice's first k.
 // CONV: A is gathered from an image (ConvDirect), B holds the filters K-inner, C is the output image.
+// ZFILL: the launch also writes zeros over the caller's split-K partial buffers (a declined split).  A template
+// flag and not a run-time test, so that the plain kernels carry none of it: the compiler's code for their stage
+// loop has reacted to a few instructions added elsewhere in the kernel before.
 template <bool A_KIN, bool B_KIN, int WM, int WN, int TM, int TN, int KT, int NS, int OCC, bool BIAS, bool SPLIT,
-          bool CONV = false>
+          bool CONV = false, bool ZFILL = false>
 __global__ __launch_bounds__(NTHREADS, OCC)
 void gemm_f32_mfma_streamk(const GemmParams p) {
     static_assert(!CONV || (A_KIN && B_KIN && !SPLIT), "the convolution is an A * B^T product, unsplit");
@@ -217,6 +237,17 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
     const int wm = wave / WN, wn = wave % WN;
     const unsigned long long a_step8 = (unsigned long long)LoadA::k_advance(p.lda) * 4;
     const unsigned long long b_step8 = (unsigned long long)LoadB::k_advance(p.ldb) * 4;
+
+    if constexpr (ZFILL) {
+        // A split-K call whose split was declined: this launch computes the whole product, and its workgroups
+        // first write zeros over the partial buffers the caller will fold into C afterwards (16 bytes per
+        // thread, the launch's threads side by side).  First of all, so that these stores are the oldest
+        // vector-memory operations of the wave: the waits on the transfers below then never wait on them.
+        static_assert(!SPLIT && !CONV && !BIAS, "only the plain unsplit product stands in for a split one");
+        const long long n4 = p.zero_floats >> 2, step = (long long)gridDim.x * NTHREADS;
+        v4f* z = (v4f*)p.zero_buf;
+        for (long long i = (long long)blockIdx.x * NTHREADS + t; i < n4; i += step) z[i] = (v4f)(0.0f);
+    }
 
     const int S = p.sk_S;
     // tile -> its stage count and first unit, unit -> tile (two regimes under SPLIT: the slices before the last
@@ -529,6 +560,7 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     // once, by whoever holds the whole sum)
     constexpr bool CAN_BIAS = (A_KIN && !B_KIN) || CONV;
     if (CONV && p.split) return hipErrorOutOfMemory;
+    if (p.zero_floats > 0 && (CONV || p.split || p.bias != nullptr)) return hipErrorOutOfMemory;
     if (p.bias != nullptr && (!CAN_BIAS || p.split)) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
@@ -575,6 +607,14 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
                            dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
         return hipGetLastError();
     }
+    if constexpr (!CONV && !(WM == 4)) {   // every 2-D shape; the 256 x 64 tile is a batch's
+        if (p.zero_floats > 0) {
+            hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false, false, false, true>),
+                               dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
+            return hipGetLastError();
+        }
+    }
+    if (p.zero_floats > 0) return hipErrorOutOfMemory;   // no zero-filling form of this shape: the caller keeps the split
     hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, false, false>),
                        dim3((unsigned)grid), dim3(NTHREADS), 0, stream, p);
     return hipGetLastError();
@@ -594,10 +634,29 @@ static hipError_t launch_streamk_variant(const GemmParams& p, int tile, hipStrea
     }
 }
 
-// ---- the workspace: one per (device, stream), made at the first balanced launch on that stream ----
+// ---- the workspace: one per (device, stream), made at the first balanced launch on that stream, released
+// when the stream is deleted through the runtime bridge (or by gemm_streamk_release_workspaces) ----
 struct Workspace { float* ptr; size_t floats; };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
+std::atomic<long long> g_ws_refused{0};   // balanced launches that found the table full and took another kernel
+
+__global__ void sk_zero_counters_kernel(int* counters, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) counters[i] = 0;
+}
+
+// the device a stream belongs to (the current one for the null stream)
+int device_of(hipStream_t stream) {
+    int dev = 0;
+    if (stream != nullptr) {
+        hipDevice_t d = 0;
+        if (hipStreamGetDevice(stream, &d) == hipSuccess) return (int)d;
+        (void)hipGetLastError();
+    }
+    if (hipGetDevice(&dev) != hipSuccess) return -1;
+    return dev;
+}
 
 }  // namespace
 
@@ -605,8 +664,6 @@ size_t gemm_streamk_workspace_floats(int num_cu) { return SK_MAX_TILES + (size_t
 static_assert(GEMM_SK_WS_FLOATS_256CU == SK_MAX_TILES + (size_t)2 * 256 * 128 * 128, "the constant in the header");
 
 float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     // Not under a stream capture: nothing may be allocated there, and a graph may later be launched on ANOTHER
     // stream, next to eager launches that use this stream's workspace -- two launches on one workspace at a
     // time would mix their pieces.  The caller takes the tile-per-workgroup kernel instead.
@@ -618,6 +675,8 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
         (void)hipGetLastError();
         return nullptr;
     }
+    const int dev = device_of(stream);
+    if (dev < 0) return nullptr;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     auto it = g_ws.find({dev, stream});
     if (it != g_ws.end()) {
@@ -626,16 +685,27 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
     }
     const int num_cu = gemm_device_num_cu();
     if (num_cu <= 0) return nullptr;
-    // a host that keeps making streams with new handles does not make the library hold ever more memory
-    if (g_ws.size() >= SK_MAX_WORKSPACES) return nullptr;
+    // a host that keeps making streams without deleting them does not make the library hold ever more memory
+    if (g_ws.size() >= SK_MAX_WORKSPACES) {
+        g_ws_refused.fetch_add(1, std::memory_order_relaxed);
+        return nullptr;
+    }
     Workspace w = {nullptr, gemm_streamk_workspace_floats(num_cu)};
-    if (hipMalloc((void**)&w.ptr, w.floats * sizeof(float)) != hipSuccess) {
+    // Another host thread may be capturing a graph in the global mode, which forbids allocations from every
+    // thread: for the length of the allocation this thread steps out of that rule (its own stream is not
+    // capturing, checked above).
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    const hipError_t em = hipMalloc((void**)&w.ptr, w.floats * sizeof(float));
+    if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    if (em != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
-    // the arrival counters start at zero and every launch leaves them there
-    if (hipMemset(w.ptr, 0, SK_MAX_TILES * sizeof(int)) != hipSuccess) {
-        (void)hipGetLastError();
+    // the arrival counters start at zero and every launch leaves them there.  Cleared by a kernel on the launch
+    // stream itself: in order before the launch that follows, and no other stream is made to wait.
+    hipLaunchKernelGGL(sk_zero_counters_kernel, dim3(SK_MAX_TILES / 256), dim3(256), 0, stream, (int*)w.ptr, SK_MAX_TILES);
+    if (hipGetLastError() != hipSuccess) {
         (void)hipFree(w.ptr);
         return nullptr;
     }
@@ -643,6 +713,64 @@ float* gemm_streamk_workspace(hipStream_t stream, size_t* floats) {
     *floats = w.floats;
     return w.ptr;
 }
+
+void gemm_streamk_release_workspace(hipStream_t stream) {
+    const int dev = device_of(stream);
+    Workspace w = {nullptr, 0};
+    {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        auto it = g_ws.find({dev, stream});
+        if (it == g_ws.end()) return;
+        w = it->second;
+        g_ws.erase(it);
+    }
+    // the stream's launches may still be using it
+    (void)hipStreamSynchronize(stream);
+    (void)hipFree(w.ptr);
+}
+
+int gemm_streamk_release_workspaces() {
+    std::map<std::pair<int, hipStream_t>, Workspace> all;
+    {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        all.swap(g_ws);
+    }
+    int prev = -1;
+    (void)hipGetDevice(&prev);
+    for (auto& kv : all) {
+        // a workspace is freed on its own device, after that device's work (the launches that use it) is done
+        if (hipSetDevice(kv.first.first) != hipSuccess) continue;
+        (void)hipDeviceSynchronize();
+        (void)hipFree(kv.second.ptr);
+    }
+    if (prev >= 0) (void)hipSetDevice(prev);
+    return (int)all.size();
+}
+
+int gemm_streamk_workspace_count() {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    return (int)g_ws.size();
+}
+long long gemm_streamk_workspaces_refused() { return g_ws_refused.load(std::memory_order_relaxed); }
+
+namespace {
+// The three fitted times for t64 tiles of 64 x 64 with S stages each on num_cu units (see below): tile per
+// workgroup, balanced with one workgroup per unit, balanced with two (1e300 where its runs are not whole tiles).
+struct FewTilesEstimate { double t_tiles, t_one, t_two; };
+FewTilesEstimate few_tiles_estimate(long long t64, long long S, int num_cu, int variant) {
+    const long long units = t64 * S;
+    const long long run1 = (units + num_cu - 1) / num_cu;
+    const bool whole1 = t64 % num_cu == 0;
+    const double pieces = run1 < S ? (double)S / (double)run1 : 0.0;
+    FewTilesEstimate e;
+    e.t_one = (whole1 ? 3.0 : 7.5 + 0.4 * (pieces > 2.0 ? pieces - 2.0 : 0.0)) + 0.5 * (double)run1;
+    const bool whole2 = t64 % (2LL * num_cu) == 0;
+    e.t_two = whole2 ? 3.5 + 0.92 * (double)(units / (2LL * num_cu)) : 1e300;
+    const double per_unit = (double)((t64 + num_cu - 1) / num_cu);
+    e.t_tiles = 4.5 + (variant == GEMM_T1 ? 0.615 : 0.575) * (double)S * per_unit;
+    return e;
+}
+}  // namespace
 
 // Fitted to times measured on MI355X (256 ... 2048-wide squares and panels, 1000 x 780 x 1532, K from 64 to
 // 131072, all three layouts), in microseconds, with S = 32-k stages per tile and `run` = stages per workgroup:
@@ -710,7 +838,6 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
     const long long S = ((long long)k + 31) / 32;
     const long long units = t64 * S;
     if (units < 2LL * num_cu) return -1;
-    const long long run1 = (units + num_cu - 1) / num_cu;
     const bool whole1 = t64 % num_cu == 0;
     // Many tiles with a long K whose runs are not whole tiles: neighbouring workgroups then sit at different k of
     // the same operand panels, nothing is shared through the L2, and 64 x 64 tiles -- 16 FLOP per byte staged --
@@ -722,15 +849,43 @@ int gemm_choose_streamk(int rows, int cols, int nz, int k, int num_cu, int varia
         const bool tall = (double)(rm * 128) * (double)(cn64 * 64) <= (double)(rm64 * 64) * (double)(cn * 128);
         return tall ? TILE_SK_128x64 : TILE_SK_64x128;
     }
-    const double pieces = run1 < S ? (double)S / (double)run1 : 0.0;
-    const double t_one = (whole1 ? 3.0 : 7.5 + 0.4 * (pieces > 2.0 ? pieces - 2.0 : 0.0)) + 0.5 * (double)run1;
-    const bool whole2 = t64 % (2LL * num_cu) == 0;
-    const double t_two = whole2 ? 3.5 + 0.92 * (double)(units / (2LL * num_cu)) : 1e300;
-    const double per_unit = (double)((t64 + num_cu - 1) / num_cu);
-    const double t_tiles = 4.5 + (variant == GEMM_T1 ? 0.615 : 0.575) * (double)S * per_unit;
-    const double t_balanced = t_two < t_one ? t_two : t_one;
-    if (t_balanced > 0.97 * t_tiles) return -1;
-    return t_two < t_one ? TILE_SK_64x64_O2 : TILE_SK_64x64;
+    const FewTilesEstimate est = few_tiles_estimate(t64, S, num_cu, variant);
+    const double t_balanced = est.t_two < est.t_one ? est.t_two : est.t_one;
+    if (t_balanced > 0.97 * est.t_tiles) return -1;
+    return est.t_two < est.t_one ? TILE_SK_64x64_O2 : TILE_SK_64x64;
+}
+
+double gemm_estimate_us(int rows, int cols, int nz, int k, int num_cu, int variant) {
+    if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return 0.0;
+    const long long rm64 = (rows + 63) / 64, cn64 = (cols + 63) / 64;
+    const long long t64 = rm64 * cn64 * nz;
+    const long long S = ((long long)k + 31) / 32;
+    if (t64 <= 2LL * num_cu) {
+        const FewTilesEstimate est = few_tiles_estimate(t64, S, num_cu, variant);
+        double t = est.t_tiles;
+        if (t64 * S >= 2LL * num_cu) {   // the balanced kernel's floor of two stages per unit
+            if (est.t_one < t) t = est.t_one;
+            if (est.t_two < t) t = est.t_two;
+        }
+        return t;
+    }
+    // more tiles: the matrix work of the padded tiles at 90 % of the chip's rate (256 FLOP per clock and unit,
+    // 2400 clocks per microsecond) and what a launch of that size costs beside it
+    const double flop = 2.0 * (double)(rm64 * 64) * (double)(cn64 * 64) * (double)nz * (double)k;
+    return flop / (0.9 * 614400.0 * (double)num_cu) + 4.0;
+}
+
+bool gemm_split_loses(int variant, int rows, int cols, int gz, int k, int k_slice, int num_cu) {
+    if (gz < 2 || k_slice < 32 || num_cu <= 0) return false;
+    // only where the unsplit product takes the balanced kernel: the tile-per-workgroup kernels deal whole tiles,
+    // and few of them leave units idle -- that is what the host's split is for
+    if (gemm_choose_streamk(rows, cols, 1, k, num_cu, variant) < 0) return false;
+    const long long t64 = (long long)((rows + 63) / 64) * ((cols + 63) / 64);
+    // equal runs of 128-class tiles' stages: a split adds nothing there but its fold
+    if (t64 > 2LL * num_cu) return true;
+    // the fold: a launch, and gz + 1 passes over C at about 5.5 TB/s
+    const double fold = 2.5 + 4.0 * (double)(gz + 1) * (double)rows * (double)cols / 5.5e6;
+    return gemm_estimate_us(rows, cols, 1, k, num_cu, variant) <= gemm_estimate_us(rows, cols, gz, k_slice, num_cu, variant) + fold;
 }
 
 hipError_t gemm_launch_streamk_conv(const GemmParams& p0, int tile, hipStream_t stream) {

@@ -12,6 +12,9 @@
 #include "../../include/dragon_hip_testing.h"
 #include "runtime_internal.h"
 
+namespace dragon {
+void gemm_streamk_release_workspace(hipStream_t stream);   // gemm_mfma_streamk.hip
+}
 namespace {
 // per host thread, like the runtime's own last error (cudaGetLastError in the reference,
 // Cuda/Cuda/Cuda_Exception.cuh:21-27): one thread never takes another thread's error code
@@ -76,7 +79,10 @@ int64_t dragon_Cuda_malloc(int64_t size) {
     if (note(hipMalloc(&p, (size_t)size)) != 0) return 0;
     return (int64_t)(intptr_t)p;
 }
-int dragon_Cuda_free(int64_t address) { return note(hipFree(as_ptr(address))); }
+int dragon_Cuda_free(int64_t address) {
+    dragon::split_ledger_touch(as_ptr(address), 0);
+    return note(hipFree(as_ptr(address)));
+}
 int64_t dragon_Cuda_mallocHost(int64_t size) {
     void* p = nullptr;
     if (size <= 0) { note(hipErrorInvalidValue); return 0; }
@@ -85,9 +91,11 @@ int64_t dragon_Cuda_mallocHost(int64_t size) {
 }
 int dragon_Cuda_freeHost(int64_t address) { return note(hipHostFree(as_ptr(address))); }
 int dragon_Cuda_memsetAsync(int64_t stream, int64_t address, int32_t value, int64_t size) {
+    dragon::split_ledger_touch(as_ptr(address), (size_t)size);
     return note(hipMemsetAsync(as_ptr(address), value, (size_t)size, as_stream(stream)));
 }
 static int copy_async(int64_t stream, int64_t dst, int64_t src, int64_t size, hipMemcpyKind kind) {
+    dragon::split_ledger_touch(as_ptr(dst), (size_t)size);   // a host destination never matches a device range
     return note(hipMemcpyAsync(as_ptr(dst), as_ptr(src), (size_t)size, kind, as_stream(stream)));
 }
 int dragon_Cuda_memcpyAsyncHostToDevice(int64_t s, int64_t dst, int64_t src, int64_t size) {
@@ -137,14 +145,18 @@ int64_t dragon_Cuda_newStream_NonBlocking(void) {
     if (note(hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) != 0) return 0;
     return (int64_t)(intptr_t)s;
 }
+// A stream that has launched the balanced product kernel owns a workspace in device memory (the library's only
+// allocation); it goes with the stream.
 int dragon_Cuda_deleteStream(int64_t stream) {
     if (stream == 0) return 0;  // the default stream is never destroyed
+    dragon::gemm_streamk_release_workspace(as_stream(stream));
     return note(hipStreamDestroy(as_stream(stream)));
 }
 int dragon_Cuda_deleteStreams(const int64_t* streams, int32_t length) {
     int rc = 0;
     for (int i = 0; i < length; i++) {
         if (streams[i] == 0) continue;
+        dragon::gemm_streamk_release_workspace(as_stream(streams[i]));
         int e = note(hipStreamDestroy(as_stream(streams[i])));
         if (e && !rc) rc = e;
     }
@@ -237,6 +249,7 @@ int32_t dragon_Cuda_getLastExceptionType(void) {
 // ---- float fill / transfer ---------------------------------------------------------
 int dragon_Cuda_set1D_value(int64_t stream, int64_t address, float value, int32_t length) {
     if (address == 0 || length <= 0) return note(hipErrorInvalidValue);
+    dragon::split_ledger_touch(as_ptr(address), (size_t)length * 4);
     hipLaunchKernelGGL(fill1d_kernel, dim3(launch_blocks(length, 256)), dim3(256), 0,
                        as_stream(stream), (float*)as_ptr(address), value, length);
     return note(hipGetLastError());
@@ -244,16 +257,25 @@ int dragon_Cuda_set1D_value(int64_t stream, int64_t address, float value, int32_
 int dragon_Cuda_set2D_value(int64_t stream, int64_t address, float value, int32_t height,
                             int32_t width, int32_t stride) {
     if (address == 0 || height <= 0 || width <= 0 || stride < width) return note(hipErrorInvalidValue);
+    dragon::split_ledger_touch(as_ptr(address), (size_t)height * stride * 4);
     hipLaunchKernelGGL(fill2d_kernel, dim3(launch_blocks((long long)height * stride, 256)),
                        dim3(256), 0, as_stream(stream), (float*)as_ptr(address), value, height,
                        width, stride);
     return note(hipGetLastError());
 }
 
+int dragon_test_mem_get_info(int64_t* free_bytes, int64_t* total_bytes) {
+    size_t f = 0, t = 0;
+    const int e = note(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = (int64_t)f;
+    if (total_bytes) *total_bytes = (int64_t)t;
+    return e;
+}
 int dragon_test_copy1D_kernel(int64_t stream, int64_t dst, int64_t src, int64_t length) {
     if (dst == 0 || src == 0 || length <= 0 || (length & 3) || ((dst | src) & 15))
         return note(hipErrorInvalidValue);
     const long long n4 = length >> 2;
+    dragon::split_ledger_touch(as_ptr(dst), (size_t)length * 4);
     hipLaunchKernelGGL(copy4_kernel, dim3(launch_blocks(n4, 256)), dim3(256), 0, as_stream(stream),
                        (v4f*)as_ptr(dst), (const v4f*)as_ptr(src), n4);
     return note(hipGetLastError());

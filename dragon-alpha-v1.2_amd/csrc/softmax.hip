@@ -9,6 +9,7 @@
 //     the tensor five times; the optional scale folds the preceding sdiv launch in as well.
 // Both are bound by HBM.
 #include <hip/hip_runtime.h>
+#include "runtime_internal.h"
 #include <stdint.h>
 #include "../../include/dragon_hip_gemm.h"
 
@@ -140,6 +141,7 @@ int dragon_Cuda_function_linear2D(int64_t stream, float alpha, int64_t dX, float
     if (lengthv <= 0 || (lengthv & 3) || stride <= 0 || (stride & 3) || width <= 0 || width > stride ||
         lengthv % stride != 0)
         return hipErrorInvalidValue;
+    dragon::split_ledger_touch((const void*)(intptr_t)dY, (size_t)lengthv * 4);
     const int length4 = lengthv >> 2;
     // one 16-byte element per thread, workgroups in address order: measured on a 1 GiB tensor in place 6.0 TB/s,
     // against 4.7 for 8192 workgroups that stride over the tensor (neighbours in time then touch addresses far apart)
@@ -158,6 +160,7 @@ int dragon_Cuda_reduce_softmax2D(int64_t stream, int64_t dX, int64_t dY, int32_t
     hipStream_t s = (hipStream_t)(intptr_t)stream;
     const float* X = (const float*)(intptr_t)dX;
     float* Y = (float*)(intptr_t)dY;
+    dragon::split_ledger_touch(Y, (size_t)field_length * row_lengthv * 4);
     const dim3 grid4((field_length + 3) / 4), block(256);
 #define WAVE_CASE(NV)                                                                                    \
     hipLaunchKernelGGL(softmax_wave_kernel<NV>, grid4, block, 0, s, X, Y, field_length, row_lengthv, width, \

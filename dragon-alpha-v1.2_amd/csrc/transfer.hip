@@ -274,6 +274,7 @@ int dragon_Cuda_get1D(int64_t stream, int64_t address, float* value, int32_t len
 }
 int dragon_Cuda_set1D(int64_t stream, int64_t address, const float* value, int32_t length) {
     if (address == 0 || value == nullptr || length <= 0) return note(hipErrorInvalidValue);
+    dragon::split_ledger_touch(as_ptr(address), (size_t)length * 4);
     hipStream_t s = as_stream(stream);
     int e = note(hipMemcpyAsync(as_ptr(address), value, sizeof(float) * (size_t)length, hipMemcpyHostToDevice, s));
     return e ? e : sync(s);
@@ -284,6 +285,7 @@ int dragon_Cuda_get1D_v2(int64_t stream, int64_t address, float* value, int64_t 
 }
 int dragon_Cuda_set1D_v2(int64_t stream, int64_t address, const float* value, int64_t buf, int32_t length) {
     if (address == 0 || value == nullptr || buf == 0 || length <= 0) return note(hipErrorInvalidValue);
+    dragon::split_ledger_touch(as_ptr(address), (size_t)length * 4);
     return upload_linear(as_stream(stream), (float*)as_ptr(address), value, (float*)as_ptr(buf), length);
 }
 
@@ -300,6 +302,7 @@ int dragon_Cuda_get2D_v2(int64_t stream, int64_t address, float* value, int64_t 
 int dragon_Cuda_set2D_v2(int64_t stream, int64_t address, const float* value, int64_t buf, int32_t height,
                          int32_t width, int32_t stride) {
     if (bad2d(address, value, height, width, stride) || buf == 0) return note(hipErrorInvalidValue);
+    dragon::split_ledger_touch(as_ptr(address), (size_t)height * stride * 4);
     hipStream_t s = as_stream(stream);
     float* dX = (float*)as_ptr(address);
     float* b = (float*)as_ptr(buf);
@@ -321,6 +324,7 @@ int dragon_Cuda_set2D(int64_t stream, int64_t address, const float* value, int32
                       int32_t stride) {
     if (bad2d(address, value, height, width, stride)) return note(hipErrorInvalidValue);
     if (width == stride) return dragon_Cuda_set1D(stream, address, value, height * width);
+    dragon::split_ledger_touch(as_ptr(address), (size_t)height * stride * 4);
     std::vector<float> staging((size_t)height * stride);
     return upload_staged(as_stream(stream), (float*)as_ptr(address), value, staging.data(), height, width,
                          stride);

@@ -14,6 +14,7 @@
 //     strided stores (its own comments quote a third of the row-copy rate for it).
 // Both are bound by HBM: one read and one write of the tensor.
 #include <hip/hip_runtime.h>
+#include "runtime_internal.h"
 #include <stdint.h>
 #include "../../include/dragon_hip_gemm.h"
 
@@ -117,6 +118,7 @@ int transpose_launch(int64_t stream, int64_t dX, int64_t dY, Dims4 xd, int i1, i
     hipStream_t s = (hipStream_t)(intptr_t)stream;
     const float* X = (const float*)(intptr_t)dX;
     float* Y = (float*)(intptr_t)dY;
+    dragon::split_ledger_touch(Y, (size_t)yd.d[0] * yd.d[1] * yd.d[2] * (size_t)strideY * 4);
     if (i2 < 3) {
         if (strideX != strideY) return hipErrorInvalidValue;
         const long long rows = (long long)xd.d[0] * xd.d[1] * xd.d[2];

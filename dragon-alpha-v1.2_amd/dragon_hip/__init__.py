@@ -453,6 +453,53 @@ def force_tile(tile):
     lib.dragon_gemm_force_tile(int(tile))
 
 
+def split_policy(mode):
+    """How the split-K entries treat GridZ: -1 the estimate decides, 0 always as asked, 1 declined where possible."""
+    lib.dragon_gemm_split_policy(int(mode))
+
+
+def fold_skip(on):
+    """Whether the no-op fold after a declined split is elided (default on).  Test hook."""
+    lib.dragon_gemm_fold_skip(int(bool(on)))
+
+
+def folds_skipped():
+    return lib.dragon_gemm_folds_skipped()
+
+
+def declined_splits():
+    return lib.dragon_gemm_declined_splits()
+
+
+def split_loses(variant, N, M, GZ, K, num_cu=256):
+    return lib.dragon_gemm_split_loses(variant, N, M, GZ, K, num_cu)
+
+
+def estimate_us(variant, rows, cols, nz, k, num_cu=256):
+    return lib.dragon_gemm_estimate_us(variant, rows, cols, nz, k, num_cu)
+
+
+def workspace_count():
+    return lib.dragon_gemm_workspace_count()
+
+
+def workspaces_refused():
+    return lib.dragon_gemm_workspaces_refused()
+
+
+def release_workspaces():
+    """Frees every per-stream workspace of the balanced kernel; returns how many there were."""
+    return lib.dragon_gemm_release_workspaces()
+
+
+def mem_get_info():
+    """(free, total) bytes of device memory on the current device."""
+    import ctypes
+    f, t = ctypes.c_int64(0), ctypes.c_int64(0)
+    _check(lib.dragon_test_mem_get_info(ctypes.byref(f), ctypes.byref(t)))
+    return f.value, t.value
+
+
 def choose_tile(variant, rows, cols, nz, k, num_cu=256):
     """The tile shape the automatic choice takes (host arithmetic only)."""
     return lib.dragon_gemm_choose_tile(variant, rows, cols, nz, k, num_cu)

@@ -79,6 +79,16 @@ SIGNATURES = {
     "dragon_Cuda_matMul_nstream": (i32, [i32, i32]),
     "dragon_Cuda_batchMatMul_streamSize": (i32, [i32, i32]),
     "dragon_gemm_force_tile": (None, [i32]),
+    "dragon_test_mem_get_info": (i32, [POINTER(i64), POINTER(i64)]),
+    "dragon_gemm_split_policy": (None, [i32]),
+    "dragon_gemm_fold_skip": (None, [i32]),
+    "dragon_gemm_folds_skipped": (i64, []),
+    "dragon_gemm_declined_splits": (i64, []),
+    "dragon_gemm_split_loses": (i32, [i32, i32, i32, i32, i32, i32]),
+    "dragon_gemm_estimate_us": (ctypes.c_double, [i32, i32, i32, i32, i32, i32]),
+    "dragon_gemm_workspace_count": (i32, []),
+    "dragon_gemm_workspaces_refused": (i64, []),
+    "dragon_gemm_release_workspaces": (i32, []),
     "dragon_gemm_choose_tile": (i32, [i32, i32, i32, i32, i32, i32]),
     "dragon_gemm_paired_form_fits": (i32, [i32, i32, i32, i32, i32]),
     "dragon_gemm_tile_divisor": (None, [ctypes.c_uint32, POINTER(ctypes.c_uint32), POINTER(ctypes.c_uint32)]),

@@ -21,11 +21,14 @@
  *     aligned; no caller memory is freed or retained here.  The one thing the library allocates:
  *     for large products (K from 768 on), for products with few tiles and a long K (at most two
  *     64 x 64 tiles of C per compute unit) and for their split-K forms the first call on a stream
- *     makes a 32 MiB workspace that later calls on the same stream handle reuse (partial tiles of
- *     workgroups that share the K range of a tile pass through it); it is kept until the process
- *     ends, at most 64 of them exist, and none is made or used while the stream is being
- *     captured into a graph -- such a call runs the ordinary kernel instead, as does every call
- *     when the allocation fails.
+ *     makes a 32 MiB workspace (one hipMalloc, and a small kernel on that stream that clears its
+ *     counters; nothing waits and no other stream is touched) that later calls on the same stream
+ *     handle reuse (partial tiles of workgroups that share the K range of a tile pass through it).
+ *     The workspace belongs to the stream: dragon_Cuda_deleteStream / deleteStreams give it back,
+ *     dragon_gemm_release_workspaces() below gives all of them back.  At most 64 exist at a time
+ *     (a launch on a 65th stream runs the ordinary kernel), and none is made or used while the
+ *     stream is being captured into a graph -- such a call runs the ordinary kernel instead, as
+ *     does every call when the allocation fails.
  *   - C is overwritten (no alpha/beta).  Padded rows/columns of C receive exact zeros.
  *   - streams[0..length) are valid stream handles, 1 <= length <= 10.  Work is issued
  *     asynchronously on streams[0]; the other handles are left idle (the caller joins
@@ -75,6 +78,21 @@ int dragon_Cuda_matMul_matMulT2(const int64_t* streams, int32_t length,
 /* ---- split-K stage 1: K is cut into GridZ slices of K_slice = (K/GridZ)>>3<<3, the
  * last slice takes the remainder; slice 0 is written to C, slice z >= 1 to
  * Cbuf + (z-1)*N*M.  Cbuf holds (GridZ-1)*N*M floats.  GridZ >= 1.
+ * What the caller may rely on is the SUM: C + sum over the GridZ-1 partials of Cbuf is the
+ * product, and every float of C and Cbuf is written.  Where the library estimates that the
+ * unsplit product is faster than the slices plus their fold (its balanced kernel deals equal
+ * shares of K to the compute units by itself; e.g. 1000 x 780 x 1532 with GridZ 2), it declines
+ * the split: the whole product goes to C and Cbuf gets exact zeros, in the same launch, so that
+ * SKbuf_summary afterwards leaves C as it is.  Where the split wins (256 x 256 x 131072 in 128
+ * slices) the slices are computed as asked.
+ * The library remembers a declined call (stream, Cbuf, C, GridZ-1, N*M): the SKbuf_summary call
+ * with exactly these arguments on streams[0] -- the one the reference's host issues next,
+ * CudaFloat32EngineBase.java:1565-1588 -- would add zeros and returns without launching
+ * anything.  The memory is forgotten at its first use, when any entry point of this library
+ * writes to or frees memory that overlaps that C or Cbuf, and when 64 later declined calls
+ * exist; a fold with other arguments, or after the entry is gone, runs as usual and finds the
+ * zeros.  Only writes that bypass this library (another library's kernels writing into Cbuf
+ * between the two calls) are invisible to it: a host that does that must not rely on the fold.
  * Replace ..._Cuda_1matMul_matMulSK / matMulT1SK / matMulT2SK (MM/A.cu:59-79, 108-128,
  * 157-178; JM/Cuda_matMul.java:137, 251, 343; slice rule MM/micro.cuh:92 and
  * MM/matMulSK_kernel.cuh:124-131). */
@@ -95,6 +113,13 @@ int dragon_Cuda_matMul_matMulT2SK(const int64_t* streams, int32_t length, int32_
  * kernel MM/SKbufsum.cuh:29-81). */
 int dragon_Cuda_matMul_SKbuf_summary(int64_t stream, int64_t dCbuf, int64_t dC,
                                      int32_t part, int32_t sizeC);
+
+/* Gives back every per-stream workspace the library holds (see the conventions above), on every
+ * device, after synchronising that device; returns how many there were.  For hosts that keep their
+ * streams for the life of the process and want the memory back in between; streams that run a large or
+ * few-tile product again get a new workspace.  No counterpart in the reference, whose natives own no
+ * device memory (engine-cuda-base/Cuda/Cuda/Cuda_Stream.cuh:55-75 destroys a stream and that is all). */
+int32_t dragon_gemm_release_workspaces(void);
 
 /* ---- the complete split-K product without any allocation: stage 1 as above (variant 0 = A*B,
  * 1 = A^T*B, 2 = A*B^T), the GridZ-1 partial products in a workspace that is part of the library's

@@ -27,7 +27,9 @@ extern "C" {
  * convolutions): 18 = 64x64, 19 = 128x64, 20 = 64x128, 21 = 128x128 with one workgroup per
  * compute unit, 22 = 64x64 and 23 = 128x64 with two, 25 = 256x64 with one.  24: the band kernel
  * for a K of at most 64 under a large C (a band of 128 rows of A stays in LDS; a longer K falls
- * back to the automatic choice). */
+ * back to the automatic choice).  26: the resident-K kernel for a K of 89 ... 144 (64x64 tiles whose whole K
+ * sits in LDS, the rim of C -- 1 ... 4 rows / columns past a multiple of 64 -- as strips of 4x4 MFMA blocks;
+ * another K falls back to the automatic choice). */
 void dragon_gemm_force_tile(int32_t tile);
 /* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
  * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the
@@ -42,6 +44,31 @@ void dragon_gemm_tile_divisor(uint32_t d, uint32_t* mul, uint32_t* shift);
  * Pure host arithmetic (no device needed); returns the forced shape while the calling thread forces one,
  * -1 on bad arguments. */
 int32_t dragon_gemm_choose_tile(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu);
+/* How the split-K entry points (matMulSK, matMulT1SK, matMulT2SK, matMulSK_static) treat the caller's GridZ,
+ * for the following calls OF THE CALLING THREAD: -1 (default) the library's estimate decides -- where the
+ * unsplit product through the balanced kernel is estimated to beat the slices plus their fold, the whole
+ * product goes to C and the partial buffers get exact zeros; 0 the K slices always as asked; 1 declined
+ * wherever the unsplit product can take the balanced kernel.  A forced tile shape always honours the split. */
+void dragon_gemm_split_policy(int32_t mode);
+/* 0: SKbuf_summary always launches its kernel; 1 (default): the fold that follows a declined split with the
+ * same stream, Cbuf, C, part and sizeC -- which would add zeros -- returns without launching (see
+ * dragon_hip_gemm.h).  Process-wide.  And the number of folds elided so far. */
+void dragon_gemm_fold_skip(int32_t on);
+int64_t dragon_gemm_folds_skipped(void);
+/* Split-K calls of this process that ran unsplit (with zeroed partial buffers) so far. */
+int64_t dragon_gemm_declined_splits(void);
+/* 1 if the estimate declines GridZ slices of the 2-D product N x M x K (all multiples of 4) on num_cu compute
+ * units, 0 if it honours them, -1 on bad arguments; and the estimate itself in microseconds for `nz` products
+ * (or K slices) of rows x cols x k.  Host arithmetic only. */
+int32_t dragon_gemm_split_loses(int32_t variant, int32_t N, int32_t M, int32_t GridZ, int32_t K, int32_t num_cu);
+double dragon_gemm_estimate_us(int32_t variant, int32_t rows, int32_t cols, int32_t nz, int32_t k, int32_t num_cu);
+/* The balanced kernel's per-stream workspaces (device memory the library owns, see dragon_hip_gemm.h):
+ * how many it holds now, and how many balanced launches found the table of 64 full and took a
+ * tile-per-workgroup kernel instead. */
+int32_t dragon_gemm_workspace_count(void);
+int64_t dragon_gemm_workspaces_refused(void);
+/* Free and total device memory of the current device in bytes (hipMemGetInfo). */
+int dragon_test_mem_get_info(int64_t* free_bytes, int64_t* total_bytes);
 /* Device-to-device copy of `length` floats (a multiple of 4, 16-byte aligned) done by an ordinary
  * kernel rather than the copy engine: the known-size copy that hardware byte counters are
  * calibrated against when profiling. */

@@ -207,7 +207,13 @@ def test_tile_choice_on_the_documented_shapes(dh):
     # many tiles, a long K, runs that are not whole tiles: the half-size tile (fewer bytes staged per FLOP)
     assert ct(NN, 1000, 780, 1, 8192) == 19 and ct(NN, 768, 768, 1, 8192) == 19 and ct(NN, 1280, 1280, 1, 4096) in (19, 20)
     assert ct(NN, 640, 640, 1, 4096) == 18 and ct(NN, 1000, 780, 1, 3072) == 18 and ct(NN, 1024, 1024, 1, 4096) == 18
-    assert ct(NN, 257, 388, 36, 129) == 1                       # batch of small ragged products: 64x64
+    # a batch of ragged products with a K of 89 ... 144: the resident-K kernel (26) where C has a rim of 1 ... 4 rows
+    # or columns past a multiple of 64 and there are at least two 64x64 tiles per unit
+    for v in (NN, T1, T2):
+        assert ct(v, 257, 388, 36, 129) == 26 and ct(v, 257, 388, 36, 132) == 26 and ct(v, 961, 772, 4, 100) == 26
+        assert ct(v, 257, 388, 36, 88) != 26 and ct(v, 257, 388, 36, 148) != 26 and ct(v, 256, 384, 36, 129) != 26
+        assert ct(v, 257, 388, 8, 129) != 26                   # 192 tiles: too few
+    assert ct(NN, 257, 388, 36, 64) == 1                        # a shorter K: 64x64 tiles with the rim beside them
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
     if ct(NN, *shape) in (5 + P, 9 + P):
@@ -226,7 +232,7 @@ def test_tile_choice_stays_inside_what_the_kernels_accept(dh):
     # that fits its one stage, and every id is one that exists
     rng = np.random.default_rng(20240607)
     dims = {18: (64, 64), 19: (128, 64), 20: (64, 128), 21: (128, 128), 22: (64, 64), 23: (128, 64), 25: (256, 64)}
-    valid = set(range(0, 26)) | set(range(256, 266))
+    valid = set(range(0, 27)) | set(range(256, 266))
     dh.force_tile(-1)
     seen = set()
     for _ in range(20000):
@@ -243,4 +249,6 @@ def test_tile_choice_stays_inside_what_the_kernels_accept(dh):
                 assert -(-rows // bm) * -(-cols // bn) * nz <= 65536, (v, rows, cols, nz, k, t)
             if t == 24:
                 assert 56 < k <= 64 and cols % 32 == 0, (v, rows, cols, nz, k)
+            if t == 26:
+                assert 88 < k <= 144, (v, rows, cols, nz, k)
     assert {21, 24} <= seen and seen & {18, 22} and seen & {19, 20, 23}      # the sample reaches every family

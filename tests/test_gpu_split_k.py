@@ -3,9 +3,19 @@ import numpy as np
 import pytest
 
 from oracle import oracle
-from helpers import NN, T1, T2, VARIANT_NAMES, assert_within_tolerance, logical_operands, pad2, rel_fro
+from helpers import NN, T1, T2, VARIANT_NAMES, assert_within_tolerance, gpu_matmul_2d, logical_operands, pad2, rel_fro
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _slices_as_asked(gpu):
+    """The tests of the slice rule need the slices: the entry points are told to honour every GridZ (they
+    otherwise decline a split they estimate to lose; that behaviour has tests of its own below)."""
+    gpu.split_policy(0)
+    yield
+    gpu.split_policy(-1)
+    gpu.force_tile(-1)
 
 
 def run_sk(gpu, variant, A, B, GZ, summary=True, fill=9.0):
@@ -133,3 +143,148 @@ def test_degenerate_slices(gpu):
     MM.matMulT1SK([0], 1, 1, dA.address, dB.address, dC.address, 0, 32, 36, 24)
     gpu.Cuda.streamSynchronize(0)
     assert np.array_equal(dC.get((32, 36)), oracle.matmul(T1, A, B))
+
+
+# ---- a split that loses is declined: the whole product in C, exact zeros in the partial buffers ----
+
+DECLINED = [((1000, 780, 1532), 2), ((512, 512, 4096), 2), ((1024, 768, 2048), 2)]
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("shape_gz", DECLINED)
+def test_a_losing_split_is_declined(gpu, variant, shape_gz):
+    """The host's policy asks for GridZ slices of a product that the balanced kernel runs faster unsplit (the
+    three shapes: two 64 x 64 tiles per unit at most and a K long enough): C then holds the whole product --
+    the very bits of the unsplit entry point --, every float of Cbuf is +0, and the fold leaves C as it is."""
+    (N, M, K), GZ = shape_gz
+    assert gpu.split_loses(variant, N, M, GZ, K, gpu.Cuda.multiProcessorCount(0)) == 1
+    gpu.split_policy(-1)
+    rng = np.random.default_rng(N + GZ + variant)
+    for dist in ("int", "uniform"):
+        A, B = logical_operands(variant, rng, N, M, K, dist=dist)
+        before = gpu.declined_splits()
+        C, Cbuf = run_sk(gpu, variant, A, B, GZ, summary=False)
+        assert gpu.declined_splits() == before + 1
+        assert not Cbuf.view(np.uint32).any(), "the partial buffers of a declined split hold exact zeros"
+        unsplit, _ = gpu_matmul_2d(gpu, variant, A, B)
+        assert np.array_equal(C.view(np.uint32), unsplit.view(np.uint32))
+        folded, _ = run_sk(gpu, variant, A, B, GZ, summary=True)
+        assert np.array_equal(folded.view(np.uint32), C.view(np.uint32))
+        R = oracle.matmul(variant, A, B)
+        if dist == "int":
+            assert np.array_equal(C, R)
+        else:
+            assert_within_tolerance(C, R, K, A, B, "%s declined GZ=%d" % (VARIANT_NAMES[variant], GZ))
+        # the same call with the slices forced: C + the partials is the same product
+        gpu.split_policy(0)
+        C0, Cb0 = run_sk(gpu, variant, A, B, GZ, summary=False)
+        gpu.split_policy(-1)
+        total = C0.astype(np.float64) + Cb0.astype(np.float64).sum(axis=0)
+        assert_within_tolerance(total, R, K, A, B, "%s honoured GZ=%d" % (VARIANT_NAMES[variant], GZ))
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_a_winning_split_is_honoured(gpu, variant):
+    """256 x 256 x 8192 in 32 slices: 512 (slice, tile) pairs deal whole to the units, the unsplit product has
+    sixteen workgroups per tile to put together -- the slices stay, bit for bit where the oracle puts them."""
+    (N, M, K), GZ = (256, 256, 8192), 32
+    assert gpu.split_loses(variant, N, M, GZ, K, gpu.Cuda.multiProcessorCount(0)) == 0
+    gpu.split_policy(-1)
+    rng = np.random.default_rng(17 + variant)
+    A, B = logical_operands(variant, rng, N, M, K, dist="int")
+    before = gpu.declined_splits()
+    C, Cbuf = run_sk(gpu, variant, A, B, GZ, summary=False)
+    assert gpu.declined_splits() == before
+    C0, Cb0 = oracle.matMulSK(variant, GZ, A, B)
+    assert np.array_equal(C, C0) and np.array_equal(Cbuf, Cb0)
+
+
+def test_a_forced_decline_and_a_bias_row(gpu):
+    """Policy 1 declines wherever the unsplit product can take the balanced kernel, whatever the estimate
+    says; shapes it cannot take (too few stages) keep their slices."""
+    gpu.split_policy(1)
+    rng = np.random.default_rng(2)
+    A, B = logical_operands(T1, rng, 256, 256, 8192, dist="int")
+    C, Cbuf = run_sk(gpu, T1, A, B, 32, summary=False)
+    assert not Cbuf.view(np.uint32).any() and np.array_equal(C, oracle.matmul(T1, A, B))
+    A, B = logical_operands(NN, rng, 64, 64, 256, dist="int")
+    C, Cbuf = run_sk(gpu, NN, A, B, 2, summary=False)
+    C0, Cb0 = oracle.matMulSK(NN, 2, A, B)
+    assert np.array_equal(C, C0) and np.array_equal(Cbuf, Cb0)
+
+
+def test_the_fold_after_a_declined_split_is_elided_only_when_it_is_a_no_op(gpu):
+    """SKbuf_summary with the stream, Cbuf, C, part and sizeC of the declined call just before returns without
+    a launch; any other fold, and the same fold after the library has seen a write to C or Cbuf, runs."""
+    MM, Cuda = gpu.Cuda_matMul, gpu.Cuda
+    N, M, K, GZ = 1000, 780, 1532, 2
+    rng = np.random.default_rng(31)
+    A, B = logical_operands(NN, rng, N, M, K, dist="int")
+    R = oracle.matmul(NN, A, B)
+    dA, dB = gpu.DeviceArray(A), gpu.DeviceArray(B)
+    dC, dCbuf = gpu.DeviceArray(size=N * M), gpu.DeviceArray(size=N * M)
+    s1, s2 = Cuda.newStream_NonBlocking(), Cuda.newStream_NonBlocking()
+    gpu.split_policy(-1)
+
+    def declined_call():
+        before = gpu.declined_splits()
+        MM.matMulSK([s1], 1, GZ, dA.address, dB.address, dC.address, dCbuf.address, N, M, K)
+        assert gpu.declined_splits() == before + 1
+
+    # 1. the reference's sequence: elided, C is the product
+    declined_call()
+    n0 = gpu.folds_skipped()
+    MM.SKbuf_summary(s1, dCbuf.address, dC.address, GZ - 1, N * M)
+    assert gpu.folds_skipped() == n0 + 1
+    Cuda.streamSynchronize(s1)
+    assert np.array_equal(dC.get((N, M)), R)
+    # 2. the same fold once more: the memory was used up, the kernel runs (adds the zeros in Cbuf)
+    MM.SKbuf_summary(s1, dCbuf.address, dC.address, GZ - 1, N * M)
+    assert gpu.folds_skipped() == n0 + 1
+    Cuda.streamSynchronize(s1)
+    assert np.array_equal(dC.get((N, M)), R)
+    # 3. the host overwrites Cbuf through the library between the two calls: the fold must add what is there now
+    declined_call()
+    Cuda.streamSynchronize(s1)
+    ones = np.ones(N * M, np.float32)
+    Cuda.set1D(s1, dCbuf.address, ones, N * M)
+    MM.SKbuf_summary(s1, dCbuf.address, dC.address, GZ - 1, N * M)
+    assert gpu.folds_skipped() == n0 + 1
+    Cuda.streamSynchronize(s1)
+    assert np.array_equal(dC.get((N, M)), R + 1.0)
+    # 4. other arguments (another stream; another part): the kernel runs
+    declined_call()
+    Cuda.streamSynchronize(s1)
+    MM.SKbuf_summary(s2, dCbuf.address, dC.address, GZ - 1, N * M)
+    assert gpu.folds_skipped() == n0 + 1
+    Cuda.streamSynchronize(s2)
+    assert np.array_equal(dC.get((N, M)), R)
+    # 5. C written by another product of the library in between: the entry is gone, the fold runs on what C holds
+    declined_call()
+    MM.matMul([s1], 1, dA.address, dB.address, dC.address, N, M, K)
+    MM.SKbuf_summary(s1, dCbuf.address, dC.address, GZ - 1, N * M)
+    assert gpu.folds_skipped() == n0 + 1
+    # 6. switched off: every fold is launched
+    gpu.fold_skip(0)
+    try:
+        declined_call()
+        MM.SKbuf_summary(s1, dCbuf.address, dC.address, GZ - 1, N * M)
+        assert gpu.folds_skipped() == n0 + 1
+        Cuda.streamSynchronize(s1)
+        assert np.array_equal(dC.get((N, M)), R)
+    finally:
+        gpu.fold_skip(1)
+    # 7. freed memory takes its entry along: a new allocation at the same address is not mistaken for it
+    declined_call()
+    Cuda.streamSynchronize(s1)
+    address = dCbuf.address
+    dCbuf.free()
+    dCbuf = gpu.DeviceArray(np.full(N * M, 2.0, np.float32))
+    MM.SKbuf_summary(s1, dCbuf.address, dC.address, GZ - 1, N * M)
+    assert gpu.folds_skipped() == n0 + 1
+    Cuda.streamSynchronize(s1)
+    assert np.array_equal(dC.get((N, M)), R + 2.0), "reused address %x / %x" % (address, dCbuf.address)
+    for x in (dA, dB, dC, dCbuf):
+        x.free()
+    Cuda.deleteStream(s1)
+    Cuda.deleteStream(s2)

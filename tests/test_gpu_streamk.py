@@ -135,6 +135,100 @@ def test_two_streams_have_a_workspace_each(gpu):
         Cuda.deleteStream(s)
 
 
+@pytest.mark.parametrize("tile", [18, 22, 23])
+def test_two_thousand_overlapping_launches_give_one_answer(gpu, tile):
+    """A bounded soak of the hand-over of shared tiles' pieces between workgroups, which rests on the order in
+    which the hardware makes stores visible rather than on fences: 2000 launches of two products whose tiles
+    are shared (1000 x 777 x 1531 and 257 x 385 x 4100), the two on a stream each so that launches overlap on
+    the device, twenty in flight at a time, every result compared bit for bit with the first launch's.  Stops
+    at the first mismatch."""
+    Cuda, MM = gpu.Cuda, gpu.Cuda_matMul
+    rng = np.random.default_rng(900 + tile)
+    streams = [Cuda.newStream_NonBlocking(), Cuda.newStream_NonBlocking()]
+    IN_FLIGHT, ROUNDS = 10, 100
+    jobs = []
+    for (N, M, K) in ((1000, 777, 1531), (257, 385, 4100)):
+        A, B = logical_operands(T1, rng, N, M, K, dist="normal")
+        Ap, Bp, dims = padded(T1, A, B)
+        jobs.append((gpu.DeviceArray(Ap), gpu.DeviceArray(Bp), [gpu.DeviceArray(size=dims[0] * dims[1]) for _ in range(IN_FLIGHT)], dims))
+    gpu.force_tile(tile)
+    first = [None, None]
+    launches = 0
+    try:
+        for rnd in range(ROUNDS):
+            for i in range(IN_FLIGHT):
+                for s, (dA, dB, dCs, (N, M, K)) in zip(streams, jobs):
+                    MM.matMulT1([s], 1, dA.address, dB.address, dCs[i].address, N, M, K)
+            for s in streams:
+                Cuda.streamSynchronize(s)
+            for j, (dA, dB, dCs, (N, M, K)) in enumerate(jobs):
+                for i in range(IN_FLIGHT):
+                    got = dCs[i].get((N, M)).view(np.uint32)
+                    launches += 1
+                    if first[j] is None:
+                        first[j] = got
+                    assert np.array_equal(first[j], got), "tile %d, product %d: launch %d differs from the first" % (tile, j, launches)
+                    dCs[i].fill(-1.0)
+        assert launches == 2 * IN_FLIGHT * ROUNDS
+    finally:
+        gpu.force_tile(-1)
+        for dA, dB, dCs, _ in jobs:
+            for x in [dA, dB] + dCs:
+                x.free()
+        for s in streams:
+            Cuda.deleteStream(s)
+
+
+def test_a_stream_takes_its_workspace_with_it(gpu):
+    """The balanced kernel's workspace belongs to the stream that first needed it: a hundred streams made, used
+    for a balanced launch and deleted leave the device's free memory where it was (to within one workspace),
+    the table of workspaces never fills up, and the hundredth stream still gets the balanced kernel."""
+    Cuda, MM = gpu.Cuda, gpu.Cuda_matMul
+    rng = np.random.default_rng(4)
+    N, M, K = 512, 512, 1024
+    A = rng.integers(-3, 4, (N, K)).astype(np.float32)
+    B = rng.integers(-3, 4, (K, M)).astype(np.float32)
+    R = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32)
+    dA, dB, dC = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(size=N * M)
+    gpu.release_workspaces()
+    held0, refused0 = gpu.workspace_count(), gpu.workspaces_refused()
+    assert held0 == 0
+    free0, _ = gpu.mem_get_info()
+    gpu.force_tile(21)
+    try:
+        for i in range(100):
+            s = Cuda.newStream_NonBlocking()
+            dC.fill(7.0)
+            MM.matMul([s], 1, dA.address, dB.address, dC.address, N, M, K)
+            Cuda.streamSynchronize(s)
+            assert gpu.workspace_count() == 1, "stream %d: the balanced kernel made no workspace" % i
+            if i % 33 == 0 or i == 99:
+                assert np.array_equal(dC.get((N, M)), R)
+            Cuda.deleteStream(s)
+            assert gpu.workspace_count() == 0
+    finally:
+        gpu.force_tile(-1)
+    assert gpu.workspaces_refused() == refused0
+    free1, _ = gpu.mem_get_info()
+    workspace_bytes = 4 * (65536 + 2 * Cuda.multiProcessorCount(0) * 128 * 128)
+    assert free0 - free1 <= workspace_bytes, "device memory not given back: %d bytes" % (free0 - free1)
+    # streams that are kept: release on request
+    s = Cuda.newStream_NonBlocking()
+    gpu.force_tile(21)
+    MM.matMul([s], 1, dA.address, dB.address, dC.address, N, M, K)
+    Cuda.streamSynchronize(s)
+    gpu.force_tile(-1)
+    assert gpu.workspace_count() == 1 and gpu.release_workspaces() == 1 and gpu.workspace_count() == 0
+    gpu.force_tile(21)
+    MM.matMul([s], 1, dA.address, dB.address, dC.address, N, M, K)     # and a new one on the next launch
+    Cuda.streamSynchronize(s)
+    gpu.force_tile(-1)
+    assert np.array_equal(dC.get((N, M)), R) and gpu.workspace_count() == 1
+    Cuda.deleteStream(s)
+    for x in (dA, dB, dC):
+        x.free()
+
+
 def test_host_threads_force_tiles_independently(gpu):
     """The forced tile is a setting of the calling thread: a second thread that forces another shape (or none)
     does not change what this thread's launches run, and its own choice is reported back to it."""
