@@ -148,7 +148,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the split-K / batched / ragged workloads")
-    ap.add_argument("--configs", default="3,4,5,sizes,bias,attention,conv,hbm,transpose,transfer,engine",
+    ap.add_argument("--configs", default="3,4,5,sizes,skinny,bias,attention,conv,hbm,transpose,transfer,engine",
                     help="which of the other workloads to time (default all): BASELINE configs 3, 4, 5, other sizes, "
                          "the biased fully-connected layer, the attention chain, the forward convolution, "
                          "dimension swaps, tensor upload / download, the host mirror's own overhead")
@@ -411,6 +411,35 @@ def main():
                 ms = timer.per_launch_ms(lambda: fn(S, 1, dA.address, dB.address, dC.address, r, c, k), iters=20)
                 record("%s %dx%dx%d" % (name, r, c, k), 2.0 * r * c * k, ms)
         for x in (dA, dB, dC):
+            x.free()
+
+    if "skinny" in extra:
+        # a C of 4 or 8 columns (or rows) under a long other side: the long operand is read once, so the figure that
+        # matters is bytes per second against the 8 TB/s of HBM.  The operands of the first three shapes fit or nearly
+        # fit the 256 MB Infinity Cache (134 ... 268 MB); the 1 GiB ones do not.
+        log("skinny products ...")
+        shapes = [(65536, 4, 1024), (8192, 8, 4096), (4, 65536, 1024), (8, 8192, 4096), (262144, 4, 1024), (262144, 8, 1024),
+                  (4, 262144, 1024), (8, 65536, 4096)]
+        nl = max(max(r, c) * k for r, c, k in shapes)
+        g = synthetic.stream_for(9)
+        block = g.normal((1 << 24,), 0.0, 1.0)          # the long operand repeats a 64 MiB block of normals
+        dL = dh.DeviceArray(np.tile(block, (nl + block.size - 1) // block.size)[:nl])
+        dS, dC = dh.DeviceArray(g.normal((8 * 8192,), 0.0, 1.0)), dh.DeviceArray(size=8 * 262144)
+        del block
+        for (r, c, k) in shapes:
+            long_is_a = r > c
+            da, db = (dL, dS) if long_is_a else (dS, dL)
+            nbytes = 4.0 * (r * k + k * c + r * c)
+            for name, fn in products:
+                for tile, label in ((-1, ""), (4 if long_is_a else 5, " through the %s tile kernel" % ("128x64" if long_is_a else "64x128"))):
+                    dh.force_tile(tile)
+                    ms = timer.per_launch_ms(lambda: fn(S, 1, da.address, db.address, dC.address, r, c, k), iters=10)
+                    dh.force_tile(-1)
+                    key = "%s %dx%dx%d%s" % (name, r, c, k, label)
+                    record(key, 2.0 * r * c * k, ms, nbytes)
+                    per_config[key]["pct_hbm_peak"] = round(100.0 * per_config[key]["alg_GBps"] / 8000.0, 1)
+                    per_config[key]["bound"] = "hbm" if 4.0 * max(r, c) * k > 300e6 else "hbm (operand near the Infinity Cache's 256 MB)"
+        for x in (dL, dS, dC):
             x.free()
 
     if "bias" in extra:

@@ -9,7 +9,7 @@ HIPFLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Wall -Wno-unused-function 
 mkdir -p build
 OBJS=""
 PIDS=""
-for s in gemm_mfma.hip gemm_mfma_biased.hip gemm_mfma_dma.hip gemm_mfma_streamk.hip gemm_mfma_band.hip gemm_mfma_shortk.hip gemm_mfma_conv.hip skbuf_summary.hip bias_row.hip c_abi_gemm.hip c_abi_conv.hip runtime.hip transfer.hip transpose.hip softmax.hip attention.hip; do
+for s in gemm_mfma.hip gemm_mfma_biased.hip gemm_mfma_dma.hip gemm_mfma_streamk.hip gemm_mfma_band.hip gemm_mfma_shortk.hip gemm_skinny.hip gemm_mfma_conv.hip skbuf_summary.hip bias_row.hip c_abi_gemm.hip c_abi_conv.hip runtime.hip transfer.hip transpose.hip softmax.hip attention.hip; do
   o=build/${s%.hip}.o
   # the host pass does not know the packed-fp32 target feature and says so: harmless
   if [ "$s" = gemm_mfma_streamk.hip ]; then

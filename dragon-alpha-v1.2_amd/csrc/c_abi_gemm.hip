@@ -489,6 +489,7 @@ int32_t dragon_Cuda_batchMatMul_streamSize(int32_t N, int32_t M) {
 }
 
 void dragon_gemm_force_tile(int32_t tile) { gemm_force_tile(tile); }
+void dragon_gemm_skinny_form(int32_t form) { gemm_skinny_form(form); }
 int32_t dragon_gemm_release_workspaces(void) { return gemm_streamk_release_workspaces(); }
 int32_t dragon_gemm_workspace_count(void) { return gemm_streamk_workspace_count(); }
 int64_t dragon_gemm_workspaces_refused(void) { return gemm_streamk_workspaces_refused(); }

@@ -106,6 +106,8 @@ static const TileTraits kTiles[TILE_ALL_COUNT] = {
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant) {
     const int forced = gemm_forced_tile();
     if (forced != TILE_AUTO) return forced;
+    const int skinny = gemm_choose_skinny(rows, cols, nz);
+    if (skinny >= 0) return skinny;
     const int band = gemm_choose_band(rows, cols, nz, k, num_cu, variant);
     if (band >= 0) return band;
     const int shortk = gemm_choose_shortk(rows, cols, nz, k, num_cu, variant);
@@ -173,11 +175,12 @@ int gemm_choose_tile_per_workgroup(int rows, int cols, int nz, int k, int num_cu
 
 hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t stream) {
     if (!gemm_pitches_addressable(p)) return hipErrorInvalidValue;
-    if (gemm_tile_is_streamk(tile) || gemm_tile_is_band(tile) || gemm_tile_is_shortk(tile)) {
+    if (gemm_tile_is_streamk(tile) || gemm_tile_is_band(tile) || gemm_tile_is_shortk(tile) || gemm_tile_is_skinny(tile)) {
         // where the product cannot take the balanced kernel (K slices shorter than a stage; a capturing
         // stream that has no workspace yet; a bias row on a transposed product) or the band kernel (a K beyond one stage, K slices, a
         // bias row) a tile-per-workgroup kernel takes over
-        const hipError_t e = gemm_tile_is_band(tile)     ? gemm_launch_band(variant, p, stream)
+        const hipError_t e = gemm_tile_is_skinny(tile)   ? gemm_launch_skinny(variant, p, stream)
+                             : gemm_tile_is_band(tile)   ? gemm_launch_band(variant, p, stream)
                              : gemm_tile_is_shortk(tile) ? gemm_launch_shortk(variant, p, stream)
                                                          : gemm_launch_streamk(variant, p, tile, stream);
         if (e != hipErrorOutOfMemory) return e;

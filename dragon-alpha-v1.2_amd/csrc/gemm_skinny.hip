@@ -1,0 +1,378 @@
+// Skinny products: a C of at most 8 columns (N x 4, N x 8) or at most 8 rows (4 x M, 8 x M) under a long other
+// side -- matrix times a few vectors.  The reference sends a C of 4 columns to kernels of their own
+// (MM/matMul_sernel.cuh:17-30, dispatched at MM/matMul.cuh:100-102) and thin row strips to k18 / k14 / k12
+// (MM/matMul.cuh:104-106).
+//
+// Such a product reads its long operand X (L lines of K) once and does next to nothing with it: it is bound by
+// HBM, and a 64 x 64 MFMA tile would multiply sixteen times the columns that exist.  Here every wavefront streams
+// lines of X from memory straight into registers -- no LDS, no barrier in the stream, two register buffers so that
+// the loads of one run under the arithmetic of the other -- and multiplies them with v_mfma_f32_4x4x1_16B_f32:
+// sixteen independent 4 x 4 x 1 products per instruction, i.e. 64 lanes' values of X against 4 lines of the short
+// operand S with no padded work.
+//   X K-outer (k is the row: A of A^T*B, B of A*B and A^T*B): a lane owns W lines (W = 1 or 4 consecutive outputs);
+//       the wavefront reads 64 W consecutive floats of a k row per instruction and adds k after k into the same
+//       4 x 4 blocks.  The sum of an output runs k-ascending.
+//   X K-inner (k contiguous: A of A*B and A*B^T, B of A*B^T): per instruction the wavefront reads 8 lines x 128
+//       bytes: lane l holds the 4 k at 4 * (l >> 3) of line (l & 7), two such instructions (lines 0-7, 8-15) make
+//       the 16 lines of a wavefront.  The 8 classes of k of a line meet at the end through three lane exchanges.
+// S's values come from memory as well (they stay in the L1: a few floats per k, the same for every wavefront).
+// Where the lines are too few to give every compute unit enough wavefronts, the 4 or 16 wavefronts of a workgroup
+// share their lines and split K; their sums meet in LDS and are added share after share, a fixed order.
+#include "gemm_mfma_kernel.h"
+
+namespace dragon {
+namespace {
+
+struct SkinnyParams {
+    const float* X;     // the long operand: L lines of K
+    const float* S;     // the short operand: T lines of K
+    float* C;
+    int L, K;           // lines of X (exact), contraction length (a multiple of 4)
+    int ldx, lds, ldc;  // leading strides in floats
+    int x_lines;        // lines X has in memory (rows of a K-inner X / row length of a K-outer one)
+    int s_lines;        // the same for S (<= T)
+    int k_share;        // 0: a wavefront takes its lines' whole K; else the k of each wavefront of a workgroup (a multiple of 32)
+    int out_rows;       // the short side is C's row index (C is T x L), else its column index (C is L x T)
+};
+
+typedef float sk_v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t skinny_rsrc(const float* base, long long bytes) {
+    const long long capped = bytes > 0xfffffff0LL ? 0xfffffff0LL : (bytes < 0 ? 0 : bytes);
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(unsigned)capped, RSRC_FLAGS);
+}
+__device__ __forceinline__ float ld1(__amdgpu_buffer_rsrc_t r, int off, int soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, soff, 0));
+}
+__device__ __forceinline__ sk_v4f ld4(__amdgpu_buffer_rsrc_t r, int off, int soff) {
+    return __builtin_bit_cast(sk_v4f, __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, 0));
+}
+template <int W> struct XVal;
+template <> struct XVal<1> { float v; __device__ __forceinline__ float at(int) const { return v; } };
+template <> struct XVal<4> { sk_v4f v; __device__ __forceinline__ float at(int c) const { const float value = v[c]; return value; } };
+
+__device__ __forceinline__ void skinny_put(const SkinnyParams& p, int line, int col, float value) {
+    if (line < p.L) {
+        if (p.out_rows) p.C[(size_t)col * p.ldc + line] = value;
+        else p.C[(size_t)line * p.ldc + col] = value;
+    }
+}
+
+// W: floats of a K-outer X a lane reads per k row (1 or 4), or sets of 8 lines of a K-inner X per wavefront (2 or 4).
+// CL: classes of k among the lanes of a K-outer X with W = 1 (2: lanes 0-31 take the even k rows of 32 lines, lanes
+// 32-63 the odd ones).  NW: wavefronts of a workgroup.
+template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
+__global__ __launch_bounds__(NW * 64)
+void gemm_f32_skinny(const SkinnyParams p) {
+    static_assert(T == 4 || T == 8, "4 or 8 short lines");
+    static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || (CL == 2 && W == 1)), "forms");
+    constexpr int LS = 8, PK = 32;                         // K-inner X: lines per read, k per panel
+    constexpr int H = T / 4;                               // groups of 4 short lines
+    constexpr int LINES = X_KIN ? LS * W : 64 * W / CL;    // lines of X per wavefront
+    constexpr int ACCS = W * H;                            // 4 x 4 accumulator blocks per lane
+    constexpr int MEET_LANES = X_KIN ? LS : 64 / CL;       // lanes that hold outputs once the classes of k have met
+    __shared__ float meet_lds[NW][ACCS * 4][MEET_LANES];
+
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const bool shared = p.k_share > 0;
+    const int unit = shared ? blockIdx.x : blockIdx.x * NW + wave;     // which run of LINES lines
+    const int line0 = unit * LINES;
+    const int k_begin = shared ? wave * p.k_share : 0;
+    const int k_end = shared ? min(p.K, k_begin + p.k_share) : p.K;
+    const int j = lane & 3;
+
+    // S(k, j): rows beyond K (K-outer) or lines beyond those S has (K-inner) lie beyond the descriptor's end
+    const __amdgpu_buffer_rsrc_t rs = skinny_rsrc(p.S, S_KIN ? (long long)p.s_lines * p.lds * 4 : ((long long)(p.K - 1) * p.lds + p.s_lines) * 4);
+    sk_v4f d[ACCS];
+#pragma unroll
+    for (int a = 0; a < ACCS; a++) d[a] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
+
+    if (line0 < p.L && k_begin < k_end) {
+        if constexpr (!X_KIN) {
+            // ---- a lane owns W lines: X[k][line0 + W * lane + c] (CL = 2: X[k + class][line0 + (lane & 31)]);
+            //      U loads (U * CL k rows) per register buffer ----
+            constexpr int U = W == 4 ? 8 : 16;
+            const int cls = CL == 2 ? lane >> 5 : 0;
+            const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, ((long long)(p.K - 1) * p.ldx + p.x_lines) * 4);
+            const int x_step = p.ldx * 4;
+            const int x_off = CL == 2 ? (line0 + (lane & 31)) * 4 + cls * x_step : (line0 + W * lane) * 4;
+            // the lane's short line j (and j + 4) at k: K-outer S[k][j], K-inner S[j][k]
+            const int s_step = S_KIN ? 4 : p.lds * 4;
+            int s_off[H];
+#pragma unroll
+            for (int h = 0; h < H; h++)
+                s_off[h] = (4 * h + j < p.s_lines) ? (S_KIN ? (4 * h + j) * p.lds * 4 : (4 * h + j) * 4) + cls * s_step : OOB_OFFSET;
+            struct Buf { XVal<W> x[U]; float s[H][U]; };
+            // k rows at or beyond k_end are not this wavefront's (another share's, or beyond K): zeros instead.  K and
+            // the shares are even, so the two classes of a load stand or fall together.
+            auto load = [&](Buf& b, int k) {
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const int off = (k + CL * u < k_end) ? x_off : OOB_OFFSET;
+                    if constexpr (W == 4) b.x[u].v = ld4(rx, off, (k + CL * u) * x_step);
+                    else b.x[u].v = ld1(rx, off, (k + CL * u) * x_step);
+                }
+#pragma unroll
+                for (int h = 0; h < H; h++) {
+                    if constexpr (S_KIN && CL == 1) {
+#pragma unroll
+                        for (int u = 0; u < U; u += 4) {
+                            const sk_v4f v = ld4(rs, (k + u < k_end) ? s_off[h] : OOB_OFFSET, (k + u) * 4);
+                            b.s[h][u] = v.x; b.s[h][u + 1] = v.y; b.s[h][u + 2] = v.z; b.s[h][u + 3] = v.w;
+                        }
+                    } else {   // (single floats also for the two classes of a K-inner S: measured faster than four k per read)
+#pragma unroll
+                        for (int u = 0; u < U; u++) b.s[h][u] = ld1(rs, (k + CL * u < k_end) ? s_off[h] : OOB_OFFSET, (k + CL * u) * s_step);
+                    }
+                }
+            };
+            auto compute = [&](const Buf& b) {
+#pragma unroll
+                for (int u = 0; u < U; u++)
+#pragma unroll
+                    for (int c = 0; c < W; c++)
+#pragma unroll
+                        for (int h = 0; h < H; h++)
+                            d[c * H + h] = __builtin_amdgcn_mfma_f32_4x4x1f32(b.x[u].at(c), b.s[h][u], d[c * H + h], 0, 0, 0);
+            };
+            Buf b0, b1;
+            load(b0, k_begin);
+            for (int k = k_begin; k < k_end; k += 2 * U * CL) {
+                load(b1, k + U * CL);
+                compute(b0);
+                load(b0, k + 2 * U * CL);
+                compute(b1);
+            }
+            if constexpr (CL == 2) {   // the two classes of k meet: lanes l and l ^ 32 hold the same outputs
+#pragma unroll
+                for (int a = 0; a < ACCS; a++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float v = d[a][r];
+                        v += __shfl_xor(v, 32);
+                        d[a][r] = v;
+                    }
+            }
+        } else {
+            // ---- per instruction 8 lines x 8 classes of k: X[line0 + 8 * set + (lane & 7)][k0 + 4 * (lane >> 3) + 0 .. 3];
+            //      U 32-k panels per register buffer ----
+            constexpr int U = (NW == 16 || W == 4) ? 2 : 4;
+            const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, (long long)p.x_lines * p.ldx * 4);
+            const int kk4 = 4 * (lane / LS);
+            int x_off[W];
+#pragma unroll
+            for (int set = 0; set < W; set++) x_off[set] = ((line0 + LS * set + (lane & (LS - 1))) * p.ldx + kk4) * 4;
+            int s_off[H];
+#pragma unroll
+            for (int h = 0; h < H; h++)
+                s_off[h] = (4 * h + j < p.s_lines) ? (S_KIN ? ((4 * h + j) * p.lds + kk4) * 4 : (kk4 * p.lds + 4 * h + j) * 4) : OOB_OFFSET;
+            const int s_step = S_KIN ? 4 : p.lds * 4;
+            struct Buf { sk_v4f x[U][W]; sk_v4f s[H][U]; };
+            // a lane's 4 k at or beyond k_end are not read (what lies there is the next line, or another share)
+            auto load = [&](Buf& b, int k) {
+#pragma unroll
+                for (int q = 0; q < U; q++) {
+                    const bool on = k + PK * q + kk4 < k_end;
+#pragma unroll
+                    for (int set = 0; set < W; set++) b.x[q][set] = ld4(rx, on ? x_off[set] : OOB_OFFSET, (k + PK * q) * 4);
+#pragma unroll
+                    for (int h = 0; h < H; h++) {
+                        if constexpr (S_KIN) {
+                            b.s[h][q] = ld4(rs, on ? s_off[h] : OOB_OFFSET, (k + PK * q) * 4);
+                        } else {
+                            const int so = on ? s_off[h] : OOB_OFFSET, ss = (k + PK * q) * s_step;
+                            sk_v4f v;
+                            v.x = ld1(rs, so, ss);
+                            v.y = ld1(rs, so, ss + s_step);
+                            v.z = ld1(rs, so, ss + 2 * s_step);
+                            v.w = ld1(rs, so, ss + 3 * s_step);
+                            b.s[h][q] = v;
+                        }
+                    }
+                }
+            };
+            auto compute = [&](const Buf& b) {
+#pragma unroll
+                for (int q = 0; q < U; q++)
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+#pragma unroll
+                        for (int set = 0; set < W; set++)
+#pragma unroll
+                            for (int h = 0; h < H; h++) {
+                                const float xv = b.x[q][set][u], sv = b.s[h][q][u];
+                                d[set * H + h] = __builtin_amdgcn_mfma_f32_4x4x1f32(xv, sv, d[set * H + h], 0, 0, 0);
+                            }
+            };
+            Buf b0, b1;
+            load(b0, k_begin);
+            for (int k = k_begin; k < k_end; k += 2 * PK * U) {
+                load(b1, k + PK * U);
+                compute(b0);
+                load(b0, k + 2 * PK * U);
+                compute(b1);
+            }
+            // the eight classes of k meet: lanes l, l ^ 8, l ^ 16, ... hold the same outputs
+#pragma unroll
+            for (int a = 0; a < ACCS; a++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float v = d[a][r];
+                    v += __shfl_xor(v, 8);
+                    v += __shfl_xor(v, 16);
+                    v += __shfl_xor(v, 32);
+                    d[a][r] = v;
+                }
+        }
+    }
+
+    if (shared) {
+        // the wavefronts' shares of K meet in LDS and are added in k order by the first
+        if (lane < MEET_LANES) {
+#pragma unroll
+            for (int a = 0; a < ACCS; a++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) { const float value = d[a][r]; meet_lds[wave][a * 4 + r][lane] = value; }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+        if (lane < MEET_LANES) {
+#pragma unroll
+            for (int a = 0; a < ACCS; a++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float v = meet_lds[0][a * 4 + r][lane];
+                    for (int w = 1; w < NW; w++) v += meet_lds[w][a * 4 + r][lane];
+                    d[a][r] = v;
+                }
+        }
+    }
+    // the lane's outputs.  K-outer X: accumulator c * H + h, element r is line line0 + W * (4 * (lane >> 2) + r) + c;
+    // K-inner X (lanes 0 .. 7): accumulator set * H + h, element r is line line0 + 8 * set + 4 * (lane >> 2) + r;
+    // both at the short line 4 * h + j
+    if (lane < MEET_LANES) {
+#pragma unroll
+        for (int a = 0; a < ACCS; a++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int h = a % H, hi = a / H;
+                const int line = X_KIN ? line0 + LS * hi + 4 * (lane >> 2) + r : line0 + W * (4 * (lane >> 2) + r) + hi;
+                const float value = d[a][r];
+                skinny_put(p, line, 4 * h + j, value);
+            }
+    }
+}
+
+template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
+hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream) {
+    constexpr int LINES = X_KIN ? 8 * W : 64 * W / CL;
+    const long long units = ((long long)p.L + LINES - 1) / LINES;
+    p.k_share = shared ? ((p.K + NW - 1) / NW + 31) / 32 * 32 : 0;
+    const long long grid = shared ? units : (units + NW - 1) / NW;
+    if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((gemm_f32_skinny<X_KIN, S_KIN, T, W, NW, CL>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    return hipGetLastError();
+}
+
+thread_local int t_skinny_form = -1;
+
+// Which form (gemm_skinny_form's numbering): enough wavefronts on every compute unit with the widest reads that
+// allow it.  With too few runs of lines the wavefronts of a workgroup share a run and split K, sixteen of them
+// where even that leaves compute units without a run.
+template <bool X_KIN, bool S_KIN, int T>
+hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    int form = t_skinny_form;
+    constexpr int W0 = X_KIN ? 2 : 1;     // the narrow form: 16 lines of a K-inner X, 64 of a K-outer one
+    if (form < 0) {
+        // measured on 134 MB ... 1 GiB operands: the long runs wherever they give every compute unit a workgroup;
+        // a K-inner X also then prefers the four wavefronts of a workgroup on the same lines (a K-outer one only
+        // below four runs per compute unit); short of that the narrow runs, and 32-line runs of a K-outer X
+        const long long narrow = ((long long)p.L + (X_KIN ? 15 : 63)) / (X_KIN ? 16 : 64);
+        const long long wide = ((long long)p.L + (X_KIN ? 31 : 255)) / (X_KIN ? 32 : 256);
+        if (p.K < 128) form = wide >= 4LL * num_cu ? 3 : 0;
+        else if (wide >= 4LL * num_cu) form = X_KIN ? 4 : 3;
+        else if (wide >= num_cu) form = 4;
+        else if (narrow >= num_cu || p.K < 512) form = 1;
+        else form = X_KIN ? 2 : 5;
+    }
+    switch (form) {
+        case 0: return launch_one<X_KIN, S_KIN, T, W0, 4>(p, false, stream);
+        case 1: return launch_one<X_KIN, S_KIN, T, W0, 4>(p, true, stream);
+        case 2: return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
+        case 3: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, false, stream);
+        case 4: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, true, stream);
+        default:
+            if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
+            else return launch_one<X_KIN, S_KIN, T, 1, 16, 2>(p, true, stream);
+    }
+}
+
+template <bool X_KIN, bool S_KIN>
+hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
+    return T == 4 ? launch_skinny<X_KIN, S_KIN, 4>(p, stream) : launch_skinny<X_KIN, S_KIN, 8>(p, stream);
+}
+
+}  // namespace
+
+// Force a form of the skinny kernel for the calling thread's launches: 0 = a wavefront per run of lines (64 of a
+// K-outer long operand, 16 of a K-inner one) with the whole K, 1 = the four wavefronts of a workgroup share a run
+// and split K, 2 = sixteen wavefronts do, 3 and 4 = as 0 and 1 with runs four (K-inner: two) times as long,
+// 5 = as 2 with runs of 32 lines of a K-outer operand (two classes of k among the lanes; K-inner: as 2);
+// -1 = the automatic choice.
+void gemm_skinny_form(int form) { t_skinny_form = (form >= 0 && form <= 5) ? form : -1; }
+
+int gemm_choose_skinny(int rows, int cols, int nz) {
+    if (nz != 1) return -1;
+    const bool thin_cols = (cols == 4 || cols == 8) && rows >= 256;
+    const bool thin_rows = (rows == 4 || rows == 8) && cols >= 256;
+    return thin_cols || thin_rows ? TILE_SKINNY : -1;
+}
+
+// True where the product is one for the skinny kernel: one unsplit 2-D product without a bias row whose C has
+// 4 or 8 columns under at least 256 rows, or 4 or 8 rows over at least 256 columns, and whose operands' byte
+// offsets (with the reads a register buffer runs ahead, and the lines of a last, partly filled run) fit 32 bits.
+static bool gemm_skinny_applies(int variant, const GemmParams& p) {
+    if (p.split || p.bias != nullptr || gemm_choose_skinny(p.rows, p.cols, p.nz) < 0) return false;
+    const bool thin_cols = (p.cols == 4 || p.cols == 8) && p.rows >= 256;
+    const bool a_kin = variant != GEMM_T1, b_kin = variant == GEMM_T2;
+    // a K-inner operand is addressed line * ld + k, a K-outer one k * ld + line
+    const long long a_span = a_kin ? (long long)(thin_cols ? p.rows : 8) * p.lda : (long long)p.k_total * p.lda;
+    const long long b_span = b_kin ? (long long)(thin_cols ? 8 : p.cols) * p.ldb : (long long)p.k_total * p.ldb;
+    const long long ld = p.lda > p.ldb ? p.lda : p.ldb;
+    return ld <= (1 << 20) && (a_span + 64 * ld) * 4 < 0x7fff0000LL && (b_span + 64 * ld) * 4 < 0x7fff0000LL;
+}
+
+hipError_t gemm_launch_skinny(int variant, const GemmParams& g, hipStream_t stream) {
+    if (!gemm_skinny_applies(variant, g)) return hipErrorOutOfMemory;   // the caller takes a tile kernel
+    const bool a_kin = variant != GEMM_T1, b_kin = variant == GEMM_T2;
+    const bool thin_cols = (g.cols == 4 || g.cols == 8) && g.rows >= 256;
+    SkinnyParams p = {};
+    p.C = g.C; p.ldc = g.ldc;
+    p.K = min(g.k_total, min(a_kin ? g.a_inner : g.a_outer, b_kin ? g.b_inner : g.b_outer));
+    if (p.K <= 0) return hipErrorInvalidValue;
+    if (thin_cols) {          // X = A (lines = rows of C), S = B (lines = columns of C)
+        p.X = g.A; p.ldx = g.lda; p.x_lines = a_kin ? g.a_outer : g.a_inner;
+        p.S = g.B; p.lds = g.ldb; p.s_lines = min(b_kin ? g.b_outer : g.b_inner, g.cols);
+        p.L = g.rows; p.out_rows = 0;
+        switch ((a_kin ? 2 : 0) | (b_kin ? 1 : 0)) {
+            case 0: return launch_skinny_t<false, false>(p, g.cols, stream);
+            case 1: return launch_skinny_t<false, true>(p, g.cols, stream);
+            case 2: return launch_skinny_t<true, false>(p, g.cols, stream);
+            default: return launch_skinny_t<true, true>(p, g.cols, stream);
+        }
+    }
+    // X = B (lines = columns of C), S = A (lines = rows of C)
+    p.X = g.B; p.ldx = g.ldb; p.x_lines = b_kin ? g.b_outer : g.b_inner;
+    p.S = g.A; p.lds = g.lda; p.s_lines = min(a_kin ? g.a_outer : g.a_inner, g.rows);
+    p.L = g.cols; p.out_rows = 1;
+    switch ((b_kin ? 2 : 0) | (a_kin ? 1 : 0)) {
+        case 0: return launch_skinny_t<false, false>(p, g.rows, stream);
+        case 1: return launch_skinny_t<false, true>(p, g.rows, stream);
+        case 2: return launch_skinny_t<true, false>(p, g.rows, stream);
+        default: return launch_skinny_t<true, true>(p, g.rows, stream);
+    }
+}
+
+}  // namespace dragon

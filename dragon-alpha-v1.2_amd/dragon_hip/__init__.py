@@ -453,6 +453,11 @@ def force_tile(tile):
     lib.dragon_gemm_force_tile(int(tile))
 
 
+def skinny_form(form):
+    """Force a form of the skinny kernel (0..4, -1 = automatic).  Benchmark / test hook."""
+    lib.dragon_gemm_skinny_form(int(form))
+
+
 def split_policy(mode):
     """How the split-K entries treat GridZ: -1 the estimate decides, 0 always as asked, 1 declined where possible."""
     lib.dragon_gemm_split_policy(int(mode))

@@ -79,6 +79,7 @@ SIGNATURES = {
     "dragon_Cuda_matMul_nstream": (i32, [i32, i32]),
     "dragon_Cuda_batchMatMul_streamSize": (i32, [i32, i32]),
     "dragon_gemm_force_tile": (None, [i32]),
+    "dragon_gemm_skinny_form": (None, [i32]),
     "dragon_test_mem_get_info": (i32, [POINTER(i64), POINTER(i64)]),
     "dragon_gemm_split_policy": (None, [i32]),
     "dragon_gemm_fold_skip": (None, [i32]),

@@ -1,0 +1,115 @@
+"""GPU parity of the skinny kernel (gemm_skinny.hip): a C of 4 or 8 columns under many rows, or of 4 or 8 rows over
+many columns -- what the reference sends to its 4-column kernels (MM/matMul_sernel.cuh:17-30, dispatched at
+MM/matMul.cuh:100-102) and to k18 / k14 / k12 (MM/matMul.cuh:104-106).  Wavefronts stream the long operand from
+memory into 4 x 4 x 1 MFMA blocks; integer inputs pin the indexing bit for bit: lines per wavefront, the classes
+of k, the K tail, K shared between the wavefronts of a workgroup, both orientations of C."""
+import numpy as np
+import pytest
+
+from helpers import NN, T1, T2, VARIANT_NAMES, assert_within_tolerance, gpu_matmul_2d, logical_operands, oracle_2d
+
+pytestmark = pytest.mark.gpu
+
+SKINNY = 27
+
+
+@pytest.fixture(autouse=True)
+def _auto_tile(gpu):
+    yield
+    gpu.force_tile(-1)
+    gpu.skinny_form(-1)
+
+
+def check(gpu, variant, N, M, K, seed, fill=-77.0):
+    rng = np.random.default_rng(seed)
+    A, B = logical_operands(variant, rng, N, M, K, "int")
+    C, Cp = gpu_matmul_2d(gpu, variant, A, B, fill=fill)
+    R = oracle_2d(variant, A, B)
+    what = "%s %d x %d x %d" % (VARIANT_NAMES[variant], N, M, K)
+    if not np.array_equal(C, R):
+        bad = np.argwhere(C != R)
+        raise AssertionError("%s: %d wrong outputs, first at %s (got %s, want %s); rows %s cols %s" % (
+            what, len(bad), bad[0], C[tuple(bad[0])], R[tuple(bad[0])], sorted(set(bad[:, 0]))[:12],
+            sorted(set(bad[:, 1]))[:12]))
+    assert np.count_nonzero(Cp[N:]) == 0 and np.count_nonzero(Cp[:, M:]) == 0, what + ": pads must come out zero"
+
+
+def test_the_automatic_choice_names_the_kernel(gpu):
+    cu = 256
+    for (rows, cols) in ((65536, 4), (8192, 8), (256, 4), (4, 65536), (8, 256), (4, 1000)):
+        for variant in (NN, T1, T2):
+            assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
+    # not skinny enough, too short, or a batch / K slices
+    for (rows, cols, nz) in ((65536, 12, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (65536, 4, 2), (4, 65536, 3)):
+        assert gpu.choose_tile(NN, rows, cols, nz, 1024, cu) != SKINNY
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("thin", [1, 2, 3, 4, 5, 7, 8])
+def test_thin_columns_bitwise(gpu, variant, thin, form):
+    """C of 1 ... 8 columns (stored 4 or 8) under row counts around the 16, 64 and 256 lines a wavefront takes,
+    in every form of the kernel: a wavefront per run of lines, K shared between 4 or 16 wavefronts, one or four
+    lines per lane."""
+    gpu.skinny_form(form)
+    for (N, K) in ((256, 64), (1000, 1028), (4099, 36), (40000, 100), (20000, 260)):
+        check(gpu, variant, N, thin, K, 100 * thin + N + K + variant)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("thin", [1, 3, 4, 6, 8])
+def test_thin_rows_bitwise(gpu, variant, thin, form):
+    gpu.skinny_form(form)
+    for (M, K) in ((256, 64), (1001, 1028), (4100, 36), (40001, 100), (20000, 260)):
+        check(gpu, variant, thin, M, K, 200 * thin + M + K + variant)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("K", [1, 3, 4, 5, 8, 12, 15, 16, 17, 28, 31, 32, 33, 60, 64, 68, 127, 128, 129, 252, 255, 256, 257, 300, 511, 513, 1000])
+def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
+    """K around the k rows / 32-k panels of a register buffer, the 4-k chunks of a lane, the shares of a K split
+    between 4 or 16 wavefronts; in every form."""
+    for form in (0, 1, 2, 3, 4, 5):
+        gpu.skinny_form(form)
+        check(gpu, variant, 700, 4, K, 3000 + K + variant)
+        check(gpu, variant, 8, 900, K, 4000 + K + variant)
+    gpu.skinny_form(-1)
+    if K <= 64:
+        check(gpu, variant, 70000, 7, K, 5000 + K + variant)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_long_shapes_against_both_oracles(gpu, variant):
+    """Uniform inputs at the benchmark's shapes, scaled down 4 x along the long side, within the FP32 tolerance
+    (relative Frobenius error <= 1e-5, elements within 1e-4 * sqrt(K) * max|A| * max|B|); and the same launch
+    twice gives the same bits."""
+    for (N, M, K) in ((16384, 4, 1024), (2048, 8, 4096), (4, 16384, 1024), (8, 2048, 4096)):
+        rng = np.random.default_rng(N + M + K + variant)
+        A, B = logical_operands(variant, rng, N, M, K)
+        C, _ = gpu_matmul_2d(gpu, variant, A, B)
+        C2, _ = gpu_matmul_2d(gpu, variant, A, B)
+        R = oracle_2d(variant, A, B)
+        assert_within_tolerance(C, R, K, A, B, "%s %d x %d x %d" % (VARIANT_NAMES[variant], N, M, K))
+        assert np.array_equal(C, C2)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_forced_on_another_shape_falls_back(gpu, variant):
+    gpu.force_tile(SKINNY)
+    check(gpu, variant, 300, 12, 64, 77 + variant)
+    check(gpu, variant, 100, 4, 64, 78 + variant)
+    check(gpu, variant, 8, 8, 64, 79 + variant)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_agrees_with_the_tile_kernels(gpu, variant):
+    """The same integer product through the skinny kernel and through a 64 x 64 tile kernel: equal bits."""
+    rng = np.random.default_rng(9 + variant)
+    for (N, M, K) in ((5000, 8, 516), (4, 5000, 516)):
+        A, B = logical_operands(variant, rng, N, M, K, "int")
+        C, _ = gpu_matmul_2d(gpu, variant, A, B)
+        gpu.force_tile(1)
+        C1, _ = gpu_matmul_2d(gpu, variant, A, B)
+        gpu.force_tile(-1)
+        assert np.array_equal(C, C1)
