@@ -230,7 +230,8 @@ def main():
     rec_kernel = rec.get("per_launch", {}).get(slowest)
     variant_id = {"A*B": 0, "A^T*B": 1, "A*B^T": 2}[slowest]
     tile_id = dh.choose_tile(variant_id, n, n, 1, n, SM)
-    kernel_name = ("gemm_f32_mfma_streamk" if 18 <= tile_id < 24 or tile_id == 25 else "gemm_f32_mfma_band" if tile_id == 24
+    kernel_name = ("gemm_f32_mfma_streamk" if 18 <= tile_id < 24 or tile_id == 25 else "gemm_f32_mfma_band" if tile_id in (24, 28)
+                   else "gemm_f32_mfma_shortk" if tile_id == 26 else "gemm_f32_skinny" if tile_id == 27
                    else "gemm_f32_mfma_dma" if 15 <= tile_id < 18 else "gemm_f32_mfma")
     roofline = {"bound": "mfma", "kernel": "%s (tile id %d) %s 4096^3" % (kernel_name, tile_id, slowest),
                 "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -342,6 +343,11 @@ def main():
         ms = timer.per_launch_ms(lambda: BMM.batchMatMulT2_texture(
             S, 1, dQ.address, dK.address, dO.address, Bt, Sq, Sq, Sq, D), iters=50)
         record("cfg4 batch64 Q.K^T 1024x64", fl4, ms, by4)
+        dh.force_tile(28)      # the band kernel with bands of 64 rows under tiles of 256 columns
+        ms = timer.per_launch_ms(lambda: BMM.batchMatMulT2_texture(
+            S, 1, dQ.address, dK.address, dO.address, Bt, Sq, Sq, Sq, D), iters=50)
+        dh.force_tile(-1)
+        record("cfg4 batch64 Q.K^T 1024x64, bands of 64 rows x tiles of 256 columns (forced)", fl4, ms, by4)
         ms = timer.per_launch_ms(lambda: BMM.batchMatMul_texture(
             S, 1, dS.address, dV.address, dO.address, Bt, Sq, D, Sq, Sq), iters=50)
         record("cfg4 batch64 scores.V 1024x1024 by 1024x64", fl4, ms, by4)
@@ -675,6 +681,30 @@ def main():
             per_config["engine.matMulT1 256x256 K=131072 (GridZ %d), %s" % (eg.get_param("last_gridZ"), name)] = {
                 "ms": round(ms, 4), "tflops": round(2.0 * N3 * N3 * K3 / ms / 1e9, 2),
                 "pct_peak": round(100 * 2.0 * N3 * N3 * K3 / ms / 1e9 / PEAK_TFLOPS, 1)}
+            if pool_bytes:
+                # the same calls with the engine in its asynchronous mode (sync(false)): a call returns once its
+                # launches are issued and the wait for a result comes one call later, so the device always has
+                # the next product queued -- the per-call cost without the blocking round trip (launch latency to
+                # an idle device + wake-up: 12.5 us for an empty product)
+                eg.sync(False)
+                prev = None
+                for _ in range(40):
+                    cur = eg.matMulT1(tA, tB)
+                    if prev is not None:
+                        eg.delete(prev)
+                    prev = cur
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    cur = eg.matMulT1(tA, tB)
+                    eg.delete(prev)
+                    prev = cur
+                ms = (time.perf_counter() - t0) / reps * 1e3
+                eg.delete(prev)
+                eg.sync(True)
+                per_config["engine.matMulT1 256x256 K=131072 (GridZ %d), %s, asynchronous mode, one call queued behind the wait" % (
+                    eg.get_param("last_gridZ"), name)] = {
+                    "ms": round(ms, 4), "tflops": round(2.0 * N3 * N3 * K3 / ms / 1e9, 2),
+                    "pct_peak": round(100 * 2.0 * N3 * N3 * K3 / ms / 1e9 / PEAK_TFLOPS, 1)}
             eg.close()
 
     Cuda.deleteStream(stream)

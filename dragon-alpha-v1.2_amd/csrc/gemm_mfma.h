@@ -52,13 +52,15 @@ enum GemmTile {
     // A C of 4 or 8 columns (or rows) under a long other side: wavefronts stream the long operand from memory into
     // 4 x 4 x 1 MFMA blocks, no tiles and no LDS staging (gemm_skinny.hip)
     TILE_SKINNY = 27,
+    // the band kernel with bands of 64 rows under tiles of 256 columns
+    TILE_BAND_64x256 = 28,
     // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
     // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
     // short K; gemm_choose_tile sets it.
     TILE_PAIRED = 0x100
 };
 inline bool gemm_tile_is_streamk(int tile) { return (tile >= TILE_SK_64x64 && tile < TILE_SK_END) || tile == TILE_SK_256x64; }
-inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128; }
+inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128 || tile == TILE_BAND_64x256; }
 inline bool gemm_tile_is_shortk(int tile) { return tile == TILE_SHORTK_64x64; }
 inline bool gemm_tile_is_skinny(int tile) { return tile == TILE_SKINNY; }
 inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
@@ -113,6 +115,9 @@ struct GemmParams {
     // zero) instead of the stream's
     float* sk_ws_given;
     size_t sk_ws_given_floats;
+    // few tiles under a very long K, dealt in whole runs per tile: sk_kmajor_rpt runs per tile (0: off) of
+    // sk_kmajor_tiles tiles; the workgroups that share an XCD then take the same k ranges of different tiles
+    int sk_kmajor_rpt, sk_kmajor_tiles;
     // K slices: the tiles from number sk_T1 on (the last slice's) have sk_S_last stages
     int sk_S_last, sk_T1;
     unsigned sk_div_Sl_mul, sk_div_Sl_shift;
@@ -206,10 +211,10 @@ void gemm_streamk_release_workspace(hipStream_t stream);
 int gemm_streamk_release_workspaces();
 int gemm_streamk_workspace_count();               // workspaces held now
 long long gemm_streamk_workspaces_refused();      // balanced launches that found the table full and took another kernel
-// The band kernel (tile id TILE_BAND_128x128) for the three products, batched too, with K <= 64.
-// hipErrorOutOfMemory says that the product cannot go this way (a longer K, K slices, a bias row) and the
-// caller takes a tile-per-workgroup kernel instead.
-hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream);
+// The band kernel (tile ids TILE_BAND_128x128, and TILE_BAND_64x256 with `wide`) for the three products, batched
+// too, with K <= 64.  hipErrorOutOfMemory says that the product cannot go this way (a longer K, K slices, a bias
+// row) and the caller takes a tile-per-workgroup kernel instead.
+hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream, bool wide = false);
 // TILE_BAND_128x128 where the band kernel is the better choice, else -1
 int gemm_choose_band(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
 // how the band kernel deals a band's column tiles to workgroups

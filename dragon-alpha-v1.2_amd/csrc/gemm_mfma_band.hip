@@ -40,7 +40,7 @@
 namespace dragon {
 namespace {
 
-constexpr int BD_BM = 128, BD_BN = 128, BD_KT = 64, BD_THREADS = 512;
+constexpr int BD_KT = 64, BD_THREADS = 512;
 // Cache policy of the C stores: streaming (nt).  Measured on batch 64 of 1024 x 1024 x 64: 73 us, against 91-96 us
 // with plain stores or with the scope bits alone (C's lines then stay in the L2 and compete with the operands).
 constexpr int BD_STORE_AUX = 2;
@@ -102,10 +102,12 @@ __device__ __forceinline__ v4u band_descriptor(const float* base, int rows, int 
     return rsrc;
 }
 
-template <bool A_KIN, bool B_KIN>
+// BM x BN: 128 x 128 (bands of 128 rows), or 64 x 256 (bands of 64 rows under tiles of 256 columns: the stores of a
+// tile then run along 1 KiB of a row of C instead of 512 bytes)
+template <bool A_KIN, bool B_KIN, int BM, int BN>
 __global__ __launch_bounds__(BD_THREADS, 1)
 void gemm_f32_mfma_band(const GemmParams p) {
-    constexpr int NT = BD_THREADS, WN = 2, TN = 2, BM = BD_BM, BN = BD_BN, KT = BD_KT;
+    constexpr int NT = BD_THREADS, TN = 2, WN = BN / (TN * 32), KT = BD_KT;
     static_assert(NT / 64 == (BM / 32) * WN && BN == WN * TN * 32, "the wavefronts cover the tile");
     constexpr int GR = KT / 8;                 // k groups per tile
     constexpr int NM = 4 * TN;                 // MFMAs per group: 4 k steps of TN blocks
@@ -383,7 +385,7 @@ void gemm_f32_mfma_band(const GemmParams p) {
     }
 }
 
-template <bool A_KIN, bool B_KIN>
+template <bool A_KIN, bool B_KIN, int BD_BM, int BD_BN>
 static hipError_t launch_band_cfg(GemmParams p, hipStream_t stream) {
     if (p.split || p.bias != nullptr || p.k_total > BD_KT) return hipErrorOutOfMemory;   // the caller falls back
     p.tiles_m = (p.rows + BD_BM - 1) / BD_BM;
@@ -395,7 +397,7 @@ static hipError_t launch_band_cfg(GemmParams p, hipStream_t stream) {
     gemm_band_split(bands, p.tiles_n, num_cu, p.bd_chunks, p.bd_chunk_tiles);
     const long long units = bands * p.bd_chunks;
     const long long grid = units < num_cu ? units : num_cu;
-    hipLaunchKernelGGL((gemm_f32_mfma_band<A_KIN, B_KIN>), dim3((unsigned)grid), dim3(BD_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((gemm_f32_mfma_band<A_KIN, B_KIN, BD_BM, BD_BN>), dim3((unsigned)grid), dim3(BD_THREADS), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -427,6 +429,7 @@ int gemm_choose_band(int rows, int cols, int nz, int k, int num_cu, int variant)
     if (rows <= 0 || cols <= 0 || nz <= 0 || k <= 0 || num_cu <= 0) return -1;
     if (k > BD_KT || k <= BD_KT - 8) return -1;
     if (cols % 32 != 0) return -1;
+    constexpr int BD_BM = 128, BD_BN = 128;
     const long long tiles_m = (rows + BD_BM - 1) / BD_BM, tiles_n = (cols + BD_BN - 1) / BD_BN;
     if (tiles_n < 2 || tiles_m * nz * tiles_n < 2LL * num_cu) return -1;
     // rows and columns that fill their tiles: the padded part of a ragged C is multiplied too
@@ -434,11 +437,19 @@ int gemm_choose_band(int rows, int cols, int nz, int k, int num_cu, int variant)
     return TILE_BAND_128x128;
 }
 
-hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream) {
+hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream, bool wide) {
+    if (wide) {
+        switch (variant) {
+            case GEMM_NN: return launch_band_cfg<true, false, 64, 256>(p, stream);
+            case GEMM_T1: return launch_band_cfg<false, false, 64, 256>(p, stream);
+            case GEMM_T2: return launch_band_cfg<true, true, 64, 256>(p, stream);
+            default: return hipErrorInvalidValue;
+        }
+    }
     switch (variant) {
-        case GEMM_NN: return launch_band_cfg<true, false>(p, stream);
-        case GEMM_T1: return launch_band_cfg<false, false>(p, stream);
-        case GEMM_T2: return launch_band_cfg<true, true>(p, stream);
+        case GEMM_NN: return launch_band_cfg<true, false, 128, 128>(p, stream);
+        case GEMM_T1: return launch_band_cfg<false, false, 128, 128>(p, stream);
+        case GEMM_T2: return launch_band_cfg<true, true, 128, 128>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -275,8 +275,16 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
         }
         return c;
     };
-    // neighbouring runs share a tile's operands: keep them on one XCD (one L2)
-    const int w = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // neighbouring runs share a tile's operands: keep them on one XCD (one L2).  Where every tile is cut into the
+    // same whole number of runs (few tiles, a very long K), a tile's runs share nothing -- but the runs of the
+    // same k range of the tiles of a row read the same rows of A, those of a column the same of B: there the
+    // workgroups of an XCD take neighbouring k ranges of all the tiles, and the L2 serves each operand row to
+    // its tiles from one fetch.
+    int w = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    if (p.sk_kmajor_rpt > 0) {
+        const int k_range = w / p.sk_kmajor_tiles, tile = w - k_range * p.sk_kmajor_tiles;
+        w = tile * p.sk_kmajor_rpt + k_range;
+    }
     const int u0 = sk_first_unit(w, p.sk_q, p.sk_rem);
     const int n = p.sk_q + (w < p.sk_rem ? 1 : 0);             // >= 1: the grid never exceeds the unit count
 
@@ -590,6 +598,10 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     gemm_magic_divisor((unsigned)S_last, p.sk_div_Sl_mul, p.sk_div_Sl_shift);
     p.sk_q = (int)(units / grid);
     p.sk_rem = (int)(units % grid);
+    p.sk_kmajor_rpt = 0;
+    p.sk_kmajor_tiles = (int)tiles;
+    if (!CONV && !p.split && p.nz == 1 && tiles >= 2 && p.sk_rem == 0 && grid % tiles == 0 && grid / tiles >= 2 && S % (grid / tiles) == 0)
+        p.sk_kmajor_rpt = (int)(grid / tiles);
     if constexpr (CAN_BIAS) {
         if (p.bias != nullptr) {
             hipLaunchKernelGGL((gemm_f32_mfma_streamk<A_KIN, B_KIN, WM, WN, TM, TN, KT, NS, OCC, true, false, CONV>),

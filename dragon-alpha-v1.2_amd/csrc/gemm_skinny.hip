@@ -17,7 +17,10 @@
 //       the 16 lines of a wavefront.  The 8 classes of k of a line meet at the end through three lane exchanges.
 // S's values come from memory as well (they stay in the L1: a few floats per k, the same for every wavefront).
 // Where the lines are too few to give every compute unit enough wavefronts, the 4 or 16 wavefronts of a workgroup
-// share their lines and split K; their sums meet in LDS and are added share after share, a fixed order.
+// share their lines and split K; their sums meet in LDS and are added share after share, a fixed order.  With
+// fewer runs of lines than compute units K is cut across up to 8 workgroups per run as well: each leaves its sum
+// in the stream's workspace (the balanced kernel's, with its arrival counters) and the one counted last adds them
+// in k order -- one launch, the same bits every time.
 #include "gemm_mfma_kernel.h"
 
 namespace dragon {
@@ -33,9 +36,15 @@ struct SkinnyParams {
     int s_lines;        // the same for S (<= T)
     int k_share;        // 0: a wavefront takes its lines' whole K; else the k of each wavefront of a workgroup (a multiple of 32)
     int out_rows;       // the short side is C's row index (C is T x L), else its column index (C is L x T)
+    // K cut across workgroups (few lines under a long K): k_cuts workgroups per run of lines take k_cut k each (a
+    // multiple of 128, shared among a workgroup's wavefronts as k_share says); their sums meet in ws, counted in count
+    int k_cuts, k_cut, units;
+    float* ws;
+    int* count;
 };
 
 typedef float sk_v4f __attribute__((ext_vector_type(4)));
+constexpr int SKINNY_MAX_CUTS = 8;    // workgroups that cut one run's K
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t skinny_rsrc(const float* base, long long bytes) {
     const long long capped = bytes > 0xfffffff0LL ? 0xfffffff0LL : (bytes < 0 ? 0 : bytes);
@@ -65,7 +74,7 @@ template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny(const SkinnyParams p) {
     static_assert(T == 4 || T == 8, "4 or 8 short lines");
-    static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || (CL == 2 && W == 1)), "forms");
+    static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || ((CL == 2 || CL == 4) && W == 1)), "forms");
     constexpr int LS = 8, PK = 32;                         // K-inner X: lines per read, k per panel
     constexpr int H = T / 4;                               // groups of 4 short lines
     constexpr int LINES = X_KIN ? LS * W : 64 * W / CL;    // lines of X per wavefront
@@ -75,10 +84,13 @@ void gemm_f32_skinny(const SkinnyParams p) {
 
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const bool shared = p.k_share > 0;
-    const int unit = shared ? blockIdx.x : blockIdx.x * NW + wave;     // which run of LINES lines
+    // which run of LINES lines; neighbouring runs of a shared K read the halves of the same 128-byte lines: one XCD
+    const int wg = shared ? xcd_contiguous_id(blockIdx.x, gridDim.x) : 0;
+    const int cut = p.k_cuts > 1 ? wg / p.units : 0;           // neighbouring workgroups: neighbouring lines, the same k
+    const int unit = shared ? wg - cut * p.units : blockIdx.x * NW + wave;
     const int line0 = unit * LINES;
-    const int k_begin = shared ? wave * p.k_share : 0;
-    const int k_end = shared ? min(p.K, k_begin + p.k_share) : p.K;
+    const int k_begin = shared ? cut * p.k_cut + wave * p.k_share : 0;
+    const int k_end = shared ? min(min(p.K, (cut + 1) * p.k_cut), k_begin + p.k_share) : p.K;
     const int j = lane & 3;
 
     // S(k, j): rows beyond K (K-outer) or lines beyond those S has (K-inner) lie beyond the descriptor's end
@@ -92,10 +104,10 @@ void gemm_f32_skinny(const SkinnyParams p) {
             // ---- a lane owns W lines: X[k][line0 + W * lane + c] (CL = 2: X[k + class][line0 + (lane & 31)]);
             //      U loads (U * CL k rows) per register buffer ----
             constexpr int U = W == 4 ? 8 : 16;
-            const int cls = CL == 2 ? lane >> 5 : 0;
+            const int cls = CL == 4 ? lane >> 4 : CL == 2 ? lane >> 5 : 0;
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, ((long long)(p.K - 1) * p.ldx + p.x_lines) * 4);
             const int x_step = p.ldx * 4;
-            const int x_off = CL == 2 ? (line0 + (lane & 31)) * 4 + cls * x_step : (line0 + W * lane) * 4;
+            const int x_off = CL > 1 ? (line0 + (lane & (64 / CL - 1))) * 4 + cls * x_step : (line0 + W * lane) * 4;
             // the lane's short line j (and j + 4) at k: K-outer S[k][j], K-inner S[j][k]
             const int s_step = S_KIN ? 4 : p.lds * 4;
             int s_off[H];
@@ -143,12 +155,13 @@ void gemm_f32_skinny(const SkinnyParams p) {
                 load(b0, k + 2 * U * CL);
                 compute(b1);
             }
-            if constexpr (CL == 2) {   // the two classes of k meet: lanes l and l ^ 32 hold the same outputs
+            if constexpr (CL > 1) {   // the classes of k meet: lanes l, l ^ 32 (and l ^ 16) hold the same outputs
 #pragma unroll
                 for (int a = 0; a < ACCS; a++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         float v = d[a][r];
+                        if constexpr (CL == 4) v += __shfl_xor(v, 16);
                         v += __shfl_xor(v, 32);
                         d[a][r] = v;
                     }
@@ -246,6 +259,54 @@ void gemm_f32_skinny(const SkinnyParams p) {
                     d[a][r] = v;
                 }
         }
+        if constexpr (ACCS * 4 <= 16 && NW == 4) if (p.k_cuts > 1) {
+            // The workgroups that cut this run's K meet in memory: every one leaves its sum in its slot and is
+            // counted; whoever is counted last adds the slots -- its own included -- in k order and stores.  The
+            // hand-over is the balanced kernel's (gemm_mfma_streamk.hip, store_partial): device-scope stores that
+            // have all been acknowledged (vmcnt 0) before this wavefront's count, device-scope loads after it.
+            float* const slots = p.ws + (size_t)unit * p.k_cuts * (ACCS * 4 * MEET_LANES);
+            if (lane < MEET_LANES) {
+                float* const mine = slots + (size_t)cut * (ACCS * 4 * MEET_LANES) + lane;
+#pragma unroll
+                for (int a = 0; a < ACCS; a++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const float value = d[a][r];
+                        __hip_atomic_store(mine + (a * 4 + r) * MEET_LANES, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            asm volatile("" ::: "memory");
+            int arrived = 0;
+            if (lane == 0) {
+                arrived = atomicAdd(p.count + unit, 1);
+                if (arrived == p.k_cuts - 1) atomicExch(p.count + unit, 0);     // zero again for the next launch
+            }
+            arrived = __builtin_amdgcn_readfirstlane(arrived);
+            if (arrived != p.k_cuts - 1) return;
+            asm volatile("" ::: "memory");
+            if (lane < MEET_LANES) {
+                float v[SKINNY_MAX_CUTS][ACCS * 4];
+#pragma unroll
+                for (int c = 0; c < SKINNY_MAX_CUTS; c++)
+                    if (c < p.k_cuts) {
+#pragma unroll
+                        for (int i = 0; i < ACCS * 4; i++)
+                            v[c][i] = __hip_atomic_load(slots + (size_t)c * (ACCS * 4 * MEET_LANES) + i * MEET_LANES + lane,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                for (int a = 0; a < ACCS; a++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float sum = v[0][a * 4 + r];
+#pragma unroll
+                        for (int c = 1; c < SKINNY_MAX_CUTS; c++)
+                            if (c < p.k_cuts) sum += v[c][a * 4 + r];
+                        d[a][r] = sum;
+                    }
+            }
+        }
     }
     // the lane's outputs.  K-outer X: accumulator c * H + h, element r is line line0 + W * (4 * (lane >> 2) + r) + c;
     // K-inner X (lanes 0 .. 7): accumulator set * H + h, element r is line line0 + 8 * set + 4 * (lane >> 2) + r;
@@ -263,18 +324,40 @@ void gemm_f32_skinny(const SkinnyParams p) {
     }
 }
 
+// cuts > 1: that many workgroups per run of lines take a part of K each (narrow forms only, at most
+// SKINNY_MAX_CUTS); they meet through the stream's workspace of the balanced kernel -- without one (the stream
+// is being captured before it has one, the table is full) the run's K stays with one workgroup.
 template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
-hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream) {
+hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream, int cuts = 1) {
     constexpr int LINES = X_KIN ? 8 * W : 64 * W / CL;
+    constexpr int SLOT = W * (T / 4) * 4 * (X_KIN ? 8 : 64 / CL);      // floats a workgroup leaves in the workspace
     const long long units = ((long long)p.L + LINES - 1) / LINES;
     p.k_share = shared ? ((p.K + NW - 1) / NW + 31) / 32 * 32 : 0;
-    const long long grid = shared ? units : (units + NW - 1) / NW;
+    p.units = (int)units;
+    p.k_cuts = 1;
+    p.k_cut = p.K;
+    long long grid = shared ? units : (units + NW - 1) / NW;
+    if (shared && cuts > 1 && NW == 4 && W * (T / 4) * 4 <= 16 && units <= 65536) {
+        if (cuts > SKINNY_MAX_CUTS) cuts = SKINNY_MAX_CUTS;
+        const int k_cut = ((p.K + cuts - 1) / cuts + 32 * NW - 1) / (32 * NW) * (32 * NW);
+        const int real = (p.K + k_cut - 1) / k_cut;
+        size_t floats = 0;
+        float* ws = real > 1 ? gemm_streamk_workspace(stream, &floats) : nullptr;
+        if (ws != nullptr && 65536 + (size_t)units * real * SLOT <= floats) {
+            p.k_cuts = real;
+            p.k_cut = k_cut;
+            p.k_share = k_cut / NW;
+            p.count = (int*)ws;          // the workspace's arrival counters, zero between launches
+            p.ws = ws + 65536;
+            grid = units * real;
+        }
+    }
     if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
     hipLaunchKernelGGL((gemm_f32_skinny<X_KIN, S_KIN, T, W, NW, CL>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
 
-thread_local int t_skinny_form = -1;
+thread_local int t_skinny_form = -1, t_skinny_cuts = 0;
 
 // Which form (gemm_skinny_form's numbering): enough wavefronts on every compute unit with the widest reads that
 // allow it.  With too few runs of lines the wavefronts of a workgroup share a run and split K, sixteen of them
@@ -295,7 +378,10 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
         else if (wide >= 4LL * num_cu) form = X_KIN ? 4 : 3;
         else if (wide >= num_cu) form = 4;
         else if (narrow >= num_cu || p.K < 512) form = 1;
-        else form = X_KIN ? 2 : 5;
+        // fewer narrow runs than compute units: K is cut across workgroups as well -- except for 128 ... 255 runs of
+        // a K-outer X beside a K-outer S, where sixteen wavefronts on 32-line runs measured 10 % ahead
+        else if (!X_KIN && !S_KIN && 2 * narrow >= num_cu) form = 5;
+        else form = 7;
     }
     switch (form) {
         case 0: return launch_one<X_KIN, S_KIN, T, W0, 4>(p, false, stream);
@@ -303,6 +389,13 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
         case 2: return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
         case 3: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, false, stream);
         case 4: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, true, stream);
+        case 6:
+            if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
+            else return launch_one<X_KIN, S_KIN, T, 1, 16, 4>(p, true, stream);
+        case 7: {   // two workgroups per compute unit
+            const long long narrow = ((long long)p.L + (X_KIN ? 15 : 63)) / (X_KIN ? 16 : 64);
+            return launch_one<X_KIN, S_KIN, T, W0, 4>(p, true, stream, (int)((t_skinny_cuts > 0 ? t_skinny_cuts : (2LL * num_cu + narrow - 1) / narrow)));
+        }
         default:
             if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
             else return launch_one<X_KIN, S_KIN, T, 1, 16, 2>(p, true, stream);
@@ -319,9 +412,14 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
 // Force a form of the skinny kernel for the calling thread's launches: 0 = a wavefront per run of lines (64 of a
 // K-outer long operand, 16 of a K-inner one) with the whole K, 1 = the four wavefronts of a workgroup share a run
 // and split K, 2 = sixteen wavefronts do, 3 and 4 = as 0 and 1 with runs four (K-inner: two) times as long,
-// 5 = as 2 with runs of 32 lines of a K-outer operand (two classes of k among the lanes; K-inner: as 2);
+// 5 and 6 = as 2 with runs of 32 and 16 lines of a K-outer operand (two and four classes of k among the lanes;
+// K-inner: as 2), 7 = as 1 with K cut across workgroups too (two workgroups per compute unit; 100 + c: c cuts);
 // -1 = the automatic choice.
-void gemm_skinny_form(int form) { t_skinny_form = (form >= 0 && form <= 5) ? form : -1; }
+void gemm_skinny_form(int form) {
+    t_skinny_cuts = form >= 100 ? form % 100 : 0;
+    if (form >= 100) form = 7;
+    t_skinny_form = (form >= 0 && form <= 7) ? form : -1;
+}
 
 int gemm_choose_skinny(int rows, int cols, int nz) {
     if (nz != 1) return -1;

@@ -32,20 +32,30 @@ std::string fmt(const char* f, long long a = 0, long long b = 0) {
     return buf;
 }
 
-// an event that is deleted when the scope ends, also when an exception leaves it
+// an event of the pool that goes back when the scope ends, also when an exception leaves it
 struct ScopedEvent {
+    CudaStreamPool* pool;
     int64_t handle;
-    ScopedEvent() : handle(cu_handle(dragon_Cuda_newEvent_DisableTiming())) {}
-    ~ScopedEvent() { if (handle) dragon_Cuda_deleteEvent(handle); }
+    explicit ScopedEvent(CudaStreamPool* p) : pool(p), handle(p->getEvent()) {}
+    ~ScopedEvent() { if (handle) pool->returnEvent(handle); }
     ScopedEvent(const ScopedEvent&) = delete;
     ScopedEvent& operator=(const ScopedEvent&) = delete;
 };
 
-// streams -> streams[0]  (CudaFloat32EngineBase.java:649-654)
-void sync_streamArray_2_stream0(const std::vector<int64_t>& streams) {
-    ScopedEvent event1;
+// streams -> streams[0]  (CudaFloat32EngineBase.java:649-654).  With a single stream there is nothing to
+// join: what follows on it is ordered behind what was issued.
+void sync_streamArray_2_stream0(CudaStreamPool* pool, const std::vector<int64_t>& streams) {
+    if (streams.size() < 2) return;
+    ScopedEvent event1(pool);
     cu(dragon_Cuda_eventRecord_streams(event1.handle, streams.data(), (int)streams.size()));
     cu(dragon_Cuda_streamWaitEvent_default(streams[0], event1.handle));
+}
+
+// wait for a syncer's event and hand it back to the pool
+void wait_and_recycle(CudaStreamPool* pool, int64_t event) {
+    const int rc = dragon_Cuda_eventSynchronize(event);
+    pool->returnEvent(event);
+    cu(rc);
 }
 
 // CudaFloat32EngineBase.java:657-694
@@ -53,8 +63,8 @@ class StreamArraySyncer : public Syncer {
 public:
     StreamArraySyncer(CudaStreamPool* pool, std::vector<int64_t> streams)
         : pool_(pool), streams_(std::move(streams)) {
-        sync_streamArray_2_stream0(streams_);
-        event_ = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        sync_streamArray_2_stream0(pool_, streams_);
+        event_ = pool_->getEvent();
         cu(dragon_Cuda_eventRecord(event_, streams_[0]));
     }
     // The reference's finalizer drops the event without waiting; waiting is the safe
@@ -66,7 +76,7 @@ public:
         {
             std::lock_guard<std::mutex> g(mu_);
             if (called_) return;
-            cu(dragon_Cuda_eventSync_Del(event_));
+            wait_and_recycle(pool_, event_);
             called_ = true;
         }
         pool_->returnStreamArray(streams_);
@@ -86,7 +96,7 @@ public:
     SplitKSyncer(EngineCore* core, EngineCore::Block block, CudaStreamPool* pool,
                  std::vector<int64_t> streams)
         : core_(core), block_(block), pool_(pool), streams_(std::move(streams)) {
-        event_ = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        event_ = pool_->getEvent();
         cu(dragon_Cuda_eventRecord(event_, streams_[0]));
     }
     ~SplitKSyncer() override {
@@ -96,7 +106,7 @@ public:
         {
             std::lock_guard<std::mutex> g(mu_);
             if (called_) return;
-            cu(dragon_Cuda_eventSync_Del(event_));
+            wait_and_recycle(pool_, event_);
             called_ = true;
         }
         core_->free(block_.size, block_.address);
@@ -116,7 +126,7 @@ private:
 class StreamSyncer : public Syncer {
 public:
     StreamSyncer(CudaStreamPool* pool, int64_t stream) : pool_(pool), stream_(stream) {
-        event_ = cu_handle(dragon_Cuda_newEvent_DisableTiming());
+        event_ = pool_->getEvent();
         cu(dragon_Cuda_eventRecord(event_, stream_));
     }
     ~StreamSyncer() override {
@@ -124,7 +134,7 @@ public:
     }
     void sync() override {
         if (called_) return;
-        cu(dragon_Cuda_eventSync_Del(event_));
+        wait_and_recycle(pool_, event_);
         called_ = true;
         pool_->returnStream(stream_);
     }
@@ -170,7 +180,27 @@ CudaStreamPool::CudaStreamPool(const CudaDevice& dev, int max_streamsize, int ma
     if (max_getsize_oneturn_ > max_streamsize_) max_getsize_oneturn_ = max_streamsize_;
 }
 CudaStreamPool::~CudaStreamPool() {
+    for (int64_t e : events_) dragon_Cuda_deleteEvent(e);
     if (!gc_.empty()) dragon_Cuda_deleteStreams(gc_.data(), (int)gc_.size());
+}
+int64_t CudaStreamPool::getEvent() {
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        if (!events_.empty()) { const int64_t e = events_.back(); events_.pop_back(); return e; }
+    }
+    std::lock_guard<std::mutex> g(g_cuda_class_lock);
+    cu(dragon_Cuda_setDevice(dev_id_));
+    return cu_handle(dragon_Cuda_newEvent_DisableTiming());
+}
+void CudaStreamPool::returnEvent(int64_t event) {
+    if (event == 0) return;
+    std::lock_guard<std::mutex> g(mu_);
+    if (events_.size() < 256) { events_.push_back(event); return; }
+    dragon_Cuda_deleteEvent(event);
+}
+int CudaStreamPool::pooled_event_count() {
+    std::lock_guard<std::mutex> g(mu_);
+    return (int)events_.size();
 }
 void CudaStreamPool::init() {
     std::lock_guard<std::mutex> g(g_cuda_class_lock);
@@ -495,9 +525,7 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
             } else {
                 cu(mma ? dragon_Cuda_matMul_matMul_mma(streamArray.data(), n, A, B, C, N, M, K)
                        : dragon_Cuda_matMul_matMul(streamArray.data(), n, A, B, C, N, M, K));
-                ScopedEvent event;
-                cu(dragon_Cuda_eventRecord_streams(event.handle, streamArray.data(), n));
-                cu(dragon_Cuda_streamWaitEvent_default(streamArray[0], event.handle));
+                sync_streamArray_2_stream0(streamPool_.get(), streamArray);
                 cu(dragon_Cuda_function_linear_dual2D_row(streamArray[0], C, Bias, M, 1.0f, 1.0f, 0.0f,
                                                           C, lengthv, width, M));
             }
@@ -538,11 +566,7 @@ SyncerPtr CudaFloat32EngineBase::run_2d(int variant, int GridZ, int64_t C, int64
         cu(rc);
         // stage 2: global reduction on streams[0] once every stream has finished stage 1
         const int64_t stream = streamArray[0];
-        {
-            ScopedEvent event;
-            cu(dragon_Cuda_eventRecord_streams(event.handle, streamArray.data(), n));
-            cu(dragon_Cuda_streamWaitEvent_default(stream, event.handle));
-        }
+        sync_streamArray_2_stream0(streamPool_.get(), streamArray);
         cu(dragon_Cuda_matMul_SKbuf_summary(stream, Cbuf, C, part, sizeC));
         // stage 3 of matMul_biased: the bias row, after the reduction
         if (Bias != 0)
@@ -590,7 +614,7 @@ SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, 
         try {
             stream = streamPool_->getStream();
             cu(dragon_Cuda_conv3D_kernel_remode(stream, W, block.address, FH, FW, OC, IC));
-            ScopedEvent event;
+            ScopedEvent event(streamPool_.get());
             cu(dragon_Cuda_eventRecord(event.handle, stream));
             s = streamPool_->getStreamArray(policy_conv3D_GEMM_nstream(GM, OC));
             const int n = (int)s.size();
@@ -605,7 +629,7 @@ SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, 
                 cu(dragon_Cuda_conv3D_conv3D_GemmR(s.data(), n, X, IH, IW, W, block.address, FH, FW, Y, OH, OW,
                                                    N, IC, OC, sh, sw, ph, pw));
             if (Bias) {   // stage 3 on the first stream, after stage 2
-                ScopedEvent event2;
+                ScopedEvent event2(streamPool_.get());
                 cu(dragon_Cuda_eventRecord_streams(event2.handle, s.data(), n));
                 cu(dragon_Cuda_streamWaitEvent_default(stream, event2.handle));
                 cu(dragon_Cuda_function_linear_dual2D_row(stream, Y, Bias, OC, 1.0f, 1.0f, 0.0f, Y, lengthv,
@@ -653,7 +677,7 @@ SyncerPtr CudaFloat32EngineBase::run_conv(int64_t Y, int OH, int OW, int64_t X, 
                 cu(dragon_Cuda_conv3D_conv3D(s.data(), n, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw,
                                              ph, pw));
             if (Bias) {   // the second launch, on streams[0] after every stream of the first
-                ScopedEvent event;
+                ScopedEvent event(streamPool_.get());
                 cu(dragon_Cuda_eventRecord_streams(event.handle, s.data(), n));
                 cu(dragon_Cuda_streamWaitEvent_default(s[0], event.handle));
                 cu(dragon_Cuda_function_linear_dual2D_row(s[0], Y, Bias, OC, 1.0f, 1.0f, 0.0f, Y, lengthv,

@@ -57,10 +57,18 @@ public:
     void returnStream(int64_t) {}
     void returnStreamArray(const std::vector<int64_t>&) {}
     int total_stream_size();
+    // Events without timing, recycled: the reference creates and destroys one per call
+    // (CudaFloat32EngineBase.java:649-694, 1008-1054); handing the same few out again saves the two driver
+    // calls.  An event may go back as soon as its waits are enqueued: a stream's wait refers to the record
+    // that preceded it, not to later ones.
+    int64_t getEvent();
+    void returnEvent(int64_t event);
+    int pooled_event_count();
 private:
     void init();
     int dev_id_, max_streamsize_, max_getsize_oneturn_;
     std::vector<int64_t> gc_;
+    std::vector<int64_t> events_;     // idle events
     int gc_index_ = 0;
     bool inited_ = false;
     std::mutex mu_;

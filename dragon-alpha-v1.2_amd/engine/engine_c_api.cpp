@@ -124,6 +124,7 @@ int32_t dragon_engine_get_param(dragon_engine* eg, const char* name) {
         else if (n == "last_stream_count") out = b.last_stream_count;
         else if (n == "live_blocks") out = (int32_t)eg->eg.engineCore().live_blocks();
         else if (n == "stream_pool_size") out = b.streamPool().total_stream_size();
+        else if (n == "pooled_events") out = b.streamPool().pooled_event_count();
         else if (n == "buf_physical_blocks") out = b.buf_mempool() ? b.buf_mempool()->physical_block_num() : -1;
         else if (n == "buf_buffered_blocks") out = b.buf_mempool() ? b.buf_mempool()->buffered_block_num() : -1;
         else if (n == "buf_used_mem_size") out = b.buf_mempool() ? (int32_t)b.buf_mempool()->used_mem_size() : -1;

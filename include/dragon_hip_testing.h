@@ -31,12 +31,15 @@ extern "C" {
  * sits in LDS, the rim of C -- 1 ... 4 rows / columns past a multiple of 64 -- as strips of 4x4 MFMA blocks;
  * another K falls back to the automatic choice).  27: the skinny kernel for a 2-D product whose C has 4 or 8 columns
  * under at least 256 rows, or 4 or 8 rows over at least 256 columns (wavefronts stream the long operand into 4x4x1
- * MFMA blocks; what the automatic choice takes there; another shape falls back to the automatic choice). */
+ * MFMA blocks; what the automatic choice takes there; another shape falls back to the automatic choice).  28: the band
+ * kernel with bands of 64 rows under tiles of 256 columns (never chosen automatically: measured level with 24). */
 void dragon_gemm_force_tile(int32_t tile);
 /* Force a form of the skinny kernel for the following launches OF THE CALLING THREAD: 0 = a wavefront per run of
- * lines of the long operand with the whole K, 1 = the four wavefronts of a workgroup share a run and split K,
- * 2 = sixteen wavefronts do, 3 and 4 = as 0 and 1 with four lines per lane (a long operand whose k is the row
- * index; as 0 and 1 otherwise); -1 restores the automatic choice. */
+ * lines of the long operand (64 lines where k is its row index, 16 where k is contiguous) with the whole K, 1 = the
+ * four wavefronts of a workgroup share a run and split K, 2 = sixteen wavefronts do, 3 and 4 = as 0 and 1 with runs
+ * four (two) times as long, 5 and 6 = as 2 with runs of 32 and 16 lines (k the row index; else as 2), 7 = as 1 with K
+ * cut across workgroups as well, two workgroups per compute unit (100 + c: c cuts, at most 8; needs the stream's
+ * workspace); -1 restores the automatic choice. */
 void dragon_gemm_skinny_form(int32_t form);
 /* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
  * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the

@@ -12,7 +12,9 @@ from helpers import NN, T1, T2, VARIANT_NAMES, assert_within_tolerance, logical_
 from test_gpu_batched import make_case, run
 
 pytestmark = pytest.mark.gpu
-BAND = 24
+BAND = 24           # bands of 128 rows, tiles of 128 columns
+BAND_WIDE = 28      # bands of 64 rows, tiles of 256 columns
+BANDS = [BAND, BAND_WIDE]
 
 
 @pytest.fixture(autouse=True)
@@ -21,15 +23,17 @@ def _auto_tile(gpu):
     gpu.force_tile(-1)
 
 
+@pytest.mark.parametrize("band", BANDS)
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-def test_two_dimensional_shapes_bitwise(gpu, variant):
+def test_two_dimensional_shapes_bitwise(gpu, variant, band):
     """One tile; one band with an odd and an even number of tiles; more bands than compute units (a
     workgroup walks several bands: the A buffers take turns); bands cut into runs (few bands, many column
     tiles); rows, columns and K 1..3 past a tile or short of one."""
     rng = np.random.default_rng(8100 + variant)
-    gpu.force_tile(BAND)
+    gpu.force_tile(band)
     for (N, M, K) in ((4, 4, 4), (128, 128, 64), (128, 384, 64), (128, 512, 60), (100, 1000, 33), (257, 1029, 64),
-                      (40000, 260, 64), (33000, 131, 12), (256, 8200, 56), (131, 5000, 61), (1024, 1024, 64)):
+                      (40000, 260, 64), (33000, 131, 12), (256, 8200, 56), (131, 5000, 61), (1024, 1024, 64),
+                      (64, 256, 64), (65, 257, 64), (200, 768, 64), (190, 770, 57)):
         A, B = logical_operands(variant, rng, N, M, K, dist="int")
         C, Cp = gpu_matmul_2d(gpu, variant, A, B, fill=91.0)
         R = oracle.matmul_f64(variant, A, B).astype(np.float32)     # small integers: every order is exact
@@ -38,10 +42,11 @@ def test_two_dimensional_shapes_bitwise(gpu, variant):
         assert np.count_nonzero(Cp[N:, :]) == 0 and np.count_nonzero(Cp[:, M:]) == 0, what
 
 
+@pytest.mark.parametrize("band", BANDS)
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-def test_batched_shapes_bitwise(gpu, variant):
+def test_batched_shapes_bitwise(gpu, variant, band):
     rng = np.random.default_rng(8200 + variant)
-    gpu.force_tile(BAND)
+    gpu.force_tile(band)
     for (Batch, N, M, K) in ((1, 1, 1, 1), (3, 5, 6, 7), (15, 82, 96, 9), (4, 128, 128, 64), (37, 1024, 1024, 64),
                              (33, 257, 385, 61), (6, 300, 1000, 36), (70, 260, 520, 64)):
         A, B, dims, cshape, B4 = make_case(variant, rng, Batch, N, M, K, "int")
@@ -52,11 +57,12 @@ def test_batched_shapes_bitwise(gpu, variant):
         assert np.count_nonzero(C[Batch:]) == 0 and np.count_nonzero(C[:, :, M:]) == 0, what
 
 
+@pytest.mark.parametrize("band", BANDS)
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-def test_a_longer_k_takes_another_kernel(gpu, variant):
+def test_a_longer_k_takes_another_kernel(gpu, variant, band):
     # the band kernel holds K in one stage of 64: a forced choice falls back for a longer K
     rng = np.random.default_rng(8300 + variant)
-    gpu.force_tile(BAND)
+    gpu.force_tile(band)
     A, B = logical_operands(variant, rng, 300, 520, 68, dist="int")
     C, _ = gpu_matmul_2d(gpu, variant, A, B)
     assert np.array_equal(C, oracle.matmul_f64(variant, A, B).astype(np.float32))

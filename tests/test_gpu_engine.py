@@ -105,6 +105,28 @@ def test_split_k_through_the_engine_frees_its_buffer(eg):
     eg.delete(tA, tB, tC)
 
 
+def test_events_are_recycled(eg):
+    """The syncers' events (CudaFloat32EngineBase.java:657-694, 1008-1054 create and destroy one per call) come
+    from a pool and go back to it: after many calls, split and unsplit, in both modes, the pool holds a few idle
+    events rather than one per call, and the results stay right."""
+    rng = np.random.default_rng(5)
+    K, N, M = 4096, 256, 256
+    A = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    B = rng.integers(-3, 4, (K, M)).astype(np.float32)
+    tA, tB = eg.tensor(A, K, N), eg.tensor(B, K, M)
+    R = oracle.matmul(1, A, B)
+    for sync in (True, False, True):
+        eg.sync(sync)
+        for _ in range(40):
+            tC = eg.matMulT1(tA, tB)
+            tS = eg.matMul(tC, tC)                           # an unsplit product behind the split one
+            assert np.array_equal(eg.valueOf(tC).reshape(N, M), R)
+            eg.delete(tC, tS)
+    eg.sync(True)
+    assert 1 <= eg.get_param("pooled_events") <= 8
+    eg.delete(tA, tB)
+
+
 def test_policy_follows_the_unit_count(eg):
     real = eg.get_param("multiProcessorCount")
     try:

@@ -45,7 +45,7 @@ def test_the_automatic_choice_names_the_kernel(gpu):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108])
 @pytest.mark.parametrize("thin", [1, 2, 3, 4, 5, 7, 8])
 def test_thin_columns_bitwise(gpu, variant, thin, form):
     """C of 1 ... 8 columns (stored 4 or 8) under row counts around the 16, 64 and 256 lines a wavefront takes,
@@ -57,7 +57,7 @@ def test_thin_columns_bitwise(gpu, variant, thin, form):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108])
 @pytest.mark.parametrize("thin", [1, 3, 4, 6, 8])
 def test_thin_rows_bitwise(gpu, variant, thin, form):
     gpu.skinny_form(form)
@@ -70,7 +70,7 @@ def test_thin_rows_bitwise(gpu, variant, thin, form):
 def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
     """K around the k rows / 32-k panels of a register buffer, the 4-k chunks of a lane, the shares of a K split
     between 4 or 16 wavefronts; in every form."""
-    for form in (0, 1, 2, 3, 4, 5):
+    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108):
         gpu.skinny_form(form)
         check(gpu, variant, 700, 4, K, 3000 + K + variant)
         check(gpu, variant, 8, 900, K, 4000 + K + variant)
@@ -92,6 +92,25 @@ def test_long_shapes_against_both_oracles(gpu, variant):
         R = oracle_2d(variant, A, B)
         assert_within_tolerance(C, R, K, A, B, "%s %d x %d x %d" % (VARIANT_NAMES[variant], N, M, K))
         assert np.array_equal(C, C2)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
+    """Fewer runs of lines than compute units: the automatic choice cuts K across workgroups, which meet through
+    the stream's workspace and its arrival counters.  Bitwise on integers, the same bits launch after launch
+    (the counters are back at zero each time), and a balanced-kernel launch on the same stream in between."""
+    for (N, M, K) in ((8, 4096, 4096), (4, 2048, 8192), (2048, 4, 16384), (1000, 8, 3000), (8, 1000, 5000)):
+        check(gpu, variant, N, M, K, 600 + N + M + K + variant)
+    rng = np.random.default_rng(31 + variant)
+    A, B = logical_operands(variant, rng, 8, 4096, 4096)
+    first, _ = gpu_matmul_2d(gpu, variant, A, B)
+    A2, B2 = logical_operands(variant, rng, 1000, 780, 1532, "int")
+    for _ in range(20):
+        C, _ = gpu_matmul_2d(gpu, variant, A, B)
+        assert np.array_equal(C, first)
+        C2, _ = gpu_matmul_2d(gpu, variant, A2, B2)             # the balanced kernel: same workspace, same counters
+        assert np.array_equal(C2, oracle_2d(variant, A2, B2))
+    assert_within_tolerance(first, oracle_2d(variant, A, B), 4096, A, B, "%s 8 x 4096 x 4096" % VARIANT_NAMES[variant])
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
