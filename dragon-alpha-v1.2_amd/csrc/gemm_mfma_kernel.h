@@ -643,7 +643,7 @@ __device__ __forceinline__ void rim_job(const GemmParams& p, float* lds, int job
         const int i = row_job ? R0 + x : seg * 64 + lane, j = row_job ? seg * 64 + lane : C0 + x;
         const bool inside = row_job ? (x < rr && j < C0 + rc) : (x < rc && i < R0);
         float value = (ok && (row_job ? i < a_rows : j < b_cols)) ? sum : 0.0f;
-        if constexpr (BIAS) {   // as the tiles' epilogue adds it (see store_tile_rows)
+        if constexpr (BIAS) {   // as the tiles' epilogue adds it (see store_tile)
             if (inside && i < p.bias_rows) value = (value + (j < p.bias_width ? p.bias[j] : 0.0f)) + 0.0f;
         }
         if (inside) C[(size_t)i * p.ldc + j] = value;

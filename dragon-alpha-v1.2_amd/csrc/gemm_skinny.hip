@@ -1,5 +1,5 @@
-// Skinny products: a C of at most 8 columns (N x 4, N x 8) or at most 8 rows (4 x M, 8 x M) under a long other
-// side -- matrix times a few vectors.  The reference sends a C of 4 columns to kernels of their own
+// Skinny products: a C of at most 16 columns (N x 4 ... N x 16) or at most 16 rows (4 x M ... 16 x M) under a long
+// other side -- matrix times a few vectors.  The reference sends a C of 4 columns to kernels of their own
 // (MM/matMul_sernel.cuh:17-30, dispatched at MM/matMul.cuh:100-102) and thin row strips to k18 / k14 / k12
 // (MM/matMul.cuh:104-106).
 //
@@ -73,7 +73,7 @@ __device__ __forceinline__ void skinny_put(const SkinnyParams& p, int line, int 
 template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny(const SkinnyParams p) {
-    static_assert(T == 4 || T == 8, "4 or 8 short lines");
+    static_assert(T == 4 || T == 8 || T == 12 || T == 16, "4, 8, 12 or 16 short lines");
     static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || ((CL == 2 || CL == 4) && W == 1)), "forms");
     constexpr int LS = 8, PK = 32;                         // K-inner X: lines per read, k per panel
     constexpr int H = T / 4;                               // groups of 4 short lines
@@ -103,7 +103,7 @@ void gemm_f32_skinny(const SkinnyParams p) {
         if constexpr (!X_KIN) {
             // ---- a lane owns W lines: X[k][line0 + W * lane + c] (CL = 2: X[k + class][line0 + (lane & 31)]);
             //      U loads (U * CL k rows) per register buffer ----
-            constexpr int U = W == 4 ? 8 : 16;
+            constexpr int U = (W == 4 || (NW == 16 && H > 2)) ? 8 : 16;     // (the workgroups of 16 wavefronts have 128 registers a lane)
             const int cls = CL == 4 ? lane >> 4 : CL == 2 ? lane >> 5 : 0;
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, ((long long)(p.K - 1) * p.ldx + p.x_lines) * 4);
             const int x_step = p.ldx * 4;
@@ -169,7 +169,7 @@ void gemm_f32_skinny(const SkinnyParams p) {
         } else {
             // ---- per instruction 8 lines x 8 classes of k: X[line0 + 8 * set + (lane & 7)][k0 + 4 * (lane >> 3) + 0 .. 3];
             //      U 32-k panels per register buffer ----
-            constexpr int U = (NW == 16 || W == 4) ? 2 : 4;
+            constexpr int U = (NW == 16 && H > 2) ? 1 : (NW == 16 || W == 4) ? 2 : 4;
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, (long long)p.x_lines * p.ldx * 4);
             const int kk4 = 4 * (lane / LS);
             int x_off[W];
@@ -259,7 +259,7 @@ void gemm_f32_skinny(const SkinnyParams p) {
                     d[a][r] = v;
                 }
         }
-        if constexpr (ACCS * 4 <= 16 && NW == 4) if (p.k_cuts > 1) {
+        if constexpr (W == (X_KIN ? 2 : 1) && CL == 1 && NW == 4) if (p.k_cuts > 1) {    // the narrow forms only
             // The workgroups that cut this run's K meet in memory: every one leaves its sum in its slot and is
             // counted; whoever is counted last adds the slots -- its own included -- in k order and stores.  The
             // hand-over is the balanced kernel's (gemm_mfma_streamk.hip, store_partial): device-scope stores that
@@ -286,25 +286,28 @@ void gemm_f32_skinny(const SkinnyParams p) {
             if (arrived != p.k_cuts - 1) return;
             asm volatile("" ::: "memory");
             if (lane < MEET_LANES) {
-                float v[SKINNY_MAX_CUTS][ACCS * 4];
+                // eight outputs of a lane at a time: every cut's floats of them are read before any is added
+                constexpr int CH = ACCS * 4 < 8 ? ACCS * 4 : 8;
 #pragma unroll
-                for (int c = 0; c < SKINNY_MAX_CUTS; c++)
-                    if (c < p.k_cuts) {
+                for (int base = 0; base < ACCS * 4; base += CH) {
+                    float v[SKINNY_MAX_CUTS][CH];
 #pragma unroll
-                        for (int i = 0; i < ACCS * 4; i++)
-                            v[c][i] = __hip_atomic_load(slots + (size_t)c * (ACCS * 4 * MEET_LANES) + i * MEET_LANES + lane,
-                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
+                    for (int c = 0; c < SKINNY_MAX_CUTS; c++)
+                        if (c < p.k_cuts) {
 #pragma unroll
-                for (int a = 0; a < ACCS; a++)
+                            for (int i = 0; i < CH; i++)
+                                v[c][i] = __hip_atomic_load(slots + (size_t)c * (ACCS * 4 * MEET_LANES) + (base + i) * MEET_LANES + lane,
+                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        float sum = v[0][a * 4 + r];
+                    for (int i = 0; i < CH; i++) {
+                        float sum = v[0][i];
 #pragma unroll
                         for (int c = 1; c < SKINNY_MAX_CUTS; c++)
-                            if (c < p.k_cuts) sum += v[c][a * 4 + r];
-                        d[a][r] = sum;
+                            if (c < p.k_cuts) sum += v[c][i];
+                        d[(base + i) / 4][(base + i) % 4] = sum;
                     }
+                }
             }
         }
     }
@@ -337,7 +340,7 @@ hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream, int cuts 
     p.k_cuts = 1;
     p.k_cut = p.K;
     long long grid = shared ? units : (units + NW - 1) / NW;
-    if (shared && cuts > 1 && NW == 4 && W * (T / 4) * 4 <= 16 && units <= 65536) {
+    if (shared && cuts > 1 && NW == 4 && W == (X_KIN ? 2 : 1) && CL == 1 && units <= 65536) {
         if (cuts > SKINNY_MAX_CUTS) cuts = SKINNY_MAX_CUTS;
         const int k_cut = ((p.K + cuts - 1) / cuts + 32 * NW - 1) / (32 * NW) * (32 * NW);
         const int real = (p.K + k_cut - 1) / k_cut;
@@ -404,7 +407,13 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
 
 template <bool X_KIN, bool S_KIN>
 hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
-    return T == 4 ? launch_skinny<X_KIN, S_KIN, 4>(p, stream) : launch_skinny<X_KIN, S_KIN, 8>(p, stream);
+    switch (T) {
+        case 4: return launch_skinny<X_KIN, S_KIN, 4>(p, stream);
+        case 8: return launch_skinny<X_KIN, S_KIN, 8>(p, stream);
+        case 12: return launch_skinny<X_KIN, S_KIN, 12>(p, stream);
+        case 16: return launch_skinny<X_KIN, S_KIN, 16>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace
@@ -421,23 +430,35 @@ void gemm_skinny_form(int form) {
     t_skinny_form = (form >= 0 && form <= 7) ? form : -1;
 }
 
-int gemm_choose_skinny(int rows, int cols, int nz) {
+// 4, 8, 12 or 16 stored lines on the short side
+static bool skinny_short(int n) { return n >= 4 && n <= 16 && n % 4 == 0; }
+
+// 4 or 8 short lines: every layout.  12 or 16: measured ahead of the tile kernels (46 - 50 us against 67 - 70 on
+// 65536 lines of 1024, 202 - 211 against 252 - 269 on 262144) only where the long operand is K-outer and has at
+// least a run of 256 lines per compute unit; a K-inner long operand shares its short operand's values among too
+// few lines per wavefront there (59 - 83 us against 68 - 77).
+int gemm_choose_skinny(int rows, int cols, int nz, int variant, int num_cu) {
     if (nz != 1) return -1;
-    const bool thin_cols = (cols == 4 || cols == 8) && rows >= 256;
-    const bool thin_rows = (rows == 4 || rows == 8) && cols >= 256;
-    return thin_cols || thin_rows ? TILE_SKINNY : -1;
+    const bool thin_cols = skinny_short(cols) && rows >= 256;
+    const bool thin_rows = !thin_cols && skinny_short(rows) && cols >= 256;
+    if (!thin_cols && !thin_rows) return -1;
+    if ((thin_cols ? cols : rows) <= 8) return TILE_SKINNY;
+    const bool x_kouter = thin_cols ? variant == GEMM_T1 : (variant == GEMM_NN || variant == GEMM_T1);
+    return x_kouter && (long long)(thin_cols ? rows : cols) >= 256LL * num_cu ? TILE_SKINNY : -1;
 }
 
 // True where the product is one for the skinny kernel: one unsplit 2-D product without a bias row whose C has
-// 4 or 8 columns under at least 256 rows, or 4 or 8 rows over at least 256 columns, and whose operands' byte
-// offsets (with the reads a register buffer runs ahead, and the lines of a last, partly filled run) fit 32 bits.
+// 4 ... 16 stored columns under at least 256 rows, or 4 ... 16 stored rows over at least 256 columns, and whose
+// operands' byte offsets (with the reads a register buffer runs ahead, and the lines of a last, partly filled
+// run) fit 32 bits.
 static bool gemm_skinny_applies(int variant, const GemmParams& p) {
-    if (p.split || p.bias != nullptr || gemm_choose_skinny(p.rows, p.cols, p.nz) < 0) return false;
-    const bool thin_cols = (p.cols == 4 || p.cols == 8) && p.rows >= 256;
+    // (a forced choice takes every shape the kernel can run: up to 16 short lines in every layout)
+    if (p.split || p.bias != nullptr || gemm_choose_skinny(p.rows, p.cols, p.nz, GEMM_T1, 1) < 0) return false;
+    const bool thin_cols = skinny_short(p.cols) && p.rows >= 256;
     const bool a_kin = variant != GEMM_T1, b_kin = variant == GEMM_T2;
     // a K-inner operand is addressed line * ld + k, a K-outer one k * ld + line
-    const long long a_span = a_kin ? (long long)(thin_cols ? p.rows : 8) * p.lda : (long long)p.k_total * p.lda;
-    const long long b_span = b_kin ? (long long)(thin_cols ? 8 : p.cols) * p.ldb : (long long)p.k_total * p.ldb;
+    const long long a_span = a_kin ? (long long)(thin_cols ? p.rows : 16) * p.lda : (long long)p.k_total * p.lda;
+    const long long b_span = b_kin ? (long long)(thin_cols ? 16 : p.cols) * p.ldb : (long long)p.k_total * p.ldb;
     const long long ld = p.lda > p.ldb ? p.lda : p.ldb;
     return ld <= (1 << 20) && (a_span + 64 * ld) * 4 < 0x7fff0000LL && (b_span + 64 * ld) * 4 < 0x7fff0000LL;
 }
@@ -445,7 +466,7 @@ static bool gemm_skinny_applies(int variant, const GemmParams& p) {
 hipError_t gemm_launch_skinny(int variant, const GemmParams& g, hipStream_t stream) {
     if (!gemm_skinny_applies(variant, g)) return hipErrorOutOfMemory;   // the caller takes a tile kernel
     const bool a_kin = variant != GEMM_T1, b_kin = variant == GEMM_T2;
-    const bool thin_cols = (g.cols == 4 || g.cols == 8) && g.rows >= 256;
+    const bool thin_cols = skinny_short(g.cols) && g.rows >= 256;
     SkinnyParams p = {};
     p.C = g.C; p.ldc = g.ldc;
     p.K = min(g.k_total, min(a_kin ? g.a_inner : g.a_outer, b_kin ? g.b_inner : g.b_outer));

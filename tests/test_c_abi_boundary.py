@@ -214,10 +214,14 @@ def test_tile_choice_on_the_documented_shapes(dh):
         assert ct(v, 257, 388, 36, 88) != 26 and ct(v, 257, 388, 36, 148) != 26 and ct(v, 256, 384, 36, 129) != 26
         assert ct(v, 257, 388, 8, 129) != 26                   # 192 tiles: too few
     assert ct(NN, 257, 388, 36, 64) == 1                        # a shorter K: 64x64 tiles with the rim beside them
-    # a C of 4 or 8 columns (or rows) under at least 256 lines of the other side, one 2-D product: the skinny kernel
+    # a C of 4, 8, 12 or 16 columns (or rows) under at least 256 lines of the other side, one 2-D product: the skinny kernel
     for v in (NN, T1, T2):
         assert ct(v, 65536, 4, 1, 1024) == 27 and ct(v, 8, 8192, 1, 4096) == 27 and ct(v, 256, 8, 1, 4) == 27
-        assert ct(v, 65536, 12, 1, 1024) != 27 and ct(v, 65536, 4, 2, 1024) != 27 and ct(v, 252, 4, 1, 1024) != 27
+    # 12 or 16: only beside a K-outer long operand (A of A^T*B, B of A*B and A^T*B) with 256 lines per compute unit
+    assert ct(T1, 65536, 16, 1, 1024) == 27 and ct(NN, 16, 65536, 1, 1024) == 27 and ct(T1, 12, 65536, 1, 1024) == 27
+    assert ct(NN, 65536, 16, 1, 1024) != 27 and ct(T2, 16, 65536, 1, 1024) != 27 and ct(T1, 32768, 16, 1, 1024) != 27
+    for v in (NN, T1, T2):
+        assert ct(v, 65536, 20, 1, 1024) != 27 and ct(v, 65536, 4, 2, 1024) != 27 and ct(v, 252, 4, 1, 1024) != 27
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
     if ct(NN, *shape) in (5 + P, 9 + P):
@@ -255,7 +259,7 @@ def test_tile_choice_stays_inside_what_the_kernels_accept(dh):
                 assert 56 < k <= 64 and cols % 32 == 0, (v, rows, cols, nz, k)
             if t == 26:
                 assert 88 < k <= 144, (v, rows, cols, nz, k)
-            if t == 27:     # the skinny kernel: one 2-D product with a C of 4 or 8 columns (rows) and a long other side
-                assert nz == 1 and ((cols in (4, 8) and rows >= 256) or (rows in (4, 8) and cols >= 256)), (v, rows, cols, nz, k)
+            if t == 27:     # the skinny kernel: one 2-D product with a C of 4 ... 16 columns (rows) and a long other side
+                assert nz == 1 and ((cols in (4, 8, 12, 16) and rows >= 256) or (rows in (4, 8, 12, 16) and cols >= 256)), (v, rows, cols, nz, k)
     assert 27 in seen
     assert {21, 24} <= seen and seen & {18, 22} and seen & {19, 20, 23}      # the sample reaches every family

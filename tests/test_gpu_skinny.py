@@ -1,4 +1,4 @@
-"""GPU parity of the skinny kernel (gemm_skinny.hip): a C of 4 or 8 columns under many rows, or of 4 or 8 rows over
+"""GPU parity of the skinny kernel (gemm_skinny.hip): a C of 4 ... 16 columns under many rows, or of 4 ... 16 rows over
 many columns -- what the reference sends to its 4-column kernels (MM/matMul_sernel.cuh:17-30, dispatched at
 MM/matMul.cuh:100-102) and to k18 / k14 / k12 (MM/matMul.cuh:104-106).  Wavefronts stream the long operand from
 memory into 4 x 4 x 1 MFMA blocks; integer inputs pin the indexing bit for bit: lines per wavefront, the classes
@@ -39,28 +39,38 @@ def test_the_automatic_choice_names_the_kernel(gpu):
     for (rows, cols) in ((65536, 4), (8192, 8), (256, 4), (4, 65536), (8, 256), (4, 1000)):
         for variant in (NN, T1, T2):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
+    # 12 or 16 short lines: only beside a K-outer long operand of at least 256 lines per compute unit
+    assert gpu.choose_tile(T1, 65536, 16, 1, 1024, cu) == SKINNY and gpu.choose_tile(T1, 65536, 12, 1, 1024, cu) == SKINNY
+    assert gpu.choose_tile(NN, 16, 65536, 1, 1024, cu) == SKINNY and gpu.choose_tile(T1, 12, 70000, 1, 1024, cu) == SKINNY
+    assert gpu.choose_tile(NN, 65536, 16, 1, 1024, cu) != SKINNY and gpu.choose_tile(T2, 65536, 16, 1, 1024, cu) != SKINNY
+    assert gpu.choose_tile(T2, 16, 65536, 1, 1024, cu) != SKINNY and gpu.choose_tile(T1, 32768, 16, 1, 1024, cu) != SKINNY
     # not skinny enough, too short, or a batch / K slices
-    for (rows, cols, nz) in ((65536, 12, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (65536, 4, 2), (4, 65536, 3)):
-        assert gpu.choose_tile(NN, rows, cols, nz, 1024, cu) != SKINNY
+    for (rows, cols, nz) in ((65536, 20, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (16, 252, 1), (65536, 4, 2), (4, 65536, 3)):
+        for variant in (NN, T1, T2):
+            assert gpu.choose_tile(variant, rows, cols, nz, 1024, cu) != SKINNY
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
 @pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108])
-@pytest.mark.parametrize("thin", [1, 2, 3, 4, 5, 7, 8])
+@pytest.mark.parametrize("thin", [1, 2, 3, 4, 5, 7, 8, 9, 12, 13, 16])
 def test_thin_columns_bitwise(gpu, variant, thin, form):
-    """C of 1 ... 8 columns (stored 4 or 8) under row counts around the 16, 64 and 256 lines a wavefront takes,
+    """C of 1 ... 16 columns (stored 4, 8, 12 or 16) under row counts around the 16, 64 and 256 lines a wavefront takes,
     in every form of the kernel: a wavefront per run of lines, K shared between 4 or 16 wavefronts, one or four
     lines per lane."""
     gpu.skinny_form(form)
+    if form >= 0:
+        gpu.force_tile(SKINNY)      # 12 and 16 columns beside a K-inner long operand are not the automatic choice
     for (N, K) in ((256, 64), (1000, 1028), (4099, 36), (40000, 100), (20000, 260)):
         check(gpu, variant, N, thin, K, 100 * thin + N + K + variant)
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
 @pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108])
-@pytest.mark.parametrize("thin", [1, 3, 4, 6, 8])
+@pytest.mark.parametrize("thin", [1, 3, 4, 6, 8, 10, 12, 15, 16])
 def test_thin_rows_bitwise(gpu, variant, thin, form):
     gpu.skinny_form(form)
+    if form >= 0:
+        gpu.force_tile(SKINNY)
     for (M, K) in ((256, 64), (1001, 1028), (4100, 36), (40001, 100), (20000, 260)):
         check(gpu, variant, thin, M, K, 200 * thin + M + K + variant)
 
@@ -70,11 +80,15 @@ def test_thin_rows_bitwise(gpu, variant, thin, form):
 def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
     """K around the k rows / 32-k panels of a register buffer, the 4-k chunks of a lane, the shares of a K split
     between 4 or 16 wavefronts; in every form."""
+    gpu.force_tile(SKINNY)
     for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108):
         gpu.skinny_form(form)
         check(gpu, variant, 700, 4, K, 3000 + K + variant)
         check(gpu, variant, 8, 900, K, 4000 + K + variant)
+        check(gpu, variant, 530, 16, K, 3500 + K + variant)
+        check(gpu, variant, 12, 300, K, 4500 + K + variant)
     gpu.skinny_form(-1)
+    gpu.force_tile(-1)
     if K <= 64:
         check(gpu, variant, 70000, 7, K, 5000 + K + variant)
 
@@ -84,7 +98,7 @@ def test_long_shapes_against_both_oracles(gpu, variant):
     """Uniform inputs at the benchmark's shapes, scaled down 4 x along the long side, within the FP32 tolerance
     (relative Frobenius error <= 1e-5, elements within 1e-4 * sqrt(K) * max|A| * max|B|); and the same launch
     twice gives the same bits."""
-    for (N, M, K) in ((16384, 4, 1024), (2048, 8, 4096), (4, 16384, 1024), (8, 2048, 4096)):
+    for (N, M, K) in ((16384, 4, 1024), (2048, 8, 4096), (4, 16384, 1024), (8, 2048, 4096), (16384, 16, 1024), (12, 16384, 1024)):
         rng = np.random.default_rng(N + M + K + variant)
         A, B = logical_operands(variant, rng, N, M, K)
         C, _ = gpu_matmul_2d(gpu, variant, A, B)
@@ -101,6 +115,10 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
     (the counters are back at zero each time), and a balanced-kernel launch on the same stream in between."""
     for (N, M, K) in ((8, 4096, 4096), (4, 2048, 8192), (2048, 4, 16384), (1000, 8, 3000), (8, 1000, 5000)):
         check(gpu, variant, N, M, K, 600 + N + M + K + variant)
+    gpu.force_tile(SKINNY)
+    for (N, M, K) in ((16, 4096, 2048), (1000, 12, 3000)):
+        check(gpu, variant, N, M, K, 700 + N + M + K + variant)
+    gpu.force_tile(-1)
     rng = np.random.default_rng(31 + variant)
     A, B = logical_operands(variant, rng, 8, 4096, 4096)
     first, _ = gpu_matmul_2d(gpu, variant, A, B)
@@ -116,7 +134,7 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
 @pytest.mark.parametrize("variant", [NN, T1, T2])
 def test_forced_on_another_shape_falls_back(gpu, variant):
     gpu.force_tile(SKINNY)
-    check(gpu, variant, 300, 12, 64, 77 + variant)
+    check(gpu, variant, 300, 20, 64, 77 + variant)
     check(gpu, variant, 100, 4, 64, 78 + variant)
     check(gpu, variant, 8, 8, 64, 79 + variant)
 
