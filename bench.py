@@ -343,11 +343,14 @@ def main():
         ms = timer.per_launch_ms(lambda: BMM.batchMatMulT2_texture(
             S, 1, dQ.address, dK.address, dO.address, Bt, Sq, Sq, Sq, D), iters=50)
         record("cfg4 batch64 Q.K^T 1024x64", fl4, ms, by4)
-        dh.force_tile(28)      # the band kernel with bands of 64 rows under tiles of 256 columns
-        ms = timer.per_launch_ms(lambda: BMM.batchMatMulT2_texture(
-            S, 1, dQ.address, dK.address, dO.address, Bt, Sq, Sq, Sq, D), iters=50)
-        dh.force_tile(-1)
-        record("cfg4 batch64 Q.K^T 1024x64, bands of 64 rows x tiles of 256 columns (forced)", fl4, ms, by4)
+        # two other builds of the band kernel, never chosen automatically: measured level with it
+        for forced, what in ((28, "bands of 64 rows x tiles of 256 columns"),
+                             (29, "the band's rows of A in registers, two workgroups of four wavefronts per unit")):
+            dh.force_tile(forced)
+            ms = timer.per_launch_ms(lambda: BMM.batchMatMulT2_texture(
+                S, 1, dQ.address, dK.address, dO.address, Bt, Sq, Sq, Sq, D), iters=50)
+            dh.force_tile(-1)
+            record("cfg4 batch64 Q.K^T 1024x64, %s (forced)" % what, fl4, ms, by4)
         ms = timer.per_launch_ms(lambda: BMM.batchMatMul_texture(
             S, 1, dS.address, dV.address, dO.address, Bt, Sq, D, Sq, Sq), iters=50)
         record("cfg4 batch64 scores.V 1024x1024 by 1024x64", fl4, ms, by4)

@@ -54,13 +54,15 @@ enum GemmTile {
     TILE_SKINNY = 27,
     // the band kernel with bands of 64 rows under tiles of 256 columns
     TILE_BAND_64x256 = 28,
+    // the band kernel with the band's rows of A in registers: 128 x 128 tiles, four wavefronts, two workgroups per unit
+    TILE_BAND_REGS = 29,
     // Flag on the ids 0..9: the stages of a long K run two by two, with the LDS buffer known at compile
     // time and without the per-lane K test (see the kernel).  Faster from about K = 512 on, slower on a
     // short K; gemm_choose_tile sets it.
     TILE_PAIRED = 0x100
 };
 inline bool gemm_tile_is_streamk(int tile) { return (tile >= TILE_SK_64x64 && tile < TILE_SK_END) || tile == TILE_SK_256x64; }
-inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128 || tile == TILE_BAND_64x256; }
+inline bool gemm_tile_is_band(int tile) { return tile == TILE_BAND_128x128 || tile == TILE_BAND_64x256 || tile == TILE_BAND_REGS; }
 inline bool gemm_tile_is_shortk(int tile) { return tile == TILE_SHORTK_64x64; }
 inline bool gemm_tile_is_skinny(int tile) { return tile == TILE_SKINNY; }
 inline bool gemm_tile_is_dma(int tile) { return tile >= TILE_DMA_128x128_S4 && tile <= TILE_DMA_64x64_K32_S4; }
@@ -214,7 +216,7 @@ long long gemm_streamk_workspaces_refused();      // balanced launches that foun
 // The band kernel (tile ids TILE_BAND_128x128, and TILE_BAND_64x256 with `wide`) for the three products, batched
 // too, with K <= 64.  hipErrorOutOfMemory says that the product cannot go this way (a longer K, K slices, a bias
 // row) and the caller takes a tile-per-workgroup kernel instead.
-hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream, bool wide = false);
+hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream, bool wide = false, bool regs = false);
 // TILE_BAND_128x128 where the band kernel is the better choice, else -1
 int gemm_choose_band(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
 // how the band kernel deals a band's column tiles to workgroups

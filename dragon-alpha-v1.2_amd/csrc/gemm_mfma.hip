@@ -180,7 +180,7 @@ hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t s
         // stream that has no workspace yet; a bias row on a transposed product) or the band kernel (a K beyond one stage, K slices, a
         // bias row) a tile-per-workgroup kernel takes over
         const hipError_t e = gemm_tile_is_skinny(tile)   ? gemm_launch_skinny(variant, p, stream)
-                             : gemm_tile_is_band(tile)   ? gemm_launch_band(variant, p, stream, tile == TILE_BAND_64x256)
+                             : gemm_tile_is_band(tile)   ? gemm_launch_band(variant, p, stream, tile == TILE_BAND_64x256, tile == TILE_BAND_REGS)
                              : gemm_tile_is_shortk(tile) ? gemm_launch_shortk(variant, p, stream)
                                                          : gemm_launch_streamk(variant, p, tile, stream);
         if (e != hipErrorOutOfMemory) return e;

@@ -385,6 +385,244 @@ void gemm_f32_mfma_band(const GemmParams p) {
     }
 }
 
+// ---- the band's rows of A in registers ----
+// With K <= 64 a wavefront's share of A -- 64 rows x 64 k -- is 64 floats a lane: it is read from memory once per
+// band straight into registers (lane half h takes the k of [32h, 32h + 32), so a lane's floats of a row are
+// contiguous) and stays there while the workgroup walks the band's column tiles.  LDS then holds only the two
+// B tiles (64 KiB), a workgroup is four wavefronts of 64 x 64 (half the LDS reads per MFMA of the 32 x 64 share
+// above) with about 170 registers, and TWO workgroups fit a compute unit: while one waits at its barrier, reads
+// its fragments or loads a band, the other one's MFMAs keep the pipes busy.  A tile is multiplied block after
+// block (32 x 32 outputs, the whole K: 32 MFMAs in a row into one accumulator): a finished block's 16 stores go
+// out between the MFMAs of the next block, so one accumulator set is enough and the write path sees an even
+// stream; a lane's B values of a column block (32 floats) are read from LDS as the values before them have had
+// their last use.
+template <bool A_KIN, bool B_KIN>
+__global__ __launch_bounds__(256, 2)
+void gemm_f32_mfma_band_regs(const GemmParams p) {
+    constexpr int NT = 256, BM = 128, BN = 128, KT = BD_KT, TM = 2, TN = 2;
+    constexpr int GR = KT / 8;                 // groups of 4 k steps (a step = one MFMA's two k: s and 32 + s)
+    using LanesB = BandLanes<B_KIN, BN, KT, NT>;
+    constexpr int PB = LanesB::PASSES, B_BYTES = BN * KT * 4;
+    __shared__ __attribute__((aligned(16))) float smemB[2 * BN * KT];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int k_a = min(p.k_total, A_KIN ? p.a_inner : p.a_outer), k_b = min(p.k_total, B_KIN ? p.b_inner : p.b_outer);
+
+    LanesB lb;
+    lb.init(t, p.ldb, k_b);
+    const unsigned lds_b0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float*)smemB;
+    const unsigned lds_wave_b = lds_b0 + wave * 1024;
+
+    // B fragments of step group g (steps 4g .. 4g + 3: k = 32h + 4g + q): K-inner logical chunk 8h + g of the lane's
+    // column; K-outer k row 32h + 4g + q, the lane's column.  Block j is 32 columns on.
+    unsigned b_rd[B_KIN ? GR : 1];
+    if constexpr (B_KIN) {
+#pragma unroll
+        for (int g = 0; g < GR; g++) b_rd[g] = pinned(lds_b0 + ((wn * 64 + r) * KT + ((8 * h + g) ^ kin_swizzle<KT>(r)) * 4) * 4);
+    } else {
+        b_rd[0] = pinned(lds_b0 + (32 * h * BN + wn * 64 + r) * 4);
+    }
+    // the lane's B values of one 32-column block for the whole K: fb[s] = B(k = 32 h + s, the lane's column)
+    float fb[32];
+    // steps 4g .. 4g + 3 of block j from B buffer PB_
+    auto read_group = [&](auto g_c, auto j_c, auto pb_c) __attribute__((always_inline)) {
+        constexpr int g = decltype(g_c)::value, j = decltype(j_c)::value, PB_ = decltype(pb_c)::value;
+        if constexpr (B_KIN) {
+            const v4f v = *(lds_v4f)(b_rd[g] + PB_ * B_BYTES + j * 32 * KT * 4);
+            fb[4 * g] = v.x; fb[4 * g + 1] = v.y; fb[4 * g + 2] = v.z; fb[4 * g + 3] = v.w;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; q++) fb[4 * g + q] = *(lds_f32)(b_rd[0] + PB_ * B_BYTES + ((4 * g + q) * BN + j * 32) * 4);
+        }
+    };
+
+    const int ldc4 = p.ldc * 4;
+    const int c_lane = (int)pinned((unsigned)((wm * 64 + 4 * h) * ldc4 + (wn * 64 + r) * 4));
+    const int c_col = wn * 64 + r;
+
+    const int G = gridDim.x;
+    const int U = p.nz * p.tiles_m * p.bd_chunks;
+    int u = xcd_contiguous_id(blockIdx.x, G);   // G <= U
+    int z, m, n, n_end;
+    auto decode_unit = [&](int unit) __attribute__((always_inline)) {
+        const int per_z = p.tiles_m * p.bd_chunks;
+        z = __builtin_amdgcn_readfirstlane(unit / per_z);
+        const int rem = unit - z * per_z;
+        m = __builtin_amdgcn_readfirstlane(rem / p.bd_chunks);
+        n = (rem - m * p.bd_chunks) * p.bd_chunk_tiles;
+        n_end = min(n + p.bd_chunk_tiles, p.tiles_n);
+    };
+    auto b_descriptor = [&](bool live) __attribute__((always_inline)) {
+        const float* base = p.B + (size_t)z * p.sB + (B_KIN ? (size_t)n * BN * p.ldb : (size_t)n * BN);
+        return band_descriptor<B_KIN>(base, live ? (B_KIN ? p.b_outer : p.b_inner) - n * BN : 0, BN, p.ldb);
+    };
+
+    // ---- the band's A: a[i][s] = A(row 64 wm + 32 i + r of the band, k = 32 h + s); zero beyond the operand ----
+    float a[TM][32];
+    auto load_a = [&]() __attribute__((always_inline)) {
+        if constexpr (A_KIN) {
+            const int rows_left = p.a_outer - m * BM;
+            const float* base = p.A + (size_t)z * p.sA + (size_t)m * BM * p.lda;
+            const int rows = rows_left > BM ? BM : rows_left;
+            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, rows > 0 ? rows * p.lda * 4 : 0, RSRC_FLAGS);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    const int k = 32 * h + 4 * c;
+                    const int off = k < k_a ? ((wm * 64 + 32 * i + r) * p.lda + k) * 4 : OOB_OFFSET;
+                    const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ra, off, 0, 0));
+                    a[i][4 * c] = v.x; a[i][4 * c + 1] = v.y; a[i][4 * c + 2] = v.z; a[i][4 * c + 3] = v.w;
+                }
+        } else {
+            const float* base = p.A + (size_t)z * p.sA + (size_t)m * BM;
+            const int cols_left = p.a_inner - m * BM;
+            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, RSRC_RECORDS, RSRC_FLAGS);
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const int col = wm * 64 + 32 * i + r;
+#pragma unroll
+                for (int s2 = 0; s2 < 32; s2++) {
+                    const int k = 32 * h + s2;     // differs between the lane halves: it travels in the lanes' offset
+                    const int off = (col < cols_left && k < k_a) ? (k * p.lda + col) * 4 : OOB_OFFSET;
+                    a[i][s2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra, off, 0, 0));
+                }
+            }
+        }
+    };
+    auto issue_b = [&](auto pc, const v4u& rb) __attribute__((always_inline)) {
+        constexpr int P = decltype(pc)::value;
+        const int left = p.b_inner - n * BN;
+        static_for<PB>([&](auto ic) {
+            constexpr int s2 = decltype(ic)::value;
+            dma_f4_lean<P * B_BYTES + s2 * NT * 16>(rb, lds_wave_b, (B_KIN || lb.first < left) ? lb.off[s2] : OOB_OFFSET);
+        });
+    };
+
+    v16f acc[TM][TN];
+
+    // ---- prologue ----
+    decode_unit(u);
+    load_a();
+    issue_b(std::integral_constant<int, 0>{}, b_descriptor(true));
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    static_for<GR>([&](auto gc) { read_group(gc, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
+    bool has_next = true;
+    // the block on its way out: the descriptor of its tile (no rows before the first tile: every store is dropped)
+    __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.C, 0, 0, RSRC_FLAGS);
+    int out_off[TN] = {OOB_OFFSET, OOB_OFFSET};
+
+    // 16 stores of block (I, J), one behind every second MFMA of the block that follows it
+    auto store_e = [&](auto ic, auto jc, auto ec) __attribute__((always_inline)) {
+        constexpr int I = decltype(ic)::value, J = decltype(jc)::value, e = decltype(ec)::value;
+        const float value = acc[I][J][e];
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), out_rsrc, out_off[J],
+                                              (32 * I + 8 * (e / 4) + e % 4) * ldc4, BD_STORE_AUX);
+    };
+    // One block: 32 dependent MFMAs into acc[I][J] from a[I] and fb, with the stores of block (SI, SJ) between them
+    // and, where NEXT_J >= 0, fb's next contents read group by group as the values there have had their last use
+    // (block NEXT_J of B buffer NEXT_P).
+    auto block = [&](auto ic, auto jc, auto sic, auto sjc, auto njc, auto npc) __attribute__((always_inline)) {
+        constexpr int I = decltype(ic)::value, J = decltype(jc)::value, SI = decltype(sic)::value, SJ = decltype(sjc)::value;
+        constexpr int NEXT_J = decltype(njc)::value;
+        static_for<32>([&](auto sc) {
+            constexpr int s2 = decltype(sc)::value;
+            if constexpr (s2 == 0)
+                acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[I][s2], fb[s2], (v16f)(0.0f), 0, 0, 0);
+            else
+                acc[I][J] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[I][s2], fb[s2], acc[I][J], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (s2 % 2 == 1) store_e(sic, sjc, std::integral_constant<int, s2 / 2>{});
+            if constexpr (NEXT_J >= 0 && s2 % 4 == 3)
+                read_group(std::integral_constant<int, s2 / 4>{}, std::integral_constant<int, (NEXT_J >= 0 ? NEXT_J : 0)>{}, npc);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using CN = std::integral_constant<int, -1>;
+
+    // One tile from B buffer P, block after block: (0,0) (1,0) (0,1) (1,1).
+    auto tile = [&](auto pc) __attribute__((always_inline)) {
+        constexpr int P = decltype(pc)::value;
+        float* const cur_c = p.C + (size_t)z * p.sC + (size_t)m * BM * p.ldc + (size_t)n * BN;
+        const int cur_rows = p.rows - m * BM, cur_cols = p.cols - n * BN;
+        // -- the tile after this one: its B goes to the other buffer now --
+        bool new_band = false;
+        if (++n == n_end) {
+            u += G;
+            if (u < U) {
+                decode_unit(u);
+                new_band = true;
+            } else {
+                has_next = false;
+                n = 0;
+            }
+        }
+        issue_b(std::integral_constant<int, P ^ 1>{}, b_descriptor(has_next));
+        __builtin_amdgcn_sched_barrier(0);
+
+        // block (0,0), with the last block of the tile before on its way out
+        block(C0{}, C0{}, C1{}, C1{}, CN{}, C0{});
+        // from here on the stores are this tile's: rows beyond C are cut off by the descriptor, columns by the offsets
+        {
+            const unsigned long long pc_at = (unsigned long long)cur_c;
+            const int rows_in = cur_rows > BM ? BM : cur_rows;
+            const unsigned out_lo = __builtin_amdgcn_readfirstlane((unsigned)pc_at), out_hi = __builtin_amdgcn_readfirstlane((unsigned)(pc_at >> 32));
+            out_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(((unsigned long long)out_hi << 32) | out_lo), 0,
+                                                         __builtin_amdgcn_readfirstlane(rows_in > 0 ? rows_in * ldc4 : 0), RSRC_FLAGS);
+#pragma unroll
+            for (int j = 0; j < TN; j++) out_off[j] = (c_col + j * 32 < cur_cols) ? c_lane + j * 128 : OOB_OFFSET;
+        }
+        // block (1,0): fb's values have their last use for column block 0; block 1's come in behind them
+        block(C1{}, C0{}, C0{}, C0{}, C1{}, pc);
+        block(C0{}, C1{}, C1{}, C0{}, CN{}, C0{});
+        // The next tile's B was requested before this tile's 48 stores so far, and vector-memory operations retire
+        // in issue order: with at most those outstanding it has landed.  The barrier makes every wavefront's part
+        // visible; everybody has read the last of this tile's B (block 1's values) before its block (0,1) ended.
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(48));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // block (1,1): the next tile's column block 0 comes in behind fb's last uses
+        block(C1{}, C1{}, C0{}, C1{}, C0{}, std::integral_constant<int, P ^ 1>{});
+        // the next band's A replaces this one's (every MFMA that read it has been issued)
+        if (new_band) {
+            load_a();
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    for (;;) {
+        tile(std::integral_constant<int, 0>{});
+        if (!has_next) break;
+        tile(std::integral_constant<int, 1>{});
+        if (!has_next) break;
+    }
+    // the last block of the last tile
+    static_for<16>([&](auto ec) { store_e(C1{}, C1{}, ec); });
+}
+
+template <bool A_KIN, bool B_KIN>
+static hipError_t launch_band_regs_cfg(GemmParams p, hipStream_t stream) {
+    if (p.split || p.bias != nullptr || p.k_total > BD_KT) return hipErrorOutOfMemory;   // the caller falls back
+    p.tiles_m = (p.rows + 127) / 128;
+    p.tiles_n = (p.cols + 127) / 128;
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return hipErrorNoDevice;
+    const long long bands = (long long)p.tiles_m * p.nz;
+    if (bands <= 0 || bands * p.tiles_n > 0x3fffffffLL) return hipErrorOutOfMemory;
+    gemm_band_split(bands, p.tiles_n, 2 * num_cu, p.bd_chunks, p.bd_chunk_tiles);    // two workgroups per unit
+    const long long units = bands * p.bd_chunks;
+    const long long grid = units < 2LL * num_cu ? units : 2LL * num_cu;
+    hipLaunchKernelGGL((gemm_f32_mfma_band_regs<A_KIN, B_KIN>), dim3((unsigned)grid), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
 template <bool A_KIN, bool B_KIN, int BD_BM, int BD_BN>
 static hipError_t launch_band_cfg(GemmParams p, hipStream_t stream) {
     if (p.split || p.bias != nullptr || p.k_total > BD_KT) return hipErrorOutOfMemory;   // the caller falls back
@@ -437,7 +675,15 @@ int gemm_choose_band(int rows, int cols, int nz, int k, int num_cu, int variant)
     return TILE_BAND_128x128;
 }
 
-hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream, bool wide) {
+hipError_t gemm_launch_band(int variant, const GemmParams& p, hipStream_t stream, bool wide, bool regs) {
+    if (regs) {
+        switch (variant) {
+            case GEMM_NN: return launch_band_regs_cfg<true, false>(p, stream);
+            case GEMM_T1: return launch_band_regs_cfg<false, false>(p, stream);
+            case GEMM_T2: return launch_band_regs_cfg<true, true>(p, stream);
+            default: return hipErrorInvalidValue;
+        }
+    }
     if (wide) {
         switch (variant) {
             case GEMM_NN: return launch_band_cfg<true, false, 64, 256>(p, stream);

@@ -74,7 +74,7 @@ template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny(const SkinnyParams p) {
     static_assert(T == 4 || T == 8 || T == 12 || T == 16, "4, 8, 12 or 16 short lines");
-    static_assert(X_KIN ? (W == 2 || W == 4 || W == 8) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || ((CL == 2 || CL == 4) && W == 1)), "forms");
+    static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || ((CL == 2 || CL == 4) && W == 1)), "forms");
     constexpr int LS = 8, PK = 32;                         // K-inner X: lines per read, k per panel
     constexpr int H = T / 4;                               // groups of 4 short lines
     constexpr int LINES = X_KIN ? LS * W : 64 * W / CL;    // lines of X per wavefront
@@ -175,7 +175,7 @@ void gemm_f32_skinny(const SkinnyParams p) {
         } else {
             // ---- per instruction 8 lines x 8 classes of k: X[line0 + 8 * set + (lane & 7)][k0 + 4 * (lane >> 3) + 0 .. 3];
             //      U 32-k panels per register buffer ----
-            constexpr int U = ((NW == 16 && H > 2) || W == 8) ? 1 : (NW == 16 || W == 4) ? 2 : 4;
+            constexpr int U = (NW == 16 && H > 2) ? 1 : (NW == 16 || W == 4) ? 2 : 4;
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, (long long)p.x_lines * p.ldx * 4);
             const int kk4 = 4 * (lane / LS);
             int x_off[W];
@@ -402,8 +402,6 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
         case 2: return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
         case 3: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, false, stream);
         case 4: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, true, stream);
-        case 8: if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, 8, 4>(p, false, stream); else return hipErrorInvalidValue;
-        case 9: if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, 8, 4>(p, true, stream); else return hipErrorInvalidValue;
         case 6:
             if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
             else return launch_one<X_KIN, S_KIN, T, 1, 16, 4>(p, true, stream);
@@ -439,7 +437,7 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
 void gemm_skinny_form(int form) {
     t_skinny_cuts = form >= 100 ? form % 100 : 0;
     if (form >= 100) form = 7;
-    t_skinny_form = (form >= 0 && form <= 9) ? form : -1;
+    t_skinny_form = (form >= 0 && form <= 7) ? form : -1;
 }
 
 // 4, 8, 12 or 16 stored lines on the short side

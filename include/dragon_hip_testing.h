@@ -32,7 +32,9 @@ extern "C" {
  * another K falls back to the automatic choice).  27: the skinny kernel for a 2-D product whose C has 4, 8, 12 or 16
  * columns under at least 256 rows, or as many rows over at least 256 columns (wavefronts stream the long operand into 4x4x1
  * MFMA blocks; what the automatic choice takes there; another shape falls back to the automatic choice).  28: the band
- * kernel with bands of 64 rows under tiles of 256 columns (never chosen automatically: measured level with 24). */
+ * kernel with bands of 64 rows under tiles of 256 columns, 29: the band kernel with the band's rows of A in registers
+ * (four wavefronts, two workgroups per compute unit, a tile multiplied block after block); neither is chosen
+ * automatically: both measure level with 24. */
 void dragon_gemm_force_tile(int32_t tile);
 /* Force a form of the skinny kernel for the following launches OF THE CALLING THREAD: 0 = a wavefront per run of
  * lines of the long operand (64 lines where k is its row index, 16 where k is contiguous) with the whole K, 1 = the

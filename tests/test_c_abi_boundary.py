@@ -240,7 +240,7 @@ def test_tile_choice_stays_inside_what_the_kernels_accept(dh):
     # that fits its one stage, and every id is one that exists
     rng = np.random.default_rng(20240607)
     dims = {18: (64, 64), 19: (128, 64), 20: (64, 128), 21: (128, 128), 22: (64, 64), 23: (128, 64), 25: (256, 64)}
-    valid = set(range(0, 29)) | set(range(256, 266))
+    valid = set(range(0, 30)) | set(range(256, 266))
     dh.force_tile(-1)
     seen = set()
     for _ in range(20000):

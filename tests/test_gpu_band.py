@@ -14,7 +14,8 @@ from test_gpu_batched import make_case, run
 pytestmark = pytest.mark.gpu
 BAND = 24           # bands of 128 rows, tiles of 128 columns
 BAND_WIDE = 28      # bands of 64 rows, tiles of 256 columns
-BANDS = [BAND, BAND_WIDE]
+BAND_REGS = 29      # the band's rows of A in registers: four wavefronts, two workgroups per compute unit
+BANDS = [BAND, BAND_WIDE, BAND_REGS]
 
 
 @pytest.fixture(autouse=True)

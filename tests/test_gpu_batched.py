@@ -58,7 +58,7 @@ SHAPES = [(1, 1, 1, 1), (3, 5, 6, 7), (5, 24, 21, 8), (15, 82, 96, 9), (4, 128, 
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("tile", list(range(-1, 29)) + list(range(256, 266)))
+@pytest.mark.parametrize("tile", list(range(-1, 30)) + list(range(256, 266)))
 def test_batched_integer_inputs_bitwise(gpu, variant, tile):
     rng = np.random.default_rng(900 + variant * 10 + tile)
     gpu.force_tile(tile)
