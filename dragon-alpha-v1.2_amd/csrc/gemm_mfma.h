@@ -120,6 +120,9 @@ struct GemmParams {
     // few tiles under a very long K, dealt in whole runs per tile: sk_kmajor_rpt runs per tile (0: off) of
     // sk_kmajor_tiles tiles; the workgroups that share an XCD then take the same k ranges of different tiles
     int sk_kmajor_rpt, sk_kmajor_tiles;
+    // a launch of the balanced kernel over the tiles sk_tile_base ... sk_tile_base + sk_tile_count - 1 only
+    // (sk_tile_count 0: all of them): see gemm_launch_streamk
+    int sk_tile_base, sk_tile_count;
     // K slices: the tiles from number sk_T1 on (the last slice's) have sk_S_last stages
     int sk_S_last, sk_T1;
     unsigned sk_div_Sl_mul, sk_div_Sl_shift;

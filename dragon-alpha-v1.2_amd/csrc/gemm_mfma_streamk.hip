@@ -268,7 +268,7 @@ void gemm_f32_mfma_streamk(const GemmParams p) {
         return div_by(u, p.sk_div_S_mul, p.sk_div_S_shift);
     };
     auto decode = [&](int tile) __attribute__((always_inline)) -> TileCtx {
-        TileCtx c = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, tile);
+        TileCtx c = decode_tile<A_KIN, B_KIN, BM, BN, KT, LoadA, LoadB>(p, tile + p.sk_tile_base);
         if constexpr (SPLIT) {   // K limits relative to the slice's first k, like the stage index
             c.ka_lim -= c.k0;
             c.kb_lim -= c.k0;
@@ -572,7 +572,9 @@ static hipError_t launch_streamk_cfg(GemmParams p, hipStream_t stream, float* ws
     if (p.bias != nullptr && (!CAN_BIAS || p.split)) return hipErrorOutOfMemory;   // no balanced form: the caller falls back
     p.tiles_m = (p.rows + BM - 1) / BM;
     p.tiles_n = (p.cols + BN - 1) / BN;
-    const long long tiles = (long long)p.tiles_m * p.tiles_n * p.nz;
+    const long long all_tiles = (long long)p.tiles_m * p.tiles_n * p.nz;
+    if (p.sk_tile_count > 0 && (p.split || CONV || p.zero_floats > 0 || p.sk_tile_base + (long long)p.sk_tile_count > all_tiles)) return hipErrorInvalidValue;
+    const long long tiles = p.sk_tile_count > 0 ? p.sk_tile_count : all_tiles;
     // K slices: every slice but the last is k_slice long, the last takes the rest of K
     const long long k_first = p.split ? p.k_slice : p.k_total;
     const long long k_last = p.split ? (long long)p.k_total - (long long)(p.nz - 1) * p.k_slice : p.k_total;
@@ -934,16 +936,51 @@ hipError_t gemm_launch_streamk_conv(const GemmParams& p0, int tile, hipStream_t 
     }
 }
 
-hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream) {
-    size_t floats = p.sk_ws_given_floats;
-    float* ws = p.sk_ws_given != nullptr ? p.sk_ws_given : gemm_streamk_workspace(stream, &floats);
-    if (ws == nullptr) return hipErrorOutOfMemory;
+static hipError_t launch_streamk_any(int variant, const GemmParams& p, int tile, hipStream_t stream, float* ws, size_t floats) {
     switch (variant) {
         case GEMM_NN: return launch_streamk_variant<true, false>(p, tile, stream, ws, floats);
         case GEMM_T1: return launch_streamk_variant<false, false>(p, tile, stream, ws, floats);
         case GEMM_T2: return launch_streamk_variant<true, true>(p, tile, stream, ws, floats);
         default: return hipErrorInvalidValue;
     }
+}
+
+// Many 128 x 128 tiles that do not divide among the workgroups (3072^3: 576 tiles for 256; 5120^3: 1600): dealt in
+// equal runs, every workgroup starts inside a tile at a k of its own, neighbours on an XCD no longer read the same
+// operand panels at the same time, and the L2 serves next to nothing (measured: 2 % and 1.3 % hits against 71 % at
+// 4096^3, 24 x and 40 x the operands' bytes fetched through the fabric).  Such a product goes out as TWO launches:
+// the largest multiple of the workgroup count as whole tiles (every workgroup the same number, in step, the band
+// order's sharing intact), then the remaining tiles -- fewer than workgroups -- shared out in runs of stages, where
+// the k ranges of all tiles sit together on an XCD (sk_kmajor_rpt) whenever the counts divide.
+static bool streamk_two_launches(const GemmParams& p, int tile, long long& first_count, long long& all_tiles) {
+    if (tile != TILE_SK_128x128 || p.split || p.zero_floats > 0 || p.sk_tile_count > 0) return false;
+    const int num_cu = gemm_device_num_cu();
+    if (num_cu <= 0) return false;
+    all_tiles = (long long)((p.rows + 127) / 128) * ((p.cols + 127) / 128) * p.nz;
+    first_count = all_tiles / num_cu * num_cu;
+    const long long rest = all_tiles - first_count;
+    // Worth a second launch from two whole tiles per workgroup on (with one it measured -2 ... +2 %) and a K of at
+    // least 3072: 3072^3 414 -> 402 us, 5120^3 1871 -> 1800, 4096 x 11008 x 4096 2588 -> 2481; with K = 1024 ... 2048
+    // (3072^2, 5120^2, 3584^2 x 1536, 2000 x 5000 x 1100) the launches' ends cost what the L2 gives back, -3 ... +1 %.
+    return first_count >= 2LL * num_cu && rest > 0 && p.k_total >= 3072;
+}
+
+hipError_t gemm_launch_streamk(int variant, const GemmParams& p, int tile, hipStream_t stream) {
+    size_t floats = p.sk_ws_given_floats;
+    float* ws = p.sk_ws_given != nullptr ? p.sk_ws_given : gemm_streamk_workspace(stream, &floats);
+    if (ws == nullptr) return hipErrorOutOfMemory;
+    long long first_count = 0, all_tiles = 0;
+    if (streamk_two_launches(p, tile, first_count, all_tiles)) {
+        GemmParams q = p;
+        q.sk_tile_base = 0;
+        q.sk_tile_count = (int)first_count;
+        const hipError_t e = launch_streamk_any(variant, q, tile, stream, ws, floats);
+        if (e != hipSuccess) return e;
+        q.sk_tile_base = (int)first_count;
+        q.sk_tile_count = (int)(all_tiles - first_count);
+        return launch_streamk_any(variant, q, tile, stream, ws, floats);
+    }
+    return launch_streamk_any(variant, p, tile, stream, ws, floats);
 }
 
 }  // namespace dragon

@@ -157,6 +157,20 @@ def test_fused_bias_equals_two_launches_bitwise(dh, gpu, tile):
         assert np.abs(C1[:N, :M] - Rb[:, :M]).max() <= 1e-4 * np.sqrt(K) + 1e-6
 
 
+def test_fused_bias_through_two_launches_of_the_balanced_kernel(dh, gpu):
+    """640 tiles of 128 x 128 for 256 compute units: whole tiles first, the remaining 128 in a second launch; the
+    bias row is added once, by whoever stores a tile, in both."""
+    rng = np.random.default_rng(77)
+    N, M, K = 2000, 5000, 3100
+    A = rng.integers(-3, 4, (N, K)).astype(np.float32)
+    B = rng.integers(-3, 4, (K, M)).astype(np.float32)
+    bias = rng.integers(-5, 6, M).astype(np.float32)
+    C1, C2 = _biased_both_ways(dh, A, B, bias, -1)
+    assert np.array_equal(C1.view(np.uint32), C2.view(np.uint32))
+    assert np.array_equal(C1[:N, :M], oracle.matmul_f64(0, A, B).astype(np.float32) + bias[None, :])
+    assert not C1[N:].any() and not C1[:, M:].any()
+
+
 def test_fused_bias_large_and_negative_zero(dh, gpu):
     rng = np.random.default_rng(3)
     N, M, K = 1000, 780, 256

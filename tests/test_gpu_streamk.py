@@ -267,3 +267,20 @@ def test_batched_products_through_the_balanced_kernel(gpu):
         assert np.array_equal(dC.get((B4, N, M4)), R), BALANCED[tile]
         for x in (dA, dB, dC):
             x.free()
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
+def test_tiles_that_do_not_divide_among_the_workgroups_go_out_as_two_launches(gpu, variant):
+    """Many 128 x 128 tiles, not a multiple of the compute units, K >= 3072: whole tiles first (every workgroup the
+    same number), then the remaining tiles shared out in runs of stages -- two launches on the caller's stream.
+    Every bit against the exact product (small integers), ragged rows and columns, and twice in a row (the
+    second launch's arrival counters are back at zero)."""
+    rng = np.random.default_rng(640 + variant)
+    for (N, M, K) in ((3072, 3072, 3072), (2000, 5000, 3100), (3300, 2900, 3076)):
+        assert gpu.choose_tile(variant, N, (M + 3) // 4 * 4, 1, (K + 3) // 4 * 4) == 21
+        A, B = logical_operands(variant, rng, N, M, K, dist="int")
+        R = oracle.matmul_f64(variant, A, B).astype(np.float32)
+        for _ in range(2):
+            C, Cp = gpu_matmul_2d(gpu, variant, A, B, fill=3.0)
+            assert np.array_equal(C, R), "%s %s" % (VARIANT_NAMES[variant], (N, M, K))
+            assert np.count_nonzero(Cp[N:, :]) == 0 and np.count_nonzero(Cp[:, M:]) == 0
