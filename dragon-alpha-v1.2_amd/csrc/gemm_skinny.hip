@@ -45,6 +45,7 @@ struct SkinnyParams {
 
 typedef float sk_v4f __attribute__((ext_vector_type(4)));
 constexpr int SKINNY_MAX_CUTS = 8;    // workgroups that cut one run's K
+constexpr int SKINNY_STAGED_FLOATS = 12288;   // of a K-inner short operand in LDS (48 KiB)
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t skinny_rsrc(const float* base, long long bytes) {
     const long long capped = bytes > 0xfffffff0LL ? 0xfffffff0LL : (bytes < 0 ? 0 : bytes);
@@ -70,9 +71,12 @@ __device__ __forceinline__ void skinny_put(const SkinnyParams& p, int line, int 
 // W: floats of a K-outer X a lane reads per k row (1 or 4), or sets of 8 lines of a K-inner X per wavefront (2 or 4).
 // CL: classes of k among the lanes of a K-outer X with W = 1 (2: lanes 0-31 take the even k rows of 32 lines, lanes
 // 32-63 the odd ones).  NW: wavefronts of a workgroup.
-template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
+// SL: the workgroup's part of a K-inner S (T lines x its k range, at most 48 KiB) is staged in LDS once and read from
+// there: the short operand's lines are K floats apart -- with K a power of two, lines of the L1 that fall into one set.
+template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1, bool SL = false>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny(const SkinnyParams p) {
+    static_assert(!SL || (!X_KIN && S_KIN && W == 1 && NW == 4 && CL == 1), "the staged form");
     static_assert(T == 4 || T == 8 || T == 12 || T == 16, "4, 8, 12 or 16 short lines");
     static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || ((CL == 2 || CL == 4) && W == 1)), "forms");
     constexpr int LS = 8, PK = 32;                         // K-inner X: lines per read, k per panel
@@ -81,6 +85,9 @@ void gemm_f32_skinny(const SkinnyParams p) {
     constexpr int ACCS = W * H;                            // 4 x 4 accumulator blocks per lane
     constexpr int MEET_LANES = X_KIN ? LS : 64 / CL;       // lanes that hold outputs once the classes of k have met
     __shared__ float meet_lds[NW][ACCS * 4][MEET_LANES];
+    constexpr int SL_KMAX = SL ? SKINNY_STAGED_FLOATS / T : 4;     // k per short line in LDS; 4 zeros behind each line
+    constexpr int SL_KS = SL_KMAX + 4;
+    __shared__ __attribute__((aligned(16))) float s_lds[SL ? T * SL_KS + 64 : 4];
 
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const bool shared = p.k_share > 0;
@@ -99,6 +106,20 @@ void gemm_f32_skinny(const SkinnyParams p) {
 #pragma unroll
     for (int a = 0; a < ACCS; a++) d[a] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
+    // the workgroup's k range of S, line after line (the launcher made sure that it fits)
+    const int k_wg0 = (shared && p.k_cuts > 1) ? cut * p.k_cut : 0;
+    if constexpr (SL) {
+        const int k_len = min(p.K, (shared && p.k_cuts > 1) ? k_wg0 + p.k_cut : p.K) - k_wg0;
+        const int chunks = k_len >> 2;
+        for (int idx = t; idx < T * chunks; idx += NW * 64) {
+            const int jj = idx / chunks, c = idx - jj * chunks;
+            const sk_v4f v = ld4(rs, jj < p.s_lines ? (jj * p.lds + k_wg0 + 4 * c) * 4 : OOB_OFFSET, 0);
+            *(sk_v4f*)&s_lds[jj * SL_KS + 4 * c] = v;
+        }
+        if (t < T) *(sk_v4f*)&s_lds[t * SL_KS + SL_KMAX] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        __syncthreads();
+    }
+
     if (line0 < p.L && k_begin < k_end) {
         if constexpr (!X_KIN) {
             // ---- a lane owns W lines: X[k][line0 + W * lane + c] (CL = 2: X[k + class][line0 + (lane & 31)]);
@@ -114,6 +135,9 @@ void gemm_f32_skinny(const SkinnyParams p) {
 #pragma unroll
             for (int h = 0; h < H; h++)
                 s_off[h] = (4 * h + j < p.s_lines) ? (S_KIN ? (4 * h + j) * p.lds * 4 : (4 * h + j) * 4) + cls * s_step : OOB_OFFSET;
+            int sl_base[H];      // staged S: the lane's line, as an index that k - k_wg0 is added to
+#pragma unroll
+            for (int h = 0; h < H; h++) sl_base[h] = (4 * h + j) * SL_KS;
             struct Buf { XVal<W> x[U]; float s[H][U]; };
             // k rows at or beyond k_end are not this wavefront's (another share's, or beyond K): zeros instead.  K and
             // the shares are even, so the two classes of a load stand or fall together.
@@ -126,7 +150,13 @@ void gemm_f32_skinny(const SkinnyParams p) {
                 }
 #pragma unroll
                 for (int h = 0; h < H; h++) {
-                    if constexpr (S_KIN && CL == 1) {
+                    if constexpr (SL) {
+#pragma unroll
+                        for (int u = 0; u < U; u += 4) {     // beyond k_end: the zeros behind the line
+                            const sk_v4f v = *(const sk_v4f*)&s_lds[sl_base[h] + ((k + u < k_end) ? k + u - k_wg0 : SL_KMAX)];
+                            b.s[h][u] = v.x; b.s[h][u + 1] = v.y; b.s[h][u + 2] = v.z; b.s[h][u + 3] = v.w;
+                        }
+                    } else if constexpr (S_KIN && CL == 1) {
 #pragma unroll
                         for (int u = 0; u < U; u += 4) {
                             const sk_v4f v = ld4(rs, (k + u < k_end) ? s_off[h] : OOB_OFFSET, (k + u) * 4);
@@ -366,6 +396,13 @@ hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream, int cuts 
         }
     }
     if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    if constexpr (!X_KIN && S_KIN && W == 1 && NW == 4 && CL == 1) {
+        // the wavefronts share their lines and the workgroup's part of S is small enough: S from LDS
+        if (shared && (p.k_cuts > 1 ? p.k_cut : p.K) <= SKINNY_STAGED_FLOATS / T) {
+            hipLaunchKernelGGL((gemm_f32_skinny<X_KIN, S_KIN, T, W, NW, CL, true>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+            return hipGetLastError();
+        }
+    }
     hipLaunchKernelGGL((gemm_f32_skinny<X_KIN, S_KIN, T, W, NW, CL>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
@@ -390,6 +427,10 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
         if (p.K < 128) form = wide >= 4LL * num_cu ? 3 : 0;
         else if (wide >= 4LL * num_cu) form = X_KIN ? 4 : 3;
         else if (wide >= num_cu) form = 4;
+        // (8 or more lines of a K-inner S beside a K-outer X: K cut so that a workgroup's part of S fits the LDS,
+        // 8 x 16384 x 2048 35.8 -> 28.9 us; with 4 lines the cut costs more than the staging gives, 43.6 -> 47.2)
+        else if (!X_KIN && S_KIN && T >= 8 && p.K >= 512 && narrow < 4LL * num_cu && p.K > SKINNY_STAGED_FLOATS / T &&
+                 (p.K + SKINNY_STAGED_FLOATS / T - 1) / (SKINNY_STAGED_FLOATS / T) <= SKINNY_MAX_CUTS) form = 7;
         else if (narrow >= num_cu || p.K < 512) form = 1;
         // fewer narrow runs than compute units: K is cut across workgroups as well -- except for 128 ... 255 runs of
         // a K-outer X beside a K-outer S, where sixteen wavefronts on 32-line runs measured 10 % ahead
@@ -407,7 +448,13 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
             else return launch_one<X_KIN, S_KIN, T, 1, 16, 4>(p, true, stream);
         case 7: {   // two workgroups per compute unit
             const long long narrow = ((long long)p.L + (X_KIN ? 15 : 63)) / (X_KIN ? 16 : 64);
-            return launch_one<X_KIN, S_KIN, T, W0, 4>(p, true, stream, (int)((t_skinny_cuts > 0 ? t_skinny_cuts : (2LL * num_cu + narrow - 1) / narrow)));
+            long long cuts = t_skinny_cuts > 0 ? t_skinny_cuts : narrow < 2LL * num_cu ? (2LL * num_cu + narrow - 1) / narrow : 1;
+            // a K-inner S beside a K-outer X is staged in LDS where a cut's part of it fits: enough cuts for that
+            if (!X_KIN && S_KIN && t_skinny_cuts == 0) {
+                const long long fit = ((long long)p.K + SKINNY_STAGED_FLOATS / T - 1) / (SKINNY_STAGED_FLOATS / T);
+                if (fit > cuts && fit <= SKINNY_MAX_CUTS) cuts = fit;
+            }
+            return launch_one<X_KIN, S_KIN, T, W0, 4>(p, true, stream, (int)cuts);
         }
         default:
             if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
