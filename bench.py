@@ -448,7 +448,27 @@ def main():
                     record(key, 2.0 * r * c * k, ms, nbytes)
                     per_config[key]["pct_hbm_peak"] = round(100.0 * per_config[key]["alg_GBps"] / 8000.0, 1)
                     per_config[key]["bound"] = "hbm" if 4.0 * max(r, c) * k > 300e6 else "hbm (operand near the Infinity Cache's 256 MB)"
-        for x in (dL, dS, dC):
+        # the shapes with few lines are the ones the unchanged host policy splits (8 x 4096 x 4096: GridZ 16): what
+        # the engine's call sequence takes with the split declined by the library (default) and with it honoured
+        dCb = dh.DeviceArray(size=32 * 8 * 8192)
+        for (r, c, k) in ((8, 4096, 4096), (8, 8192, 4096), (8192, 8, 4096)):
+            da, db = (dL, dS) if r > c else (dS, dL)
+            nbytes = 4.0 * (r * k + k * c + r * c)
+            GZs = host_policy.gridZ(host_policy.MATMUL, r, c, k, SM)
+            if GZs < 2:
+                continue
+
+            def sk_call():
+                MM.matMulSK(S, 1, GZs, da.address, db.address, dC.address, dCb.address, r, c, k)
+                MM.SKbuf_summary(stream, dCb.address, dC.address, GZs - 1, r * c)
+            for mode, label in ((-1, "split declined: the skinny kernel, fold elided"), (0, "split honoured: %d slices + fold" % GZs)):
+                dh.split_policy(mode)
+                ms = timer.per_launch_ms(sk_call, iters=10)
+                dh.split_policy(-1)
+                key = "A*B %dx%dx%d as the host policy calls it (GridZ %d), %s" % (r, c, k, GZs, label)
+                record(key, 2.0 * r * c * k, ms, nbytes)
+                per_config[key]["pct_hbm_peak"] = round(100.0 * per_config[key]["alg_GBps"] / 8000.0, 1)
+        for x in (dL, dS, dC, dCb):
             x.free()
 
     if "bias" in extra:

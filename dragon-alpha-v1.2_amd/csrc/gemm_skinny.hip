@@ -41,6 +41,9 @@ struct SkinnyParams {
     int k_cuts, k_cut, units;
     float* ws;
     int* count;
+    // a split-K call whose split was declined: zero_floats floats (a multiple of 4) of the caller's partial buffers get zeros
+    float* zero_buf;
+    long long zero_floats;
 };
 
 typedef float sk_v4f __attribute__((ext_vector_type(4)));
@@ -106,6 +109,11 @@ void gemm_f32_skinny(const SkinnyParams p) {
 #pragma unroll
     for (int a = 0; a < ACCS; a++) d[a] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
+    if (p.zero_floats > 0) {
+        sk_v4f* const z = (sk_v4f*)p.zero_buf;
+        const long long n4 = p.zero_floats >> 2, step = (long long)gridDim.x * (NW * 64);
+        for (long long i = (long long)blockIdx.x * (NW * 64) + t; i < n4; i += step) z[i] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    }
     // the workgroup's k range of S, line after line (the launcher made sure that it fits)
     const int k_wg0 = (shared && p.k_cuts > 1) ? cut * p.k_cut : 0;
     if constexpr (SL) {
@@ -526,6 +534,7 @@ hipError_t gemm_launch_skinny(int variant, const GemmParams& g, hipStream_t stre
     const bool thin_cols = skinny_short(g.cols) && g.rows >= 256;
     SkinnyParams p = {};
     p.C = g.C; p.ldc = g.ldc;
+    p.zero_buf = g.zero_buf; p.zero_floats = g.zero_floats;
     p.K = min(g.k_total, min(a_kin ? g.a_inner : g.a_outer, b_kin ? g.b_inner : g.b_outer));
     if (p.K <= 0) return hipErrorInvalidValue;
     if (thin_cols) {          // X = A (lines = rows of C), S = B (lines = columns of C)

@@ -184,6 +184,40 @@ def test_a_losing_split_is_declined(gpu, variant, shape_gz):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("shape_gz", [((8, 4096, 4096), 16), ((4100, 8, 2052), 8), ((8, 1000, 1028), 4), ((3000, 4, 516), 3)])
+def test_the_split_of_a_skinny_product_is_declined(gpu, variant, shape_gz):
+    """The host's policy splits the skinny products with few lines (8 x 4096 x 4096: GridZ 16).  The skinny kernel
+    cuts K among its workgroups itself: the whole product goes to C through it -- the bits of the unsplit entry
+    point --, the partial buffers get exact zeros from the same launch, the fold leaves C as it is; with the
+    slices forced the same product comes out of C plus the partials."""
+    (N, M, K), GZ = shape_gz
+    gpu.split_policy(-1)
+    rng = np.random.default_rng(N + M + GZ + variant)
+    for dist in ("int", "uniform"):
+        A, B = logical_operands(variant, rng, N, M, K, dist=dist)
+        before = gpu.declined_splits()
+        C, Cbuf = run_sk(gpu, variant, A, B, GZ, summary=False)
+        assert gpu.declined_splits() == before + 1
+        assert not Cbuf.view(np.uint32).any(), "the partial buffers of a declined split hold exact zeros"
+        unsplit, _ = gpu_matmul_2d(gpu, variant, A, B)
+        assert np.array_equal(C.view(np.uint32), unsplit.view(np.uint32))
+        skipped = gpu.folds_skipped()
+        folded, _ = run_sk(gpu, variant, A, B, GZ, summary=True)
+        assert gpu.folds_skipped() == skipped + 1
+        assert np.array_equal(folded.view(np.uint32), C.view(np.uint32))
+        R = oracle.matmul(variant, A, B)
+        if dist == "int":
+            assert np.array_equal(C, R)
+        else:
+            assert_within_tolerance(C, R, K, A, B, "%s skinny declined GZ=%d" % (VARIANT_NAMES[variant], GZ))
+        gpu.split_policy(0)
+        C0, Cb0 = run_sk(gpu, variant, A, B, GZ, summary=False)
+        gpu.split_policy(-1)
+        total = C0.astype(np.float64) + Cb0.astype(np.float64).sum(axis=0)
+        assert_within_tolerance(total, R, K, A, B, "%s skinny honoured GZ=%d" % (VARIANT_NAMES[variant], GZ))
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
 def test_a_winning_split_is_honoured(gpu, variant):
     """256 x 256 x 8192 in 32 slices: 512 (slice, tile) pairs deal whole to the units, the unsplit product has
     sixteen workgroups per tile to put together -- the slices stay, bit for bit where the oracle puts them."""
