@@ -105,6 +105,25 @@ def test_split_k_through_the_engine_frees_its_buffer(eg):
     eg.delete(tA, tB, tC)
 
 
+def test_a_skinny_product_through_the_engine(eg, gpu):
+    """Engine.matMul of 8 rows by a 2048 x 4096 matrix: the unchanged policy splits it (GridZ >= 2), the library
+    declines the split and runs the skinny kernel; the engine's sequence (stage 1, fold, syncer, buffer release)
+    is the same and the result is the exact product."""
+    rng = np.random.default_rng(12)
+    N, K, M = 8, 2048, 4096
+    A = rng.integers(-3, 4, (N, K)).astype(np.float32)
+    B = rng.integers(-3, 4, (K, M)).astype(np.float32)
+    tA, tB = eg.tensor(A, N, K), eg.tensor(B, K, M)
+    base = eg.get_param("live_blocks")
+    before = gpu.declined_splits()
+    tC = eg.matMul(tA, tB)
+    assert eg.get_param("last_gridZ") >= 2
+    assert gpu.declined_splits() == before + 1
+    assert np.array_equal(eg.valueOf(tC).reshape(N, M), oracle.matmul_f64(0, A, B).astype(np.float32))
+    assert eg.get_param("live_blocks") == base + 1          # the partial buffer went back
+    eg.delete(tA, tB, tC)
+
+
 def test_events_are_recycled(eg):
     """The syncers' events (CudaFloat32EngineBase.java:657-694, 1008-1054 create and destroy one per call) come
     from a pool and go back to it: after many calls, split and unsplit, in both modes, the pool holds a few idle
