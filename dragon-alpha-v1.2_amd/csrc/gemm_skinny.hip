@@ -44,6 +44,9 @@ struct SkinnyParams {
     // a split-K call whose split was declined: zero_floats floats (a multiple of 4) of the caller's partial buffers get zeros
     float* zero_buf;
     long long zero_floats;
+    // optional row vector added to C[i][j] for i < bias_rows, j < bias_width (the forward product's bias)
+    const float* bias;
+    int bias_rows, bias_width;
 };
 
 typedef float sk_v4f __attribute__((ext_vector_type(4)));
@@ -66,8 +69,10 @@ template <> struct XVal<4> { sk_v4f v; __device__ __forceinline__ float at(int c
 
 __device__ __forceinline__ void skinny_put(const SkinnyParams& p, int line, int col, float value) {
     if (line < p.L) {
-        if (p.out_rows) p.C[(size_t)col * p.ldc + line] = value;
-        else p.C[(size_t)line * p.ldc + col] = value;
+        const int ci = p.out_rows ? col : line, cj = p.out_rows ? line : col;      // row and column of C
+        // the bias row as the tile kernels' epilogue adds it: "+ 0.0f" is the gamma term of the separate launch
+        if (p.bias != nullptr && ci < p.bias_rows) value = (value + (cj < p.bias_width ? p.bias[cj] : 0.0f)) + 0.0f;
+        p.C[(size_t)ci * p.ldc + cj] = value;
     }
 }
 
@@ -512,13 +517,13 @@ int gemm_choose_skinny(int rows, int cols, int nz, int variant, int num_cu) {
     return x_kouter && (long long)(thin_cols ? rows : cols) >= 256LL * num_cu ? TILE_SKINNY : -1;
 }
 
-// True where the product is one for the skinny kernel: one unsplit 2-D product without a bias row whose C has
+// True where the product is one for the skinny kernel: one unsplit 2-D product (a bias row on A*B only) whose C has
 // 4 ... 16 stored columns under at least 256 rows, or 4 ... 16 stored rows over at least 256 columns, and whose
 // operands' byte offsets (with the reads a register buffer runs ahead, and the lines of a last, partly filled
 // run) fit 32 bits.
 static bool gemm_skinny_applies(int variant, const GemmParams& p) {
     // (a forced choice takes every shape the kernel can run: up to 16 short lines in every layout)
-    if (p.split || p.bias != nullptr || gemm_choose_skinny(p.rows, p.cols, p.nz, GEMM_T1, 1) < 0) return false;
+    if (p.split || (p.bias != nullptr && variant != GEMM_NN) || gemm_choose_skinny(p.rows, p.cols, p.nz, GEMM_T1, 1) < 0) return false;
     const bool thin_cols = skinny_short(p.cols) && p.rows >= 256;
     const bool a_kin = variant != GEMM_T1, b_kin = variant == GEMM_T2;
     // a K-inner operand is addressed line * ld + k, a K-outer one k * ld + line
@@ -535,6 +540,7 @@ hipError_t gemm_launch_skinny(int variant, const GemmParams& g, hipStream_t stre
     SkinnyParams p = {};
     p.C = g.C; p.ldc = g.ldc;
     p.zero_buf = g.zero_buf; p.zero_floats = g.zero_floats;
+    p.bias = g.bias; p.bias_rows = g.bias_rows; p.bias_width = g.bias_width;
     p.K = min(g.k_total, min(a_kin ? g.a_inner : g.a_outer, b_kin ? g.b_inner : g.b_outer));
     if (p.K <= 0) return hipErrorInvalidValue;
     if (thin_cols) {          // X = A (lines = rows of C), S = B (lines = columns of C)

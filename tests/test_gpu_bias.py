@@ -157,6 +157,26 @@ def test_fused_bias_equals_two_launches_bitwise(dh, gpu, tile):
         assert np.abs(C1[:N, :M] - Rb[:, :M]).max() <= 1e-4 * np.sqrt(K) + 1e-6
 
 
+def test_fused_bias_on_skinny_products(dh, gpu):
+    """A C of at most 8 rows or columns goes through the skinny kernel, whose epilogue adds the bias row like the
+    tile kernels' does: the bits of the product followed by linear_dual2D_row, pads left at zero."""
+    rng = np.random.default_rng(91)
+    for (N, M, K) in ((8, 5000, 516), (5000, 8, 516), (3, 4097, 100), (4100, 5, 2052), (8, 4096, 4096)):
+        assert dh.choose_tile(0, (N + 3) // 4 * 4, (M + 3) // 4 * 4, 1, (K + 3) // 4 * 4) == 27
+        A = rng.integers(-3, 4, (N, K)).astype(np.float32)
+        B = rng.integers(-3, 4, (K, M)).astype(np.float32)
+        bias = rng.integers(-5, 6, M).astype(np.float32)
+        C1, C2 = _biased_both_ways(dh, A, B, bias, -1)
+        assert np.array_equal(C1.view(np.uint32), C2.view(np.uint32)), (N, M, K)
+        assert np.array_equal(C1[:N, :M], oracle.matmul_f64(0, A, B).astype(np.float32) + bias[None, :])
+        assert not C1[N:].any() and not C1[:, M:].any()
+    # a sum of -0 and a bias of +0: the gamma term of the separate launch turns it into +0 in both
+    A = np.zeros((8, 512), np.float32); A[:, 0] = -1.0
+    B = np.zeros((512, 300), np.float32)
+    C1, C2 = _biased_both_ways(dh, A, B, np.zeros(300, np.float32), -1)
+    assert np.array_equal(C1.view(np.uint32), C2.view(np.uint32))
+
+
 def test_fused_bias_through_two_launches_of_the_balanced_kernel(dh, gpu):
     """640 tiles of 128 x 128 for 256 compute units: whole tiles first, the remaining 128 in a second launch; the
     bias row is added once, by whoever stores a tile, in both."""
