@@ -173,7 +173,7 @@ int gemm_choose_shortk(int rows, int cols, int nz, int k, int num_cu, int varian
 hipError_t gemm_launch_skinny(int variant, const GemmParams& p, hipStream_t stream);
 // TILE_SKINNY for such a shape, else -1
 int gemm_choose_skinny(int rows, int cols, int nz, int variant, int num_cu);
-// force one of the kernel's forms (0..4, see gemm_skinny.hip) for the calling thread's launches; -1 = automatic
+// force one of the kernel's forms (0..11, see gemm_skinny.hip) for the calling thread's launches; -1 = automatic
 void gemm_skinny_form(int form);
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)
 hipError_t gemm_launch_dma(int variant, const GemmParams& p, int tile, hipStream_t stream);

@@ -15,6 +15,9 @@
 //   X K-inner (k contiguous: A of A*B and A*B^T, B of A*B^T): per instruction the wavefront reads 8 lines x 128
 //       bytes: lane l holds the 4 k at 4 * (l >> 3) of line (l & 7), two such instructions (lines 0-7, 8-15) make
 //       the 16 lines of a wavefront.  The 8 classes of k of a line meet at the end through three lane exchanges.
+// With 8 or more short lines (and a long operand of at most 512 MiB, or a K-inner one) the same stream feeds
+// v_mfma_f32_16x16x4_f32 instead: 16 lines of X against all 16 short lines over 4 k per instruction, the k classes
+// added inside the instruction (gemm_f32_skinny16 below).
 // S's values come from memory as well (they stay in the L1: a few floats per k, the same for every wavefront).
 // Where the lines are too few to give every compute unit enough wavefronts, the 4 or 16 wavefronts of a workgroup
 // share their lines and split K; their sums meet in LDS and are added share after share, a fixed order.  With
@@ -47,9 +50,11 @@ struct SkinnyParams {
     // optional row vector added to C[i][j] for i < bias_rows, j < bias_width (the forward product's bias)
     const float* bias;
     int bias_rows, bias_width;
+    int short_stored;   // lines C stores on its short side (4, 8, 12 or 16; >= s_lines)
 };
 
 typedef float sk_v4f __attribute__((ext_vector_type(4)));
+typedef float sk_v2f __attribute__((ext_vector_type(2)));
 constexpr int SKINNY_MAX_CUTS = 8;    // workgroups that cut one run's K
 constexpr int SKINNY_STAGED_FLOATS = 12288;   // of a K-inner short operand in LDS (48 KiB)
 
@@ -63,8 +68,12 @@ __device__ __forceinline__ float ld1(__amdgpu_buffer_rsrc_t r, int off, int soff
 __device__ __forceinline__ sk_v4f ld4(__amdgpu_buffer_rsrc_t r, int off, int soff) {
     return __builtin_bit_cast(sk_v4f, __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, 0));
 }
+__device__ __forceinline__ sk_v2f ld2(__amdgpu_buffer_rsrc_t r, int off, int soff) {
+    return __builtin_bit_cast(sk_v2f, __builtin_amdgcn_raw_buffer_load_b64(r, off, soff, 0));
+}
 template <int W> struct XVal;
 template <> struct XVal<1> { float v; __device__ __forceinline__ float at(int) const { return v; } };
+template <> struct XVal<2> { sk_v2f v; __device__ __forceinline__ float at(int c) const { const float value = v[c]; return value; } };
 template <> struct XVal<4> { sk_v4f v; __device__ __forceinline__ float at(int c) const { const float value = v[c]; return value; } };
 
 __device__ __forceinline__ void skinny_put(const SkinnyParams& p, int line, int col, float value) {
@@ -380,6 +389,217 @@ void gemm_f32_skinny(const SkinnyParams p) {
     }
 }
 
+// Sixteen short lines at once: v_mfma_f32_16x16x4_f32 multiplies 16 lines of X by the 16 lines of S over 4 k per
+// instruction (lane l supplies line l & 15 at k class l >> 4 of either operand; element v of the result in lane l
+// is X line 4 * (l >> 4) + v against S line l & 15).  A quarter of the 4 x 4 x 1 blocks' instructions per byte of X
+// for 16 short lines, the k classes add up inside the instruction (no lane exchange), and the lanes of a line's
+// outputs are 16 consecutive floats of C.  Fewer short lines than 16 are multiplied as zeros and not stored.
+//   X K-inner: a lane reads the 4 k at k0 + 4 * (l >> 4) of line l & 15 of each of its W sets of 16 lines (16 lines x
+//       64 bytes per instruction); the four floats feed four instructions.
+//   X K-outer: a lane reads W consecutive lines at row k0 + 4 * (l >> 4) + m, m = 0 .. 3 (4 rows x 64 W bytes per
+//       instruction); its W floats feed W accumulators (lines W * i + e, i the MFMA's row).
+// ROWS: the short side is C's row index (C is 16 x L).  Then S is the instruction's first operand and X its second:
+// element v of the result in lane l is S line 4 * (l >> 4) + v against X line l & 15 -- the lanes of a store run
+// along a row of C.
+template <bool X_KIN, bool S_KIN, int W, int NW, bool ROWS, int U = (W == 4 ? 2 : 4)>
+__global__ __launch_bounds__(NW * 64)
+void gemm_f32_skinny16(const SkinnyParams p) {
+    static_assert(W == 2 || W == 4, "sets of 16 lines (K-inner X) or floats a lane reads of a row (K-outer X)");
+    constexpr int LINES = 16 * W, PK = 16;                 // U: 16-k panels per register buffer
+    __shared__ float meet_lds[NW][W * 4][64];
+
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const bool shared = p.k_share > 0;
+    const int wg = shared ? xcd_contiguous_id(blockIdx.x, gridDim.x) : 0;
+    const int unit = shared ? wg : blockIdx.x * NW + wave;
+    const int line0 = unit * LINES;
+    const int k_begin = shared ? wave * p.k_share : 0;
+    const int k_end = shared ? min(p.K, k_begin + p.k_share) : p.K;
+    const int r = lane & 15, c4 = 4 * (lane >> 4);
+
+    const __amdgpu_buffer_rsrc_t rs = skinny_rsrc(p.S, S_KIN ? (long long)p.s_lines * p.lds * 4 : ((long long)(p.K - 1) * p.lds + p.s_lines) * 4);
+    sk_v4f d[W];
+#pragma unroll
+    for (int a = 0; a < W; a++) d[a] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
+
+    if (p.zero_floats > 0) {
+        sk_v4f* const z = (sk_v4f*)p.zero_buf;
+        const long long n4 = p.zero_floats >> 2, step = (long long)gridDim.x * (NW * 64);
+        for (long long i = (long long)blockIdx.x * (NW * 64) + t; i < n4; i += step) z[i] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    if (line0 < p.L && k_begin < k_end) {
+        // the lane's short line r at its class of k: K-inner S[r][k + c4 + m], K-outer S[k + c4 + m][r]
+        const int s_off = r < p.s_lines ? (S_KIN ? (r * p.lds + c4) * 4 : (c4 * p.lds + r) * 4) : OOB_OFFSET;
+        const int s_step = S_KIN ? 4 : p.lds * 4;
+        auto load_s = [&](int k, bool on) {
+            sk_v4f v;
+            if constexpr (S_KIN) {
+                v = ld4(rs, on ? s_off : OOB_OFFSET, k * 4);
+            } else {
+                const int so = on ? s_off : OOB_OFFSET, ss = k * s_step;
+                v.x = ld1(rs, so, ss);
+                v.y = ld1(rs, so, ss + s_step);
+                v.z = ld1(rs, so, ss + 2 * s_step);
+                v.w = ld1(rs, so, ss + 3 * s_step);
+            }
+            return v;
+        };
+        if constexpr (X_KIN) {
+            const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, (long long)p.x_lines * p.ldx * 4);
+            int x_off[W];
+#pragma unroll
+            for (int set = 0; set < W; set++) x_off[set] = ((line0 + 16 * set + r) * p.ldx + c4) * 4;
+            struct Buf { sk_v4f x[U][W]; sk_v4f s[U]; };
+            // a lane's 4 k at or beyond k_end are not read (what lies there is the next line, or another share)
+            auto load = [&](Buf& b, int k) {
+#pragma unroll
+                for (int set = 0; set < W; set++)
+#pragma unroll
+                    for (int q = 0; q < U; q++)          // (the halves of a 128-byte line one after the other)
+                        b.x[q][set] = ld4(rx, (k + PK * q + c4 < k_end) ? x_off[set] : OOB_OFFSET, (k + PK * q) * 4);
+#pragma unroll
+                for (int q = 0; q < U; q++) b.s[q] = load_s(k + PK * q, k + PK * q + c4 < k_end);
+            };
+            auto compute = [&](const Buf& b) {
+#pragma unroll
+                for (int q = 0; q < U; q++)
+#pragma unroll
+                    for (int m = 0; m < 4; m++)
+#pragma unroll
+                        for (int set = 0; set < W; set++) {
+                            const float xv = b.x[q][set][m], sv = b.s[q][m];
+                            d[set] = ROWS ? __builtin_amdgcn_mfma_f32_16x16x4f32(sv, xv, d[set], 0, 0, 0)
+                                          : __builtin_amdgcn_mfma_f32_16x16x4f32(xv, sv, d[set], 0, 0, 0);
+                        }
+            };
+            Buf b0, b1;
+            load(b0, k_begin);
+            for (int k = k_begin; k < k_end; k += 2 * PK * U) {
+                load(b1, k + PK * U);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(b0);
+                __builtin_amdgcn_sched_barrier(0);
+                load(b0, k + 2 * PK * U);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(b1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, ((long long)(p.K - 1) * p.ldx + p.x_lines) * 4);
+            const int x_step = p.ldx * 4;
+            const int x_off = (c4 * p.ldx + line0 + W * r) * 4;
+            struct Buf { XVal<W> x[U][4]; sk_v4f s[U]; };
+            // (K and the shares are multiples of 4: the lane's rows k + c4 + 0 .. 3 stand or fall together)
+            auto load = [&](Buf& b, int k) {
+#pragma unroll
+                for (int q = 0; q < U; q++) {
+                    const bool on = k + PK * q + c4 < k_end;
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        if constexpr (W == 4) b.x[q][m].v = ld4(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
+                        else b.x[q][m].v = ld2(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
+                    }
+                    b.s[q] = load_s(k + PK * q, on);
+                }
+            };
+            auto compute = [&](const Buf& b) {
+#pragma unroll
+                for (int q = 0; q < U; q++)
+#pragma unroll
+                    for (int m = 0; m < 4; m++)
+#pragma unroll
+                        for (int e = 0; e < W; e++) {
+                            const float xv = b.x[q][m].at(e), sv = b.s[q][m];
+                            d[e] = ROWS ? __builtin_amdgcn_mfma_f32_16x16x4f32(sv, xv, d[e], 0, 0, 0)
+                                        : __builtin_amdgcn_mfma_f32_16x16x4f32(xv, sv, d[e], 0, 0, 0);
+                        }
+            };
+            Buf b0, b1;
+            load(b0, k_begin);
+            for (int k = k_begin; k < k_end; k += 2 * PK * U) {
+                load(b1, k + PK * U);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(b0);
+                __builtin_amdgcn_sched_barrier(0);
+                load(b0, k + 2 * PK * U);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(b1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+
+    if (shared) {
+        // the wavefronts' shares of K meet in LDS and are added in k order by the first
+#pragma unroll
+        for (int a = 0; a < W; a++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) { const float value = d[a][v]; meet_lds[wave][a * 4 + v][lane] = value; }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int a = 0; a < W; a++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                float sum = meet_lds[0][a * 4 + v][lane];
+                for (int w = 1; w < NW; w++) sum += meet_lds[w][a * 4 + v][lane];
+                d[a][v] = sum;
+            }
+    }
+    if constexpr (!ROWS) {
+        // element v of accumulator a: K-inner X line line0 + 16 * a + c4 + v, K-outer X line line0 + W * (c4 + v) + a;
+        // the short line is r
+        if (r < p.short_stored) {
+#pragma unroll
+            for (int a = 0; a < W; a++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int line = X_KIN ? line0 + 16 * a + c4 + v : line0 + W * (c4 + v) + a;
+                    const float value = d[a][v];
+                    skinny_put(p, line, r, value);
+                }
+        }
+    } else {
+        // element v of accumulator a: short line c4 + v at K-inner X line line0 + 16 * a + r, K-outer X line
+        // line0 + W * r + a -- there a lane's W accumulators are W consecutive floats of a row of C
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            if (c4 + v >= p.short_stored) continue;
+            if constexpr (!X_KIN && W == 4) {
+                const int line = line0 + W * r;
+                if (p.bias == nullptr && line + 3 < p.L) {
+                    const sk_v4f out = {d[0][v], d[1][v], d[2][v], d[3][v]};
+                    *(sk_v4f*)&p.C[(size_t)(c4 + v) * p.ldc + line] = out;
+                    continue;
+                }
+            }
+#pragma unroll
+            for (int a = 0; a < W; a++) {
+                const int line = X_KIN ? line0 + 16 * a + r : line0 + W * r + a;
+                const float value = d[a][v];
+                skinny_put(p, line, c4 + v, value);
+            }
+        }
+    }
+}
+
+template <bool X_KIN, bool S_KIN, int W, int NW, int U = (W == 4 ? 2 : 4)>
+hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream) {
+    if ((p.ldc & 3) != 0 || ((size_t)p.C & 15) != 0) return hipErrorInvalidValue;
+    constexpr int LINES = 16 * W;
+    const long long units = ((long long)p.L + LINES - 1) / LINES;
+    p.k_share = shared ? ((p.K + NW - 1) / NW + 31) / 32 * 32 : 0;
+    p.units = (int)units;
+    p.k_cuts = 1;
+    p.k_cut = p.K;
+    const long long grid = shared ? units : (units + NW - 1) / NW;
+    if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    return hipGetLastError();
+}
+
 // cuts > 1: that many workgroups per run of lines take a part of K each (narrow forms only, at most
 // SKINNY_MAX_CUTS); they meet through the stream's workspace of the balanced kernel -- without one (the stream
 // is being captured before it has one, the table is full) the run's K stays with one workgroup.
@@ -477,6 +697,30 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
 
 template <bool X_KIN, bool S_KIN>
 hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
+    int form = t_skinny_form;
+    if (form < 0) {
+        // The 16-line blocks, measured against the 4 x 4 blocks on 32 MB ... 1 GiB operands: always for 12 or 16
+        // short lines (16 x 65536 x 4096 192 - 268 -> 176 - 187 us), except 12 beside a long K-outer operand
+        // (level); for 8 beside a K-inner long operand (65536 x 8 x 1024 50 -> 41 us) and beside a K-outer one up to
+        // 512 MiB (8192 x 8 x 4096 29.8 -> 23.9); not for 4 (level), nor under 32 lines per compute unit.
+        const int num_cu = gemm_device_num_cu();
+        if (num_cu <= 0) return hipErrorNoDevice;
+        const long long runs = ((long long)p.L + 63) / 64;
+        bool blocks16 = false;
+        if (T >= 12) blocks16 = X_KIN || T == 16 || p.L < 256LL * num_cu;
+        else if (T == 8) blocks16 = p.L >= 32LL * num_cu && (X_KIN || (long long)p.L * p.K <= (1LL << 27));
+        if (blocks16) {
+            if (p.K < 128) form = runs >= 4LL * num_cu ? 8 : 10;
+            else form = runs >= 4LL * num_cu ? (X_KIN ? 9 : 8) : runs >= num_cu ? 9 : 11;
+        }
+    }
+    switch (form) {     // the 16-line blocks: runs of 64 lines with the whole K, or shared; runs of 32
+        case 8: return launch_16<X_KIN, S_KIN, 4, 4>(p, false, stream);
+        case 9: return launch_16<X_KIN, S_KIN, 4, 4>(p, true, stream);
+        case 10: return launch_16<X_KIN, S_KIN, 2, 4>(p, false, stream);
+        case 11: return launch_16<X_KIN, S_KIN, 2, 4>(p, true, stream);
+        default: break;
+    }
     switch (T) {
         case 4: return launch_skinny<X_KIN, S_KIN, 4>(p, stream);
         case 8: return launch_skinny<X_KIN, S_KIN, 8>(p, stream);
@@ -493,28 +737,27 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
 // and split K, 2 = sixteen wavefronts do, 3 and 4 = as 0 and 1 with runs four (K-inner: two) times as long,
 // 5 and 6 = as 2 with runs of 32 and 16 lines of a K-outer operand (two and four classes of k among the lanes;
 // K-inner: as 2), 7 = as 1 with K cut across workgroups too (two workgroups per compute unit; 100 + c: c cuts);
-// -1 = the automatic choice.
+// 8 ... 11 = the 16-line blocks: 8 = a wavefront per run of 64 lines with the whole K, 9 = the four wavefronts of a
+// workgroup share a run, 10 and 11 = as 8 and 9 with runs of 32 lines; -1 = the automatic choice.
 void gemm_skinny_form(int form) {
     t_skinny_cuts = form >= 100 ? form % 100 : 0;
     if (form >= 100) form = 7;
-    t_skinny_form = (form >= 0 && form <= 7) ? form : -1;
+    t_skinny_form = (form >= 0 && form <= 11) ? form : -1;
 }
 
 // 4, 8, 12 or 16 stored lines on the short side
 static bool skinny_short(int n) { return n >= 4 && n <= 16 && n % 4 == 0; }
 
-// 4 or 8 short lines: every layout.  12 or 16: measured ahead of the tile kernels (46 - 50 us against 67 - 70 on
-// 65536 lines of 1024, 202 - 211 against 252 - 269 on 262144) only where the long operand is K-outer and has at
-// least a run of 256 lines per compute unit; a K-inner long operand shares its short operand's values among too
-// few lines per wavefront there (59 - 83 us against 68 - 77).
+// 4 or 8 short lines: every layout from 256 lines on.  12 or 16: from 16 lines of the long operand per compute unit
+// on (4096 x 16 x 4096 20 - 24 us against the tile kernels' 24; 2048 x 16 x 8192 33 - 45 against 24 - 26).
 int gemm_choose_skinny(int rows, int cols, int nz, int variant, int num_cu) {
+    (void)variant;
     if (nz != 1) return -1;
     const bool thin_cols = skinny_short(cols) && rows >= 256;
     const bool thin_rows = !thin_cols && skinny_short(rows) && cols >= 256;
     if (!thin_cols && !thin_rows) return -1;
     if ((thin_cols ? cols : rows) <= 8) return TILE_SKINNY;
-    const bool x_kouter = thin_cols ? variant == GEMM_T1 : (variant == GEMM_NN || variant == GEMM_T1);
-    return x_kouter && (long long)(thin_cols ? rows : cols) >= 256LL * num_cu ? TILE_SKINNY : -1;
+    return (long long)(thin_cols ? rows : cols) >= 16LL * num_cu ? TILE_SKINNY : -1;
 }
 
 // True where the product is one for the skinny kernel: one unsplit 2-D product (a bias row on A*B only) whose C has
@@ -546,7 +789,7 @@ hipError_t gemm_launch_skinny(int variant, const GemmParams& g, hipStream_t stre
     if (thin_cols) {          // X = A (lines = rows of C), S = B (lines = columns of C)
         p.X = g.A; p.ldx = g.lda; p.x_lines = a_kin ? g.a_outer : g.a_inner;
         p.S = g.B; p.lds = g.ldb; p.s_lines = min(b_kin ? g.b_outer : g.b_inner, g.cols);
-        p.L = g.rows; p.out_rows = 0;
+        p.L = g.rows; p.out_rows = 0; p.short_stored = g.cols;
         switch ((a_kin ? 2 : 0) | (b_kin ? 1 : 0)) {
             case 0: return launch_skinny_t<false, false>(p, g.cols, stream);
             case 1: return launch_skinny_t<false, true>(p, g.cols, stream);
@@ -557,7 +800,7 @@ hipError_t gemm_launch_skinny(int variant, const GemmParams& g, hipStream_t stre
     // X = B (lines = columns of C), S = A (lines = rows of C)
     p.X = g.B; p.ldx = g.ldb; p.x_lines = b_kin ? g.b_outer : g.b_inner;
     p.S = g.A; p.lds = g.lda; p.s_lines = min(a_kin ? g.a_outer : g.a_inner, g.rows);
-    p.L = g.cols; p.out_rows = 1;
+    p.L = g.cols; p.out_rows = 1; p.short_stored = g.rows;
     switch ((b_kin ? 2 : 0) | (a_kin ? 1 : 0)) {
         case 0: return launch_skinny_t<false, false>(p, g.rows, stream);
         case 1: return launch_skinny_t<false, true>(p, g.rows, stream);

@@ -31,7 +31,7 @@ extern "C" {
  * sits in LDS, the rim of C -- 1 ... 4 rows / columns past a multiple of 64 -- as strips of 4x4 MFMA blocks;
  * another K falls back to the automatic choice).  27: the skinny kernel for a 2-D product whose C has 4, 8, 12 or 16
  * columns under at least 256 rows, or as many rows over at least 256 columns (wavefronts stream the long operand into 4x4x1
- * MFMA blocks; what the automatic choice takes there; another shape falls back to the automatic choice).  28: the band
+ * or 16x16x4 MFMA blocks; what the automatic choice takes there; another shape falls back to the automatic choice).  28: the band
  * kernel with bands of 64 rows under tiles of 256 columns, 29: the band kernel with the band's rows of A in registers
  * (four wavefronts, two workgroups per compute unit, a tile multiplied block after block); neither is chosen
  * automatically: both measure level with 24. */
@@ -41,7 +41,10 @@ void dragon_gemm_force_tile(int32_t tile);
  * four wavefronts of a workgroup share a run and split K, 2 = sixteen wavefronts do, 3 and 4 = as 0 and 1 with runs
  * four (two) times as long, 5 and 6 = as 2 with runs of 32 and 16 lines (k the row index; else as 2), 7 = as 1 with K
  * cut across workgroups as well, two workgroups per compute unit (100 + c: c cuts, at most 8; needs the stream's
- * workspace); -1 restores the automatic choice. */
+ * workspace); 8 ... 11 = 16x16x4 MFMA blocks (16 lines against all short lines per instruction; what the automatic
+ * choice takes for 12 or 16 short lines and for most products with 8): 8 = a wavefront per run of 64 lines with the
+ * whole K, 9 = the four wavefronts of a workgroup share a run, 10 and 11 = as 8 and 9 with runs of 32 lines;
+ * -1 restores the automatic choice. */
 void dragon_gemm_skinny_form(int32_t form);
 /* 1 if the paired-stage form can address the 2-D product (variant 0 = A*B, 1 = A^T*B, 2 = A*B^T, cut into
  * GridZ K slices): it reaches a tile's stages by 32-bit byte offsets, so the longest K range times the

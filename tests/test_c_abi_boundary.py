@@ -217,9 +217,10 @@ def test_tile_choice_on_the_documented_shapes(dh):
     # a C of 4, 8, 12 or 16 columns (or rows) under at least 256 lines of the other side, one 2-D product: the skinny kernel
     for v in (NN, T1, T2):
         assert ct(v, 65536, 4, 1, 1024) == 27 and ct(v, 8, 8192, 1, 4096) == 27 and ct(v, 256, 8, 1, 4) == 27
-    # 12 or 16: only beside a K-outer long operand (A of A^T*B, B of A*B and A^T*B) with 256 lines per compute unit
+    # 12 or 16: from 16 lines of the long side per compute unit on
     assert ct(T1, 65536, 16, 1, 1024) == 27 and ct(NN, 16, 65536, 1, 1024) == 27 and ct(T1, 12, 65536, 1, 1024) == 27
-    assert ct(NN, 65536, 16, 1, 1024) != 27 and ct(T2, 16, 65536, 1, 1024) != 27 and ct(T1, 32768, 16, 1, 1024) != 27
+    assert ct(NN, 65536, 16, 1, 1024) == 27 and ct(T2, 16, 65536, 1, 1024) == 27 and ct(T1, 4096, 16, 1, 1024) == 27
+    assert ct(NN, 4092, 16, 1, 1024) != 27 and ct(T2, 12, 2048, 1, 1024) != 27
     for v in (NN, T1, T2):
         assert ct(v, 65536, 20, 1, 1024) != 27 and ct(v, 65536, 4, 2, 1024) != 27 and ct(v, 252, 4, 1, 1024) != 27
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise

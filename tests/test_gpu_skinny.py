@@ -39,11 +39,12 @@ def test_the_automatic_choice_names_the_kernel(gpu):
     for (rows, cols) in ((65536, 4), (8192, 8), (256, 4), (4, 65536), (8, 256), (4, 1000)):
         for variant in (NN, T1, T2):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
-    # 12 or 16 short lines: only beside a K-outer long operand of at least 256 lines per compute unit
-    assert gpu.choose_tile(T1, 65536, 16, 1, 1024, cu) == SKINNY and gpu.choose_tile(T1, 65536, 12, 1, 1024, cu) == SKINNY
-    assert gpu.choose_tile(NN, 16, 65536, 1, 1024, cu) == SKINNY and gpu.choose_tile(T1, 12, 70000, 1, 1024, cu) == SKINNY
-    assert gpu.choose_tile(NN, 65536, 16, 1, 1024, cu) != SKINNY and gpu.choose_tile(T2, 65536, 16, 1, 1024, cu) != SKINNY
-    assert gpu.choose_tile(T2, 16, 65536, 1, 1024, cu) != SKINNY and gpu.choose_tile(T1, 32768, 16, 1, 1024, cu) != SKINNY
+    # 12 or 16 short lines: from 16 lines of the long operand per compute unit on, in every layout
+    for variant in (NN, T1, T2):
+        for (rows, cols) in ((65536, 16), (4096, 12), (16, 65536), (12, 4096)):
+            assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
+        for (rows, cols) in ((4092, 16), (16, 4000), (256, 12)):
+            assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) != SKINNY
     # not skinny enough, too short, or a batch / K slices
     for (rows, cols, nz) in ((65536, 20, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (16, 252, 1), (65536, 4, 2), (4, 65536, 3)):
         for variant in (NN, T1, T2):
@@ -51,7 +52,7 @@ def test_the_automatic_choice_names_the_kernel(gpu):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108, 8, 9, 10, 11])
 @pytest.mark.parametrize("thin", [1, 2, 3, 4, 5, 7, 8, 9, 12, 13, 16])
 def test_thin_columns_bitwise(gpu, variant, thin, form):
     """C of 1 ... 16 columns (stored 4, 8, 12 or 16) under row counts around the 16, 64 and 256 lines a wavefront takes,
@@ -59,13 +60,13 @@ def test_thin_columns_bitwise(gpu, variant, thin, form):
     lines per lane."""
     gpu.skinny_form(form)
     if form >= 0:
-        gpu.force_tile(SKINNY)      # 12 and 16 columns beside a K-inner long operand are not the automatic choice
+        gpu.force_tile(SKINNY)      # (a forced form also runs shapes the automatic choice leaves to the tile kernels)
     for (N, K) in ((256, 64), (1000, 1028), (4099, 36), (40000, 100), (20000, 260)):
         check(gpu, variant, N, thin, K, 100 * thin + N + K + variant)
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108, 8, 9, 10, 11])
 @pytest.mark.parametrize("thin", [1, 3, 4, 6, 8, 10, 12, 15, 16])
 def test_thin_rows_bitwise(gpu, variant, thin, form):
     gpu.skinny_form(form)
@@ -81,7 +82,7 @@ def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
     """K around the k rows / 32-k panels of a register buffer, the 4-k chunks of a lane, the shares of a K split
     between 4 or 16 wavefronts; in every form."""
     gpu.force_tile(SKINNY)
-    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108):
+    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108, 8, 9, 10, 11):
         gpu.skinny_form(form)
         check(gpu, variant, 700, 4, K, 3000 + K + variant)
         check(gpu, variant, 8, 900, K, 4000 + K + variant)
