@@ -143,11 +143,11 @@ int matmul_2d(int variant, const int64_t* streams, int length, int gz, int64_t d
     // whole product goes to C and the partial buffers get zeros -- SKbuf_summary then adds zeros and leaves C
     // as it is (the caller sees the sum it asked for; which slice holds what is the kernel's business).  A
     // forced tile shape (tests, tuning) always honours the split.
-    // A skinny product (a C of 4 or 8 columns or rows, ...) that the host policy asks to split -- it does, by 4 to 16,
+    // A skinny product (a C of 4 ... 32 columns or rows, ...) that the host policy asks to split -- it does, by 4 to 16,
     // for the shapes with few lines: 8 x 4096 x 4096 gets GridZ 16 -- goes to the skinny kernel whole, which cuts K
     // among its workgroups itself; the partial buffers get zeros from the same launch and the fold is elided.
     if (gz > 1 && dBias == 0 && sk_ws == nullptr && gemm_forced_tile() == TILE_AUTO && t_split_policy != 0 &&
-        gemm_choose_skinny(N, M, 1, variant, num_cu) >= 0) {
+        gemm_choose_skinny(N, M, 1, K, variant, num_cu) >= 0) {
         GemmParams q = p;
         q.nz = 1; q.split = 0; q.k_slice = 0; q.sizeC = 0; q.Cbuf = nullptr;
         q.zero_buf = p.Cbuf;

@@ -167,12 +167,12 @@ hipError_t gemm_launch(int variant, const GemmParams& p, int tile, hipStream_t s
 hipError_t gemm_launch_shortk(int variant, const GemmParams& p, hipStream_t stream);
 // TILE_SHORTK_64x64 where that kernel is the better choice, else -1
 int gemm_choose_shortk(int rows, int cols, int nz, int k, int num_cu, int variant = -1);
-// The skinny kernel (tile id TILE_SKINNY) for the three 2-D products whose C has 4, 8, 12 or 16 columns under at
+// The skinny kernel (tile id TILE_SKINNY) for the three 2-D products whose C has 4, 8, ... 32 columns under at
 // least 256 rows, or as many rows over at least 256 columns.  hipErrorOutOfMemory says that the product cannot go this way
 // (another shape, a batch, K slices, a bias row) and the caller takes a tile-per-workgroup kernel instead.
 hipError_t gemm_launch_skinny(int variant, const GemmParams& p, hipStream_t stream);
 // TILE_SKINNY for such a shape, else -1
-int gemm_choose_skinny(int rows, int cols, int nz, int variant, int num_cu);
+int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_cu);
 // force one of the kernel's forms (0..11, see gemm_skinny.hip) for the calling thread's launches; -1 = automatic
 void gemm_skinny_form(int form);
 // the three products through the direct-to-LDS kernel (tile ids TILE_DMA_*)

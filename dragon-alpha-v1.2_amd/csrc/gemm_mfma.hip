@@ -106,7 +106,7 @@ static const TileTraits kTiles[TILE_ALL_COUNT] = {
 int gemm_choose_tile(int rows, int cols, int nz, int k, int num_cu, int variant) {
     const int forced = gemm_forced_tile();
     if (forced != TILE_AUTO) return forced;
-    const int skinny = gemm_choose_skinny(rows, cols, nz, variant, num_cu);
+    const int skinny = gemm_choose_skinny(rows, cols, nz, k, variant, num_cu);
     if (skinny >= 0) return skinny;
     const int band = gemm_choose_band(rows, cols, nz, k, num_cu, variant);
     if (band >= 0) return band;

@@ -1,4 +1,4 @@
-// Skinny products: a C of at most 16 columns (N x 4 ... N x 16) or at most 16 rows (4 x M ... 16 x M) under a long
+// Skinny products: a C of at most 32 columns (N x 4 ... N x 32) or at most 32 rows (4 x M ... 32 x M) under a long
 // other side -- matrix times a few vectors.  The reference sends a C of 4 columns to kernels of their own
 // (MM/matMul_sernel.cuh:17-30, dispatched at MM/matMul.cuh:100-102) and thin row strips to k18 / k14 / k12
 // (MM/matMul.cuh:104-106).
@@ -16,8 +16,8 @@
 //       bytes: lane l holds the 4 k at 4 * (l >> 3) of line (l & 7), two such instructions (lines 0-7, 8-15) make
 //       the 16 lines of a wavefront.  The 8 classes of k of a line meet at the end through three lane exchanges.
 // With 8 or more short lines (and a long operand of at most 512 MiB, or a K-inner one) the same stream feeds
-// v_mfma_f32_16x16x4_f32 instead: 16 lines of X against all 16 short lines over 4 k per instruction, the k classes
-// added inside the instruction (gemm_f32_skinny16 below).
+// v_mfma_f32_16x16x4_f32 instead: 16 lines of X against 16 short lines over 4 k per instruction, the k classes
+// added inside the instruction (gemm_f32_skinny16 below; 20 ... 32 short lines as two groups of 16).
 // S's values come from memory as well (they stay in the L1: a few floats per k, the same for every wavefront).
 // Where the lines are too few to give every compute unit enough wavefronts, the 4 or 16 wavefronts of a workgroup
 // share their lines and split K; their sums meet in LDS and are added share after share, a fixed order.  With
@@ -401,12 +401,14 @@ void gemm_f32_skinny(const SkinnyParams p) {
 // ROWS: the short side is C's row index (C is 16 x L).  Then S is the instruction's first operand and X its second:
 // element v of the result in lane l is S line 4 * (l >> 4) + v against X line l & 15 -- the lanes of a store run
 // along a row of C.
-template <bool X_KIN, bool S_KIN, int W, int NW, bool ROWS, int U = (W == 4 ? 2 : 4)>
+// G: groups of 16 short lines (1, or 2 for 20 ... 32 short lines: every value of X feeds G instructions).
+template <bool X_KIN, bool S_KIN, int W, int NW, bool ROWS, int G = 1, int U = (W == 4 ? 2 : 4)>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny16(const SkinnyParams p) {
     static_assert(W == 2 || W == 4, "sets of 16 lines (K-inner X) or floats a lane reads of a row (K-outer X)");
+    static_assert(G == 1 || G == 2, "up to 32 short lines");
     constexpr int LINES = 16 * W, PK = 16;                 // U: 16-k panels per register buffer
-    __shared__ float meet_lds[NW][W * 4][64];
+    __shared__ float meet_lds[NW][W * G * 4][64];
 
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const bool shared = p.k_share > 0;
@@ -418,9 +420,11 @@ void gemm_f32_skinny16(const SkinnyParams p) {
     const int r = lane & 15, c4 = 4 * (lane >> 4);
 
     const __amdgpu_buffer_rsrc_t rs = skinny_rsrc(p.S, S_KIN ? (long long)p.s_lines * p.lds * 4 : ((long long)(p.K - 1) * p.lds + p.s_lines) * 4);
-    sk_v4f d[W];
+    sk_v4f d[W][G];
 #pragma unroll
-    for (int a = 0; a < W; a++) d[a] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    for (int a = 0; a < W; a++)
+#pragma unroll
+        for (int g = 0; g < G; g++) d[a][g] = (sk_v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
     if (p.zero_floats > 0) {
         sk_v4f* const z = (sk_v4f*)p.zero_buf;
@@ -429,15 +433,18 @@ void gemm_f32_skinny16(const SkinnyParams p) {
     }
 
     if (line0 < p.L && k_begin < k_end) {
-        // the lane's short line r at its class of k: K-inner S[r][k + c4 + m], K-outer S[k + c4 + m][r]
-        const int s_off = r < p.s_lines ? (S_KIN ? (r * p.lds + c4) * 4 : (c4 * p.lds + r) * 4) : OOB_OFFSET;
+        // the lane's short line 16 g + r at its class of k: K-inner S[line][k + c4 + m], K-outer S[k + c4 + m][line]
+        int s_off[G];
+#pragma unroll
+        for (int g = 0; g < G; g++)
+            s_off[g] = 16 * g + r < p.s_lines ? (S_KIN ? ((16 * g + r) * p.lds + c4) * 4 : (c4 * p.lds + 16 * g + r) * 4) : OOB_OFFSET;
         const int s_step = S_KIN ? 4 : p.lds * 4;
-        auto load_s = [&](int k, bool on) {
+        auto load_s = [&](int g, int k, bool on) {
             sk_v4f v;
             if constexpr (S_KIN) {
-                v = ld4(rs, on ? s_off : OOB_OFFSET, k * 4);
+                v = ld4(rs, on ? s_off[g] : OOB_OFFSET, k * 4);
             } else {
-                const int so = on ? s_off : OOB_OFFSET, ss = k * s_step;
+                const int so = on ? s_off[g] : OOB_OFFSET, ss = k * s_step;
                 v.x = ld1(rs, so, ss);
                 v.y = ld1(rs, so, ss + s_step);
                 v.z = ld1(rs, so, ss + 2 * s_step);
@@ -445,12 +452,16 @@ void gemm_f32_skinny16(const SkinnyParams p) {
             }
             return v;
         };
+        auto mfma = [&](sk_v4f& acc, float xv, float sv) {
+            acc = ROWS ? __builtin_amdgcn_mfma_f32_16x16x4f32(sv, xv, acc, 0, 0, 0)
+                       : __builtin_amdgcn_mfma_f32_16x16x4f32(xv, sv, acc, 0, 0, 0);
+        };
         if constexpr (X_KIN) {
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, (long long)p.x_lines * p.ldx * 4);
             int x_off[W];
 #pragma unroll
             for (int set = 0; set < W; set++) x_off[set] = ((line0 + 16 * set + r) * p.ldx + c4) * 4;
-            struct Buf { sk_v4f x[U][W]; sk_v4f s[U]; };
+            struct Buf { sk_v4f x[U][W]; sk_v4f s[U][G]; };
             // a lane's 4 k at or beyond k_end are not read (what lies there is the next line, or another share)
             auto load = [&](Buf& b, int k) {
 #pragma unroll
@@ -459,7 +470,9 @@ void gemm_f32_skinny16(const SkinnyParams p) {
                     for (int q = 0; q < U; q++)          // (the halves of a 128-byte line one after the other)
                         b.x[q][set] = ld4(rx, (k + PK * q + c4 < k_end) ? x_off[set] : OOB_OFFSET, (k + PK * q) * 4);
 #pragma unroll
-                for (int q = 0; q < U; q++) b.s[q] = load_s(k + PK * q, k + PK * q + c4 < k_end);
+                for (int q = 0; q < U; q++)
+#pragma unroll
+                    for (int g = 0; g < G; g++) b.s[q][g] = load_s(g, k + PK * q, k + PK * q + c4 < k_end);
             };
             auto compute = [&](const Buf& b) {
 #pragma unroll
@@ -467,11 +480,12 @@ void gemm_f32_skinny16(const SkinnyParams p) {
 #pragma unroll
                     for (int m = 0; m < 4; m++)
 #pragma unroll
-                        for (int set = 0; set < W; set++) {
-                            const float xv = b.x[q][set][m], sv = b.s[q][m];
-                            d[set] = ROWS ? __builtin_amdgcn_mfma_f32_16x16x4f32(sv, xv, d[set], 0, 0, 0)
-                                          : __builtin_amdgcn_mfma_f32_16x16x4f32(xv, sv, d[set], 0, 0, 0);
-                        }
+                        for (int set = 0; set < W; set++)
+#pragma unroll
+                            for (int g = 0; g < G; g++) {
+                                const float xv = b.x[q][set][m], sv = b.s[q][g][m];
+                                mfma(d[set][g], xv, sv);
+                            }
             };
             Buf b0, b1;
             load(b0, k_begin);
@@ -489,7 +503,7 @@ void gemm_f32_skinny16(const SkinnyParams p) {
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, ((long long)(p.K - 1) * p.ldx + p.x_lines) * 4);
             const int x_step = p.ldx * 4;
             const int x_off = (c4 * p.ldx + line0 + W * r) * 4;
-            struct Buf { XVal<W> x[U][4]; sk_v4f s[U]; };
+            struct Buf { XVal<W> x[U][4]; sk_v4f s[U][G]; };
             // (K and the shares are multiples of 4: the lane's rows k + c4 + 0 .. 3 stand or fall together)
             auto load = [&](Buf& b, int k) {
 #pragma unroll
@@ -500,7 +514,8 @@ void gemm_f32_skinny16(const SkinnyParams p) {
                         if constexpr (W == 4) b.x[q][m].v = ld4(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
                         else b.x[q][m].v = ld2(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
                     }
-                    b.s[q] = load_s(k + PK * q, on);
+#pragma unroll
+                    for (int g = 0; g < G; g++) b.s[q][g] = load_s(g, k + PK * q, on);
                 }
             };
             auto compute = [&](const Buf& b) {
@@ -509,11 +524,12 @@ void gemm_f32_skinny16(const SkinnyParams p) {
 #pragma unroll
                     for (int m = 0; m < 4; m++)
 #pragma unroll
-                        for (int e = 0; e < W; e++) {
-                            const float xv = b.x[q][m].at(e), sv = b.s[q][m];
-                            d[e] = ROWS ? __builtin_amdgcn_mfma_f32_16x16x4f32(sv, xv, d[e], 0, 0, 0)
-                                        : __builtin_amdgcn_mfma_f32_16x16x4f32(xv, sv, d[e], 0, 0, 0);
-                        }
+                        for (int e = 0; e < W; e++)
+#pragma unroll
+                            for (int g = 0; g < G; g++) {
+                                const float xv = b.x[q][m].at(e), sv = b.s[q][g][m];
+                                mfma(d[e][g], xv, sv);
+                            }
             };
             Buf b0, b1;
             load(b0, k_begin);
@@ -535,56 +551,64 @@ void gemm_f32_skinny16(const SkinnyParams p) {
 #pragma unroll
         for (int a = 0; a < W; a++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) { const float value = d[a][v]; meet_lds[wave][a * 4 + v][lane] = value; }
+            for (int g = 0; g < G; g++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) { const float value = d[a][g][v]; meet_lds[wave][(a * G + g) * 4 + v][lane] = value; }
         __syncthreads();
         if (wave != 0) return;
 #pragma unroll
         for (int a = 0; a < W; a++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                float sum = meet_lds[0][a * 4 + v][lane];
-                for (int w = 1; w < NW; w++) sum += meet_lds[w][a * 4 + v][lane];
-                d[a][v] = sum;
-            }
-    }
-    if constexpr (!ROWS) {
-        // element v of accumulator a: K-inner X line line0 + 16 * a + c4 + v, K-outer X line line0 + W * (c4 + v) + a;
-        // the short line is r
-        if (r < p.short_stored) {
-#pragma unroll
-            for (int a = 0; a < W; a++)
+            for (int g = 0; g < G; g++)
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const int line = X_KIN ? line0 + 16 * a + c4 + v : line0 + W * (c4 + v) + a;
-                    const float value = d[a][v];
-                    skinny_put(p, line, r, value);
+                    float sum = meet_lds[0][(a * G + g) * 4 + v][lane];
+                    for (int w = 1; w < NW; w++) sum += meet_lds[w][(a * G + g) * 4 + v][lane];
+                    d[a][g][v] = sum;
                 }
-        }
-    } else {
-        // element v of accumulator a: short line c4 + v at K-inner X line line0 + 16 * a + r, K-outer X line
-        // line0 + W * r + a -- there a lane's W accumulators are W consecutive floats of a row of C
+    }
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            if (c4 + v >= p.short_stored) continue;
-            if constexpr (!X_KIN && W == 4) {
-                const int line = line0 + W * r;
-                if (p.bias == nullptr && line + 3 < p.L) {
-                    const sk_v4f out = {d[0][v], d[1][v], d[2][v], d[3][v]};
-                    *(sk_v4f*)&p.C[(size_t)(c4 + v) * p.ldc + line] = out;
-                    continue;
-                }
+    for (int g = 0; g < G; g++) {
+        if constexpr (!ROWS) {
+            // element v of accumulator a: K-inner X line line0 + 16 * a + c4 + v, K-outer X line line0 + W * (c4 + v) + a;
+            // the short line is 16 g + r
+            if (16 * g + r < p.short_stored) {
+#pragma unroll
+                for (int a = 0; a < W; a++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int line = X_KIN ? line0 + 16 * a + c4 + v : line0 + W * (c4 + v) + a;
+                        const float value = d[a][g][v];
+                        skinny_put(p, line, 16 * g + r, value);
+                    }
             }
+        } else {
+            // element v of accumulator a: short line 16 g + c4 + v at K-inner X line line0 + 16 * a + r, K-outer X line
+            // line0 + W * r + a -- there a lane's W accumulators are W consecutive floats of a row of C
 #pragma unroll
-            for (int a = 0; a < W; a++) {
-                const int line = X_KIN ? line0 + 16 * a + r : line0 + W * r + a;
-                const float value = d[a][v];
-                skinny_put(p, line, c4 + v, value);
+            for (int v = 0; v < 4; v++) {
+                const int row = 16 * g + c4 + v;
+                if (row >= p.short_stored) continue;
+                if constexpr (!X_KIN && W == 4) {
+                    const int line = line0 + W * r;
+                    if (p.bias == nullptr && line + 3 < p.L) {
+                        const sk_v4f out = {d[0][g][v], d[1][g][v], d[2][g][v], d[3][g][v]};
+                        *(sk_v4f*)&p.C[(size_t)row * p.ldc + line] = out;
+                        continue;
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < W; a++) {
+                    const int line = X_KIN ? line0 + 16 * a + r : line0 + W * r + a;
+                    const float value = d[a][g][v];
+                    skinny_put(p, line, row, value);
+                }
             }
         }
     }
 }
 
-template <bool X_KIN, bool S_KIN, int W, int NW, int U = (W == 4 ? 2 : 4)>
+template <bool X_KIN, bool S_KIN, int W, int NW, int G>
 hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream) {
     if ((p.ldc & 3) != 0 || ((size_t)p.C & 15) != 0) return hipErrorInvalidValue;
     constexpr int LINES = 16 * W;
@@ -595,8 +619,8 @@ hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream) {
     p.k_cut = p.K;
     const long long grid = shared ? units : (units + NW - 1) / NW;
     if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
-    else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -707,18 +731,19 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
         if (num_cu <= 0) return hipErrorNoDevice;
         const long long runs = ((long long)p.L + 63) / 64;
         bool blocks16 = false;
-        if (T >= 12) blocks16 = X_KIN || T == 16 || p.L < 256LL * num_cu;
+        if (T >= 12) blocks16 = X_KIN || T >= 16 || p.L < 256LL * num_cu;
         else if (T == 8) blocks16 = p.L >= 32LL * num_cu && (X_KIN || (long long)p.L * p.K <= (1LL << 27));
         if (blocks16) {
             if (p.K < 128) form = runs >= 4LL * num_cu ? 8 : 10;
             else form = runs >= 4LL * num_cu ? (X_KIN ? 9 : 8) : runs >= num_cu ? 9 : 11;
         }
     }
+    if (T > 16 && (form < 8 || form > 11)) form = 9;        // (the 4 x 4 blocks stop at 16 short lines)
     switch (form) {     // the 16-line blocks: runs of 64 lines with the whole K, or shared; runs of 32
-        case 8: return launch_16<X_KIN, S_KIN, 4, 4>(p, false, stream);
-        case 9: return launch_16<X_KIN, S_KIN, 4, 4>(p, true, stream);
-        case 10: return launch_16<X_KIN, S_KIN, 2, 4>(p, false, stream);
-        case 11: return launch_16<X_KIN, S_KIN, 2, 4>(p, true, stream);
+        case 8: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, false, stream) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, false, stream);
+        case 9: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, true, stream) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, true, stream);
+        case 10: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, false, stream) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, false, stream);
+        case 11: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, true, stream) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, true, stream);
         default: break;
     }
     switch (T) {
@@ -745,33 +770,36 @@ void gemm_skinny_form(int form) {
     t_skinny_form = (form >= 0 && form <= 11) ? form : -1;
 }
 
-// 4, 8, 12 or 16 stored lines on the short side
-static bool skinny_short(int n) { return n >= 4 && n <= 16 && n % 4 == 0; }
+// 4, 8, ... 32 stored lines on the short side
+static bool skinny_short(int n) { return n >= 4 && n <= 32 && n % 4 == 0; }
 
 // 4 or 8 short lines: every layout from 256 lines on.  12 or 16: from 16 lines of the long operand per compute unit
-// on (4096 x 16 x 4096 20 - 24 us against the tile kernels' 24; 2048 x 16 x 8192 33 - 45 against 24 - 26).
-int gemm_choose_skinny(int rows, int cols, int nz, int variant, int num_cu) {
+// on (4096 x 16 x 4096 20 - 24 us against the tile kernels' 24; 2048 x 16 x 8192 33 - 45 against 24 - 26).  20 ... 32:
+// from 32 lines per compute unit on and a K of at least 256 (8192 x 32 x 4096 31 - 35 us against 39 - 41).
+int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_cu) {
     (void)variant;
     if (nz != 1) return -1;
     const bool thin_cols = skinny_short(cols) && rows >= 256;
     const bool thin_rows = !thin_cols && skinny_short(rows) && cols >= 256;
     if (!thin_cols && !thin_rows) return -1;
-    if ((thin_cols ? cols : rows) <= 8) return TILE_SKINNY;
-    return (long long)(thin_cols ? rows : cols) >= 16LL * num_cu ? TILE_SKINNY : -1;
+    const int t = thin_cols ? cols : rows;
+    if (t <= 8) return TILE_SKINNY;
+    if (t > 16 && k < 256) return -1;      // (16384 x 32 x 128: 8.1 us against the balanced kernel's 5.2)
+    return (long long)(thin_cols ? rows : cols) >= (t <= 16 ? 16LL : 32LL) * num_cu ? TILE_SKINNY : -1;
 }
 
 // True where the product is one for the skinny kernel: one unsplit 2-D product (a bias row on A*B only) whose C has
-// 4 ... 16 stored columns under at least 256 rows, or 4 ... 16 stored rows over at least 256 columns, and whose
+// 4 ... 32 stored columns under at least 256 rows, or 4 ... 32 stored rows over at least 256 columns, and whose
 // operands' byte offsets (with the reads a register buffer runs ahead, and the lines of a last, partly filled
 // run) fit 32 bits.
 static bool gemm_skinny_applies(int variant, const GemmParams& p) {
     // (a forced choice takes every shape the kernel can run: up to 16 short lines in every layout)
-    if (p.split || (p.bias != nullptr && variant != GEMM_NN) || gemm_choose_skinny(p.rows, p.cols, p.nz, GEMM_T1, 1) < 0) return false;
     const bool thin_cols = skinny_short(p.cols) && p.rows >= 256;
+    if (p.split || p.nz != 1 || (p.bias != nullptr && variant != GEMM_NN) || !(thin_cols || (skinny_short(p.rows) && p.cols >= 256))) return false;
     const bool a_kin = variant != GEMM_T1, b_kin = variant == GEMM_T2;
     // a K-inner operand is addressed line * ld + k, a K-outer one k * ld + line
-    const long long a_span = a_kin ? (long long)(thin_cols ? p.rows : 16) * p.lda : (long long)p.k_total * p.lda;
-    const long long b_span = b_kin ? (long long)(thin_cols ? 16 : p.cols) * p.ldb : (long long)p.k_total * p.ldb;
+    const long long a_span = a_kin ? (long long)(thin_cols ? p.rows : 32) * p.lda : (long long)p.k_total * p.lda;
+    const long long b_span = b_kin ? (long long)(thin_cols ? 32 : p.cols) * p.ldb : (long long)p.k_total * p.ldb;
     const long long ld = p.lda > p.ldb ? p.lda : p.ldb;
     return ld <= (1 << 20) && (a_span + 64 * ld) * 4 < 0x7fff0000LL && (b_span + 64 * ld) * 4 < 0x7fff0000LL;
 }

@@ -29,7 +29,7 @@ extern "C" {
  * for a K of at most 64 under a large C (a band of 128 rows of A stays in LDS; a longer K falls
  * back to the automatic choice).  26: the resident-K kernel for a K of 89 ... 144 (64x64 tiles whose whole K
  * sits in LDS, the rim of C -- 1 ... 4 rows / columns past a multiple of 64 -- as strips of 4x4 MFMA blocks;
- * another K falls back to the automatic choice).  27: the skinny kernel for a 2-D product whose C has 4, 8, 12 or 16
+ * another K falls back to the automatic choice).  27: the skinny kernel for a 2-D product whose C has 4, 8, ... 32
  * columns under at least 256 rows, or as many rows over at least 256 columns (wavefronts stream the long operand into 4x4x1
  * or 16x16x4 MFMA blocks; what the automatic choice takes there; another shape falls back to the automatic choice).  28: the band
  * kernel with bands of 64 rows under tiles of 256 columns, 29: the band kernel with the band's rows of A in registers

@@ -222,7 +222,7 @@ def test_tile_choice_on_the_documented_shapes(dh):
     assert ct(NN, 65536, 16, 1, 1024) == 27 and ct(T2, 16, 65536, 1, 1024) == 27 and ct(T1, 4096, 16, 1, 1024) == 27
     assert ct(NN, 4092, 16, 1, 1024) != 27 and ct(T2, 12, 2048, 1, 1024) != 27
     for v in (NN, T1, T2):
-        assert ct(v, 65536, 20, 1, 1024) != 27 and ct(v, 65536, 4, 2, 1024) != 27 and ct(v, 252, 4, 1, 1024) != 27
+        assert ct(v, 65536, 36, 1, 1024) != 27 and ct(v, 65536, 20, 1, 1024) == 27 and ct(v, 4096, 20, 1, 1024) != 27 and ct(v, 65536, 4, 2, 1024) != 27 and ct(v, 252, 4, 1, 1024) != 27
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise
     shape = (64 * 20, 128 * 19, 1, 2048)
     if ct(NN, *shape) in (5 + P, 9 + P):

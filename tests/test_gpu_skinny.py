@@ -1,7 +1,7 @@
-"""GPU parity of the skinny kernel (gemm_skinny.hip): a C of 4 ... 16 columns under many rows, or of 4 ... 16 rows over
+"""GPU parity of the skinny kernel (gemm_skinny.hip): a C of 4 ... 32 columns under many rows, or of 4 ... 32 rows over
 many columns -- what the reference sends to its 4-column kernels (MM/matMul_sernel.cuh:17-30, dispatched at
 MM/matMul.cuh:100-102) and to k18 / k14 / k12 (MM/matMul.cuh:104-106).  Wavefronts stream the long operand from
-memory into 4 x 4 x 1 MFMA blocks; integer inputs pin the indexing bit for bit: lines per wavefront, the classes
+memory into 4 x 4 x 1 or 16 x 16 x 4 MFMA blocks; integer inputs pin the indexing bit for bit: lines per wavefront, the classes
 of k, the K tail, K shared between the wavefronts of a workgroup, both orientations of C."""
 import numpy as np
 import pytest
@@ -45,8 +45,14 @@ def test_the_automatic_choice_names_the_kernel(gpu):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
         for (rows, cols) in ((4092, 16), (16, 4000), (256, 12)):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) != SKINNY
+        # 20 ... 32: from 32 lines per compute unit on
+        for (rows, cols) in ((8192, 32), (65536, 20), (24, 8192), (28, 100000)):
+            assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
+        for (rows, cols) in ((8188, 32), (32, 4096), (65536, 36), (40, 65536)):
+            assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) != SKINNY
+        assert gpu.choose_tile(variant, 65536, 32, 1, 252, cu) != SKINNY and gpu.choose_tile(variant, 65536, 16, 1, 252, cu) == SKINNY
     # not skinny enough, too short, or a batch / K slices
-    for (rows, cols, nz) in ((65536, 20, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (16, 252, 1), (65536, 4, 2), (4, 65536, 3)):
+    for (rows, cols, nz) in ((65536, 36, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (16, 252, 1), (65536, 4, 2), (4, 65536, 3)):
         for variant in (NN, T1, T2):
             assert gpu.choose_tile(variant, rows, cols, nz, 1024, cu) != SKINNY
 
@@ -95,6 +101,18 @@ def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("form", [-1, 8, 9, 10, 11])
+@pytest.mark.parametrize("thin", [17, 20, 23, 24, 28, 29, 32])
+def test_up_to_32_short_lines_bitwise(gpu, variant, thin, form):
+    """Two groups of 16 short lines through the 16 x 16 x 4 blocks, both orientations of C."""
+    gpu.force_tile(SKINNY)
+    gpu.skinny_form(form)
+    for (L, K) in ((256, 64), (1003, 1028), (4099, 36), (20000, 260)):
+        check(gpu, variant, L, thin, K, 300 * thin + L + K + variant)
+        check(gpu, variant, thin, L + 1, K, 301 * thin + L + K + variant)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
 def test_long_shapes_against_both_oracles(gpu, variant):
     """Uniform inputs at the benchmark's shapes, scaled down 4 x along the long side, within the FP32 tolerance
     (relative Frobenius error <= 1e-5, elements within 1e-4 * sqrt(K) * max|A| * max|B|); and the same launch
@@ -135,7 +153,7 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
 @pytest.mark.parametrize("variant", [NN, T1, T2])
 def test_forced_on_another_shape_falls_back(gpu, variant):
     gpu.force_tile(SKINNY)
-    check(gpu, variant, 300, 20, 64, 77 + variant)
+    check(gpu, variant, 300, 36, 64, 77 + variant)
     check(gpu, variant, 100, 4, 64, 78 + variant)
     check(gpu, variant, 8, 8, 64, 79 + variant)
 
