@@ -62,14 +62,18 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t skinny_rsrc(const float* base,
     const long long capped = bytes > 0xfffffff0LL ? 0xfffffff0LL : (bytes < 0 ? 0 : bytes);
     return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(unsigned)capped, RSRC_FLAGS);
 }
+// AUX: the load's cache policy bits (2 = non-temporal)
+template <int AUX = 0>
 __device__ __forceinline__ float ld1(__amdgpu_buffer_rsrc_t r, int off, int soff) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, soff, 0));
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, soff, AUX));
 }
+template <int AUX = 0>
 __device__ __forceinline__ sk_v4f ld4(__amdgpu_buffer_rsrc_t r, int off, int soff) {
-    return __builtin_bit_cast(sk_v4f, __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, 0));
+    return __builtin_bit_cast(sk_v4f, __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, AUX));
 }
+template <int AUX = 0>
 __device__ __forceinline__ sk_v2f ld2(__amdgpu_buffer_rsrc_t r, int off, int soff) {
-    return __builtin_bit_cast(sk_v2f, __builtin_amdgcn_raw_buffer_load_b64(r, off, soff, 0));
+    return __builtin_bit_cast(sk_v2f, __builtin_amdgcn_raw_buffer_load_b64(r, off, soff, AUX));
 }
 template <int W> struct XVal;
 template <> struct XVal<1> { float v; __device__ __forceinline__ float at(int) const { return v; } };
@@ -90,10 +94,15 @@ __device__ __forceinline__ void skinny_put(const SkinnyParams& p, int line, int 
 // 32-63 the odd ones).  NW: wavefronts of a workgroup.
 // SL: the workgroup's part of a K-inner S (T lines x its k range, at most 48 KiB) is staged in LDS once and read from
 // there: the short operand's lines are K floats apart -- with K a power of two, lines of the L1 that fall into one set.
-template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1, bool SL = false>
+// NT: X is read with non-temporal loads -- an operand far larger than the 256 MB Infinity Cache passes through the
+// caches once and is not kept (262144 x 4 x 1024: 180 -> 154 us); a smaller one is better left to them (8192 x 8 x
+// 4096, served by that cache from launch to launch in a loop: 22.8 -> 32.4 us).
+template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1, bool SL = false, bool NT = false>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny(const SkinnyParams p) {
     static_assert(!SL || (!X_KIN && S_KIN && W == 1 && NW == 4 && CL == 1), "the staged form");
+    static_assert(!NT || (W == 4 && NW == 4 && CL == 1 && !SL), "non-temporal reads: the long forms");
+    constexpr int XA = NT ? 2 : 0;
     static_assert(T == 4 || T == 8 || T == 12 || T == 16, "4, 8, 12 or 16 short lines");
     static_assert(X_KIN ? (W == 2 || W == 4) && CL == 1 : (W == 1 || W == 4) && (CL == 1 || ((CL == 2 || CL == 4) && W == 1)), "forms");
     constexpr int LS = 8, PK = 32;                         // K-inner X: lines per read, k per panel
@@ -167,8 +176,8 @@ void gemm_f32_skinny(const SkinnyParams p) {
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     const int off = (k + CL * u < k_end) ? x_off : OOB_OFFSET;
-                    if constexpr (W == 4) b.x[u].v = ld4(rx, off, (k + CL * u) * x_step);
-                    else b.x[u].v = ld1(rx, off, (k + CL * u) * x_step);
+                    if constexpr (W == 4) b.x[u].v = ld4<XA>(rx, off, (k + CL * u) * x_step);
+                    else b.x[u].v = ld1<XA>(rx, off, (k + CL * u) * x_step);
                 }
 #pragma unroll
                 for (int h = 0; h < H; h++) {
@@ -245,7 +254,7 @@ void gemm_f32_skinny(const SkinnyParams p) {
                 for (int q = 0; q < U; q++) {
                     const bool on = k + PK * q + kk4 < k_end;
 #pragma unroll
-                    for (int set = 0; set < W; set++) b.x[q][set] = ld4(rx, on ? x_off[set] : OOB_OFFSET, (k + PK * q) * 4);
+                    for (int set = 0; set < W; set++) b.x[q][set] = ld4<XA>(rx, on ? x_off[set] : OOB_OFFSET, (k + PK * q) * 4);
 #pragma unroll
                     for (int h = 0; h < H; h++) {
                         if constexpr (S_KIN) {
@@ -394,18 +403,23 @@ void gemm_f32_skinny(const SkinnyParams p) {
 // is X line 4 * (l >> 4) + v against S line l & 15).  A quarter of the 4 x 4 x 1 blocks' instructions per byte of X
 // for 16 short lines, the k classes add up inside the instruction (no lane exchange), and the lanes of a line's
 // outputs are 16 consecutive floats of C.  Fewer short lines than 16 are multiplied as zeros and not stored.
-//   X K-inner: a lane reads the 4 k at k0 + 4 * (l >> 4) of line l & 15 of each of its W sets of 16 lines (16 lines x
-//       64 bytes per instruction); the four floats feed four instructions.
+//   X K-inner: per set of 16 lines and 32 k two reads of 8 whole 128-byte lines each (a lane's 16 bytes are 4 k and
+//       feed four instructions); what the instruction wants 8 lanes away comes by a row rotation.  (Reading 16 lines x
+//       64 bytes per instruction, everything in place, is level with ordinary loads and loses with non-temporal
+//       ones, which keep nothing for the second half of a line: 223 us against 178 on 262144 x 16 x 1024.)
 //   X K-outer: a lane reads W consecutive lines at row k0 + 4 * (l >> 4) + m, m = 0 .. 3 (4 rows x 64 W bytes per
 //       instruction); its W floats feed W accumulators (lines W * i + e, i the MFMA's row).
 // ROWS: the short side is C's row index (C is 16 x L).  Then S is the instruction's first operand and X its second:
 // element v of the result in lane l is S line 4 * (l >> 4) + v against X line l & 15 -- the lanes of a store run
 // along a row of C.
 // G: groups of 16 short lines (1, or 2 for 20 ... 32 short lines: every value of X feeds G instructions).
-template <bool X_KIN, bool S_KIN, int W, int NW, bool ROWS, int G = 1, int U = (W == 4 ? 2 : 4)>
+// NT: X is read with non-temporal loads (see gemm_f32_skinny).
+template <bool X_KIN, bool S_KIN, int W, int NW, bool ROWS, int G = 1, bool NT = false, int U = (W == 4 ? 2 : 4)>
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny16(const SkinnyParams p) {
     static_assert(W == 2 || W == 4, "sets of 16 lines (K-inner X) or floats a lane reads of a row (K-outer X)");
+    static_assert(!NT || W == 4, "non-temporal reads: the long runs");
+    constexpr int XA = NT ? 2 : 0;
     static_assert(G == 1 || G == 2, "up to 32 short lines");
     constexpr int LINES = 16 * W, PK = 16;                 // U: 16-k panels per register buffer
     __shared__ float meet_lds[NW][W * G * 4][64];
@@ -457,34 +471,57 @@ void gemm_f32_skinny16(const SkinnyParams p) {
                        : __builtin_amdgcn_mfma_f32_16x16x4f32(xv, sv, acc, 0, 0, 0);
         };
         if constexpr (X_KIN) {
+            // Two reads per set of 16 lines and 32 k, each of 8 whole 128-byte lines: in read i the lane takes line
+            // 8 i + (r & 7) at the 4 k at 16 (r >> 3) + c4.  The instruction wants line r at c4 (first 16 k) and at
+            // 16 + c4 (second 16 k) in lane r: half of that is in place, the other half sits 8 lanes away in the
+            // other read's register -- one row rotation (DPP) per operand.
+            static_assert(U % 2 == 0, "panels of 32 k");
+            constexpr int UP = U / 2;
             const __amdgpu_buffer_rsrc_t rx = skinny_rsrc(p.X, (long long)p.x_lines * p.ldx * 4);
-            int x_off[W];
+            const int kh = 16 * (r >> 3) + c4;
+            int x_off[W][2];
 #pragma unroll
-            for (int set = 0; set < W; set++) x_off[set] = ((line0 + 16 * set + r) * p.ldx + c4) * 4;
-            struct Buf { sk_v4f x[U][W]; sk_v4f s[U][G]; };
+            for (int set = 0; set < W; set++)
+#pragma unroll
+                for (int i = 0; i < 2; i++) x_off[set][i] = ((line0 + 16 * set + 8 * i + (r & 7)) * p.ldx + kh) * 4;
+            struct Buf { sk_v4f x[UP][W][2]; sk_v4f s[UP][2][G]; };
             // a lane's 4 k at or beyond k_end are not read (what lies there is the next line, or another share)
             auto load = [&](Buf& b, int k) {
 #pragma unroll
-                for (int set = 0; set < W; set++)
+                for (int q = 0; q < UP; q++)
 #pragma unroll
-                    for (int q = 0; q < U; q++)          // (the halves of a 128-byte line one after the other)
-                        b.x[q][set] = ld4(rx, (k + PK * q + c4 < k_end) ? x_off[set] : OOB_OFFSET, (k + PK * q) * 4);
+                    for (int set = 0; set < W; set++)
 #pragma unroll
-                for (int q = 0; q < U; q++)
+                        for (int i = 0; i < 2; i++)
+                            b.x[q][set][i] = ld4<XA>(rx, (k + 32 * q + kh < k_end) ? x_off[set][i] : OOB_OFFSET, (k + 32 * q) * 4);
 #pragma unroll
-                    for (int g = 0; g < G; g++) b.s[q][g] = load_s(g, k + PK * q, k + PK * q + c4 < k_end);
+                for (int q = 0; q < UP; q++)
+#pragma unroll
+                    for (int h = 0; h < 2; h++)
+#pragma unroll
+                        for (int g = 0; g < G; g++) b.s[q][h][g] = load_s(g, k + 32 * q + 16 * h, k + 32 * q + 16 * h + c4 < k_end);
+            };
+            auto rotated = [](float keep, float take, bool upper) {      // lanes 8 .. 15 (upper) or 0 .. 7 of a row take `take` from 8 lanes away
+                const int k = __builtin_bit_cast(int, keep), t = __builtin_bit_cast(int, take);
+                return __builtin_bit_cast(float, upper ? __builtin_amdgcn_update_dpp(k, t, 0x128, 0xf, 0xc, false)
+                                                       : __builtin_amdgcn_update_dpp(k, t, 0x128, 0xf, 0x3, false));
             };
             auto compute = [&](const Buf& b) {
 #pragma unroll
-                for (int q = 0; q < U; q++)
+                for (int q = 0; q < UP; q++)
 #pragma unroll
-                    for (int m = 0; m < 4; m++)
+                    for (int h = 0; h < 2; h++)
 #pragma unroll
-                        for (int set = 0; set < W; set++)
+                        for (int m = 0; m < 4; m++)
 #pragma unroll
-                            for (int g = 0; g < G; g++) {
-                                const float xv = b.x[q][set][m], sv = b.s[q][g][m];
-                                mfma(d[set][g], xv, sv);
+                            for (int set = 0; set < W; set++) {
+                                const float x0 = b.x[q][set][0][m], x1 = b.x[q][set][1][m];
+                                const float xv = h == 0 ? rotated(x0, x1, true) : rotated(x1, x0, false);
+#pragma unroll
+                                for (int g = 0; g < G; g++) {
+                                    const float sv = b.s[q][h][g][m];
+                                    mfma(d[set][g], xv, sv);
+                                }
                             }
             };
             Buf b0, b1;
@@ -511,8 +548,8 @@ void gemm_f32_skinny16(const SkinnyParams p) {
                     const bool on = k + PK * q + c4 < k_end;
 #pragma unroll
                     for (int m = 0; m < 4; m++) {
-                        if constexpr (W == 4) b.x[q][m].v = ld4(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
-                        else b.x[q][m].v = ld2(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
+                        if constexpr (W == 4) b.x[q][m].v = ld4<XA>(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
+                        else b.x[q][m].v = ld2<XA>(rx, on ? x_off : OOB_OFFSET, (k + PK * q + m) * x_step);
                     }
 #pragma unroll
                     for (int g = 0; g < G; g++) b.s[q][g] = load_s(g, k + PK * q, on);
@@ -609,7 +646,7 @@ void gemm_f32_skinny16(const SkinnyParams p) {
 }
 
 template <bool X_KIN, bool S_KIN, int W, int NW, int G>
-hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream) {
+hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream, bool nt = false) {
     if ((p.ldc & 3) != 0 || ((size_t)p.C & 15) != 0) return hipErrorInvalidValue;
     constexpr int LINES = 16 * W;
     const long long units = ((long long)p.L + LINES - 1) / LINES;
@@ -619,6 +656,13 @@ hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream) {
     p.k_cut = p.K;
     const long long grid = shared ? units : (units + NW - 1) / NW;
     if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    if constexpr (W == 4) {
+        if (nt) {
+            if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G, true>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+            else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G, true>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+            return hipGetLastError();
+        }
+    }
     if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
@@ -628,7 +672,7 @@ hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream) {
 // SKINNY_MAX_CUTS); they meet through the stream's workspace of the balanced kernel -- without one (the stream
 // is being captured before it has one, the table is full) the run's K stays with one workgroup.
 template <bool X_KIN, bool S_KIN, int T, int W, int NW, int CL = 1>
-hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream, int cuts = 1) {
+hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream, int cuts = 1, bool nt = false) {
     constexpr int LINES = X_KIN ? 8 * W : 64 * W / CL;
     constexpr int SLOT = W * (T / 4) * 4 * (X_KIN ? 8 : 64 / CL);      // floats a workgroup leaves in the workspace
     const long long units = ((long long)p.L + LINES - 1) / LINES;
@@ -660,11 +704,22 @@ hipError_t launch_one(SkinnyParams p, bool shared, hipStream_t stream, int cuts 
             return hipGetLastError();
         }
     }
+    if constexpr (W == 4 && NW == 4 && CL == 1) {
+        if (nt) {
+            hipLaunchKernelGGL((gemm_f32_skinny<X_KIN, S_KIN, T, W, NW, CL, false, true>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+            return hipGetLastError();
+        }
+    }
     hipLaunchKernelGGL((gemm_f32_skinny<X_KIN, S_KIN, T, W, NW, CL>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
 
-thread_local int t_skinny_form = -1, t_skinny_cuts = 0;
+thread_local int t_skinny_form = -1, t_skinny_cuts = 0, t_skinny_nt = -1;
+constexpr long long SKINNY_NT_BYTES = 320LL << 20;     // long operands from this size on are read non-temporally
+
+static bool skinny_nt(const SkinnyParams& p) {
+    return t_skinny_nt >= 0 ? t_skinny_nt != 0 : (long long)p.L * p.K * 4 >= SKINNY_NT_BYTES;
+}
 
 // Which form (gemm_skinny_form's numbering): enough wavefronts on every compute unit with the widest reads that
 // allow it.  With too few runs of lines the wavefronts of a workgroup share a run and split K, sixteen of them
@@ -698,8 +753,8 @@ hipError_t launch_skinny(const SkinnyParams& p, hipStream_t stream) {
         case 0: return launch_one<X_KIN, S_KIN, T, W0, 4>(p, false, stream);
         case 1: return launch_one<X_KIN, S_KIN, T, W0, 4>(p, true, stream);
         case 2: return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
-        case 3: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, false, stream);
-        case 4: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, true, stream);
+        case 3: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, false, stream, 1, skinny_nt(p));
+        case 4: return launch_one<X_KIN, S_KIN, T, 4, 4>(p, true, stream, 1, skinny_nt(p));
         case 6:
             if constexpr (X_KIN) return launch_one<X_KIN, S_KIN, T, W0, 16>(p, true, stream);
             else return launch_one<X_KIN, S_KIN, T, 1, 16, 4>(p, true, stream);
@@ -726,7 +781,8 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
         // The 16-line blocks, measured against the 4 x 4 blocks on 32 MB ... 1 GiB operands: always for 12 or 16
         // short lines (16 x 65536 x 4096 192 - 268 -> 176 - 187 us), except 12 beside a long K-outer operand
         // (level); for 8 beside a K-inner long operand (65536 x 8 x 1024 50 -> 41 us) and beside a K-outer one up to
-        // 512 MiB (8192 x 8 x 4096 29.8 -> 23.9); not for 4 (level), nor under 32 lines per compute unit.
+        // 512 MiB (8192 x 8 x 4096 29.8 -> 23.9; 1 GiB, non-temporal reads: 154 us with the 4 x 4 blocks against
+        // 161); not for 4 (level), nor under 32 lines per compute unit.
         const int num_cu = gemm_device_num_cu();
         if (num_cu <= 0) return hipErrorNoDevice;
         const long long runs = ((long long)p.L + 63) / 64;
@@ -740,8 +796,8 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
     }
     if (T > 16 && (form < 8 || form > 11)) form = 9;        // (the 4 x 4 blocks stop at 16 short lines)
     switch (form) {     // the 16-line blocks: runs of 64 lines with the whole K, or shared; runs of 32
-        case 8: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, false, stream) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, false, stream);
-        case 9: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, true, stream) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, true, stream);
+        case 8: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, false, stream, skinny_nt(p)) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, false, stream, skinny_nt(p));
+        case 9: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, true, stream, skinny_nt(p)) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, true, stream, skinny_nt(p));
         case 10: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, false, stream) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, false, stream);
         case 11: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, true, stream) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, true, stream);
         default: break;
@@ -765,6 +821,9 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
 // 8 ... 11 = the 16-line blocks: 8 = a wavefront per run of 64 lines with the whole K, 9 = the four wavefronts of a
 // workgroup share a run, 10 and 11 = as 8 and 9 with runs of 32 lines; -1 = the automatic choice.
 void gemm_skinny_form(int form) {
+    t_skinny_nt = form >= 2000 ? 0 : form >= 1000 ? 1 : -1;      // 1000 + form: non-temporal reads of X, 2000 + form: none
+    if (form >= 1000) form %= 1000;
+    if (form == 999) form = -1;                                   // (1999 / 2999: the automatic form with that policy)
     t_skinny_cuts = form >= 100 ? form % 100 : 0;
     if (form >= 100) form = 7;
     t_skinny_form = (form >= 0 && form <= 11) ? form : -1;

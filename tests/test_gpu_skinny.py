@@ -113,6 +113,20 @@ def test_up_to_32_short_lines_bitwise(gpu, variant, thin, form):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
+@pytest.mark.parametrize("form", [1003, 1004, 1008, 1009, 1999, 2999])
+def test_non_temporal_reads_bitwise(gpu, variant, form):
+    """The long forms with the long operand read non-temporally (what the automatic choice does from 320 MiB on), forced
+    on small shapes."""
+    gpu.force_tile(SKINNY)
+    gpu.skinny_form(form)
+    for thin in (4, 7, 8, 13, 16, 24, 32):
+        if thin > 16 and form in (1003, 1004):
+            continue
+        check(gpu, variant, 5003, thin, 1028, 400 * thin + form + variant)
+        check(gpu, variant, thin, 40001, 100, 401 * thin + form + variant)
+
+
+@pytest.mark.parametrize("variant", [NN, T1, T2])
 def test_long_shapes_against_both_oracles(gpu, variant):
     """Uniform inputs at the benchmark's shapes, scaled down 4 x along the long side, within the FP32 tolerance
     (relative Frobenius error <= 1e-5, elements within 1e-4 * sqrt(K) * max|A| * max|B|); and the same launch
