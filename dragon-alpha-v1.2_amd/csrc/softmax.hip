@@ -7,9 +7,10 @@
 //     reads X once and writes Y once.  The reference runs three launches with two temporary
 //     buffers (row_max, row_softmax, div2D_field: CudaFloat32EngineBase.java:5738-5774) and moves
 //     the tensor five times; the optional scale folds the preceding sdiv launch in as well.
-// Both are bound by HBM.
+// Both are bound by HBM; tensors far larger than the Infinity Cache pass through non-temporally (stream_policy.h).
 #include <hip/hip_runtime.h>
 #include "runtime_internal.h"
+#include "stream_policy.h"
 #include <stdint.h>
 #include "../../include/dragon_hip_gemm.h"
 
@@ -18,18 +19,19 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 #pragma clang fp contract(off)
+template <bool NT>
 __global__ __launch_bounds__(256) void linear2D_kernel(float alpha, const float* __restrict__ X, float beta,
                                                        float* __restrict__ Y, int length4, int width, int stride) {
     const int step = gridDim.x * blockDim.x;
     for (int i4 = blockIdx.x * blockDim.x + threadIdx.x; i4 < length4; i4 += step) {
         const int index = i4 << 2;
-        v4f y = alpha * *(const v4f*)(X + index) + beta;
+        v4f y = alpha * dragon::stream_load4<NT>(X + index) + beta;
         const int c0 = index % stride;
         y.x *= (c0 + 0 < width) ? 1.0f : 0.0f;   // the reference multiplies by the 0/1 flag
         y.y *= (c0 + 1 < width) ? 1.0f : 0.0f;   // (Cuda_function/micro.cuh:61-65)
         y.z *= (c0 + 2 < width) ? 1.0f : 0.0f;
         y.w *= (c0 + 3 < width) ? 1.0f : 0.0f;
-        *(v4f*)(Y + index) = y;
+        dragon::stream_store4<NT>(Y + index, y);
     }
 }
 
@@ -49,7 +51,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // One wavefront per field; the field (at most 256*NV floats) stays in registers between the
 // three steps max -> exp and sum -> divide.  Four fields per workgroup.
-template <int NV>
+template <int NV, bool NT>
 __global__ __launch_bounds__(256) void softmax_wave_kernel(const float* __restrict__ X, float* __restrict__ Y,
                                                            int field_length, int row_lengthv, int width,
                                                            int stride, float scale) {
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const float* __restri
         const int i = (s * 64 + lane) * 4;
         v[s] = (v4f)(NEG_BIG);
         if (i < row_lengthv) {
-            const v4f t = *(const v4f*)(x + i) * scale;
+            const v4f t = dragon::stream_load4<NT>(x + i) * scale;
             const int c0 = i % stride;
 #pragma unroll
             for (int j = 0; j < 4; j++)
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256) void softmax_wave_kernel(const float* __restri
 #pragma unroll
     for (int s = 0; s < NV; s++) {
         const int i = (s * 64 + lane) * 4;
-        if (i < row_lengthv) *(v4f*)(y + i) = v[s] / sum;
+        if (i < row_lengthv) dragon::stream_store4<NT>(y + i, v[s] / sum);
     }
 }
 
@@ -146,8 +148,14 @@ int dragon_Cuda_function_linear2D(int64_t stream, float alpha, int64_t dX, float
     // one 16-byte element per thread, workgroups in address order: measured on a 1 GiB tensor in place 6.0 TB/s,
     // against 4.7 for 8192 workgroups that stride over the tensor (neighbours in time then touch addresses far apart)
     const int blocks = (length4 + 255) / 256;
-    hipLaunchKernelGGL(linear2D_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)(intptr_t)stream, alpha,
-                       (const float*)(intptr_t)dX, beta, (float*)(intptr_t)dY, length4, width, stride);
+    const float* X = (const float*)(intptr_t)dX;
+    float* Y = (float*)(intptr_t)dY;
+    if (dragon::stream_nt(X, Y, (long long)lengthv * 4))
+        hipLaunchKernelGGL(linear2D_kernel<true>, dim3(blocks), dim3(256), 0, (hipStream_t)(intptr_t)stream, alpha, X, beta, Y,
+                           length4, width, stride);
+    else
+        hipLaunchKernelGGL(linear2D_kernel<false>, dim3(blocks), dim3(256), 0, (hipStream_t)(intptr_t)stream, alpha, X, beta, Y,
+                           length4, width, stride);
     return hipGetLastError();
 }
 
@@ -162,9 +170,14 @@ int dragon_Cuda_reduce_softmax2D(int64_t stream, int64_t dX, int64_t dY, int32_t
     float* Y = (float*)(intptr_t)dY;
     dragon::split_ledger_touch(Y, (size_t)field_length * row_lengthv * 4);
     const dim3 grid4((field_length + 3) / 4), block(256);
-#define WAVE_CASE(NV)                                                                                    \
-    hipLaunchKernelGGL(softmax_wave_kernel<NV>, grid4, block, 0, s, X, Y, field_length, row_lengthv, width, \
-                       stride, scale)
+    const bool nt = dragon::stream_nt(X, Y, (long long)field_length * row_lengthv * 4);
+#define WAVE_CASE(NV)                                                                                              \
+    do {                                                                                                           \
+        if (nt) hipLaunchKernelGGL((softmax_wave_kernel<NV, true>), grid4, block, 0, s, X, Y, field_length, row_lengthv, \
+                                   width, stride, scale);                                                          \
+        else hipLaunchKernelGGL((softmax_wave_kernel<NV, false>), grid4, block, 0, s, X, Y, field_length, row_lengthv,   \
+                                width, stride, scale);                                                             \
+    } while (0)
     if (row_lengthv <= 256) WAVE_CASE(1);
     else if (row_lengthv <= 512) WAVE_CASE(2);
     else if (row_lengthv <= 1024) WAVE_CASE(4);

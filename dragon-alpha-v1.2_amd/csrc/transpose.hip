@@ -12,9 +12,10 @@
 //     plane go through LDS, so that the reads run along X's last dimension and the writes along
 //     Y's (transpose_last_kernel).  The reference's general kernel gathers element by element with
 //     strided stores (its own comments quote a third of the row-copy rate for it).
-// Both are bound by HBM: one read and one write of the tensor.
+// Both are bound by HBM: one read and one write of the tensor (non-temporal for large tensors, stream_policy.h).
 #include <hip/hip_runtime.h>
 #include "runtime_internal.h"
+#include "stream_policy.h"
 #include <stdint.h>
 #include "../../include/dragon_hip_gemm.h"
 
@@ -25,6 +26,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 struct Dims4 { int d[4]; };
 
 // rows of `stride` floats; X rows indexed (x0, x1, x2), two of them swapped in Y
+template <bool NT>
 __global__ __launch_bounds__(256) void transpose_rows_kernel(const float* __restrict__ X, float* __restrict__ Y,
                                                              Dims4 xd, Dims4 yd, int i1, int i2, int stride,
                                                              long long rows) {
@@ -41,13 +43,14 @@ __global__ __launch_bounds__(256) void transpose_rows_kernel(const float* __rest
         x[0] = (int)t;
         const int s = x[i1]; x[i1] = x[i2]; x[i2] = s;
         const long long yrow = ((long long)x[0] * yd.d[1] + x[1]) * yd.d[2] + x[2];
-        *(v4f*)(Y + yrow * stride + 4 * c4) = *(const v4f*)(X + row * stride + 4 * c4);
+        dragon::stream_store4<NT>(Y + yrow * stride + 4 * c4, dragon::stream_load4<NT>(X + row * stride + 4 * c4));
     }
 }
 
 // dimension a (0..2) swapped with the last one.  A workgroup moves one 64x64 tile of the
 // (x_a, x_3) plane for one value of the two other indices.
 constexpr int TP = 64;
+template <bool NT>
 __global__ __launch_bounds__(256) void transpose_last_kernel(const float* __restrict__ X, float* __restrict__ Y,
                                                              Dims4 xd, Dims4 yd, int a, int strideX, int strideY,
                                                              int tiles_p, int tiles_q) {
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(256) void transpose_last_kernel(const float* __rest
         x[a] = p0 + ly + i;
         v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
         if (x[a] < P && x[3] < strideX)
-            v = *(const v4f*)(X + (((long long)x[0] * xd.d[1] + x[1]) * xd.d[2] + x[2]) * strideX + x[3]);
+            v = dragon::stream_load4<NT>(X + (((long long)x[0] * xd.d[1] + x[1]) * xd.d[2] + x[2]) * strideX + x[3]);
         tile[ly + i][4 * lx + 0] = v.x; tile[ly + i][4 * lx + 1] = v.y;
         tile[ly + i][4 * lx + 2] = v.z; tile[ly + i][4 * lx + 3] = v.w;
     }
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(256) void transpose_last_kernel(const float* __rest
         if (y[a] < Q && y[3] < strideY) {
             const v4f v = {tile[4 * lx + 0][ly + i], tile[4 * lx + 1][ly + i], tile[4 * lx + 2][ly + i],
                            tile[4 * lx + 3][ly + i]};
-            *(v4f*)(Y + (((long long)y[0] * yd.d[1] + y[1]) * yd.d[2] + y[2]) * strideY + y[3]) = v;
+            dragon::stream_store4<NT>(Y + (((long long)y[0] * yd.d[1] + y[1]) * yd.d[2] + y[2]) * strideY + y[3], v);
         }
     }
 }
@@ -119,21 +122,26 @@ int transpose_launch(int64_t stream, int64_t dX, int64_t dY, Dims4 xd, int i1, i
     const float* X = (const float*)(intptr_t)dX;
     float* Y = (float*)(intptr_t)dY;
     dragon::split_ledger_touch(Y, (size_t)yd.d[0] * yd.d[1] * yd.d[2] * (size_t)strideY * 4);
+    const bool nt = dragon::stream_nt(X, Y, (long long)yd.d[0] * yd.d[1] * yd.d[2] * (long long)strideY * 4);
     if (i2 < 3) {
         if (strideX != strideY) return hipErrorInvalidValue;
         const long long rows = (long long)xd.d[0] * xd.d[1] * xd.d[2];
         const long long blocks = (rows * (strideX >> 2) + 255) / 256;   // one 16-byte element per thread, in address order
         if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(transpose_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1, i2,
-                           strideX, rows);
+        if (nt) hipLaunchKernelGGL(transpose_rows_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1, i2,
+                                   strideX, rows);
+        else hipLaunchKernelGGL(transpose_rows_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1, i2,
+                                strideX, rows);
     } else {
         const int tiles_p = (strideY + TP - 1) / TP;      // along Y's rows, pad included
         const int tiles_q = (xd.d[3] + TP - 1) / TP;
         const int o1 = (i1 == 0) ? 1 : 0, o2 = (i1 == 2) ? 1 : 2;
         const long long blocks = (long long)tiles_p * tiles_q * xd.d[o1] * xd.d[o2];
         if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(transpose_last_kernel, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1,
-                           strideX, strideY, tiles_p, tiles_q);
+        if (nt) hipLaunchKernelGGL(transpose_last_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1,
+                                   strideX, strideY, tiles_p, tiles_q);
+        else hipLaunchKernelGGL(transpose_last_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, X, Y, xd, yd, i1,
+                                strideX, strideY, tiles_p, tiles_q);
     }
     return hipGetLastError();
 }
