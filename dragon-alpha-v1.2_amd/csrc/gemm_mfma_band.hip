@@ -528,7 +528,7 @@ void gemm_f32_mfma_band_regs(const GemmParams p) {
     // and, where NEXT_J >= 0, fb's next contents read group by group as the values there have had their last use
     // (block NEXT_J of B buffer NEXT_P).
     auto block = [&](auto ic, auto jc, auto sic, auto sjc, auto njc, auto npc) __attribute__((always_inline)) {
-        constexpr int I = decltype(ic)::value, J = decltype(jc)::value, SI = decltype(sic)::value, SJ = decltype(sjc)::value;
+        constexpr int I = decltype(ic)::value, J = decltype(jc)::value;
         constexpr int NEXT_J = decltype(njc)::value;
         static_for<32>([&](auto sc) {
             constexpr int s2 = decltype(sc)::value;

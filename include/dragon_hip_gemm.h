@@ -83,9 +83,9 @@ int dragon_Cuda_matMul_matMulT2(const int64_t* streams, int32_t length,
  * unsplit product is faster than the slices plus their fold (its balanced kernel deals equal
  * shares of K to the compute units by itself; e.g. 1000 x 780 x 1532 with GridZ 2), it declines
  * the split: the whole product goes to C and Cbuf gets exact zeros, in the same launch, so that
- * SKbuf_summary afterwards leaves C as it is.  The same goes for a product whose C has 4 or 8
- * rows or columns (8 x 4096 x 4096 with GridZ 16): the kernel for such shapes cuts K among its
- * workgroups itself.  Where the split wins (256 x 256 x 131072 in 128 slices) the slices are
+ * SKbuf_summary afterwards leaves C as it is.  The same goes for a product whose C has at most 32
+ * rows or columns beside a long other side (8 x 4096 x 4096 with GridZ 16): the kernels for such
+ * shapes share K among their wavefronts and workgroups themselves.  Where the split wins (256 x 256 x 131072 in 128 slices) the slices are
  * computed as asked.
  * The library remembers a declined call (stream, Cbuf, C, GridZ-1, N*M): the SKbuf_summary call
  * with exactly these arguments on streams[0] -- the one the reference's host issues next,

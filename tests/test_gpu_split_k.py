@@ -184,7 +184,8 @@ def test_a_losing_split_is_declined(gpu, variant, shape_gz):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("shape_gz", [((8, 4096, 4096), 16), ((4100, 8, 2052), 8), ((8, 1000, 1028), 4), ((3000, 4, 516), 3)])
+@pytest.mark.parametrize("shape_gz", [((8, 4096, 4096), 16), ((4100, 8, 2052), 8), ((8, 1000, 1028), 4), ((3000, 4, 516), 3),
+                                      ((16, 8192, 1028), 4), ((8200, 32, 516), 2), ((9000, 8, 260), 2)])
 def test_the_split_of_a_skinny_product_is_declined(gpu, variant, shape_gz):
     """The host's policy splits the skinny products with few lines (8 x 4096 x 4096: GridZ 16).  The skinny kernel
     cuts K among its workgroups itself: the whole product goes to C through it -- the bits of the unsplit entry
