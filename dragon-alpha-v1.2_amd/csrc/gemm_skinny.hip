@@ -645,7 +645,7 @@ void gemm_f32_skinny16(const SkinnyParams p) {
     }
 }
 
-template <bool X_KIN, bool S_KIN, int W, int NW, int G>
+template <bool X_KIN, bool S_KIN, int W, int NW, int G, int U = (W == 4 ? 2 : 4)>
 hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream, bool nt = false) {
     if ((p.ldc & 3) != 0 || ((size_t)p.C & 15) != 0) return hipErrorInvalidValue;
     constexpr int LINES = 16 * W;
@@ -658,13 +658,13 @@ hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream, bool nt = 
     if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
     if constexpr (W == 4) {
         if (nt) {
-            if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G, true>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
-            else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G, true>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+            if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G, true, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+            else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G, true, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
             return hipGetLastError();
         }
     }
-    if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
-    else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G, false, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
+    else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G, false, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
     return hipGetLastError();
 }
 
