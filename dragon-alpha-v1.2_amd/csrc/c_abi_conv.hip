@@ -53,7 +53,7 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     if (num_cu <= 0) return hipErrorNoDevice;
     // A 1 x 1 filter at stride 1 without padding gathers nothing: Y[N*IH*IW][OC] = X[N*IH*IW][IC] * W[OC][IC]^T is the
     // plain A * B^T product, whose loaders have no tap arithmetic (128 x 32 x 32 x 256 -> 256: 137 -> 131 us).
-    if (FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW && dBias == 0 &&
+    if (FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW &&
         gemm_forced_tile() == TILE_AUTO) {
         GemmParams q = {};
         q.A = p.A; q.B = p.B; q.C = p.C;
@@ -62,7 +62,13 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
         q.ldb = IC; q.b_outer = OC; q.b_inner = IC;
         q.ldc = OC;
         q.nz = 1;
-        return gemm_launch(GEMM_T2, q, gemm_choose_tile(q.rows, q.cols, 1, q.k_total, num_cu, GEMM_T2), (hipStream_t)(intptr_t)streams[0]);
+        if (dBias == 0)
+            return gemm_launch(GEMM_T2, q, gemm_choose_tile(q.rows, q.cols, 1, q.k_total, num_cu, GEMM_T2), (hipStream_t)(intptr_t)streams[0]);
+        // with a bias row: the tile-per-workgroup kernels' epilogue (the shapes that stage through registers)
+        q.bias = p.bias; q.bias_rows = p.bias_rows; q.bias_width = p.bias_width;
+        const int t = gemm_choose_tile_per_workgroup(q.rows, q.cols, 1, q.k_total, num_cu, GEMM_T2);
+        if (!gemm_tile_is_dma(t & ~TILE_PAIRED) && (t & ~TILE_PAIRED) <= TILE_64x128_K32)
+            return gemm_launch_t2_biased(q, t, (hipStream_t)(intptr_t)streams[0]);
     }
     int tile = gemm_forced_tile() != TILE_AUTO ? gemm_forced_tile() : gemm_choose_tile_per_workgroup(p.rows, p.cols, 1, p.k_total, num_cu);
     const bool free_choice = gemm_forced_tile() == TILE_AUTO;   // a forced shape (tests, sweeps) is taken as it is

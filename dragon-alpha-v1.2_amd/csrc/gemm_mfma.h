@@ -229,6 +229,8 @@ void gemm_band_split(long long bands, int tiles_n, int num_cu, int& chunks, int&
 hipError_t gemm_launch_conv(const GemmParams& p, int tile, hipStream_t stream);
 // the GEMM_NN product with p.bias added in the epilogue (what gemm_launch forwards to when p.bias is set)
 hipError_t gemm_launch_nn_biased(const GemmParams& p, int tile, hipStream_t stream);
+// the GEMM_T2 product with p.bias added in the epilogue, tile-per-workgroup shapes 0 .. TILE_64x128_K32 (+ TILE_PAIRED)
+hipError_t gemm_launch_t2_biased(const GemmParams& p, int tile, hipStream_t stream);
 
 // Y[i] = alpha*X1[i] + beta*X2[i % row_lengthv] + gamma over lengthv floats laid out in rows of
 // `stride`, elements at or beyond `width` in a row written as zero.

@@ -226,6 +226,34 @@ def test_conv3D_at_the_reference_speed_test_shape(dh, gpu):
     assert np.linalg.norm(got - ref) <= 1e-5 * np.linalg.norm(ref)
 
 
+@pytest.mark.parametrize("shape", [(6, 6, 5, 7, 9), (16, 16, 8, 64, 128), (32, 32, 4, 256, 256), (9, 13, 3, 130, 36), (1, 1, 1, 1, 1)])
+def test_conv3D_1x1_takes_the_plain_product(dh, gpu, shape):
+    """A 1 x 1 filter at stride 1 without padding is the product X[N*IH*IW][IC] * W[OC][IC]^T and is sent to the
+    A * B^T kernels, with the bias row in their epilogue: bit for bit on integers, the biased form equal to the
+    plain one plus the row, the W1 entry points the same bits; with padding or a stride the gathering loader stays."""
+    IH, IW, N, IC, OC = shape
+    rng = np.random.default_rng(sum(shape))
+    X = rng.integers(-3, 4, (N, IH, IW, IC)).astype(np.float32)
+    W = rng.integers(-3, 4, (OC, 1, 1, IC)).astype(np.float32)
+    bias = rng.integers(-5, 6, OC).astype(np.float32)
+    R = oracle.conv3D(X, W, 1, 1, 0, 0)
+    Y, Yp = run_conv(dh, X, W, 1, 1, 0, 0)
+    assert np.array_equal(Y, R)
+    assert not Yp[N:].any() and not Yp[..., OC:].any()
+    Yb, Ybp = run_conv(dh, X, W, 1, 1, 0, 0, entry="biased", bias=bias)
+    assert np.array_equal(Yb, R + bias[None, None, None, :])
+    assert not Ybp[N:].any() and not Ybp[..., OC:].any()
+    Yw, _ = run_conv(dh, X, W, 1, 1, 0, 0, entry="W1")
+    assert np.array_equal(Yw, R)
+    Xu = rng.uniform(-1, 1, X.shape).astype(np.float32)
+    Wu = rng.uniform(-1, 1, W.shape).astype(np.float32)
+    Yu, _ = run_conv(dh, Xu, Wu, 1, 1, 0, 0)
+    ref = oracle.conv3D(Xu, Wu, 1, 1, 0, 0)
+    assert np.abs(Yu - ref).max() <= 1e-4 * np.sqrt(IC) and np.linalg.norm(Yu - ref) <= 1e-5 * np.linalg.norm(ref) + 1e-30
+    Ys, _ = run_conv(dh, X, W, 2, 1, 0, 0)
+    assert np.array_equal(Ys, oracle.conv3D(X, W, 2, 1, 0, 0))
+
+
 def test_conv3D_biased_equals_two_launches(dh, gpu):
     rng = np.random.default_rng(9)
     X = rng.uniform(-1, 1, (3, 10, 9, 7)).astype(np.float32)
