@@ -167,8 +167,9 @@ int gemm_choose_tile_per_workgroup(int rows, int cols, int nz, int k, int num_cu
     if (best == TILE_DMA_64x64_K32_S4 && variant != GEMM_T1 && k >= 512) best = TILE_64x64_K32;
     // The paired-stage form of the kernel, measured over 2048..4096 x 2048..4096 x K in all layouts: equal
     // at K = 256, 2-5 % faster at 512..1024, 3.5-8 % at 4096; slower on a short K (8 % at K = 64).  The two
-    // 256-row shapes spill in it and gain only from K = 2048 on.
-    if (best <= TILE_64x128_K32 && k >= ((best == TILE_256x64 || best == TILE_64x256) ? 2048 : 512))
+    // 256-row shapes spill in it and gain only from K = 2048 on.  With 128 x 128 tiles of 16 k it is ahead from
+    // K = 256 on wherever C is large (1.5 - 3.5 % on 4096^2 ... 131072 x 256 under K = 256 ... 448).
+    if (best <= TILE_64x128_K32 && k >= ((best == TILE_256x64 || best == TILE_64x256) ? 2048 : best == TILE_128x128 ? 256 : 512))
         best |= TILE_PAIRED;
     return best;
 }

@@ -22,7 +22,7 @@ extern "C" {
  * 15 = 128x128 and 16 = 64x64 with 16 k, 17 = 64x64 with 32 k per stage, staged global -> LDS
  * directly through four stage buffers.  Adding 256 to a shape 0..9 selects its paired-stage form
  * (stages run two by two with compile-time LDS buffers; what the automatic choice takes from
- * K = 512 on).  18..23 and 25: the balanced kernel (workgroups share the work in equal runs of LDS
+ * K = 512 on, 256 for shape 0).  18..23 and 25: the balanced kernel (workgroups share the work in equal runs of LDS
  * stages; taken for few tiles and a long K, for large products, their K slices and large
  * convolutions): 18 = 64x64, 19 = 128x64, 20 = 64x128, 21 = 128x128 with one workgroup per
  * compute unit, 22 = 64x64 and 23 = 128x64 with two, 25 = 256x64 with one.  24: the band kernel

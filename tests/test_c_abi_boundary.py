@@ -228,7 +228,7 @@ def test_tile_choice_on_the_documented_shapes(dh):
     if ct(NN, *shape) in (5 + P, 9 + P):
         assert ct(NN, *shape) == 9 + P and ct(T2, *shape) == 9 + P and ct(T1, *shape) == 5 + P
     assert ct(NN, 3072, 3072, 1, 512) == 7 + P                  # nine 64x64 tiles per unit: still 32-k stages
-    assert ct(NN, 4096, 4096, 1, 256) == 0 and ct(NN, 4096, 4096, 1, 512) == P    # a short K keeps the plain form
+    assert ct(NN, 4096, 4096, 1, 252) == 0 and ct(NN, 4096, 4096, 1, 256) == P    # a short K keeps the plain form
     dh.force_tile(7)
     assert ct(NN, 4096, 4096, 1, 4096) == 7                     # a forced shape is reported as it is
     dh.force_tile(-1)
