@@ -418,7 +418,7 @@ template <bool X_KIN, bool S_KIN, int W, int NW, bool ROWS, int G = 1, bool NT =
 __global__ __launch_bounds__(NW * 64)
 void gemm_f32_skinny16(const SkinnyParams p) {
     static_assert(W == 2 || W == 4, "sets of 16 lines (K-inner X) or floats a lane reads of a row (K-outer X)");
-    static_assert(!NT || W == 4, "non-temporal reads: the long runs");
+
     constexpr int XA = NT ? 2 : 0;
     static_assert(G == 1 || G == 2, "up to 32 short lines");
     constexpr int LINES = 16 * W, PK = 16;                 // U: 16-k panels per register buffer
@@ -427,10 +427,11 @@ void gemm_f32_skinny16(const SkinnyParams p) {
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const bool shared = p.k_share > 0;
     const int wg = shared ? xcd_contiguous_id(blockIdx.x, gridDim.x) : 0;
-    const int unit = shared ? wg : blockIdx.x * NW + wave;
+    const int cut = p.k_cuts > 1 ? wg / p.units : 0;           // neighbouring workgroups: neighbouring lines, the same k
+    const int unit = shared ? wg - cut * p.units : blockIdx.x * NW + wave;
     const int line0 = unit * LINES;
-    const int k_begin = shared ? wave * p.k_share : 0;
-    const int k_end = shared ? min(p.K, k_begin + p.k_share) : p.K;
+    const int k_begin = shared ? cut * p.k_cut + wave * p.k_share : 0;
+    const int k_end = shared ? min(min(p.K, (cut + 1) * p.k_cut), k_begin + p.k_share) : p.K;
     const int r = lane & 15, c4 = 4 * (lane >> 4);
 
     const __amdgpu_buffer_rsrc_t rs = skinny_rsrc(p.S, S_KIN ? (long long)p.s_lines * p.lds * 4 : ((long long)(p.K - 1) * p.lds + p.s_lines) * 4);
@@ -603,6 +604,53 @@ void gemm_f32_skinny16(const SkinnyParams p) {
                     for (int w = 1; w < NW; w++) sum += meet_lds[w][(a * G + g) * 4 + v][lane];
                     d[a][g][v] = sum;
                 }
+        if constexpr (W == 2 && NW == 4) if (p.k_cuts > 1) {    // the 32-line runs only
+            // The workgroups that cut this run's K meet in memory exactly as in gemm_f32_skinny: every one leaves
+            // its sum in its slot and is counted; whoever is counted last adds the slots in k order and stores.
+            constexpr int ACC = W * G * 4;
+            float* const slots = p.ws + (size_t)unit * p.k_cuts * (ACC * 64);
+            float* const mine = slots + (size_t)cut * (ACC * 64) + lane;
+#pragma unroll
+            for (int a = 0; a < W; a++)
+#pragma unroll
+                for (int g = 0; g < G; g++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const float value = d[a][g][v];
+                        __hip_atomic_store(mine + ((a * G + g) * 4 + v) * 64, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            asm volatile("" ::: "memory");
+            int arrived = 0;
+            if (lane == 0) {
+                arrived = atomicAdd(p.count + unit, 1);
+                if (arrived == p.k_cuts - 1) atomicExch(p.count + unit, 0);     // zero again for the next launch
+            }
+            arrived = __builtin_amdgcn_readfirstlane(arrived);
+            if (arrived != p.k_cuts - 1) return;
+            asm volatile("" ::: "memory");
+            // eight outputs of a lane at a time: every cut's floats of them are read before any is added
+#pragma unroll
+            for (int base = 0; base < ACC; base += 8) {
+                float part[SKINNY_MAX_CUTS][8];
+#pragma unroll
+                for (int c = 0; c < SKINNY_MAX_CUTS; c++)
+                    if (c < p.k_cuts) {
+#pragma unroll
+                        for (int i = 0; i < 8; i++)
+                            part[c][i] = __hip_atomic_load(slots + (size_t)c * (ACC * 64) + (base + i) * 64 + lane,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float sum = part[0][i];
+#pragma unroll
+                    for (int c = 1; c < SKINNY_MAX_CUTS; c++)
+                        if (c < p.k_cuts) sum += part[c][i];
+                    d[(base + i) / (G * 4)][((base + i) / 4) % G][(base + i) % 4] = sum;
+                }
+            }
+        }
     }
 #pragma unroll
     for (int g = 0; g < G; g++) {
@@ -645,18 +693,36 @@ void gemm_f32_skinny16(const SkinnyParams p) {
     }
 }
 
+// cuts > 1 (the shared 32-line runs only): that many workgroups per run take a part of K each and meet through the
+// stream's workspace, as in launch_one below
 template <bool X_KIN, bool S_KIN, int W, int NW, int G, int U = (W == 4 ? 2 : 4)>
-hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream, bool nt = false) {
+hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream, bool nt = false, int cuts = 1) {
     if ((p.ldc & 3) != 0 || ((size_t)p.C & 15) != 0) return hipErrorInvalidValue;
     constexpr int LINES = 16 * W;
+    constexpr int SLOT = W * G * 4 * 64;       // floats a workgroup leaves in the workspace
     const long long units = ((long long)p.L + LINES - 1) / LINES;
     p.k_share = shared ? ((p.K + NW - 1) / NW + 31) / 32 * 32 : 0;
     p.units = (int)units;
     p.k_cuts = 1;
     p.k_cut = p.K;
-    const long long grid = shared ? units : (units + NW - 1) / NW;
+    long long grid = shared ? units : (units + NW - 1) / NW;
+    if (shared && cuts > 1 && W == 2 && NW == 4 && units <= 65536) {
+        if (cuts > SKINNY_MAX_CUTS) cuts = SKINNY_MAX_CUTS;
+        const int k_cut = ((p.K + cuts - 1) / cuts + 32 * NW - 1) / (32 * NW) * (32 * NW);
+        const int real = (p.K + k_cut - 1) / k_cut;
+        size_t floats = 0;
+        float* ws = real > 1 ? gemm_streamk_workspace(stream, &floats) : nullptr;
+        if (ws != nullptr && 65536 + (size_t)units * real * SLOT <= floats) {
+            p.k_cuts = real;
+            p.k_cut = k_cut;
+            p.k_share = k_cut / NW;
+            p.count = (int*)ws;          // the workspace's arrival counters, zero between launches
+            p.ws = ws + 65536;
+            grid = units * real;
+        }
+    }
     if (grid <= 0 || grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    if constexpr (W == 4) {
+    {
         if (nt) {
             if (p.out_rows) hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, true, G, true, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
             else hipLaunchKernelGGL((gemm_f32_skinny16<X_KIN, S_KIN, W, NW, false, G, true, U>), dim3((unsigned)grid), dim3(NW * 64), 0, stream, p);
@@ -798,8 +864,19 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
     switch (form) {     // the 16-line blocks: runs of 64 lines with the whole K, or shared; runs of 32
         case 8: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, false, stream, skinny_nt(p)) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, false, stream, skinny_nt(p));
         case 9: return T > 16 ? launch_16<X_KIN, S_KIN, 4, 4, 2>(p, true, stream, skinny_nt(p)) : launch_16<X_KIN, S_KIN, 4, 4, 1>(p, true, stream, skinny_nt(p));
-        case 10: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, false, stream) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, false, stream);
-        case 11: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, true, stream) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, true, stream);
+        case 10: return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, false, stream, skinny_nt(p)) : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, false, stream, skinny_nt(p));
+        case 11: {
+            // at most three runs per four compute units under a long K: K is cut across workgroups as well, a workgroup
+            // per unit (16 x 4096 x 32768: 173 - 180 -> 105 - 115 us, 16 x 4096 x 8192: 46 -> 26 - 27; two workgroups per
+            // unit measured 0 - 15 % behind that, and 250 runs are better left whole)
+            const int num_cu = gemm_device_num_cu();
+            const long long runs32 = ((long long)p.L + 31) / 32;
+            int cuts = t_skinny_cuts > 0 ? t_skinny_cuts : 1;
+            if (t_skinny_cuts == 0 && t_skinny_form < 0 && num_cu > 0 && 4 * runs32 <= 3LL * num_cu && p.K >= 2048)
+                cuts = (int)((num_cu + runs32 - 1) / runs32);
+            return T > 16 ? launch_16<X_KIN, S_KIN, 2, 4, 2>(p, true, stream, skinny_nt(p), cuts)
+                          : launch_16<X_KIN, S_KIN, 2, 4, 1>(p, true, stream, skinny_nt(p), cuts);
+        }
         default: break;
     }
     switch (T) {
@@ -819,13 +896,15 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
 // 5 and 6 = as 2 with runs of 32 and 16 lines of a K-outer operand (two and four classes of k among the lanes;
 // K-inner: as 2), 7 = as 1 with K cut across workgroups too (two workgroups per compute unit; 100 + c: c cuts);
 // 8 ... 11 = the 16-line blocks: 8 = a wavefront per run of 64 lines with the whole K, 9 = the four wavefronts of a
-// workgroup share a run, 10 and 11 = as 8 and 9 with runs of 32 lines; -1 = the automatic choice.
+// workgroup share a run, 10 and 11 = as 8 and 9 with runs of 32 lines (200 + c: as 11 with c cuts of K across
+// workgroups); -1 = the automatic choice.
 void gemm_skinny_form(int form) {
     t_skinny_nt = form >= 2000 ? 0 : form >= 1000 ? 1 : -1;      // 1000 + form: non-temporal reads of X, 2000 + form: none
     if (form >= 1000) form %= 1000;
     if (form == 999) form = -1;                                   // (1999 / 2999: the automatic form with that policy)
     t_skinny_cuts = form >= 100 ? form % 100 : 0;
-    if (form >= 100) form = 7;
+    if (form >= 200) form = 11;                                   // 200 + c: the 16-line blocks' 32-line runs with c cuts of K
+    else if (form >= 100) form = 7;
     t_skinny_form = (form >= 0 && form <= 11) ? form : -1;
 }
 
@@ -834,7 +913,8 @@ static bool skinny_short(int n) { return n >= 4 && n <= 32 && n % 4 == 0; }
 
 // 4 or 8 short lines: every layout from 256 lines on.  12 or 16: from 16 lines of the long operand per compute unit
 // on (4096 x 16 x 4096 20 - 24 us against the tile kernels' 24; 2048 x 16 x 8192 33 - 45 against 24 - 26).  20 ... 32:
-// from 32 lines per compute unit on and a K of at least 256 (8192 x 32 x 4096 31 - 35 us against 39 - 41).
+// from 32 lines per compute unit on and a K of at least 256 (8192 x 32 x 4096 31 - 35 us against 39 - 41), from 16
+// lines per unit on under a K of 2048 or more.
 int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_cu) {
     (void)variant;
     if (nz != 1) return -1;
@@ -844,7 +924,9 @@ int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_c
     const int t = thin_cols ? cols : rows;
     if (t <= 8) return TILE_SKINNY;
     if (t > 16 && k < 256) return -1;      // (16384 x 32 x 128: 8.1 us against the balanced kernel's 5.2)
-    return (long long)(thin_cols ? rows : cols) >= (t <= 16 ? 16LL : 32LL) * num_cu ? TILE_SKINNY : -1;
+    // (with a K of 2048 or more, which is cut across workgroups, 20 ... 32 short lines also from 16 lines per unit on:
+    // 4096 x 32 x 8192 36 - 38 us against 39 - 44)
+    return (long long)(thin_cols ? rows : cols) >= (t <= 16 || k >= 2048 ? 16LL : 32LL) * num_cu ? TILE_SKINNY : -1;
 }
 
 // True where the product is one for the skinny kernel: one unsplit 2-D product (a bias row on A*B only) whose C has

@@ -50,6 +50,7 @@ def test_the_automatic_choice_names_the_kernel(gpu):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
         for (rows, cols) in ((8188, 32), (32, 4096), (65536, 36), (40, 65536)):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) != SKINNY
+        assert gpu.choose_tile(variant, 4096, 32, 1, 2048, cu) == SKINNY and gpu.choose_tile(variant, 4092, 32, 1, 2048, cu) != SKINNY
         assert gpu.choose_tile(variant, 65536, 32, 1, 252, cu) != SKINNY and gpu.choose_tile(variant, 65536, 16, 1, 252, cu) == SKINNY
     # not skinny enough, too short, or a batch / K slices
     for (rows, cols, nz) in ((65536, 36, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (16, 252, 1), (65536, 4, 2), (4, 65536, 3)):
@@ -58,7 +59,7 @@ def test_the_automatic_choice_names_the_kernel(gpu):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108, 8, 9, 10, 11])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108, 8, 9, 10, 11, 203, 208])
 @pytest.mark.parametrize("thin", [1, 2, 3, 4, 5, 7, 8, 9, 12, 13, 16])
 def test_thin_columns_bitwise(gpu, variant, thin, form):
     """C of 1 ... 16 columns (stored 4, 8, 12 or 16) under row counts around the 16, 64 and 256 lines a wavefront takes,
@@ -72,7 +73,7 @@ def test_thin_columns_bitwise(gpu, variant, thin, form):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108, 8, 9, 10, 11])
+@pytest.mark.parametrize("form", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 103, 108, 8, 9, 10, 11, 203, 208])
 @pytest.mark.parametrize("thin", [1, 3, 4, 6, 8, 10, 12, 15, 16])
 def test_thin_rows_bitwise(gpu, variant, thin, form):
     gpu.skinny_form(form)
@@ -88,7 +89,7 @@ def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
     """K around the k rows / 32-k panels of a register buffer, the 4-k chunks of a lane, the shares of a K split
     between 4 or 16 wavefronts; in every form."""
     gpu.force_tile(SKINNY)
-    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108, 8, 9, 10, 11):
+    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108, 8, 9, 10, 11, 202, 207):
         gpu.skinny_form(form)
         check(gpu, variant, 700, 4, K, 3000 + K + variant)
         check(gpu, variant, 8, 900, K, 4000 + K + variant)
@@ -101,7 +102,7 @@ def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
 
 
 @pytest.mark.parametrize("variant", [NN, T1, T2])
-@pytest.mark.parametrize("form", [-1, 8, 9, 10, 11])
+@pytest.mark.parametrize("form", [-1, 8, 9, 10, 11, 204])
 @pytest.mark.parametrize("thin", [17, 20, 23, 24, 28, 29, 32])
 def test_up_to_32_short_lines_bitwise(gpu, variant, thin, form):
     """Two groups of 16 short lines through the 16 x 16 x 4 blocks, both orientations of C."""
@@ -152,6 +153,9 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
     for (N, M, K) in ((16, 4096, 2048), (1000, 12, 3000)):
         check(gpu, variant, N, M, K, 700 + N + M + K + variant)
     gpu.force_tile(-1)
+    # 12 ... 32 short lines beside 4096 ... 8191 lines under a K of 2048 or more: the 16 x 16 x 4 blocks' 32-line runs, cut
+    for (N, M, K) in ((16, 4100, 2052), (5000, 12, 4096), (8188, 32, 2048), (24, 8000, 2500)):
+        check(gpu, variant, N, M, K, 800 + N + M + K + variant)
     rng = np.random.default_rng(31 + variant)
     A, B = logical_operands(variant, rng, 8, 4096, 4096)
     first, _ = gpu_matmul_2d(gpu, variant, A, B)
