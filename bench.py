@@ -424,17 +424,18 @@ def main():
 
     if "skinny" in extra:
         # a C of 4 ... 32 columns (or rows) under a long other side: the long operand is read once, so the figure that
-        # matters is bytes per second against the 8 TB/s of HBM.  The operands of the first three shapes fit or nearly
-        # fit the 256 MB Infinity Cache (134 ... 268 MB); the 1 GiB ones do not.
+        # matters is bytes per second against the 8 TB/s of HBM.  The operands of the first seven shapes fit or nearly
+        # fit the 256 MB Infinity Cache (134 ... 268 MB); the 1 GiB ones and the last (512 MiB in 4096 lines) do not.
         log("skinny products ...")
         shapes = [(65536, 4, 1024), (8192, 8, 4096), (4, 65536, 1024), (8, 8192, 4096), (65536, 16, 1024), (16, 8192, 4096),
                   (65536, 32, 1024), (262144, 4, 1024), (262144, 8, 1024), (4, 262144, 1024), (8, 65536, 4096),
-                  (262144, 16, 1024), (16, 65536, 4096), (262144, 32, 1024), (32, 65536, 4096)]
+                  (262144, 16, 1024), (16, 65536, 4096), (262144, 32, 1024), (32, 65536, 4096), (16, 4096, 32768)]
         nl = max(max(r, c) * k for r, c, k in shapes)
         g = synthetic.stream_for(9)
         block = g.normal((1 << 24,), 0.0, 1.0)          # the long operand repeats a 64 MiB block of normals
         dL = dh.DeviceArray(np.tile(block, (nl + block.size - 1) // block.size)[:nl])
-        dS, dC = dh.DeviceArray(g.normal((32 * 4096,), 0.0, 1.0)), dh.DeviceArray(size=32 * 262144)
+        dS = dh.DeviceArray(g.normal((max(min(r, c) * k for r, c, k in shapes),), 0.0, 1.0))
+        dC = dh.DeviceArray(size=max(r * c for r, c, k in shapes))
         del block
         for (r, c, k) in shapes:
             long_is_a = r > c
