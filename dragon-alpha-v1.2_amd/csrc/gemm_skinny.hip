@@ -854,7 +854,10 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
         const long long runs = ((long long)p.L + 63) / 64;
         bool blocks16 = false;
         if (T >= 12) blocks16 = X_KIN || T >= 16 || p.L < 256LL * num_cu;
-        else if (T == 8) blocks16 = p.L >= 32LL * num_cu && (X_KIN || (long long)p.L * p.K <= (1LL << 27));
+        // (8 short lines over 8 ... 32 lines per unit under a long K: the 32-line runs with K cut across workgroups,
+        // 8 x 4096 x 32768 108 - 140 -> 97 - 112 us, 8 x 2048 x 16384 33 - 37 -> 25)
+        else if (T == 8) blocks16 = (p.L >= 32LL * num_cu && (X_KIN || (long long)p.L * p.K <= (1LL << 27))) ||
+                                    (p.L >= 8LL * num_cu && p.L < 32LL * num_cu && p.K >= 2048);
         if (blocks16) {
             if (p.K < 128) form = runs >= 4LL * num_cu ? 8 : 10;
             else form = runs >= 4LL * num_cu ? (X_KIN ? 9 : 8) : runs >= num_cu ? 9 : 11;
@@ -914,7 +917,7 @@ static bool skinny_short(int n) { return n >= 4 && n <= 32 && n % 4 == 0; }
 // 4 or 8 short lines: every layout from 256 lines on.  12 or 16: from 16 lines of the long operand per compute unit
 // on (4096 x 16 x 4096 20 - 24 us against the tile kernels' 24; 2048 x 16 x 8192 33 - 45 against 24 - 26).  20 ... 32:
 // from 32 lines per compute unit on and a K of at least 256 (8192 x 32 x 4096 31 - 35 us against 39 - 41), from 16
-// lines per unit on under a K of 2048 or more.
+// lines per unit on under a K of 2048 or more; 12 ... 32 under such a K from 8 lines per unit on.
 int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_cu) {
     (void)variant;
     if (nz != 1) return -1;
@@ -924,9 +927,9 @@ int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_c
     const int t = thin_cols ? cols : rows;
     if (t <= 8) return TILE_SKINNY;
     if (t > 16 && k < 256) return -1;      // (16384 x 32 x 128: 8.1 us against the balanced kernel's 5.2)
-    // (with a K of 2048 or more, which is cut across workgroups, 20 ... 32 short lines also from 16 lines per unit on:
-    // 4096 x 32 x 8192 36 - 38 us against 39 - 44)
-    return (long long)(thin_cols ? rows : cols) >= (t <= 16 || k >= 2048 ? 16LL : 32LL) * num_cu ? TILE_SKINNY : -1;
+    // (with a K of 2048 or more, which is cut across workgroups, from 8 lines per unit on: 2048 x 16 x 8192 16 - 17 us
+    // against 25 - 26, 4096 x 32 x 8192 36 - 38 against 39 - 44)
+    return (long long)(thin_cols ? rows : cols) >= (k >= 2048 ? 8LL : t <= 16 ? 16LL : 32LL) * num_cu ? TILE_SKINNY : -1;
 }
 
 // True where the product is one for the skinny kernel: one unsplit 2-D product (a bias row on A*B only) whose C has

@@ -50,7 +50,8 @@ def test_the_automatic_choice_names_the_kernel(gpu):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) == SKINNY
         for (rows, cols) in ((8188, 32), (32, 4096), (65536, 36), (40, 65536)):
             assert gpu.choose_tile(variant, rows, cols, 1, 1024, cu) != SKINNY
-        assert gpu.choose_tile(variant, 4096, 32, 1, 2048, cu) == SKINNY and gpu.choose_tile(variant, 4092, 32, 1, 2048, cu) != SKINNY
+        assert gpu.choose_tile(variant, 2048, 32, 1, 2048, cu) == SKINNY and gpu.choose_tile(variant, 2044, 32, 1, 2048, cu) != SKINNY
+        assert gpu.choose_tile(variant, 16, 2048, 1, 4096, cu) == SKINNY and gpu.choose_tile(variant, 16, 2048, 1, 2044, cu) != SKINNY
         assert gpu.choose_tile(variant, 65536, 32, 1, 252, cu) != SKINNY and gpu.choose_tile(variant, 65536, 16, 1, 252, cu) == SKINNY
     # not skinny enough, too short, or a batch / K slices
     for (rows, cols, nz) in ((65536, 36, 1), (252, 4, 1), (4, 252, 1), (8, 8, 1), (16, 252, 1), (65536, 4, 2), (4, 65536, 3)):
@@ -154,7 +155,7 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
         check(gpu, variant, N, M, K, 700 + N + M + K + variant)
     gpu.force_tile(-1)
     # 12 ... 32 short lines beside 4096 ... 8191 lines under a K of 2048 or more: the 16 x 16 x 4 blocks' 32-line runs, cut
-    for (N, M, K) in ((16, 4100, 2052), (5000, 12, 4096), (8188, 32, 2048), (24, 8000, 2500)):
+    for (N, M, K) in ((16, 4100, 2052), (5000, 12, 4096), (8188, 32, 2048), (24, 8000, 2500), (2048, 16, 4100), (8, 3000, 2048), (28, 2100, 3000)):
         check(gpu, variant, N, M, K, 800 + N + M + K + variant)
     rng = np.random.default_rng(31 + variant)
     A, B = logical_operands(variant, rng, 8, 4096, 4096)
