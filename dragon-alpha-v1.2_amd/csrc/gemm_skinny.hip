@@ -56,6 +56,7 @@ struct SkinnyParams {
 typedef float sk_v4f __attribute__((ext_vector_type(4)));
 typedef float sk_v2f __attribute__((ext_vector_type(2)));
 constexpr int SKINNY_MAX_CUTS = 8;    // workgroups that cut one run's K
+constexpr int SKINNY16_MAX_CUTS = 16; // the same for the 32-line runs of the 16 x 16 x 4 kernel
 constexpr int SKINNY_STAGED_FLOATS = 12288;   // of a K-inner short operand in LDS (48 KiB)
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t skinny_rsrc(const float* base, long long bytes) {
@@ -629,23 +630,23 @@ void gemm_f32_skinny16(const SkinnyParams p) {
             arrived = __builtin_amdgcn_readfirstlane(arrived);
             if (arrived != p.k_cuts - 1) return;
             asm volatile("" ::: "memory");
-            // eight outputs of a lane at a time: every cut's floats of them are read before any is added
+            // four outputs of a lane at a time: every cut's floats of them are read before any is added
 #pragma unroll
-            for (int base = 0; base < ACC; base += 8) {
-                float part[SKINNY_MAX_CUTS][8];
+            for (int base = 0; base < ACC; base += 4) {
+                float part[SKINNY16_MAX_CUTS][4];
 #pragma unroll
-                for (int c = 0; c < SKINNY_MAX_CUTS; c++)
+                for (int c = 0; c < SKINNY16_MAX_CUTS; c++)
                     if (c < p.k_cuts) {
 #pragma unroll
-                        for (int i = 0; i < 8; i++)
+                        for (int i = 0; i < 4; i++)
                             part[c][i] = __hip_atomic_load(slots + (size_t)c * (ACC * 64) + (base + i) * 64 + lane,
                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
+                for (int i = 0; i < 4; i++) {
                     float sum = part[0][i];
 #pragma unroll
-                    for (int c = 1; c < SKINNY_MAX_CUTS; c++)
+                    for (int c = 1; c < SKINNY16_MAX_CUTS; c++)
                         if (c < p.k_cuts) sum += part[c][i];
                     d[(base + i) / (G * 4)][((base + i) / 4) % G][(base + i) % 4] = sum;
                 }
@@ -707,7 +708,7 @@ hipError_t launch_16(SkinnyParams p, bool shared, hipStream_t stream, bool nt = 
     p.k_cut = p.K;
     long long grid = shared ? units : (units + NW - 1) / NW;
     if (shared && cuts > 1 && W == 2 && NW == 4 && units <= 65536) {
-        if (cuts > SKINNY_MAX_CUTS) cuts = SKINNY_MAX_CUTS;
+        if (cuts > SKINNY16_MAX_CUTS) cuts = SKINNY16_MAX_CUTS;
         const int k_cut = ((p.K + cuts - 1) / cuts + 32 * NW - 1) / (32 * NW) * (32 * NW);
         const int real = (p.K + k_cut - 1) / k_cut;
         size_t floats = 0;
@@ -854,10 +855,13 @@ hipError_t launch_skinny_t(const SkinnyParams& p, int T, hipStream_t stream) {
         const long long runs = ((long long)p.L + 63) / 64;
         bool blocks16 = false;
         if (T >= 12) blocks16 = X_KIN || T >= 16 || p.L < 256LL * num_cu;
-        // (8 short lines over 8 ... 32 lines per unit under a long K: the 32-line runs with K cut across workgroups,
-        // 8 x 4096 x 32768 108 - 140 -> 97 - 112 us, 8 x 2048 x 16384 33 - 37 -> 25)
+        // (8 short lines over fewer than 32 lines per unit under a long K: the 32-line runs with K cut across
+        // workgroups, 8 x 4096 x 32768 108 - 140 -> 97 - 112 us, 8 x 2048 x 16384 33 - 37 -> 25, 8 x 1024 x 65536
+        // 64 - 130 -> 44 - 46)
         else if (T == 8) blocks16 = (p.L >= 32LL * num_cu && (X_KIN || (long long)p.L * p.K <= (1LL << 27))) ||
-                                    (p.L >= 8LL * num_cu && p.L < 32LL * num_cu && p.K >= 2048);
+                                    (p.L < 32LL * num_cu && p.K >= 2048);
+        // (4 short lines: only the very few lines under a very long K, 4 x 1024 x 65536 48 - 77 -> 42 - 45 us)
+        else if (T == 4) blocks16 = p.L <= 8LL * num_cu && p.K >= 8192;
         if (blocks16) {
             if (p.K < 128) form = runs >= 4LL * num_cu ? 8 : 10;
             else form = runs >= 4LL * num_cu ? (X_KIN ? 9 : 8) : runs >= num_cu ? 9 : 11;

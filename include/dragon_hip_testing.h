@@ -44,7 +44,7 @@ void dragon_gemm_force_tile(int32_t tile);
  * workspace); 8 ... 11 = 16x16x4 MFMA blocks (16 lines against all short lines per instruction; what the automatic
  * choice takes for 12 or 16 short lines and for most products with 8): 8 = a wavefront per run of 64 lines with the
  * whole K, 9 = the four wavefronts of a workgroup share a run, 10 and 11 = as 8 and 9 with runs of 32 lines
- * (200 + c: as 11 with K cut across c workgroups per run, at most 8; needs the stream's workspace);
+ * (200 + c: as 11 with K cut across c workgroups per run, at most 16; needs the stream's workspace);
  * -1 restores the automatic choice.  Adding 1000 makes the long forms (3, 4, 8, 9) read the long operand with
  * non-temporal loads, adding 2000 with ordinary ones (automatic: non-temporal from 320 MiB on); 1999 and 2999 are
  * the automatic form with that policy. */

@@ -90,7 +90,7 @@ def test_every_kind_of_k_tail_bitwise(gpu, variant, K):
     """K around the k rows / 32-k panels of a register buffer, the 4-k chunks of a lane, the shares of a K split
     between 4 or 16 wavefronts; in every form."""
     gpu.force_tile(SKINNY)
-    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108, 8, 9, 10, 11, 202, 207):
+    for form in (0, 1, 2, 3, 4, 5, 6, 7, 102, 105, 108, 8, 9, 10, 11, 202, 207, 216):
         gpu.skinny_form(form)
         check(gpu, variant, 700, 4, K, 3000 + K + variant)
         check(gpu, variant, 8, 900, K, 4000 + K + variant)
@@ -155,7 +155,8 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
         check(gpu, variant, N, M, K, 700 + N + M + K + variant)
     gpu.force_tile(-1)
     # 12 ... 32 short lines beside 4096 ... 8191 lines under a K of 2048 or more: the 16 x 16 x 4 blocks' 32-line runs, cut
-    for (N, M, K) in ((16, 4100, 2052), (5000, 12, 4096), (8188, 32, 2048), (24, 8000, 2500), (2048, 16, 4100), (8, 3000, 2048), (28, 2100, 3000)):
+    for (N, M, K) in ((16, 4100, 2052), (5000, 12, 4096), (8188, 32, 2048), (24, 8000, 2500), (2048, 16, 4100), (8, 3000, 2048), (28, 2100, 3000),
+                      (8, 1024, 8192), (4, 512, 16384), (1000, 8, 4100), (260, 4, 9000), (8, 256, 20000)):
         check(gpu, variant, N, M, K, 800 + N + M + K + variant)
     rng = np.random.default_rng(31 + variant)
     A, B = logical_operands(variant, rng, 8, 4096, 4096)
