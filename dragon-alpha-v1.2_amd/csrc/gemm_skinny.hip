@@ -933,6 +933,9 @@ int gemm_choose_skinny(int rows, int cols, int nz, int k, int variant, int num_c
     if (t > 16 && k < 256) return -1;      // (16384 x 32 x 128: 8.1 us against the balanced kernel's 5.2)
     // (with a K of 2048 or more, which is cut across workgroups, from 8 lines per unit on: 2048 x 16 x 8192 16 - 17 us
     // against 25 - 26, 4096 x 32 x 8192 36 - 38 against 39 - 44)
+    // (and 12 or 16 short lines over any 256 lines or more under a K of 8192 or more, cut up to 16 times: 16 x 1024 x
+    // 65536 72 - 79 -> 46 - 49 us, 1024 x 16 x 8192 20 -> 10 - 12)
+    if (t <= 16 && k >= 8192) return TILE_SKINNY;
     return (long long)(thin_cols ? rows : cols) >= (k >= 2048 ? 8LL : t <= 16 ? 16LL : 32LL) * num_cu ? TILE_SKINNY : -1;
 }
 

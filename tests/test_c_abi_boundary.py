@@ -224,8 +224,9 @@ def test_tile_choice_on_the_documented_shapes(dh):
     # 20 ... 32: from 32 lines per unit and K = 256 on; under a K of 2048 or more (cut across workgroups) 12 ... 32 from 8
     for v in (NN, T1, T2):
         assert ct(v, 8192, 32, 1, 256) == 27 and ct(v, 8192, 32, 1, 252) != 27 and ct(v, 8188, 32, 1, 1024) != 27
-        assert ct(v, 2048, 32, 1, 2048) == 27 and ct(v, 16, 2048, 1, 8192) == 27 and ct(v, 2044, 12, 1, 8192) != 27
+        assert ct(v, 2048, 32, 1, 2048) == 27 and ct(v, 16, 2048, 1, 8192) == 27 and ct(v, 2044, 12, 1, 4096) != 27
         assert ct(v, 2048, 16, 1, 2044) != 27
+        assert ct(v, 256, 16, 1, 8192) == 27 and ct(v, 12, 1000, 1, 65536) == 27 and ct(v, 1024, 20, 1, 8192) != 27
     for v in (NN, T1, T2):
         assert ct(v, 65536, 36, 1, 1024) != 27 and ct(v, 65536, 20, 1, 1024) == 27 and ct(v, 4096, 20, 1, 1024) != 27 and ct(v, 65536, 4, 2, 1024) != 27 and ct(v, 252, 4, 1, 1024) != 27
     # 64x128 keeps its 16-k stages for A^T*B (both operands K-outer), takes 32-k stages otherwise

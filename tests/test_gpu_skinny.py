@@ -156,7 +156,7 @@ def test_few_lines_under_a_long_k_cut_across_workgroups(gpu, variant):
     gpu.force_tile(-1)
     # 12 ... 32 short lines beside 4096 ... 8191 lines under a K of 2048 or more: the 16 x 16 x 4 blocks' 32-line runs, cut
     for (N, M, K) in ((16, 4100, 2052), (5000, 12, 4096), (8188, 32, 2048), (24, 8000, 2500), (2048, 16, 4100), (8, 3000, 2048), (28, 2100, 3000),
-                      (8, 1024, 8192), (4, 512, 16384), (1000, 8, 4100), (260, 4, 9000), (8, 256, 20000)):
+                      (8, 1024, 8192), (4, 512, 16384), (1000, 8, 4100), (260, 4, 9000), (8, 256, 20000), (16, 1024, 8192), (300, 12, 9000)):
         check(gpu, variant, N, M, K, 800 + N + M + K + variant)
     rng = np.random.default_rng(31 + variant)
     A, B = logical_operands(variant, rng, 8, 4096, 4096)
