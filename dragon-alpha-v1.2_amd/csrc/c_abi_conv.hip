@@ -105,12 +105,20 @@ int conv_forward(const int64_t* streams, int length, int64_t dX, int IH, int IW,
     // faster (290 -> 276, 298 -> 267, 302 -> 263 us), level for a K below 768, and behind with 64 output
     // channels, where its 128 x 64 tiles lose to the paired tile-per-workgroup kernel (823 against 782 us on the
     // 7x7 layer).  gemm_launch_conv falls back where the stream has no workspace and may not make one.
-    if (free_choice && (IC & 31) == 0 && FH <= 32 && FW <= 32 &&
-        gemm_choose_streamk(p.rows, p.cols, 1, p.k_total, num_cu, GEMM_T2) == TILE_SK_128x128)
+    // Where the products' choice for this shape is one of the balanced kernel's smaller tiles (fewer 128 x 128 tiles
+    // than compute units: 128 images of 7 x 7 with 512 -> 512 channels, 196 tiles), that tile is taken as well from
+    // K = 768 on and more than 64 output channels: 298 -> 217 - 222 us on that layer.
+    const int sk = (free_choice && (IC & 31) == 0 && FH <= 32 && FW <= 32)
+                       ? gemm_choose_streamk(p.rows, p.cols, 1, p.k_total, num_cu, GEMM_T2) : -1;
+    const int sk_conv = sk == TILE_SK_128x64_O2 ? TILE_SK_128x64 : sk == TILE_SK_64x64_O2 ? TILE_SK_64x64 : sk;
+    if (sk == TILE_SK_128x128)
         tile = TILE_SK_128x128;
+    else if (OC > 64 && GK >= 768 && (sk_conv == TILE_SK_128x64 || sk_conv == TILE_SK_64x128 || sk_conv == TILE_SK_64x64))
+        tile = sk_conv;
     // ... and with up to 64 output channels the 256 x 64 shape of the same kernel, which has the 128 x 128 tile's
-    // ratio of matrix work to LDS traffic (the 7x7 layer of the reference's speed test: 784 -> 767 us)
-    else if (free_choice && (IC & 31) == 0 && FH <= 32 && FW <= 32 && OC <= 64 && OC > 32 && GK >= 768 &&
+    // ratio of matrix work to LDS traffic (the 7x7 layer of the reference's speed test: 784 -> 767 us; 3x3 layers
+    // with 64 -> 64 channels, K = 576: 139 -> 131 and 257 -> 241 us)
+    else if (free_choice && (IC & 31) == 0 && FH <= 32 && FW <= 32 && OC <= 64 && OC > 32 && GK >= 576 &&
              (GM + 255) / 256 >= num_cu && (GM + 255) / 256 <= 65536)
         tile = TILE_SK_256x64;
     return gemm_launch_conv(p, tile, (hipStream_t)(intptr_t)streams[0]);
